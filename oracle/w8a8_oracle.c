@@ -1,0 +1,386 @@
+/*
+ * CPU restatement of the reference's W8A8 linear arithmetic -- TEST
+ * INFRASTRUCTURE ONLY (see w8a8_oracle.h).  Plain scalar C, written to be
+ * obviously equal to the cited reference rule rather than fast.  Build with
+ * -ffp-contract=off: every f32 operation below is one IEEE rounding.
+ */
+#include "w8a8_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---- shared scalar helpers ------------------------------------------- */
+
+static int finite_f32(float v) {
+    uint32_t bits;
+    memcpy(&bits, &v, sizeof bits);
+    return ((bits >> 23) & 0xffu) != 0xffu;
+}
+
+static int scale_ok(float v) { return finite_f32(v) && v > 0.0f; }
+
+static int byte_dtype(uint32_t dtype) {
+    return dtype == VXO_DTYPE_I8 || dtype == VXO_DTYPE_U8;
+}
+
+static int zero_point_ok(int32_t zp, uint32_t dtype) {
+    if (dtype == VXO_DTYPE_I8) return zp >= -128 && zp <= 127;
+    if (dtype == VXO_DTYPE_U8) return zp >= 0 && zp <= 255;
+    return 0;
+}
+
+static int32_t load_byte(const void* p, uint32_t dtype, size_t i) {
+    return dtype == VXO_DTYPE_I8 ? (int32_t)((const int8_t*)p)[i]
+                                 : (int32_t)((const uint8_t*)p)[i];
+}
+
+static void store_byte(void* p, uint32_t dtype, size_t i, int32_t v) {
+    if (dtype == VXO_DTYPE_I8) ((int8_t*)p)[i] = (int8_t)v;
+    else ((uint8_t*)p)[i] = (uint8_t)v;
+}
+
+/* ---- w8a8_affine.h ---------------------------------------------------- */
+
+int32_t vxo_round_ties_even(float value) {
+    /* floor, then decide on the fractional part; exact ties go to even */
+    const float fl = floorf(value);
+    const int32_t lo = (int32_t)fl;
+    const float frac = value - (float)lo;
+    if (frac < 0.5f) return lo;
+    if (frac > 0.5f) return lo + 1;
+    return (lo % 2 == 0) ? lo : lo + 1;
+}
+
+int32_t vxo_requantize(float t, int32_t minimum, int32_t maximum,
+                       int32_t nan_value) {
+    if (t != t) return nan_value;
+    if (t <= (float)minimum) return minimum;
+    if (t >= (float)maximum) return maximum;
+    return vxo_round_ties_even(t);
+}
+
+float vxo_transform_accumulator(int64_t accumulator, float multiplier,
+                                int32_t output_zero_point) {
+    volatile float scaled = (float)accumulator * multiplier; /* rounding 1 */
+    volatile float shifted = scaled + (float)output_zero_point; /* rounding 2 */
+    return shifted;
+}
+
+int vxo_multiplier(float input_scale, float weight_scale, float output_scale,
+                   float* multiplier_out) {
+    volatile float product, multiplier;
+    if (!multiplier_out || !scale_ok(input_scale) || !scale_ok(weight_scale) ||
+        !scale_ok(output_scale))
+        return 0;
+    product = input_scale * weight_scale;   /* f32(s_x * s_w) */
+    multiplier = product / output_scale;    /* f32(. / s_y)   */
+    if (!scale_ok(multiplier)) return 0;
+    *multiplier_out = multiplier;
+    return 1;
+}
+
+/* ---- QLinear (requantizing epilogue) ---------------------------------- */
+
+int vxo_qlinear_i8u8(const void* input, const void* weight,
+                     const int32_t* bias, const float* weight_scales,
+                     const int32_t* weight_zero_points, void* output,
+                     int32_t* accumulators, uint32_t rows, uint32_t d_in,
+                     uint32_t d_out, float input_scale,
+                     int32_t input_zero_point, float output_scale,
+                     int32_t output_zero_point, uint32_t input_dtype,
+                     uint32_t weight_dtype, uint32_t output_dtype) {
+    if (!input || !weight || !bias || !weight_scales || !weight_zero_points ||
+        !output || !rows || !d_in || !d_out || !byte_dtype(input_dtype) ||
+        !byte_dtype(weight_dtype) || !byte_dtype(output_dtype) ||
+        !scale_ok(input_scale) || !scale_ok(output_scale) ||
+        !zero_point_ok(input_zero_point, input_dtype) ||
+        !zero_point_ok(output_zero_point, output_dtype))
+        return 0;
+    const int32_t lo = output_dtype == VXO_DTYPE_I8 ? -128 : 0;
+    const int32_t hi = output_dtype == VXO_DTYPE_I8 ? 127 : 255;
+    /* whole descriptor is validated before the first output byte */
+    for (uint32_t n = 0; n < d_out; n++) {
+        float m;
+        if (!zero_point_ok(weight_zero_points[n], weight_dtype) ||
+            !vxo_multiplier(input_scale, weight_scales[n], output_scale, &m))
+            return 0;
+    }
+    for (uint32_t r = 0; r < rows; r++) {
+        for (uint32_t n = 0; n < d_out; n++) {
+            int64_t acc = bias[n];
+            float mult;
+            vxo_multiplier(input_scale, weight_scales[n], output_scale, &mult);
+            for (uint32_t k = 0; k < d_in; k++) {
+                const int32_t x =
+                    load_byte(input, input_dtype, (size_t)r * d_in + k) -
+                    input_zero_point;
+                const int32_t w =
+                    load_byte(weight, weight_dtype, (size_t)n * d_in + k) -
+                    weight_zero_points[n];
+                acc += (int64_t)x * (int64_t)w;
+                /* every prefix must stay inside int32 */
+                if (acc < INT32_MIN || acc > INT32_MAX) return 0;
+            }
+            if (accumulators) accumulators[(size_t)r * d_out + n] = (int32_t)acc;
+            const float t =
+                vxo_transform_accumulator(acc, mult, output_zero_point);
+            store_byte(output, output_dtype, (size_t)r * d_out + n,
+                       vxo_requantize(t, lo, hi, output_zero_point));
+        }
+    }
+    return 1;
+}
+
+int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
+                              const int32_t* bias_i32, const float* bias_f32,
+                              const float* weight_scales,
+                              const int32_t* weight_zero_points, void* output,
+                              int32_t* accumulators, uint32_t rows,
+                              uint32_t d_in, uint32_t d_out,
+                              const float* row_scales, float output_scale,
+                              int32_t output_zero_point, uint32_t weight_dtype,
+                              uint32_t output_dtype) {
+    if (!input || !row_scales || !output || !rows || !d_out) return 0;
+    int32_t* row_bias = (int32_t*)calloc(d_out, sizeof *row_bias);
+    if (!row_bias) return 0;
+    const size_t out_stride = d_out; /* one byte per output element */
+    int ok = 1;
+    for (uint32_t r = 0; r < rows && ok; r++) {
+        if (bias_f32) {
+            ok = vxo_ptq_pack_bias_i32(bias_f32, (int32_t)d_out, row_scales[r],
+                                       weight_scales, row_bias) == 0;
+        } else if (bias_i32) {
+            memcpy(row_bias, bias_i32, d_out * sizeof *row_bias);
+        }
+        if (!ok) break;
+        ok = vxo_qlinear_i8u8(
+            input + (size_t)r * d_in, weight, row_bias, weight_scales,
+            weight_zero_points, (uint8_t*)output + (size_t)r * out_stride,
+            accumulators ? accumulators + (size_t)r * d_out : NULL, 1u, d_in,
+            d_out, row_scales[r], 0, output_scale, output_zero_point,
+            VXO_DTYPE_I8, weight_dtype, output_dtype);
+    }
+    free(row_bias);
+    return ok;
+}
+
+/* ---- PackedLinear W8 under DYNAMIC_I8 --------------------------------- */
+
+int32_t vxo_packed_round_i8(float value) {
+    if (value >= 127.0f) return 127;
+    if (value <= -127.0f) return -127;
+    int32_t q = (int32_t)value; /* toward zero */
+    const float rem = value - (float)q;
+    if (rem > 0.5f || (rem == 0.5f && (q & 1))) q++;
+    if (rem < -0.5f || (rem == -0.5f && (q & 1))) q--;
+    return q;
+}
+
+int vxo_packed_prepare_i8(const float* input, uint32_t k, int8_t* prepared,
+                          float* scale) {
+    float maximum = 0.0f;
+    int finite = 1;
+    for (uint32_t j = 0; j < k; j++) {
+        const float v = input[j];
+        if (!finite_f32(v)) { finite = 0; break; }
+        const float a = v < 0.0f ? -v : v;
+        if (a > maximum) maximum = a;
+    }
+    float s = maximum == 0.0f ? 1.0f : maximum / 127.0f;
+    if (s < 0x1p-126f) s = 0x1p-126f;
+    *scale = s;
+    if (!finite) {
+        memset(prepared, 0, k);
+        return 0;
+    }
+    for (uint32_t j = 0; j < k; j++) {
+        const float ratio = input[j] / s; /* true f32 division */
+        prepared[j] = (int8_t)vxo_packed_round_i8(ratio);
+    }
+    return 1;
+}
+
+static int group_size_ok(uint32_t g) {
+    return g == 32u || g == 64u || g == 128u || g == 256u;
+}
+
+static int32_t w8_code(const uint32_t* row_words, uint32_t k) {
+    return (int32_t)((row_words[k / 4u] >> ((k % 4u) * 8u)) & 255u) - 128;
+}
+
+int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
+                         const uint8_t* row_finite, const uint32_t* packed,
+                         const float* scales, const float* bias, float* output,
+                         int32_t* accumulators, uint64_t rows, uint32_t k,
+                         uint32_t n, uint32_t group_size) {
+    if (!activation || !row_scales || !packed || !scales || !output || !k ||
+        !n || !group_size_ok(group_size))
+        return -1;
+    const uint32_t words = (k + 3u) / 4u;
+    const uint32_t groups = (k + group_size - 1u) / group_size;
+    for (uint64_t r = 0; r < rows; r++) {
+        const int8_t* a = activation + r * k;
+        const float as = row_scales[r];
+        for (uint32_t o = 0; o < n; o++) {
+            if (row_finite && !row_finite[r]) {
+                output[r * n + o] = nanf("");
+                if (accumulators) accumulators[r * n + o] = 0;
+                continue;
+            }
+            const uint32_t* w = packed + (uint64_t)o * words;
+            float sum = 0.0f;
+            int64_t total = 0;
+            for (uint32_t g = 0; g < groups; g++) {
+                const uint32_t begin = g * group_size;
+                const uint32_t end = begin + group_size < k ? begin + group_size : k;
+                int32_t dot = 0;
+                for (uint32_t j = begin; j < end; j++)
+                    dot += (int32_t)a[j] * w8_code(w, j);
+                total += dot;
+                const float group_scale = as * scales[(uint64_t)o * groups + g];
+                const float term = (float)dot * group_scale;
+                sum = sum + term; /* ascending group order */
+            }
+            if (accumulators) accumulators[r * n + o] = (int32_t)total;
+            output[r * n + o] = sum + (bias ? bias[o] : 0.0f);
+        }
+    }
+    return 0;
+}
+
+int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
+                              const float* scales, const float* bias,
+                              float* output, uint64_t rows, uint32_t k,
+                              uint32_t n, uint32_t group_size) {
+    if (!input || !k || !n || !group_size_ok(group_size)) return -1;
+    int8_t* prepared = (int8_t*)malloc(k);
+    if (!prepared) return -1;
+    int status = 0;
+    for (uint64_t r = 0; r < rows && status == 0; r++) {
+        float as;
+        const uint8_t finite =
+            (uint8_t)vxo_packed_prepare_i8(input + r * k, k, prepared, &as);
+        status = vxo_packed_linear_a8(prepared, &as, &finite, packed, scales,
+                                      bias, output + r * n, NULL, 1u, k, n,
+                                      group_size);
+    }
+    free(prepared);
+    return status;
+}
+
+/* ---- Quantize / Dequantize boundaries --------------------------------- */
+
+int vxo_quantize_linear(const float* input, uint32_t elements, void* output,
+                        float scale, int32_t zero_point, uint32_t dtype) {
+    if (!input || !output || !byte_dtype(dtype) || !scale_ok(scale) ||
+        !zero_point_ok(zero_point, dtype))
+        return 0;
+    const int32_t lo = dtype == VXO_DTYPE_I8 ? -128 : 0;
+    const int32_t hi = dtype == VXO_DTYPE_I8 ? 127 : 255;
+    for (uint32_t i = 0; i < elements; i++) {
+        float v = input[i];
+        int32_t q;
+        if (v != v) {
+            q = zero_point;
+        } else {
+            const float ratio = v / scale;
+            v = ratio + (float)zero_point;
+            if (v <= (float)lo) q = lo;
+            else if (v >= (float)hi) q = hi;
+            else if (!finite_f32(v)) q = v < 0.0f ? lo : hi;
+            else q = vxo_round_ties_even(v);
+        }
+        store_byte(output, dtype, i, q);
+    }
+    return 1;
+}
+
+int vxo_dequantize_linear(const void* input, uint32_t elements, float scale,
+                          int32_t zero_point, uint32_t dtype, float* output) {
+    if (!input || !output || !byte_dtype(dtype)) return 0;
+    for (uint32_t i = 0; i < elements; i++) {
+        const double centered = (double)load_byte(input, dtype, i) - (double)zero_point;
+        output[i] = (float)(centered * (double)scale);
+    }
+    return 1;
+}
+
+/* ---- PTQ rules used to synthesise inputs ------------------------------ */
+
+static double round_ties_even_f64(double v) {
+    const double lo = floor(v);
+    const double frac = v - lo;
+    if (frac < 0.5) return lo;
+    if (frac > 0.5) return lo + 1.0;
+    return ((int64_t)lo % 2 == 0) ? lo : lo + 1.0;
+}
+
+int vxo_ptq_symmetric_scale(const float* values, int64_t count, float* scale) {
+    if (!values || count <= 0 || !scale) return -1;
+    double magnitude = 0.0;
+    for (int64_t i = 0; i < count; i++) {
+        if (!finite_f32(values[i])) return -1;
+        const double a = fabs((double)values[i]);
+        if (a > magnitude) magnitude = a;
+    }
+    const float s = (float)(magnitude == 0.0 ? 1.0 : magnitude / 127.0);
+    if (finite_f32(s) && s > 0.0f) { *scale = s; return 0; }
+    if (s == 0.0f) { *scale = 0x1p-126f; return 0; }
+    return -1;
+}
+
+int vxo_ptq_quantize_i8(const float* values, int64_t count, float scale,
+                        int32_t zero_point, int8_t* output) {
+    if (!values || !output || !scale_ok(scale) || zero_point < -128 ||
+        zero_point > 127)
+        return -1;
+    for (int64_t i = 0; i < count; i++) {
+        if (!finite_f32(values[i])) return -1;
+        double q = round_ties_even_f64((double)values[i] / (double)scale +
+                                       (double)zero_point);
+        if (q < -128.0) q = -128.0;
+        if (q > 127.0) q = 127.0;
+        output[i] = (int8_t)q;
+    }
+    return 0;
+}
+
+int vxo_ptq_pack_bias_i32(const float* values, int32_t count,
+                          float input_scale, const float* weight_scales,
+                          int32_t* output) {
+    if (count < 0 || (count > 0 && (!values || !weight_scales || !output)) ||
+        !scale_ok(input_scale))
+        return -1;
+    for (int pass = 0; pass < 2; pass++) {
+        for (int32_t i = 0; i < count; i++) {
+            if (!finite_f32(values[i]) || !scale_ok(weight_scales[i])) return -1;
+            const float acc_scale = input_scale * weight_scales[i];
+            if (!scale_ok(acc_scale)) return -1;
+            const float ratio = values[i] / acc_scale;
+            if (!finite_f32(ratio)) return -1;
+            const double q = round_ties_even_f64((double)ratio);
+            if (q < (double)INT32_MIN || q > (double)INT32_MAX) return -1;
+            if (pass) output[i] = (int32_t)q; /* nothing is written on failure */
+        }
+    }
+    return 0;
+}
+
+void vxo_pack_w8_words(const int8_t* weight, uint32_t n, uint32_t k,
+                       uint32_t* packed) {
+    const uint32_t words = (k + 3u) / 4u;
+    for (uint32_t o = 0; o < n; o++) {
+        for (uint32_t w = 0; w < words; w++) {
+            uint32_t word = 0;
+            for (uint32_t b = 0; b < 4u; b++) {
+                const uint32_t j = w * 4u + b;
+                /* a code of 128 is the value zero, which pads the tail */
+                const uint32_t code =
+                    j < k ? (uint32_t)((int32_t)weight[(uint64_t)o * k + j] + 128) : 128u;
+                word |= code << (8u * b);
+            }
+            packed[(uint64_t)o * words + w] = word;
+        }
+    }
+}

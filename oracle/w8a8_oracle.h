@@ -1,0 +1,126 @@
+/*
+ * CPU restatement of the reference's W8A8 linear arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library links, loads or
+ * calls this file; it exists so the HIP path can be checked against an
+ * independent scalar statement of the reference contract, and so a CPU
+ * baseline can be timed next to the GPU.  Each function names the reference
+ * file:line it restates (paths relative to the reference tree's native/).
+ *
+ * Parity status: every function below is pinned by the reference's own
+ * known-answer vectors (tests/golden/reference_kats.json) and, where the
+ * reference tree is available, by a byte comparison against the reference C
+ * compiled from its own sources (oracle/_ref).  The one exception is
+ * vxo_qlinear_rowscale_i8u8's f32-bias fold, which composes two pinned
+ * reference rules (the PTQ bias rule and the per-row QLinear call) into a
+ * form the reference does not ship as a single function; that composition
+ * is an extension and is labelled so where it is used.
+ */
+#ifndef VXO_W8A8_ORACLE_H
+#define VXO_W8A8_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Canonical dtype ids (include/volvoxai_enums.h:479-480). */
+#define VXO_DTYPE_U8 5u
+#define VXO_DTYPE_I8 6u
+
+/* src/kernels/w8a8_affine.h:114-120 */
+int32_t vxo_round_ties_even(float value);
+/* src/kernels/w8a8_affine.h:125-131 */
+int32_t vxo_requantize(float transformed, int32_t minimum, int32_t maximum,
+                       int32_t nan_value);
+/* src/kernels/w8a8_affine.h:139-144 */
+float vxo_transform_accumulator(int64_t accumulator, float multiplier,
+                                int32_t output_zero_point);
+/* src/kernels/w8a8_affine.h:169-181 and src/backends/qlinear_multiplier.h:12-27 */
+int vxo_multiplier(float input_scale, float weight_scale, float output_scale,
+                   float* multiplier_out);
+
+/* src/kernels/portable_inference_kernels.inc:968-1032.  Returns 1 handled,
+ * 0 declined.  `accumulators`, when non-NULL, receives the int32 accumulator
+ * (bias included) of every output element, row-major [rows, d_out]. */
+int vxo_qlinear_i8u8(const void* input, const void* weight,
+                     const int32_t* bias, const float* weight_scales,
+                     const int32_t* weight_zero_points, void* output,
+                     int32_t* accumulators, uint32_t rows, uint32_t d_in,
+                     uint32_t d_out, float input_scale,
+                     int32_t input_zero_point, float output_scale,
+                     int32_t output_zero_point, uint32_t input_dtype,
+                     uint32_t weight_dtype, uint32_t output_dtype);
+
+/* Per-token activation scales: row m is its own reference QLinear call with
+ * input_scale = row_scales[m] (portable_inference_kernels.inc:968-1032 called
+ * with rows = 1).  When bias_f32 is non-NULL the row's int32 bias is produced
+ * by the PTQ rule b_q = rne(f32(b / f32(s_m * s_w[n])))
+ * (src/training/quantization.c:391-414); otherwise bias_i32 (may be NULL = 0)
+ * is used as is.  Input zero point is 0 and input dtype I8. */
+int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
+                              const int32_t* bias_i32, const float* bias_f32,
+                              const float* weight_scales,
+                              const int32_t* weight_zero_points, void* output,
+                              int32_t* accumulators, uint32_t rows,
+                              uint32_t d_in, uint32_t d_out,
+                              const float* row_scales, float output_scale,
+                              int32_t output_zero_point, uint32_t weight_dtype,
+                              uint32_t output_dtype);
+
+/* src/kernels/packed_linear.h:108-116 */
+int32_t vxo_packed_round_i8(float value);
+/* Activation preparation of PackedLinear under DYNAMIC_I8
+ * (src/kernels/packed_linear_ops.inc:1574-1597, 97-153).  Returns the
+ * "finite" flag; on a non-finite row `prepared` is zeroed. */
+int vxo_packed_prepare_i8(const float* input, uint32_t k, int8_t* prepared,
+                          float* scale);
+
+/* PackedLinear W8 / DYNAMIC_I8 (src/kernels/packed_linear_ops.inc:1545-1621,
+ * row body :1493-1534).  packed: offset-binary I32 words [n, ceil(k/4)],
+ * scales [n, ceil(k/group)], bias [n] or NULL, output [rows, n].
+ * Returns 0 on success, -1 on a rejected descriptor (reference convention). */
+int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
+                              const float* scales, const float* bias,
+                              float* output, uint64_t rows, uint32_t k,
+                              uint32_t n, uint32_t group_size);
+
+/* Same arithmetic with the activation codes and per-row scales injected
+ * (the "prepared A8" form the reference's CUDA route keeps in x[4]/x[5],
+ * src/kernels/llm_ops.h:30-32).  row_finite may be NULL (all rows finite).
+ * group_dots, when non-NULL, receives nothing; accumulators (optional)
+ * receives the full-K int32 sum of the group dots, [rows, n]. */
+int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
+                         const uint8_t* row_finite, const uint32_t* packed,
+                         const float* scales, const float* bias, float* output,
+                         int32_t* accumulators, uint64_t rows, uint32_t k,
+                         uint32_t n, uint32_t group_size);
+
+/* src/kernels/quantize_linear_ops.inc:156-169 (scalar rule), :234-254 */
+int vxo_quantize_linear(const float* input, uint32_t elements, void* output,
+                        float scale, int32_t zero_point, uint32_t dtype);
+/* src/kernels/quantize_linear_ops.inc:9-16, :95-128 */
+int vxo_dequantize_linear(const void* input, uint32_t elements, float scale,
+                          int32_t zero_point, uint32_t dtype, float* output);
+
+/* src/training/quantization.c:142-160: symmetric per-tensor activation scale
+ * s = f32(max|x| / 127.0) computed in double; 1.0 for an all-zero tensor. */
+int vxo_ptq_symmetric_scale(const float* values, int64_t count, float* scale);
+/* src/training/quantization.c:186-211: q = clamp(rne(x / s + zp)) in double. */
+int vxo_ptq_quantize_i8(const float* values, int64_t count, float scale,
+                        int32_t zero_point, int8_t* output);
+/* src/training/quantization.c:391-414 */
+int vxo_ptq_pack_bias_i32(const float* values, int32_t count,
+                          float input_scale, const float* weight_scales,
+                          int32_t* output);
+
+/* docs/packed-linear-design.md:24-28: offset-binary W8 codes, LSB first. */
+void vxo_pack_w8_words(const int8_t* weight, uint32_t n, uint32_t k,
+                       uint32_t* packed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
