@@ -1,0 +1,257 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 linear hot path on one MI355X.
+
+A "step" is one W8A8 linear over one batch of synthetic, HBM-resident input:
+
+  headline  M=K=N=4096 prefill GEMM (BASELINE config 3): int8 A x prepacked
+            int8 B, int32 accumulation, per-token x per-channel scale, f32
+            bias, requantization to int8 at output scale 0.05 (ties to even).
+            Reported as int8 TOPS and as a fraction of the int8 MFMA peak.
+  gemv      M=1, K=4096, N=14336 decode GEMV (BASELINE config 2): dequant +
+            bias to f32.  Reported as GB/s of algorithmic bytes and as a
+            fraction of HBM peak, rotating over enough weight copies that the
+            256 MB Infinity Cache cannot serve them.
+
+Prints ONE JSON line.  The CPU column times the reference's own native CPU
+route (oracle/_ref, compiled from the reference sources) on the host cores
+with a bounded sample; it is a reported baseline, never part of the GPU path.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+METRIC = "W8A8 linear int8 TOPS (%MFMA peak) at 4096³; GB/s (%HBM) at M=1"
+PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, MI355X
+PEAK_HBM_GBS = 8000.0     # HBM3E, MI355X
+
+
+def gemv_algorithmic_bytes(m, k, n):
+    # weights once + activations + per-channel scales + bias + per-token scales + f32 output
+    return n * k + m * k + 4 * n + 4 * n + 4 * m + 4 * m * n
+
+
+def time_events(fn, steps, torch):
+    """Average device time of fn() in ms from one event pair per launch."""
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        starts[i].record()
+        fn(i)
+        stops[i].record()
+    torch.cuda.synchronize()
+    t = np.array([s.elapsed_time(e) for s, e in zip(starts, stops)])
+    return float(t.mean()), float(np.median(t)), float(t.min())
+
+
+def cpu_baseline_gemm(sample_rows, k, n, seed):
+    """Reference native CPU route (policy-selected packed or raw kernel) on a row
+    sample of the headline workload, one input scale (the reference has no
+    per-token form)."""
+    from oracle.pyoracle import Reference, Oracle, DTYPE_I8
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-127, 128, (sample_rows, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    sw = (rng.uniform(0.002, 0.01, n) / np.sqrt(k) * 4).astype(np.float32)
+    zps = np.zeros(n, np.int32)
+    bias = np.zeros(n, np.int32)
+    args = (0.03, 0, 0.05, 0, DTYPE_I8, DTYPE_I8, DTYPE_I8)
+    if Reference.available():
+        ref = Reference()
+        threads = ref.enter_pool(cores)
+        packed_route = ref.packed_preferred(sample_rows, k, n, DTYPE_I8, True)
+        packed = ref.pack_q8(w, DTYPE_I8) if packed_route else None
+        call = (lambda: ref.qlinear_packed(x, packed, bias, sw, zps, *args)) if packed_route else \
+               (lambda: ref.qlinear_native(x, w, bias, sw, zps, *args))
+        call()
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 5.0 or reps < 2:
+            ok, _ = call()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        ref.leave_pool()
+        kind = "reference"
+        route = "vx_qlinear_i8u8_packed" if packed_route else "vx_qlinear_i8u8_native"
+    else:
+        orc = Oracle()
+        threads = 1
+        t0 = time.perf_counter()
+        ok, _ = orc.qlinear(x[:8], w, bias, sw, zps, *args)
+        dt = (time.perf_counter() - t0) * sample_rows / 8
+        kind, route = "port", "vxo_qlinear_i8u8 (scalar restatement, 8 rows scaled)"
+    assert ok == 1
+    tops = 2.0 * sample_rows * k * n / dt / 1e12
+    return {"value": tops, "unit": "TOPS", "cores": threads, "kind": kind,
+            "sample": f"{route}, first {sample_rows} of 4096 rows at K=N=4096, one input scale, "
+                      f"{dt * 1e3:.1f} ms per call"}
+
+
+def cpu_baseline_gemv(k, n, seed):
+    from oracle.pyoracle import Reference, Oracle
+    import _cases as cases
+    c = cases.decode_case(1, k, n, 128, seed)
+    orc = Oracle()
+    words = orc.pack_w8_words(c["w"])
+    x = (c["a8"].astype(np.float32) * c["row_scales"][:, None]).astype(np.float32)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    if Reference.available():
+        ref = Reference()
+        threads = ref.enter_pool(cores)
+        call = lambda: ref.packed_linear(x, words, c["scales"], c["bias"], n, 128)
+        kind, route = "reference", "vx_llm_forward_f32 (PackedLinear, DYNAMIC_I8)"
+    else:
+        ref, threads = None, 1
+        call = lambda: orc.packed_linear(x, words, c["scales"], c["bias"], n, 128)
+        kind, route = "port", "vxo_packed_linear_forward"
+    call()
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 3.0 or reps < 2:
+        st, _ = call()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    if ref:
+        ref.leave_pool()
+    return {"value": gemv_algorithmic_bytes(1, k, n) / dt / 1e9, "unit": "GB/s", "cores": threads,
+            "kind": kind, "sample": f"{route}, M=1 K={k} N={n} full size, {dt * 1e3:.2f} ms per call"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["gemm", "gemv"], default=None,
+                    help="run one leg only (for profiling a single kernel)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (one kernel on one GPU's share of the "
+                 "work); --gpus N with N > 1 is not supported.")
+
+    import torch
+    import volvoxai_amd as vx
+    import _cases as cases
+    from oracle.pyoracle import Oracle
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    ctx = vx.Context(0, torch.cuda.current_stream())
+    out = {"metric": METRIC, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+           "data": "synthetic (seeded; random-init weights)"}
+
+    # ---- headline: 4096^3 prefill GEMM ------------------------------------------
+    if args.only in (None, "gemm"):
+        M = K = N = 4096
+        c = cases.rowscale_case(M, K, N, 4096)
+        lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, vx.DTYPE_I8)
+        xd = torch.from_numpy(c["x"]).cuda()
+        rs = torch.from_numpy(c["row_scales"]).cuda()
+        bd = torch.from_numpy(c["bias_f32"]).cuda()
+        yd = torch.empty((M, N), dtype=torch.int8, device="cuda")
+
+        def step(_i=0):
+            ok, _ = lin.forward_rowscale(ctx, xd, rs, c["s_out"], 0, bias_f32=bd, out=yd)
+            assert ok == 1, vx.library().vxhip_last_error()
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        mean_ms, med_ms, min_ms = time_events(step, args.steps, torch)
+        ops = 2.0 * M * K * N
+        out.update(value=ops / (wall_ms * 1e-3) / 1e12, ms_per_step=wall_ms,
+                   config={"workload": "configs[2]: prefill GEMM M=K=N=4096, int8 x int8 -> int32, per-token x "
+                                       "per-channel scale + f32 bias, requant to int8 (scale 0.05, ties-even)",
+                           "M": M, "K": K, "N": N, "variant": ctx.last_variant})
+        out["roofline"] = {"bound": "mfma", "achieved": ops / (mean_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS,
+                           "unit": "TFLOP/s", "frac": ops / (mean_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                           "traffic": None, "kernel": ctx.last_variant, "ops_per_launch": ops,
+                           "avg_kernel_ms": mean_ms, "median_kernel_ms": med_ms, "min_kernel_ms": min_ms,
+                           "note": "int8 TOP/s against the 5.0 POP/s dense int8 MFMA peak"}
+        # spot parity on the benchmarked output itself
+        orc = Oracle()
+        ridx, cidx = np.arange(0, M, 257)[:12], np.arange(3, N, 131)[:24]
+        ok2, want, _ = orc.qlinear_rowscale(c["x"][ridx], c["w"][cidx], c["scales"][cidx], c["zps"][cidx],
+                                            c["row_scales"][ridx], c["s_out"], 0, bias_f32=c["bias_f32"][cidx])
+        got = yd.cpu().numpy()[np.ix_(ridx, cidx)]
+        out["parity_spot_check"] = bool(ok2 == 1 and (got == want).all())
+        lin.close()
+        del xd, yd
+
+    # ---- decode GEMV: M=1, K=4096, N=14336 -------------------------------------
+    if args.only in (None, "gemv"):
+        Mg, Kg, Ng, G = 1, 4096, 14336, 128
+        d = cases.decode_case(Mg, Kg, Ng, G, 14336)
+        orc = Oracle()
+        words = orc.pack_w8_words(d["w"])
+        copies = 6  # 6 x 56 MiB > 256 MB Infinity Cache
+        pls = [vx.PackedLinear(words, d["scales"], d["bias"], Kg, Ng, G) for _ in range(copies)]
+        a8 = torch.from_numpy(d["a8"]).cuda()
+        ars = torch.from_numpy(d["row_scales"]).cuda()
+        yg = torch.empty((Mg, Ng), dtype=torch.float32, device="cuda")
+
+        def gstep(i=0):
+            st, _ = pls[i % copies].forward_a8(ctx, a8, ars, out=yg)
+            assert st == 0, vx.library().vxhip_last_error()
+
+        def gstep_hot(_i=0):
+            gstep(0)
+
+        for i in range(args.warmup):
+            gstep(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            gstep(i)
+        torch.cuda.synchronize()
+        gwall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        gmean, gmed, gmin = time_events(gstep, args.steps, torch)
+        hmean, hmed, hmin = time_events(gstep_hot, args.steps, torch)
+        gb = gemv_algorithmic_bytes(Mg, Kg, Ng)
+        _, want, _ = orc.packed_linear_a8(d["a8"], d["row_scales"], words, d["scales"], d["bias"], Ng, G)
+        out["gemv"] = {"workload": "configs[1]: decode GEMV M=1, K=4096, N=14336, dequant + bias to f32",
+                       "value": gb / (gwall_ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": gwall_ms,
+                       "variant": ctx.last_variant, "weight_copies_rotated": copies,
+                       "hot_in_cache_GBs": gb / (hmean * 1e-3) / 1e9,
+                       "parity_bit_exact": bool((yg.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all())}
+        out["roofline_gemv"] = {"bound": "hbm", "achieved": gb / (gmean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                                "unit": "GB/s", "frac": gb / (gmean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                                "kernel": ctx.last_variant, "bytes_per_launch": gb, "avg_kernel_ms": gmean,
+                                "median_kernel_ms": gmed, "min_kernel_ms": gmin}
+        if args.only == "gemv":
+            out.update(value=out["gemv"]["value"], unit="GB/s", ms_per_step=gwall_ms,
+                       config={"workload": out["gemv"]["workload"]}, roofline=out["roofline_gemv"])
+        for p in pls:
+            p.close()
+
+    if not args.no_cpu_baseline:
+        if args.only in (None, "gemm"):
+            out["cpu_baseline"] = cpu_baseline_gemm(256, 4096, 4096, 7)
+        if args.only in (None, "gemv"):
+            out["cpu_baseline_gemv"] = cpu_baseline_gemv(4096, 14336, 8)
+            if args.only == "gemv":
+                out["cpu_baseline"] = out["cpu_baseline_gemv"]
+    ctx.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,250 @@
+/*
+ * vxhip_w8a8 -- MI355X (gfx950) W8A8 linear backend, C ABI.
+ *
+ * Plain C, no HIP types: every pointer is either a host pointer or an opaque
+ * device address (void*), every handle is an opaque struct.  A C host (the
+ * backend provider in volvoxai_amd/provider/) or any FFI can bind this header
+ * directly.  File:line citations name the reference interface each entry
+ * point stands in for (paths relative to the reference's native/ directory).
+ *
+ * Return convention: functions that mirror a reference kernel slot keep that
+ * slot's convention (1 = handled, 0 = declined before any side effect, exactly
+ * like VxQLinearI8U8Fn).  All other entry points return a VxHipStatus whose
+ * values equal the reference's VxStatus codes (include/volvoxai_enums.h:264-288)
+ * so a provider can return them unchanged.  vxhip_last_error() gives the
+ * calling thread's last failure text.
+ *
+ * Scopes follow the provider contract (docs/backend-sdk.md:77-95):
+ *   VxHipQLinear / VxHipPackedLinear  compiled scope, immutable after create,
+ *                                     shareable by concurrent contexts;
+ *   VxHipContext                      context scope, owns a stream and the
+ *                                     mutable scratch; one thread at a time.
+ */
+#ifndef VXHIP_W8A8_H
+#define VXHIP_W8A8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VXHIP_ABI_VERSION 1u
+
+/* Canonical dtype ids (include/volvoxai_enums.h:479-480). */
+#define VXHIP_DTYPE_U8 5u
+#define VXHIP_DTYPE_I8 6u
+
+typedef int32_t VxHipStatus;
+#define VXHIP_OK                     0
+#define VXHIP_INVALID_ARGUMENT      (-1)
+#define VXHIP_OUT_OF_MEMORY         (-2)
+#define VXHIP_BACKEND_UNAVAILABLE   (-6)
+#define VXHIP_BACKEND_UNSUPPORTED   (-7)
+#define VXHIP_EXECUTION_FAILED      (-10)
+#define VXHIP_DEVICE_LOST           (-12)
+#define VXHIP_INTERNAL              (-16)
+
+typedef struct VxHipContext VxHipContext;
+typedef struct VxHipQLinear VxHipQLinear;
+typedef struct VxHipPackedLinear VxHipPackedLinear;
+
+/* ---- library / device ------------------------------------------------- */
+
+uint32_t vxhip_abi_version(void);
+/* Number of visible gfx950 devices; 0 when none (a provider then answers
+ * BACKEND_UNAVAILABLE from runtime_create, runtime/backend_sdk.c:206-213). */
+int32_t vxhip_device_count(void);
+/* "AMD Instinct MI355X (gfx950), 256 CU, ..." into buffer; VXHIP_OK or error. */
+VxHipStatus vxhip_device_name(int32_t device, char* buffer, size_t capacity);
+const char* vxhip_last_error(void);
+
+/* ---- context scope ---------------------------------------------------- */
+
+/* stream: an existing hipStream_t passed as void* (work is enqueued there and
+ * the caller owns synchronisation), or NULL for a context-owned stream. */
+VxHipStatus vxhip_context_create(int32_t device, void* stream,
+                                 VxHipContext** out_context);
+void vxhip_context_destroy(VxHipContext* context);
+VxHipStatus vxhip_context_synchronize(VxHipContext* context);
+/* Kernel-variant id chosen by the last launch on this context, e.g.
+ * "hip.qlinear.mfma-i8.t256x256" -- the string a provider reports as
+ * route_evidence (runtime/public_api_model_lifecycle.inc:748-751). */
+const char* vxhip_context_last_variant(const VxHipContext* context);
+/* Device-side fault word accumulated by kernels (non-finite multiplier seen,
+ * ...); reading it synchronises the stream.  0 = clean. */
+VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
+
+/* Device memory for hosts without HIP headers. */
+VxHipStatus vxhip_device_malloc(size_t bytes, void** out_device_pointer);
+void vxhip_device_free(void* device_pointer);
+VxHipStatus vxhip_memcpy_to_device(VxHipContext* context, void* device_dst,
+                                   const void* host_src, size_t bytes);
+VxHipStatus vxhip_memcpy_to_host(VxHipContext* context, void* host_dst,
+                                 const void* device_src, size_t bytes);
+
+/* ---- QLinear / QMatMul / QGemm: requantizing epilogue ------------------ */
+
+/* Weight prepack = the reference's vx_pack_q8_weight step
+ * (src/kernels/packed_quant_gemm.c:237-392), redone for the int8 MFMA operand
+ * layout.  All pointers are HOST pointers and are not retained.
+ *   weight  [d_out, d_in] I8/U8 row-major, weight_scales/zero_points [d_out],
+ *   bias    [d_out] int32 in the accumulator domain (may be NULL = 0). */
+VxHipStatus vxhip_qlinear_create(const void* weight, const float* weight_scales,
+                                 const int32_t* weight_zero_points,
+                                 const int32_t* bias, uint32_t d_in,
+                                 uint32_t d_out, uint32_t weight_dtype,
+                                 VxHipQLinear** out_linear);
+void vxhip_qlinear_destroy(VxHipQLinear* linear);
+/* Bytes of device memory held by the compiled weight (attestation input). */
+uint64_t vxhip_qlinear_resident_bytes(const VxHipQLinear* linear);
+
+/* Canonical QLinear on resident buffers (the resident half of
+ * cuda_graph_qlinear_i8u8, src/backends/cuda/host/
+ * cuda_graph_quantized_linear_conv_host.inc:19-106; arithmetic of
+ * qlinear_i8u8, src/kernels/portable_inference_kernels.inc:968-1032).
+ * input_dev [rows,d_in], output_dev [rows,d_out] device pointers;
+ * accumulators_dev optional int32 [rows,d_out] (bias included).
+ * Asynchronous on the context stream.  Returns 1 handled / 0 declined. */
+int vxhip_qlinear_forward(VxHipContext* context, const VxHipQLinear* linear,
+                          const void* input_dev, void* output_dev,
+                          int32_t* accumulators_dev, uint32_t rows,
+                          float input_scale, int32_t input_zero_point,
+                          float output_scale, int32_t output_zero_point,
+                          uint32_t input_dtype, uint32_t output_dtype);
+
+/* Per-token activation scales: row m behaves as its own canonical QLinear
+ * call with input_scale = row_scales_dev[m], input zero point 0, I8 input.
+ * bias_f32_dev (optional, [d_out]) is an extension with no reference
+ * counterpart: f32(bias/output_scale) is added to the transformed value
+ * before the saturating round; with it NULL the bytes equal the reference's.
+ * Returns 1 handled / 0 declined. */
+int vxhip_qlinear_forward_rowscale(VxHipContext* context,
+                                   const VxHipQLinear* linear,
+                                   const int8_t* input_dev,
+                                   const float* row_scales_dev,
+                                   const float* bias_f32_dev, void* output_dev,
+                                   int32_t* accumulators_dev, uint32_t rows,
+                                   float output_scale,
+                                   int32_t output_zero_point,
+                                   uint32_t output_dtype);
+
+/* Drop-in for the VxW8A8Ops.qlinear_i8u8 slot: identical argument order and
+ * meaning to VxQLinearI8U8Fn (src/backends/w8a8_device_ops.h:15-17), HOST
+ * pointers, synchronous.  Packs, uploads, runs and downloads on device 0.
+ * Returns 1 handled / 0 declined before any side effect. */
+int vxhip_qlinear_i8u8(const void* input, const void* weight,
+                       const float* weight_scales,
+                       const int32_t* weight_zero_points, const int32_t* bias,
+                       void* output, uint32_t rows, uint32_t d_in,
+                       uint32_t d_out, float input_scale,
+                       int32_t input_zero_point, float output_scale,
+                       int32_t output_zero_point, uint32_t input_dtype,
+                       uint32_t weight_dtype, uint32_t output_dtype);
+
+/* ---- PackedLinear W8 under DYNAMIC_I8: dequant + bias to f32 ----------- */
+
+/* packed_words [n, ceil(k/4)] offset-binary I32 words, scales [n, ceil(k/G)],
+ * bias [n] or NULL, group_size in {32,64,128,256}, weight_bits must be 8
+ * (docs/packed-linear-design.md:24-32; physical shapes as checked at
+ * src/runtime/engine_runtime_llm.inc:94-99).  HOST pointers, not retained. */
+VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words,
+                                       const float* scales, const float* bias,
+                                       uint32_t k, uint32_t n,
+                                       uint32_t group_size,
+                                       uint32_t weight_bits,
+                                       VxHipPackedLinear** out_linear);
+void vxhip_packed_linear_destroy(VxHipPackedLinear* linear);
+uint64_t vxhip_packed_linear_resident_bytes(const VxHipPackedLinear* linear);
+
+/* Activation preparation (vx_packed_prepare_i8_*, src/kernels/
+ * packed_linear_ops.inc:97-217; CUDA twin vx_packed_cuda_prepare,
+ * src/backends/cuda/kernels/cuda_forward_llm_kernels.inc:195-252):
+ * per-row absmax scale, round-half-even codes clamped to +-127, non-finite
+ * rows flagged by a NaN scale.  Device pointers; asynchronous. */
+VxHipStatus vxhip_packed_prepare_i8(VxHipContext* context,
+                                    const float* input_dev, uint32_t rows,
+                                    uint32_t k, int8_t* prepared_dev,
+                                    float* row_scales_dev);
+
+/* vx_packed_linear_forward with normalize==8, groups==8
+ * (src/kernels/packed_linear_ops.inc:1545-1621) on resident f32 rows.
+ * Returns 0 on success, -1 on a rejected descriptor (reference convention). */
+int vxhip_packed_linear_forward_f32(VxHipContext* context,
+                                    const VxHipPackedLinear* linear,
+                                    const float* input_dev, float* output_dev,
+                                    uint32_t rows);
+
+/* Same arithmetic from already prepared activations (the x[4]/x[5] form of
+ * src/kernels/llm_ops.h:30-32): int8 codes [rows,k] and one f32 scale per
+ * row; a NaN scale marks a non-finite row (whole output row NaN).
+ * accumulators_dev optional int32 [rows,n] = full-K sum of the group dots. */
+int vxhip_packed_linear_forward_a8(VxHipContext* context,
+                                   const VxHipPackedLinear* linear,
+                                   const int8_t* activation_dev,
+                                   const float* row_scales_dev,
+                                   float* output_dev,
+                                   int32_t* accumulators_dev, uint32_t rows);
+
+/* Field-for-field layout of the PackedLinear part of VxLLMOpArgs
+ * (src/kernels/llm_ops.h:38-53) is not reproduced here; this one-shot HOST
+ * entry takes the same values as plain arguments: x=input f32 [rows,k],
+ * packed_weight, scale, bias (optional), y=out [rows,n], key_dim=k,
+ * value_dim=n, rate=group_size, groups=weight_bits, normalize=8.
+ * Returns 0 / -1 like vx_llm_forward_f32 (src/kernels/llm_ops.inc:41-56). */
+int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
+                            const float* scale, const float* bias,
+                            float* output, uint64_t rows, int32_t key_dim,
+                            int32_t value_dim, int32_t rate, int32_t groups,
+                            int32_t normalize);
+
+/* ---- F32 <-> byte boundaries ------------------------------------------ */
+
+/* VxQuantizeTypedI8U8Fn / VxDequantizeTypedI8U8Fn slots
+ * (src/backends/w8a8_device_ops.h:31-32); arithmetic of
+ * quantize_linear_typed / dequantize_linear_typed
+ * (src/kernels/quantize_linear_ops.inc:234-254, 95-128).  HOST pointers,
+ * synchronous, 1 handled / 0 declined. */
+int vxhip_quantize_typed_f32_i8u8(const float* input, uint32_t elements,
+                                  void* output, float scale,
+                                  int32_t zero_point, uint32_t output_dtype);
+int vxhip_dequantize_typed_i8u8_f32(const void* input, uint32_t elements,
+                                    float scale, int32_t zero_point,
+                                    uint32_t input_dtype, float* output);
+/* Resident forms (device pointers, asynchronous on the context stream). */
+int vxhip_quantize_forward(VxHipContext* context, const float* input_dev,
+                           uint32_t elements, void* output_dev, float scale,
+                           int32_t zero_point, uint32_t output_dtype);
+int vxhip_dequantize_forward(VxHipContext* context, const void* input_dev,
+                             uint32_t elements, float scale,
+                             int32_t zero_point, uint32_t input_dtype,
+                             float* output_dev);
+
+/* ---- kernel-variant table --------------------------------------------- */
+
+/* Same record shape as VxKernelVariantRegistration
+ * (src/generated/kernel_registry.h:75-82).  `backend` is 0
+ * (VX_BACKEND_KIND_UNSPECIFIED): an external provider has no built-in kind
+ * (tests/test_kernel_registry.c:60). */
+typedef struct VxHipKernelVariant {
+    const char* id;
+    int32_t backend;
+    int32_t operator_kind;
+    const char* entrypoint_id;
+    const char* predicate_id;
+    const char* required_features;
+    int32_t priority;
+} VxHipKernelVariant;
+
+const VxHipKernelVariant* vxhip_kernel_variants(size_t* out_count);
+
+/* Tuning/diagnostic override: force a variant family by id prefix for the
+ * calling thread's later launches ("" or NULL restores automatic choice).
+ * A forced variant that cannot run the shape makes the launch decline. */
+void vxhip_force_variant(const char* id_prefix);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VXHIP_W8A8_H */

@@ -141,28 +141,49 @@ int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
                               const float* row_scales, float output_scale,
                               int32_t output_zero_point, uint32_t weight_dtype,
                               uint32_t output_dtype) {
-    if (!input || !row_scales || !output || !rows || !d_out) return 0;
-    int32_t* row_bias = (int32_t*)calloc(d_out, sizeof *row_bias);
-    if (!row_bias) return 0;
-    const size_t out_stride = d_out; /* one byte per output element */
-    int ok = 1;
-    for (uint32_t r = 0; r < rows && ok; r++) {
-        if (bias_f32) {
-            ok = vxo_ptq_pack_bias_i32(bias_f32, (int32_t)d_out, row_scales[r],
-                                       weight_scales, row_bias) == 0;
-        } else if (bias_i32) {
-            memcpy(row_bias, bias_i32, d_out * sizeof *row_bias);
+    if (!input || !weight || !weight_scales || !weight_zero_points ||
+        !row_scales || !output || !rows || !d_in || !d_out ||
+        !byte_dtype(weight_dtype) || !byte_dtype(output_dtype) ||
+        !scale_ok(output_scale) ||
+        !zero_point_ok(output_zero_point, output_dtype))
+        return 0;
+    const int32_t lo = output_dtype == VXO_DTYPE_I8 ? -128 : 0;
+    const int32_t hi = output_dtype == VXO_DTYPE_I8 ? 127 : 255;
+    for (uint32_t r = 0; r < rows; r++)
+        for (uint32_t n = 0; n < d_out; n++) {
+            float m;
+            if (!zero_point_ok(weight_zero_points[n], weight_dtype) ||
+                !vxo_multiplier(row_scales[r], weight_scales[n], output_scale, &m))
+                return 0;
         }
-        if (!ok) break;
-        ok = vxo_qlinear_i8u8(
-            input + (size_t)r * d_in, weight, row_bias, weight_scales,
-            weight_zero_points, (uint8_t*)output + (size_t)r * out_stride,
-            accumulators ? accumulators + (size_t)r * d_out : NULL, 1u, d_in,
-            d_out, row_scales[r], 0, output_scale, output_zero_point,
-            VXO_DTYPE_I8, weight_dtype, output_dtype);
+    for (uint32_t r = 0; r < rows; r++) {
+        for (uint32_t n = 0; n < d_out; n++) {
+            /* the reference loop with rows = 1 and input_scale = row_scales[r] */
+            int64_t acc = bias_i32 ? bias_i32[n] : 0;
+            float mult;
+            vxo_multiplier(row_scales[r], weight_scales[n], output_scale, &mult);
+            for (uint32_t k = 0; k < d_in; k++) {
+                const int32_t x = input[(size_t)r * d_in + k];
+                const int32_t w =
+                    load_byte(weight, weight_dtype, (size_t)n * d_in + k) -
+                    weight_zero_points[n];
+                acc += (int64_t)x * (int64_t)w;
+                if (acc < INT32_MIN || acc > INT32_MAX) return 0;
+            }
+            if (accumulators) accumulators[(size_t)r * d_out + n] = (int32_t)acc;
+            float t = vxo_transform_accumulator(acc, mult, output_zero_point);
+            if (bias_f32) {
+                /* extension (no reference counterpart): the real-valued bias in
+                 * output units, added as one more separately rounded f32 term */
+                volatile float in_output_units = bias_f32[n] / output_scale;
+                volatile float shifted = t + in_output_units;
+                t = shifted;
+            }
+            store_byte(output, output_dtype, (size_t)r * d_out + n,
+                       vxo_requantize(t, lo, hi, output_zero_point));
+        }
     }
-    free(row_bias);
-    return ok;
+    return 1;
 }
 
 /* ---- PackedLinear W8 under DYNAMIC_I8 --------------------------------- */

@@ -10,11 +10,11 @@
  * Parity status: every function below is pinned by the reference's own
  * known-answer vectors (tests/golden/reference_kats.json) and, where the
  * reference tree is available, by a byte comparison against the reference C
- * compiled from its own sources (oracle/_ref).  The one exception is
- * vxo_qlinear_rowscale_i8u8's f32-bias fold, which composes two pinned
- * reference rules (the PTQ bias rule and the per-row QLinear call) into a
- * form the reference does not ship as a single function; that composition
- * is an extension and is labelled so where it is used.
+ * compiled from its own sources (oracle/_ref).  The one exception is the
+ * optional f32 bias of vxo_qlinear_rowscale_i8u8: the reference has no
+ * real-valued bias in its requantizing linear, so that term is an extension
+ * ("parity unpinned" for that term only; with it absent the function is the
+ * reference's per-row call and is pinned like the rest).
  */
 #ifndef VXO_W8A8_ORACLE_H
 #define VXO_W8A8_ORACLE_H
@@ -55,11 +55,13 @@ int vxo_qlinear_i8u8(const void* input, const void* weight,
                      uint32_t weight_dtype, uint32_t output_dtype);
 
 /* Per-token activation scales: row m is its own reference QLinear call with
- * input_scale = row_scales[m] (portable_inference_kernels.inc:968-1032 called
- * with rows = 1).  When bias_f32 is non-NULL the row's int32 bias is produced
- * by the PTQ rule b_q = rne(f32(b / f32(s_m * s_w[n])))
- * (src/training/quantization.c:391-414); otherwise bias_i32 (may be NULL = 0)
- * is used as is.  Input zero point is 0 and input dtype I8. */
+ * input_scale = row_scales[m], input zero point 0, I8 input
+ * (portable_inference_kernels.inc:968-1032 called with rows = 1).  bias_i32
+ * (may be NULL = 0) is the reference's accumulator-domain bias.  bias_f32
+ * (may be NULL) is an EXTENSION with no reference counterpart: after the
+ * reference transform t = f32(f32(acc)*mult) + f32(zp), the term
+ * f32(bias_f32[n] / output_scale) is added with one more f32 rounding before
+ * the saturating round.  With bias_f32 == NULL the bytes are the reference's. */
 int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
                               const int32_t* bias_i32, const float* bias_f32,
                               const float* weight_scales,
@@ -90,8 +92,8 @@ int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
 /* Same arithmetic with the activation codes and per-row scales injected
  * (the "prepared A8" form the reference's CUDA route keeps in x[4]/x[5],
  * src/kernels/llm_ops.h:30-32).  row_finite may be NULL (all rows finite).
- * group_dots, when non-NULL, receives nothing; accumulators (optional)
- * receives the full-K int32 sum of the group dots, [rows, n]. */
+ * accumulators (optional) receives the full-K int32 sum of the group dots,
+ * [rows, n]. */
 int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
                          const uint8_t* row_finite, const uint32_t* packed,
                          const float* scales, const float* bias, float* output,

@@ -1,0 +1,357 @@
+"""Parity of the HIP path, called through the C ABI, with the CPU oracle and
+with the committed outputs of the reference's C kernels.  Integer, byte and
+f32 results are all held bit-exact (the f32 epilogue reproduces the
+reference's operation order, so no tolerance is needed; the north-star
+tolerance of 1e-5 rel / 1e-6 abs is therefore met with margin zero)."""
+import hashlib
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import _cases as cases
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = Path(__file__).parent / "golden"
+KATS = json.loads((GOLDEN / "reference_kats.json").read_text())
+VECTORS = json.loads((GOLDEN / "reference_vectors.json").read_text())
+I8, U8 = cases.DTYPE_I8, cases.DTYPE_U8
+DT = {"int8": I8, "uint8": U8}
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def sha(a):
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def same_f32(a, b):
+    """Bitwise equal, with any NaN matching any NaN (the reference stores a
+    default quiet NaN; payloads are not part of its contract)."""
+    na, nb = np.isnan(a), np.isnan(b)
+    return bool((na == nb).all() and (a.view(np.uint32)[~na] == b.view(np.uint32)[~nb]).all())
+
+
+def build_qcase(entry):
+    kind, p = entry["kind"], entry["params"]
+    if kind == "isa_parity":
+        return cases.isa_parity_case(**p)
+    if kind == "quant_gemm":
+        return cases.quant_gemm_case(**p)
+    return cases.qlinear_random_case(**p)
+
+
+def run_resident_qlinear(vx, ctx, c, want_acc=False):
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], c["bias"], c["w_dtype"])
+    res = lin.forward(ctx, dev(c["x"]), c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"],
+                      c["out_dtype"], want_accumulators=want_acc)
+    ctx.synchronize()
+    variant = ctx.last_variant
+    out = [res[0], host(res[1])] + ([host(res[2])] if want_acc else [])
+    lin.close()
+    return out, variant
+
+
+# ---- known-answer vectors through the drop-in entry point ----------------------------
+
+def test_kat_literal_and_halfway_through_drop_in():
+    import volvoxai_amd as vx
+    k = KATS["qlinear_literal"]
+    ok, y = vx.qlinear_i8u8(np.array(k["input"], np.int8), np.array(k["weight"], np.int8),
+                            np.array(k["weight_scales"], np.float32), np.array(k["weight_zero_points"], np.int32),
+                            np.array(k["bias"], np.int32), 2, 3, 4, k["input_scale"], k["input_zero_point"],
+                            k["output_scale"], k["output_zero_point"], I8, I8, I8)
+    assert ok == 1 and y.tolist() == k["expected"]
+    h = KATS["affine_halfway"]
+    x = np.zeros((h["rows"], h["channels"]), np.uint8)
+    x[:, :h["input_run"]["count"]] = h["input_run"]["value"]
+    x[:, h["input_run"]["count"]] = h["input_run"]["then"]
+    for wd in h["weight_dtypes"]:
+        w = np.full((h["outputs"], h["channels"]), h["weight_value"], np.int8 if wd == "int8" else np.uint8)
+        ok, y = vx.qlinear_i8u8(x, w, np.full(h["outputs"], h["weight_scale"], np.float32),
+                                np.zeros(h["outputs"], np.int32), np.zeros(h["outputs"], np.int32),
+                                h["rows"], h["channels"], h["outputs"], h["input_scale"], h["input_zero_point"],
+                                h["output_scale"], h["output_zero_point"], U8, DT[wd], I8)
+        assert ok == 1 and (y == h["expected_all"]).all(), "an FMA crept into the requantization epilogue"
+
+
+def test_kat_packed_near_tie(oracle):
+    import volvoxai_amd as vx
+    k = KATS["packed_near_tie_logits"]
+    x = np.zeros((1, k["k"]), np.float32)
+    for idx, v in k["x_nonzero"].items():
+        x[0, int(idx)] = v
+    w = np.zeros((k["n"], k["k"]), np.int8)
+    for row, col in k["weight_plus_one_at"]:
+        w[row, col] = 1
+    words = oracle.pack_w8_words(w)
+    st, y = vx.packed_linear_f32(x, words, np.array(k["scales"], np.float32), np.array(k["bias"], np.float32),
+                                 k["k"], k["n"], k["group_size"])
+    _, want = oracle.packed_linear(x, words, np.array(k["scales"], np.float32), np.array(k["bias"], np.float32),
+                                   k["n"], k["group_size"])
+    assert st == 0 and int(np.argmax(y[0])) == k["expected_argmax"] and same_f32(y, want)
+
+
+# ---- committed outputs of the reference's C kernels -----------------------------------
+
+@pytest.mark.parametrize("entry", VECTORS["qlinear"], ids=lambda e: f"{e['kind']}-{'-'.join(str(v) for v in e['params'].values())}")
+def test_qlinear_reference_vectors(ctx, oracle, entry):
+    import volvoxai_amd as vx
+    c = build_qcase(entry)
+    (ok, y, acc), variant = run_resident_qlinear(vx, ctx, c, want_acc=True)
+    assert ok == 1, vx.library().vxhip_last_error()
+    assert sha(y) == entry["expected"]["sha256"], f"bytes differ from the reference ({variant})"
+    _, _, want_acc = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"],
+                                    c["s_out"], c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"], want_acc=True)
+    assert (acc == want_acc).all()
+    # the host-pointer drop-in gives the same bytes
+    ok2, y2 = vx.qlinear_i8u8(c["x"], c["w"], c["scales"], c["zps"], c["bias"], *c["x"].shape, c["w"].shape[0],
+                              c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+    assert ok2 == 1 and (y2 == y).all()
+
+
+@pytest.mark.parametrize("entry", VECTORS["rowscale"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_rowscale_reference_vectors(ctx, oracle, entry):
+    import volvoxai_amd as vx
+    c = cases.rowscale_case(**entry["params"])
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, I8)
+    xd, rs = dev(c["x"]), dev(c["row_scales"])
+    ok, y, acc = lin.forward_rowscale(ctx, xd, rs, c["s_out"], c["zp_out"], want_accumulators=True)
+    ctx.synchronize()
+    assert ok == 1 and sha(host(y)) == entry["expected_without_bias"]["sha256"], ctx.last_variant
+    assert (host(acc) == c["x"].astype(np.int64) @ c["w"].astype(np.int64).T).all()
+    if c["bias_f32"] is not None:  # extension: checked against the oracle only
+        ok, yb = lin.forward_rowscale(ctx, xd, rs, c["s_out"], c["zp_out"], bias_f32=dev(c["bias_f32"]))
+        ctx.synchronize()
+        ok2, want, _ = oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], c["row_scales"], c["s_out"],
+                                               c["zp_out"], bias_f32=c["bias_f32"])
+        assert ok == ok2 == 1 and (host(yb) == want).all()
+    assert ctx.fault_flags() == 0
+    lin.close()
+
+
+@pytest.mark.parametrize("entry", VECTORS["packed"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_packed_reference_vectors(ctx, oracle, entry):
+    import volvoxai_amd as vx
+    c = cases.packed_case(**entry["params"])
+    words = oracle.pack_w8_words(c["w"])
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], c["k"], c["n"], c["group"])
+    st, y = pl.forward_f32(ctx, dev(c["x"]))
+    ctx.synchronize()
+    y = host(y)
+    assert st == 0
+    if not np.isnan(y).any():
+        assert sha(y) == entry["expected"]["sha256"], f"f32 bits differ from the reference ({ctx.last_variant})"
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"])
+    assert same_f32(y, want), ctx.last_variant
+    pl.close()
+
+
+# ---- both kernel families give the same bits ------------------------------------------
+
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 64), (7, 640, 100), (16, 4096, 96), (16, 48, 40)])
+def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
+    import volvoxai_amd as vx
+    c = cases.qlinear_random_case(rows, k, n, 77, I8, U8, I8, False)
+    _, want = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
+                             c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+    seen = set()
+    try:
+        for force in ("gemv.stream", "gemv.splitk", "mfma-i8.t128x128", "mfma-i8.t256x256"):
+            vx.force_variant(force)
+            (ok, y), variant = run_resident_qlinear(vx, ctx, c)
+            assert ok == 1 and (y == want).all(), variant
+            seen.add(variant)
+    finally:
+        vx.force_variant(None)
+    assert len(seen) == 4, seen
+
+
+@pytest.mark.parametrize("group", [32, 64, 128, 256])
+@pytest.mark.parametrize("rows,k,n", [(1, 4096, 48), (5, 1000, 36), (16, 1536, 130)])
+def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
+    import volvoxai_amd as vx
+    c = cases.packed_case(rows, k, n, group, 5 + group, True, special_rows=(rows >= 5))
+    words = oracle.pack_w8_words(c["w"])
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group)
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+    xd = dev(c["x"])
+    seen = set()
+    try:
+        for force in ("gemv.stream", "gemv.splitk", "a8-mfma.t128x128", "a8-mfma.t256x256"):
+            vx.force_variant(force)
+            st, y = pl.forward_f32(ctx, xd)
+            ctx.synchronize()
+            assert st == 0 and same_f32(host(y), want), ctx.last_variant
+            seen.add(ctx.last_variant)
+    finally:
+        vx.force_variant(None)
+    assert len(seen) >= 3, seen  # split-K is skipped when its ordered-sum buffer would not fit LDS
+    pl.close()
+
+
+# ---- BASELINE shapes --------------------------------------------------------------------
+
+@pytest.mark.parametrize("rows", [1, 4, 16])
+def test_decode_shape_config2(ctx, oracle, rows):
+    """M in {1,4,16}, K=4096, N=14336, prepared int8 activations, dequant+bias f32."""
+    import volvoxai_amd as vx
+    c = cases.decode_case(rows, 4096, 14336, 128, 1000 + rows)
+    words = oracle.pack_w8_words(c["w"])
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], 4096, 14336, 128)
+    st, y, acc = pl.forward_a8(ctx, dev(c["a8"]), dev(c["row_scales"]), want_accumulators=True)
+    ctx.synchronize()
+    assert st == 0 and "gemv" in ctx.last_variant
+    st2, want, want_acc = oracle.packed_linear_a8(c["a8"], c["row_scales"], words, c["scales"], c["bias"], 14336, 128)
+    y, acc = host(y), host(acc)
+    assert (acc == want_acc).all()
+    assert same_f32(y, want)
+    np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-6)  # the stated tolerance, met exactly
+    pl.close()
+
+
+def test_config1_cpu_route_shape(ctx, oracle):
+    """8x256x256: f32 activations quantized per tensor the PTQ way, QLinear, DQ."""
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(1)
+    xf = rng.normal(0, 1, (8, 256)).astype(np.float32)
+    w = rng.integers(-127, 128, (256, 256)).astype(np.int8)
+    sw = rng.uniform(0.005, 0.02, 256).astype(np.float32)
+    bf = rng.normal(0, 0.1, 256).astype(np.float32)
+    s_x = oracle.ptq_symmetric_scale(xf)
+    xq = oracle.ptq_quantize_i8(xf, s_x)
+    ok_q, xq_gpu = vx.quantize_typed_f32_i8u8(xf, s_x, 0, I8)
+    st, bq = oracle.ptq_pack_bias(bf, s_x, sw)
+    assert st == 0 and ok_q == 1
+    _, xq_rule = oracle.quantize(xf, s_x, 0, I8)
+    assert (xq_gpu == xq_rule).all()
+    zps = np.zeros(256, np.int32)
+    ok, y = vx.qlinear_i8u8(xq, w, sw, zps, bq, 8, 256, 256, s_x, 0, 0.25, 0, I8, I8, I8)
+    ok2, want = oracle.qlinear(xq, w, bq, sw, zps, s_x, 0, 0.25, 0, I8, I8, I8)
+    assert ok == ok2 == 1 and (y == want).all()
+    ok3, deq = vx.dequantize_typed_i8u8_f32(y, 0.25, 0, I8)
+    _, want_deq = oracle.dequantize(want, 0.25, 0, I8)
+    assert ok3 == 1 and same_f32(deq, want_deq)
+
+
+@pytest.mark.parametrize("rows", [512, 4096])
+def test_prefill_shape_config3_subblocks(ctx, oracle, rows):
+    """M in {512,4096}, K=N=4096, per-token x per-channel scale, requant to int8
+    at output scale 0.05.  An output sub-block depends only on its own rows of A
+    and B, so the oracle checks random sub-blocks at full problem size; the
+    int32 accumulators of the whole output are checked against an f64 GEMM."""
+    import torch
+    import volvoxai_amd as vx
+    c = cases.rowscale_case(rows, 4096, 4096, 3000 + rows)
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, I8)
+    xd = dev(c["x"])
+    ok, y, acc = lin.forward_rowscale(ctx, xd, dev(c["row_scales"]), c["s_out"], 0, bias_f32=dev(c["bias_f32"]),
+                                      want_accumulators=True)
+    ctx.synchronize()
+    assert ok == 1 and "mfma-i8-rowscale" in ctx.last_variant and ctx.fault_flags() == 0
+    exact = xd.double() @ dev(c["w"]).double().T  # |sum| < 2^53: exact in f64
+    assert torch.equal(acc.double(), exact)
+    y = host(y)
+    rng = np.random.default_rng(rows)
+    for _ in range(3):
+        rs = np.sort(rng.choice(rows, 24, replace=False))
+        cs = np.sort(rng.choice(4096, 40, replace=False))
+        ok2, want, _ = oracle.qlinear_rowscale(c["x"][rs], c["w"][cs], c["scales"][cs], c["zps"][cs],
+                                               c["row_scales"][rs], c["s_out"], 0, bias_f32=c["bias_f32"][cs])
+        assert ok2 == 1 and (y[np.ix_(rs, cs)] == want).all()
+    saturated = ((y == 127) | (y == -128)).mean()
+    assert saturated < 0.5, "inputs should exercise the rounding path, not only saturation"
+    lin.close()
+
+
+def test_outlier_large_k_config5_reduced_rows(ctx, oracle):
+    """K=14336, N=4096 with 1% outlier channels scaled x20 before the dynamic
+    per-row quantization; 96 rows here (the oracle is scalar), full K and N."""
+    import volvoxai_amd as vx
+    rows, k, n, g = 96, 14336, 4096, 128
+    rng = np.random.default_rng(55)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[:, rng.choice(k, k // 100, replace=False)] *= 20.0
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    chan = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    scales = np.repeat(chan[:, None], k // g, axis=1).copy()
+    bias = rng.normal(0, 0.1, n).astype(np.float32)
+    words = oracle.pack_w8_words(w)
+    pl = vx.PackedLinear(words, scales, bias, k, n, g)
+    st, y = pl.forward_f32(ctx, dev(x))
+    ctx.synchronize()
+    assert st == 0 and "a8-mfma" in ctx.last_variant
+    cs = np.sort(rng.choice(n, 160, replace=False))
+    _, want = oracle.packed_linear(x, np.ascontiguousarray(words[cs]), np.ascontiguousarray(scales[cs]),
+                                   np.ascontiguousarray(bias[cs]), len(cs), g)
+    assert same_f32(host(y)[:, cs], want)
+    pl.close()
+
+
+# ---- boundaries and edge cases ------------------------------------------------------------
+
+def test_prepare_matches_oracle(ctx, oracle):
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    c = cases.packed_case(9, 1283, 4, 128, 3, special_rows=True)
+    x = c["x"].copy()
+    x[7, 5] = np.nan
+    x[8, 0] = -np.inf
+    a8, s = packed_prepare_i8(ctx, dev(x))
+    ctx.synchronize()
+    want_a, want_s, fin = oracle.packed_prepare(x)
+    a8, s = host(a8), host(s)
+    assert (np.isnan(s) == (fin == 0)).all()
+    good = fin == 1
+    assert (s[good].view(np.uint32) == want_s[good].view(np.uint32)).all()
+    assert (a8[good] == want_a[good]).all() and not a8[~good].any()
+
+
+def test_quantize_dequantize_match_oracle(oracle):
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(8)
+    x = np.concatenate([rng.normal(0, 40, 5000), np.arange(-6, 6) + 0.5,
+                        [np.nan, np.inf, -np.inf, 1e30, -1e30, 0.0, -0.0]]).astype(np.float32)
+    for dt, zp in ((I8, -7), (U8, 131), (I8, 0)):
+        ok, q = vx.quantize_typed_f32_i8u8(x, 0.37, zp, dt)
+        ok2, want = oracle.quantize(x, 0.37, zp, dt)
+        assert ok == ok2 == 1 and (q == want).all()
+        ok, d = vx.dequantize_typed_i8u8_f32(want, 0.37, zp, dt)
+        _, wd = oracle.dequantize(want, 0.37, zp, dt)
+        assert ok == 1 and same_f32(d, wd)
+
+
+def test_declines_leave_output_untouched():
+    import volvoxai_amd as vx
+    c = cases.qlinear_random_case(2, 16, 4, 3)
+    base = dict(input=c["x"], weight=c["w"], weight_scales=c["scales"], weight_zero_points=c["zps"], bias=c["bias"],
+                rows=2, d_in=16, d_out=4, input_scale=c["s_in"], input_zero_point=0, output_scale=c["s_out"],
+                output_zero_point=0, input_dtype=I8, weight_dtype=I8, output_dtype=I8)
+    for patch in (dict(input_scale=0.0), dict(input_zero_point=300), dict(output_scale=float("inf")),
+                  dict(input_scale=1e-30, weight_scales=np.full(4, 1e-30, np.float32)),
+                  dict(bias=np.full(4, 2**31 - 1, np.int32)), dict(input_dtype=18)):
+        ok, y = vx.qlinear_i8u8(**{**base, **patch})
+        assert ok == 0 and not y.any(), patch
+    # K beyond the int32 proof: declined before launch
+    big = cases.qlinear_random_case(1, 40000, 4, 4, U8, U8, I8, False)
+    ok, _ = vx.qlinear_i8u8(big["x"], big["w"], big["scales"], big["zps"], big["bias"], 1, 40000, 4, big["s_in"],
+                            big["zp_in"], big["s_out"], big["zp_out"], U8, U8, I8)
+    assert ok == 0 and b"int32" in vx.library().vxhip_last_error()
+
+
+def test_context_reports_variant_and_clean_fault_word(ctx):
+    import volvoxai_amd as vx
+    c = cases.qlinear_random_case(64, 256, 128, 2)
+    (ok, _), variant = run_resident_qlinear(vx, ctx, c)
+    assert ok == 1 and variant.startswith("hip.qlinear.mfma-i8")
+    assert variant.split(".t")[0] in {r["id"] for r in vx.kernel_variants()}
+    assert ctx.fault_flags() == 0

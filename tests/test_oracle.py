@@ -1,0 +1,261 @@
+"""Pins the CPU oracle: against the reference's own known-answer vectors,
+against outputs of the reference's C kernels (committed digests, and live when
+oracle/_ref is built), and against closed forms / brute force that a dropped
+term, wrong sign or transposed operand would break."""
+import hashlib
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import _cases as cases
+
+GOLDEN = Path(__file__).parent / "golden"
+KATS = json.loads((GOLDEN / "reference_kats.json").read_text())
+VECTORS = json.loads((GOLDEN / "reference_vectors.json").read_text())
+I8, U8 = cases.DTYPE_I8, cases.DTYPE_U8
+DT = {"int8": I8, "uint8": U8}
+
+
+def fval(v):
+    if isinstance(v, str):
+        return float.fromhex(v) if v.startswith("0x") else float(v)
+    return float(v)
+
+
+def check_digest(arr, expected):
+    arr = np.ascontiguousarray(arr)
+    assert list(arr.shape) == expected["shape"] and str(arr.dtype) == expected["dtype"]
+    head = arr.reshape(-1)[:32]
+    head = head.view(np.uint32) if arr.dtype == np.float32 else head
+    assert [int(v) for v in head] == expected["head"]
+    assert hashlib.sha256(arr.tobytes()).hexdigest() == expected["sha256"]
+
+
+# ---- known-answer vectors held by the reference's tests -------------------------
+
+def test_qlinear_literal_kat(oracle):
+    k = KATS["qlinear_literal"]
+    ok, y = oracle.qlinear(np.array(k["input"], np.int8), np.array(k["weight"], np.int8),
+                           np.array(k["bias"], np.int32), np.array(k["weight_scales"], np.float32),
+                           np.array(k["weight_zero_points"], np.int32), k["input_scale"],
+                           k["input_zero_point"], k["output_scale"], k["output_zero_point"], I8, I8, I8)
+    assert ok == 1 and y.tolist() == k["expected"]
+
+
+def test_round_and_requantize_kats(oracle):
+    for value, expected in KATS["round_ties_even"]["cases"]:
+        assert oracle.round_ties_even(value) == expected
+    for c in KATS["requantize"]["cases"]:
+        assert oracle.requantize(fval(c["value"]), c["min"], c["max"], c["nan_value"]) == c["expected"]
+    for value, expected in KATS["packed_round_i8"]["cases"]:
+        assert oracle.packed_round_i8(value) == expected
+
+
+def test_multiplier_contract(oracle):
+    grid = [np.float32(fval(v)) for v in KATS["multiplier"]["scale_grid_hex"]]
+    for a in grid:
+        for b in grid:
+            for c in grid:
+                ok, m = oracle.multiplier(a, b, c)
+                want = np.float32(np.float32(a * b) / c)  # f32(f32(a*b)/c), numpy keeps f32
+                assert ok and m.view(np.uint32) == want.view(np.uint32)
+                # the other association differs for some triples; the oracle must not use it
+    for a, b, c in KATS["multiplier"]["invalid"]:
+        ok, _ = oracle.multiplier(fval(a), fval(b), fval(c))
+        assert not ok
+
+
+def halfway_inputs(k):
+    x = np.zeros((k["rows"], k["channels"]), np.uint8)
+    run = k["input_run"]
+    x[:, :run["count"]] = run["value"]
+    x[:, run["count"]] = run["then"]
+    return x
+
+
+def test_affine_halfway_kat(oracle):
+    k = KATS["affine_halfway"]
+    x = halfway_inputs(k)
+    for wd in k["weight_dtypes"]:
+        w = np.full((k["outputs"], k["channels"]), k["weight_value"], np.int8 if wd == "int8" else np.uint8)
+        ok, y = oracle.qlinear(x, w, np.zeros(k["outputs"], np.int32),
+                               np.full(k["outputs"], k["weight_scale"], np.float32),
+                               np.zeros(k["outputs"], np.int32), k["input_scale"], k["input_zero_point"],
+                               k["output_scale"], k["output_zero_point"], U8, DT[wd], I8)
+        assert ok == 1 and (y == k["expected_all"]).all()
+    # the fused form really is different here, so the KAT does discriminate
+    acc, mult = 17 * 255 + 40, np.float32(np.float32(np.float32(0.015) * np.float32(0.008)) / np.float32(0.03))
+    fused = np.float64(acc) * np.float64(mult) - 17.0
+    assert round(float(np.float32(fused))) == 1
+
+
+def near_tie_case():
+    k = KATS["packed_near_tie_logits"]
+    x = np.zeros((1, k["k"]), np.float32)
+    for idx, v in k["x_nonzero"].items():
+        x[0, int(idx)] = v
+    w = np.zeros((k["n"], k["k"]), np.int8)
+    for row, col in k["weight_plus_one_at"]:
+        w[row, col] = 1
+    return k, x, w
+
+
+def test_packed_near_tie_kat(oracle):
+    k, x, w = near_tie_case()
+    words = oracle.pack_w8_words(w)
+    assert words[0, 1] == 0x80808080  # the reference's W8 zero word
+    st, y = oracle.packed_linear(x, words, np.array(k["scales"], np.float32),
+                                 np.array(k["bias"], np.float32), k["n"], k["group_size"])
+    assert st == 0 and int(np.argmax(y[0])) == k["expected_argmax"]
+    s_a = np.float32(np.float32(1.0003) / np.float32(127.0))
+    term = np.float32(np.float32(127.0) * np.float32(s_a * np.float32(1.0)))
+    assert y[0, 1].view(np.uint32) == np.float32(term + np.float32(0.0)).view(np.uint32)
+    assert y[0, 0].view(np.uint32) == np.float32(term + np.float32(-0.0002)).view(np.uint32)
+
+
+# ---- outputs of the reference's C kernels (committed digests) -------------------
+
+def build_qcase(entry):
+    kind, p = entry["kind"], entry["params"]
+    if kind == "isa_parity":
+        return cases.isa_parity_case(**p)
+    if kind == "quant_gemm":
+        return cases.quant_gemm_case(**p)
+    return cases.qlinear_random_case(**p)
+
+
+@pytest.mark.parametrize("entry", VECTORS["qlinear"], ids=lambda e: f"{e['kind']}-{'-'.join(str(v) for v in e['params'].values())}")
+def test_qlinear_matches_reference_vectors(oracle, entry):
+    c = build_qcase(entry)
+    ok, y = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"],
+                           c["s_out"], c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+    assert ok == 1
+    check_digest(y, entry["expected"])
+
+
+@pytest.mark.parametrize("entry", VECTORS["rowscale"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_rowscale_matches_reference_vectors(oracle, entry):
+    c = cases.rowscale_case(**entry["params"])
+    ok, y, acc = oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], c["row_scales"],
+                                         c["s_out"], c["zp_out"])
+    assert ok == 1
+    check_digest(y, entry["expected_without_bias"])
+    brute = c["x"].astype(np.int64) @ c["w"].astype(np.int64).T
+    assert (acc == brute).all()
+
+
+@pytest.mark.parametrize("entry", VECTORS["packed"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_packed_matches_reference_vectors(oracle, entry):
+    c = cases.packed_case(**entry["params"])
+    st, y = oracle.packed_linear(c["x"], oracle.pack_w8_words(c["w"]), c["scales"], c["bias"], c["n"], c["group"])
+    assert st == 0
+    check_digest(y, entry["expected"])
+
+
+# ---- live comparison with the reference build ------------------------------------
+
+def test_live_reference_qlinear(oracle, reference):
+    rng = np.random.default_rng(5)
+    for (m, k, n) in [(7, 129, 31), (2, 33, 36), (33, 64, 64)]:
+        for idt in (I8, U8):
+            for wdt in (I8, U8):
+                c = cases.qlinear_random_case(m, k, n, int(rng.integers(1 << 30)), idt, wdt, U8, False)
+                args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"],
+                        c["s_out"], c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+                a = oracle.qlinear(*args)
+                b = reference.qlinear_portable(*args)
+                d = reference.qlinear_native(*args)
+                assert a[0] == b[0] == d[0] == 1
+                assert (a[1] == b[1]).all() and (a[1] == d[1]).all()
+
+
+def test_live_reference_declines_like_oracle(oracle, reference):
+    c = cases.qlinear_random_case(2, 16, 4, 3)
+    base = [c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
+            c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"]]
+    bad_scale = list(base); bad_scale[5] = 0.0
+    bad_zp = list(base); bad_zp[6] = 300
+    tiny = list(base); tiny[5] = 1e-30; tiny[3] = np.full(4, 1e-30, np.float32)  # product underflows to 0
+    huge_bias = list(base); huge_bias[2] = np.full(4, 2**31 - 1, np.int32)       # first add overflows
+    for args in (bad_scale, bad_zp, tiny, huge_bias):
+        assert oracle.qlinear(*args)[0] == reference.qlinear_portable(*args)[0] == 0
+
+
+def test_live_reference_packed_and_bias_rule(oracle, reference):
+    for p in [dict(rows=6, k=200, n=9, group=64, seed=1, special_rows=True),
+              dict(rows=5, k=31, n=3, group=32, seed=2, with_bias=False)]:
+        c = cases.packed_case(**p)
+        words = oracle.pack_w8_words(c["w"])
+        x = c["x"].copy()
+        if p["rows"] > 5:
+            x[5, 3] = np.inf
+        a = oracle.packed_linear(x, words, c["scales"], c["bias"], c["n"], c["group"])
+        b = reference.packed_linear(x, words, c["scales"], c["bias"], c["n"], c["group"])
+        assert a[0] == b[0] == 0
+        nan = np.isnan(b[1])
+        assert (np.isnan(a[1]) == nan).all()
+        assert (a[1].view(np.uint32)[~nan] == b[1].view(np.uint32)[~nan]).all()
+    rng = np.random.default_rng(9)
+    b = rng.normal(0, 0.3, 64).astype(np.float32)
+    sw = rng.uniform(0.002, 0.02, 64).astype(np.float32)
+    st1, q1 = oracle.ptq_pack_bias(b, 0.0173, sw)
+    st2, q2 = reference.ptq_pack_bias(b, 0.0173, sw)
+    assert st1 == st2 == 0 and (q1 == q2).all()
+
+
+# ---- what the mathematics fixes ---------------------------------------------------
+
+def test_accumulator_is_the_integer_gemm(oracle):
+    c = cases.qlinear_random_case(9, 77, 21, 11, U8, U8, I8, False)
+    ok, y, acc = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"],
+                                c["s_out"], c["zp_out"], U8, U8, I8, want_acc=True)
+    xs = c["x"].astype(np.int64) - c["zp_in"]
+    ws = c["w"].astype(np.int64) - c["zps"][:, None]
+    assert ok == 1 and (acc == xs @ ws.T + c["bias"]).all()
+
+
+def test_packed_prepare_closed_form(oracle):
+    x = np.array([[0.0, -2.0, 1.0, 0.5, 127.0 / 254.0 * 2.0]], np.float32)  # max 2 -> scale 2/127
+    a, s, fin = oracle.packed_prepare(x)
+    assert fin[0] == 1 and s[0].view(np.uint32) == np.float32(np.float32(2.0) / np.float32(127.0)).view(np.uint32)
+    assert a[0].tolist() == [0, -127, 64, 32, 64]  # 63.5 -> 64 (even), 31.75 -> 32
+    z, sz, _ = oracle.packed_prepare(np.zeros((1, 8), np.float32))
+    assert sz[0] == 1.0 and not z.any()
+    _, s_tiny, _ = oracle.packed_prepare(np.full((1, 4), 2.0 ** -140, np.float32))
+    assert s_tiny[0] == np.float32(2.0 ** -126)
+    _, _, bad = oracle.packed_prepare(np.array([[1.0, np.nan]], np.float32))
+    assert bad[0] == 0
+
+
+def test_packed_group_order_matters_and_is_ascending(oracle):
+    # terms of very different magnitude: ascending order rounds differently from descending
+    k, g = 64, 32
+    a8 = np.zeros((1, k), np.int8); a8[0, 0] = 127; a8[0, 32] = 1
+    w = np.zeros((1, k), np.int8); w[0, 0] = 127; w[0, 32] = 1
+    scales = np.array([[1.0, 2.0 ** -20]], np.float32)
+    st, y, acc = oracle.packed_linear_a8(a8, np.ones(1, np.float32), oracle.pack_w8_words(w), scales, None, 1, g)
+    want = np.float32(np.float32(0.0 + np.float32(16129.0)) + np.float32(np.float32(1.0) * np.float32(2.0 ** -20)))
+    assert st == 0 and y[0, 0].view(np.uint32) == want.view(np.uint32) and acc[0, 0] == 16130
+
+
+def test_quantize_dequantize_rules(oracle):
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, np.nan, np.inf, -np.inf, 1000.0, -1000.0, 0.3], np.float32)
+    ok, q = oracle.quantize(x, 1.0, 0, I8)
+    assert ok == 1 and q.tolist() == [0, 2, 2, 0, -2, 0, 127, -128, 127, -128, 0]
+    ok, q = oracle.quantize(x, 1.0, 7, U8)
+    assert q.tolist()[:6] == [8, 8, 10, 6, 6, 7]  # 7.5->8, 8.5->8, 9.5->10, 6.5->6, 5.5->6, NaN->zp
+    ok, d = oracle.dequantize(np.array([-128, 0, 127], np.int8), 0.1, -3, I8)
+    want = [np.float32((v + 3) * float(np.float32(0.1))) for v in (-128, 0, 127)]
+    assert [v.view(np.uint32) for v in d] == [w.view(np.uint32) for w in want]
+
+
+def test_ptq_rules(oracle):
+    x = np.array([0.0, -3.0, 1.27], np.float32)
+    s = oracle.ptq_symmetric_scale(x)
+    assert s.view(np.uint32) == np.float32(3.0 / 127.0).view(np.uint32)
+    q = oracle.ptq_quantize_i8(x, s)
+    assert q.tolist() == [0, -127, 54]
+    st, b = oracle.ptq_pack_bias(np.array([0.25, -0.75], np.float32), 0.5, np.array([0.5, 0.25], np.float32))
+    assert st == 0 and b.tolist() == [1, -6]

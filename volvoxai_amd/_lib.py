@@ -1,0 +1,93 @@
+"""Locates, builds and loads libvxhip_w8a8.so.  There is no fallback path: a
+missing library raises, it never degrades to a CPU implementation."""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+HEADER = ROOT.parent / "include" / "vxhip_w8a8.h"
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def library_path() -> Path:
+    return ROOT / "lib" / "libvxhip_w8a8.so"
+
+
+def build_library(clean: bool = False) -> Path:
+    """Compile the HIP sources for gfx950 (cross-compiles without a GPU)."""
+    if clean:
+        subprocess.check_call(["make", "-C", str(ROOT / "csrc"), "clean"])
+    subprocess.check_call(["make", "-C", str(ROOT / "csrc"), "-j8"])
+    return library_path()
+
+
+_lib = None
+
+
+def library() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not path.exists():
+            raise LibraryMissing(
+                f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C volvoxai_amd/csrc`. This package has no non-HIP path.")
+        _lib = C.CDLL(str(path))
+        _declare(_lib)
+    return _lib
+
+
+def _declare(L: C.CDLL) -> None:
+    vp, u32, i32, f32, sz, u64 = C.c_void_p, C.c_uint32, C.c_int32, C.c_float, C.c_size_t, C.c_uint64
+    pp = C.POINTER(C.c_void_p)
+    sig = {
+        "vxhip_abi_version": (u32, []),
+        "vxhip_device_count": (i32, []),
+        "vxhip_device_name": (i32, [i32, C.c_char_p, sz]),
+        "vxhip_last_error": (C.c_char_p, []),
+        "vxhip_context_create": (i32, [i32, vp, pp]),
+        "vxhip_context_destroy": (None, [vp]),
+        "vxhip_context_synchronize": (i32, [vp]),
+        "vxhip_context_last_variant": (C.c_char_p, [vp]),
+        "vxhip_context_fault_flags": (i32, [vp, C.POINTER(u32)]),
+        "vxhip_device_malloc": (i32, [sz, pp]),
+        "vxhip_device_free": (None, [vp]),
+        "vxhip_memcpy_to_device": (i32, [vp, vp, vp, sz]),
+        "vxhip_memcpy_to_host": (i32, [vp, vp, vp, sz]),
+        "vxhip_qlinear_create": (i32, [vp, vp, vp, vp, u32, u32, u32, pp]),
+        "vxhip_qlinear_destroy": (None, [vp]),
+        "vxhip_qlinear_resident_bytes": (u64, [vp]),
+        "vxhip_qlinear_forward": (C.c_int, [vp, vp, vp, vp, vp, u32, f32, i32, f32, i32, u32, u32]),
+        "vxhip_qlinear_forward_rowscale": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u32, f32, i32, u32]),
+        "vxhip_qlinear_i8u8": (C.c_int, [vp, vp, vp, vp, vp, vp, u32, u32, u32, f32, i32, f32, i32,
+                                         u32, u32, u32]),
+        "vxhip_packed_linear_create": (i32, [vp, vp, vp, u32, u32, u32, u32, pp]),
+        "vxhip_packed_linear_destroy": (None, [vp]),
+        "vxhip_packed_linear_resident_bytes": (u64, [vp]),
+        "vxhip_packed_prepare_i8": (i32, [vp, vp, u32, u32, vp, vp]),
+        "vxhip_packed_linear_forward_f32": (C.c_int, [vp, vp, vp, vp, u32]),
+        "vxhip_packed_linear_forward_a8": (C.c_int, [vp, vp, vp, vp, vp, vp, u32]),
+        "vxhip_packed_linear_f32": (C.c_int, [vp, vp, vp, vp, vp, u64, i32, i32, i32, i32, i32]),
+        "vxhip_quantize_typed_f32_i8u8": (C.c_int, [vp, u32, vp, f32, i32, u32]),
+        "vxhip_dequantize_typed_i8u8_f32": (C.c_int, [vp, u32, f32, i32, u32, vp]),
+        "vxhip_quantize_forward": (C.c_int, [vp, vp, u32, vp, f32, i32, u32]),
+        "vxhip_dequantize_forward": (C.c_int, [vp, vp, u32, f32, i32, u32, vp]),
+        "vxhip_kernel_variants": (vp, [C.POINTER(sz)]),
+        "vxhip_force_variant": (None, [C.c_char_p]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+
+
+def declared_symbols() -> list[str]:
+    """Every entry point the public header declares (parsed from the header)."""
+    import re
+    text = HEADER.read_text()
+    return sorted(set(re.findall(r"\b(vxhip_[a-z0-9_]+)\s*\(", text)))

@@ -1,0 +1,772 @@
+// C ABI of libvxhip_w8a8 (see include/vxhip_w8a8.h): handle lifetimes, the
+// host-side admission proofs, and the choice between the MFMA GEMM and the
+// streaming GEMV.  No arithmetic on tensor data happens on the host.
+#include "common.h"
+
+#include <limits.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+namespace vxhip {
+
+static thread_local char g_error[512] = "";
+static thread_local char g_force[64] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+}
+
+VxHipStatus hip_status(hipError_t e, const char* what) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    (void)hipGetLastError();
+    if (e == hipErrorOutOfMemory) return VXHIP_OUT_OF_MEMORY;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) return VXHIP_BACKEND_UNAVAILABLE;
+    if (e == hipErrorIllegalAddress || e == hipErrorLaunchFailure || e == hipErrorECCNotCorrectable)
+        return VXHIP_DEVICE_LOST;
+    return VXHIP_EXECUTION_FAILED;
+}
+
+const char* forced_variant() { return g_force[0] ? g_force : nullptr; }
+
+static bool byte_dtype(uint32_t d) { return d == VXHIP_DTYPE_I8 || d == VXHIP_DTYPE_U8; }
+static bool zero_point_ok(int32_t zp, uint32_t d) {
+    return d == VXHIP_DTYPE_I8 ? (zp >= -128 && zp <= 127) : (zp >= 0 && zp <= 255);
+}
+static bool scale_ok(float v) { return isfinite(v) && v > 0.0f; }
+
+// f32(f32(s_in * s_w) / s_out), each step rounded to f32
+// (native/src/backends/qlinear_multiplier.h:12-27).
+static bool multiplier_ok(float s_in, float s_w, float s_out) {
+    volatile float p = s_in * s_w;
+    volatile float m = p / s_out;
+    return scale_ok(m);
+}
+
+VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes) {
+    if (bytes <= ctx->scratch_bytes) return VXHIP_OK;
+    // earlier launches may still read the old block
+    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (ctx->scratch) VXHIP_TRY(hipFree(ctx->scratch));
+    ctx->scratch = nullptr;
+    ctx->scratch_bytes = 0;
+    const size_t want = (bytes + (1u << 20)) & ~((size_t)(1u << 20) - 1u);
+    VXHIP_TRY(hipMalloc(&ctx->scratch, want));
+    ctx->scratch_bytes = want;
+    return VXHIP_OK;
+}
+
+struct Carver {
+    char* base;
+    size_t off = 0;
+    template <class T>
+    T* take(size_t count) {
+        off = (off + 255u) & ~(size_t)255u;
+        T* p = base ? reinterpret_cast<T*>(base + off) : nullptr;
+        off += count * sizeof(T);
+        return p;
+    }
+};
+
+static VxHipContext* default_context() {
+    static thread_local VxHipContext* ctx = nullptr;
+    if (!ctx && vxhip_context_create(0, nullptr, &ctx) != VXHIP_OK) ctx = nullptr;
+    return ctx;
+}
+
+static bool use_device(int device) {
+    if (hipSetDevice(device) != hipSuccess) {
+        set_error("hipSetDevice(%d) failed", device);
+        return false;
+    }
+    return true;
+}
+
+// Picks the kernel family for the shape and launches it.
+static const char* run_linear(VxHipContext* ctx, const LinearArgs& a) {
+    const char* force = forced_variant();
+    const bool force_gemm = force && strstr(force, "mfma-i8") != nullptr && !strstr(force, "gemv");
+    const bool force_gemm_f = force && strstr(force, "a8-mfma") != nullptr;
+    const bool force_gemv = force && strstr(force, "gemv") != nullptr;
+    const char* id = nullptr;
+    if (force_gemv) return launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
+    if (force_gemm || force_gemm_f) return launch_gemm_mfma(ctx->stream, a, ctx->cu_count, force);
+    if (a.rows <= kMaxGemvRows) id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
+    if (!id) id = launch_gemm_mfma(ctx->stream, a, ctx->cu_count, force);
+    return id;
+}
+
+}  // namespace vxhip
+
+using namespace vxhip;
+
+extern "C" {
+
+uint32_t vxhip_abi_version(void) { return VXHIP_ABI_VERSION; }
+
+const char* vxhip_last_error(void) { return g_error; }
+
+int32_t vxhip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int ok = 0;
+    for (int i = 0; i < n; i++) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, i) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0)
+            ok++;
+    }
+    return ok;
+}
+
+VxHipStatus vxhip_device_name(int32_t device, char* buffer, size_t capacity) {
+    if (!buffer || !capacity) return VXHIP_INVALID_ARGUMENT;
+    hipDeviceProp_t prop;
+    VXHIP_TRY(hipGetDeviceProperties(&prop, device));
+    snprintf(buffer, capacity, "%s (%s), %d CU, %.0f GiB", prop.name, prop.gcnArchName,
+             prop.multiProcessorCount, (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+    return VXHIP_OK;
+}
+
+void vxhip_force_variant(const char* id_prefix) {
+    snprintf(g_force, sizeof g_force, "%s", id_prefix ? id_prefix : "");
+}
+
+// ---- context -----------------------------------------------------------------
+
+VxHipStatus vxhip_context_create(int32_t device, void* stream, VxHipContext** out) {
+    if (!out) return VXHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("no HIP device %d", device);
+        return VXHIP_BACKEND_UNAVAILABLE;
+    }
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+        return VXHIP_BACKEND_UNAVAILABLE;
+    }
+    VXHIP_TRY(hipSetDevice(device));
+    VxHipContext* ctx = new (std::nothrow) VxHipContext();
+    if (!ctx) return VXHIP_OUT_OF_MEMORY;
+    ctx->device = device;
+    ctx->cu_count = prop.multiProcessorCount;
+    if (stream) {
+        ctx->stream = (hipStream_t)stream;
+    } else {
+        hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            delete ctx;
+            return hip_status(e, "hipStreamCreateWithFlags");
+        }
+        ctx->own_stream = true;
+    }
+    hipError_t e = hipMalloc((void**)&ctx->fault_dev, 256);
+    if (e == hipSuccess) e = hipMemset(ctx->fault_dev, 0, 256);
+    if (e != hipSuccess) {
+        vxhip_context_destroy(ctx);
+        return hip_status(e, "fault word");
+    }
+    *out = ctx;
+    return VXHIP_OK;
+}
+
+void vxhip_context_destroy(VxHipContext* ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->fault_dev) (void)hipFree(ctx->fault_dev);
+    if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+VxHipStatus vxhip_context_synchronize(VxHipContext* ctx) {
+    if (!ctx) return VXHIP_INVALID_ARGUMENT;
+    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
+    return VXHIP_OK;
+}
+
+const char* vxhip_context_last_variant(const VxHipContext* ctx) { return ctx ? ctx->last_variant : ""; }
+
+VxHipStatus vxhip_context_fault_flags(VxHipContext* ctx, uint32_t* flags) {
+    if (!ctx || !flags) return VXHIP_INVALID_ARGUMENT;
+    VXHIP_TRY(hipMemcpyAsync(flags, ctx->fault_dev, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_device_malloc(size_t bytes, void** out) {
+    if (!out) return VXHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    VXHIP_TRY(hipMalloc(out, bytes ? bytes : 1));
+    return VXHIP_OK;
+}
+
+void vxhip_device_free(void* p) {
+    if (p) (void)hipFree(p);
+}
+
+VxHipStatus vxhip_memcpy_to_device(VxHipContext* ctx, void* dst, const void* src, size_t bytes) {
+    if (!ctx || (bytes && (!dst || !src))) return VXHIP_INVALID_ARGUMENT;
+    if (!bytes) return VXHIP_OK;
+    VXHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_memcpy_to_host(VxHipContext* ctx, void* dst, const void* src, size_t bytes) {
+    if (!ctx || (bytes && (!dst || !src))) return VXHIP_INVALID_ARGUMENT;
+    if (!bytes) return VXHIP_OK;
+    VXHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
+    return VXHIP_OK;
+}
+
+// ---- QLinear ------------------------------------------------------------------
+
+void vxhip_qlinear_destroy(VxHipQLinear* lin) {
+    if (!lin) return;
+    (void)hipSetDevice(lin->device);
+    (void)hipDeviceSynchronize();
+    if (lin->w.data) (void)hipFree(lin->w.data);
+    if (lin->scales) (void)hipFree(lin->scales);
+    if (lin->zero_points) (void)hipFree(lin->zero_points);
+    if (lin->bias) (void)hipFree(lin->bias);
+    if (lin->weight_sums) (void)hipFree(lin->weight_sums);
+    delete lin;
+}
+
+uint64_t vxhip_qlinear_resident_bytes(const VxHipQLinear* lin) { return lin ? lin->resident : 0; }
+
+VxHipStatus vxhip_qlinear_create(const void* weight, const float* weight_scales,
+                                 const int32_t* weight_zero_points, const int32_t* bias,
+                                 uint32_t d_in, uint32_t d_out, uint32_t weight_dtype,
+                                 VxHipQLinear** out) {
+    if (!out) return VXHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (!weight || !weight_scales || !weight_zero_points || !d_in || !d_out ||
+        !byte_dtype(weight_dtype)) {
+        set_error("qlinear_create: null tensor, zero extent or non-byte weight dtype");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if ((uint64_t)d_in * d_out > (uint64_t)1 << 40) return VXHIP_INVALID_ARGUMENT;
+    int device = 0;
+    VXHIP_TRY(hipGetDevice(&device));
+    const bool flip = weight_dtype == VXHIP_DTYPE_U8;
+    float smin = INFINITY, smax = 0.f;
+    bool any_zp = false;
+    int64_t bias_abs = 0;
+    const uint32_t n_pad = ((d_out + 31u) / 32u + kPanelPad - 1) / kPanelPad * kPanelPad * 32u;
+    std::vector<int32_t> zps(n_pad, 0), hbias(n_pad, 0);
+    std::vector<float> hscale(n_pad, 1.0f);
+    for (uint32_t i = 0; i < d_out; i++) {
+        if (!scale_ok(weight_scales[i]) || !zero_point_ok(weight_zero_points[i], weight_dtype)) {
+            set_error("qlinear_create: channel %u has an invalid scale or zero point", i);
+            return VXHIP_INVALID_ARGUMENT;
+        }
+        hscale[i] = weight_scales[i];
+        smin = fminf(smin, weight_scales[i]);
+        smax = fmaxf(smax, weight_scales[i]);
+        zps[i] = weight_zero_points[i] - (flip ? 128 : 0);
+        any_zp |= zps[i] != 0;
+        if (bias) {
+            hbias[i] = bias[i];
+            const int64_t b = bias[i] < 0 ? -(int64_t)bias[i] : (int64_t)bias[i];
+            if (b > bias_abs) bias_abs = b;
+        }
+    }
+    VxHipQLinear* lin = new (std::nothrow) VxHipQLinear();
+    if (!lin) return VXHIP_OUT_OF_MEMORY;
+    lin->device = device;
+    lin->weight_dtype = weight_dtype;
+    lin->any_zero_point = any_zp;
+    lin->scale_min = smin;
+    lin->scale_max = smax;
+    lin->bias_abs_max = bias_abs;
+    uint8_t* raw = nullptr;
+    int32_t* absmax_dev = nullptr;
+    const size_t raw_bytes = (size_t)d_in * d_out;
+    VxHipStatus st = VXHIP_OK;
+    auto fail = [&](VxHipStatus s) {
+        if (raw) (void)hipFree(raw);
+        if (absmax_dev) (void)hipFree(absmax_dev);
+        vxhip_qlinear_destroy(lin);
+        return s;
+    };
+#define TRY_OR_FAIL(expr)                                        \
+    do {                                                         \
+        hipError_t e_ = (expr);                                  \
+        if (e_ != hipSuccess) return fail(hip_status(e_, #expr)); \
+    } while (0)
+    TRY_OR_FAIL(hipMalloc((void**)&raw, raw_bytes));
+    TRY_OR_FAIL(hipMalloc((void**)&absmax_dev, 256));
+    TRY_OR_FAIL(hipMalloc((void**)&lin->scales, n_pad * sizeof(float)));
+    TRY_OR_FAIL(hipMalloc((void**)&lin->zero_points, n_pad * sizeof(int32_t)));
+    TRY_OR_FAIL(hipMalloc((void**)&lin->bias, n_pad * sizeof(int32_t)));
+    TRY_OR_FAIL(hipMalloc((void**)&lin->weight_sums, n_pad * sizeof(int32_t)));
+    TRY_OR_FAIL(hipMemcpy(raw, weight, raw_bytes, hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemcpy(lin->scales, hscale.data(), n_pad * sizeof(float), hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemcpy(lin->zero_points, zps.data(), n_pad * sizeof(int32_t), hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemcpy(lin->bias, hbias.data(), n_pad * sizeof(int32_t), hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemset(lin->weight_sums, 0, n_pad * sizeof(int32_t)));
+    st = weight_row_stats(nullptr, raw, d_in, d_out, d_in, flip, lin->zero_points, lin->weight_sums,
+                          absmax_dev);
+    if (st != VXHIP_OK) return fail(st);
+    st = pack_weight(nullptr, raw, d_in, d_out, d_in, flip, &lin->w);
+    if (st != VXHIP_OK) return fail(st);
+    int32_t absmax = 0;
+    TRY_OR_FAIL(hipMemcpy(&absmax, absmax_dev, sizeof absmax, hipMemcpyDeviceToHost));
+    TRY_OR_FAIL(hipDeviceSynchronize());
+#undef TRY_OR_FAIL
+    lin->weight_abs_max = absmax;
+    (void)hipFree(raw);
+    (void)hipFree(absmax_dev);
+    lin->resident = lin->w.bytes() + (uint64_t)n_pad * 16u;
+    *out = lin;
+    return VXHIP_OK;
+}
+
+// Shared by the per-tensor and the per-row entry points.
+static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* input_dev,
+                       const float* row_scales_dev, const float* bias_f32_dev, void* output_dev,
+                       int32_t* acc_dev, uint32_t rows, float input_scale, int32_t input_zp,
+                       float output_scale, int32_t output_zp, uint32_t input_dtype,
+                       uint32_t output_dtype, bool per_row) {
+    if (!ctx || !lin || !input_dev || (!output_dev && !acc_dev) || !rows) {
+        set_error("qlinear_forward: null handle/tensor or zero rows");
+        return 0;
+    }
+    if (!byte_dtype(input_dtype) || !byte_dtype(output_dtype) || !scale_ok(output_scale) ||
+        !zero_point_ok(input_zp, input_dtype) || !zero_point_ok(output_zp, output_dtype)) {
+        set_error("qlinear_forward: invalid dtype, scale or zero point");
+        return 0;
+    }
+    const uint32_t k = lin->w.k, n = lin->w.n;
+    if (!per_row) {
+        // product and quotient are monotone in s_w, so the extremes decide for every channel
+        if (!scale_ok(input_scale) || !multiplier_ok(input_scale, lin->scale_min, output_scale) ||
+            !multiplier_ok(input_scale, lin->scale_max, output_scale)) {
+            set_error("qlinear_forward: a requantization multiplier is not a positive finite f32");
+            return 0;
+        }
+    } else if (!row_scales_dev) {
+        set_error("qlinear_forward_rowscale: row scales are required");
+        return 0;
+    }
+    // int32 admission: no partial sum can leave int32 when
+    //   K * max|x - zx| * max|w - zw| + max|bias| <= INT32_MAX
+    // (the proof the reference's vector route demands, native/src/kernels/qlinear_w8a8_x86.c:80,92-99)
+    const int64_t lo = input_dtype == VXHIP_DTYPE_I8 ? -128 : 0, hi = input_dtype == VXHIP_DTYPE_I8 ? 127 : 255;
+    const int64_t xmax = llabs(lo - input_zp) > llabs(hi - input_zp) ? llabs(lo - input_zp) : llabs(hi - input_zp);
+    if ((int64_t)k * xmax * lin->weight_abs_max + lin->bias_abs_max > (int64_t)INT32_MAX) {
+        set_error("qlinear_forward: int32 accumulator bound not provable for K=%u", k);
+        return 0;
+    }
+    if (!use_device(ctx->device)) return 0;
+
+    const bool flip = input_dtype == VXHIP_DTYPE_U8;
+    const bool stage = flip || (k % 16u) != 0u || ((uintptr_t)input_dev % 16u) != 0u;
+    const uint32_t ld = stage ? (k + 15u) / 16u * 16u : k;
+    const uint32_t n_pad = lin->w.panels * 32u;
+    Carver sizes{nullptr};
+    sizes.take<int32_t>(rows);
+    sizes.take<int8_t>(stage ? (size_t)rows * ld : 0);
+    if (ensure_scratch(ctx, sizes.off + 256u) != VXHIP_OK) return 0;
+    Carver c{(char*)ctx->scratch};
+    int32_t* rowsum = c.take<int32_t>(rows);
+    int8_t* staged = c.take<int8_t>(stage ? (size_t)rows * ld : 0);
+
+    if (stage || lin->any_zero_point) {
+        if (launch_stage_activations(ctx->stream, input_dev, rows, k, flip, stage ? staged : nullptr, ld,
+                                     lin->any_zero_point ? rowsum : nullptr) != VXHIP_OK)
+            return 0;
+    }
+    LinearArgs a{};
+    a.mode = per_row ? Epilogue::RequantRow : Epilogue::RequantTensor;
+    a.x = stage ? staged : (const int8_t*)input_dev;
+    a.ldx = ld;
+    a.rows = rows;
+    a.n = n;
+    a.k = k;
+    a.w = lin->w.data;
+    a.panels = lin->w.panels;
+    a.ksteps = lin->w.ksteps;
+    a.wscale = lin->scales;
+    a.bias_i32 = lin->bias;
+    a.wsum = lin->weight_sums;
+    a.zw = lin->any_zero_point ? lin->zero_points : nullptr;
+    a.rowsum = rowsum;
+    a.row_scale = row_scales_dev;
+    a.bias_row = bias_f32_dev;
+    a.input_scale = input_scale;
+    a.input_zp = input_zp - (flip ? 128 : 0);
+    a.output_scale = output_scale;
+    a.out_zp = output_zp;
+    a.out_lo = output_dtype == VXHIP_DTYPE_I8 ? -128 : 0;
+    a.out_hi = output_dtype == VXHIP_DTYPE_I8 ? 127 : 255;
+    a.n_pad = n_pad;
+    a.y = output_dev;
+    a.acc_out = acc_dev;
+    a.fault = ctx->fault_dev;
+    const char* id = run_linear(ctx, a);
+    if (!id) {
+        set_error("qlinear_forward: no kernel variant accepts rows=%u k=%u n=%u", rows, k, n);
+        return 0;
+    }
+    ctx->last_variant = id;
+    return 1;
+}
+
+int vxhip_qlinear_forward(VxHipContext* ctx, const VxHipQLinear* lin, const void* input_dev,
+                          void* output_dev, int32_t* acc_dev, uint32_t rows, float input_scale,
+                          int32_t input_zp, float output_scale, int32_t output_zp,
+                          uint32_t input_dtype, uint32_t output_dtype) {
+    return qlinear_run(ctx, lin, input_dev, nullptr, nullptr, output_dev, acc_dev, rows, input_scale,
+                       input_zp, output_scale, output_zp, input_dtype, output_dtype, false);
+}
+
+int vxhip_qlinear_forward_rowscale(VxHipContext* ctx, const VxHipQLinear* lin, const int8_t* input_dev,
+                                   const float* row_scales_dev, const float* bias_f32_dev,
+                                   void* output_dev, int32_t* acc_dev, uint32_t rows,
+                                   float output_scale, int32_t output_zp, uint32_t output_dtype) {
+    return qlinear_run(ctx, lin, input_dev, row_scales_dev, bias_f32_dev, output_dev, acc_dev, rows,
+                       1.0f, 0, output_scale, output_zp, VXHIP_DTYPE_I8, output_dtype, true);
+}
+
+int vxhip_qlinear_i8u8(const void* input, const void* weight, const float* weight_scales,
+                       const int32_t* weight_zero_points, const int32_t* bias, void* output,
+                       uint32_t rows, uint32_t d_in, uint32_t d_out, float input_scale,
+                       int32_t input_zp, float output_scale, int32_t output_zp, uint32_t input_dtype,
+                       uint32_t weight_dtype, uint32_t output_dtype) {
+    // the reference declines a null bias (portable_inference_kernels.inc:978)
+    if (!input || !weight || !bias || !weight_scales || !weight_zero_points || !output || !rows ||
+        !d_in || !d_out || !byte_dtype(input_dtype) || !byte_dtype(weight_dtype) ||
+        !byte_dtype(output_dtype)) {
+        set_error("qlinear_i8u8: null tensor, zero extent or non-byte dtype");
+        return 0;
+    }
+    VxHipContext* ctx = default_context();
+    if (!ctx) return 0;
+    VxHipQLinear* lin = nullptr;
+    if (vxhip_qlinear_create(weight, weight_scales, weight_zero_points, bias, d_in, d_out, weight_dtype,
+                             &lin) != VXHIP_OK)
+        return 0;
+    const size_t in_bytes = (size_t)rows * d_in, out_bytes = (size_t)rows * d_out;
+    void *xd = nullptr, *yd = nullptr;
+    int ok = 0;
+    if (hipMalloc(&xd, in_bytes) == hipSuccess && hipMalloc(&yd, out_bytes) == hipSuccess &&
+        vxhip_memcpy_to_device(ctx, xd, input, in_bytes) == VXHIP_OK) {
+        ok = vxhip_qlinear_forward(ctx, lin, xd, yd, nullptr, rows, input_scale, input_zp, output_scale,
+                                   output_zp, input_dtype, output_dtype);
+        // the caller's output is written only after the whole launch succeeded
+        if (ok && vxhip_memcpy_to_host(ctx, output, yd, out_bytes) != VXHIP_OK) ok = 0;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (xd) (void)hipFree(xd);
+    if (yd) (void)hipFree(yd);
+    vxhip_qlinear_destroy(lin);
+    return ok;
+}
+
+// ---- PackedLinear ---------------------------------------------------------------
+
+void vxhip_packed_linear_destroy(VxHipPackedLinear* pl) {
+    if (!pl) return;
+    (void)hipSetDevice(pl->device);
+    (void)hipDeviceSynchronize();
+    if (pl->w.data) (void)hipFree(pl->w.data);
+    if (pl->scales_t) (void)hipFree(pl->scales_t);
+    if (pl->bias) (void)hipFree(pl->bias);
+    delete pl;
+}
+
+uint64_t vxhip_packed_linear_resident_bytes(const VxHipPackedLinear* pl) { return pl ? pl->resident : 0; }
+
+VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float* scales,
+                                       const float* bias, uint32_t k, uint32_t n, uint32_t group_size,
+                                       uint32_t weight_bits, VxHipPackedLinear** out) {
+    if (!out) return VXHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (!packed_words || !scales || !k || !n) {
+        set_error("packed_linear_create: null tensor or zero extent");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (weight_bits != 8u) {
+        set_error("packed_linear_create: only 8-bit weights run on this backend (got %u)", weight_bits);
+        return VXHIP_BACKEND_UNSUPPORTED;
+    }
+    if (group_size != 32u && group_size != 64u && group_size != 128u && group_size != 256u) {
+        set_error("packed_linear_create: group size %u is not 32/64/128/256", group_size);
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if ((uint64_t)k * n > (uint64_t)1 << 40) return VXHIP_INVALID_ARGUMENT;
+    int device = 0;
+    VXHIP_TRY(hipGetDevice(&device));
+    const uint32_t words = (k + 3u) / 4u;
+    const uint32_t groups = (k + group_size - 1u) / group_size;
+    const uint32_t n_pad = ((n + 31u) / 32u + kPanelPad - 1) / kPanelPad * kPanelPad * 32u;
+    std::vector<float> st((size_t)groups * n_pad, 1.0f), hb(n_pad, 0.0f);
+    for (uint32_t o = 0; o < n; o++) {
+        for (uint32_t g = 0; g < groups; g++) {
+            const float s = scales[(size_t)o * groups + g];
+            if (!isfinite(s)) {
+                set_error("packed_linear_create: scale [%u][%u] is not finite", o, g);
+                return VXHIP_INVALID_ARGUMENT;
+            }
+            st[(size_t)g * n_pad + o] = s;
+        }
+        if (bias) hb[o] = bias[o];
+    }
+    VxHipPackedLinear* pl = new (std::nothrow) VxHipPackedLinear();
+    if (!pl) return VXHIP_OUT_OF_MEMORY;
+    pl->device = device;
+    pl->group_size = group_size;
+    pl->groups = groups;
+    uint8_t* raw = nullptr;
+    const size_t raw_bytes = (size_t)n * words * 4u;
+    auto fail = [&](VxHipStatus s) {
+        if (raw) (void)hipFree(raw);
+        vxhip_packed_linear_destroy(pl);
+        return s;
+    };
+#define TRY_OR_FAIL(expr)                                        \
+    do {                                                         \
+        hipError_t e_ = (expr);                                  \
+        if (e_ != hipSuccess) return fail(hip_status(e_, #expr)); \
+    } while (0)
+    TRY_OR_FAIL(hipMalloc((void**)&raw, raw_bytes));
+    TRY_OR_FAIL(hipMalloc((void**)&pl->scales_t, st.size() * sizeof(float)));
+    TRY_OR_FAIL(hipMalloc((void**)&pl->bias, n_pad * sizeof(float)));
+    TRY_OR_FAIL(hipMemcpy(raw, packed_words, raw_bytes, hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemcpy(pl->scales_t, st.data(), st.size() * sizeof(float), hipMemcpyHostToDevice));
+    TRY_OR_FAIL(hipMemcpy(pl->bias, hb.data(), n_pad * sizeof(float), hipMemcpyHostToDevice));
+    // offset-binary codes: value = code - 128, i.e. the byte with its top bit flipped
+    VxHipStatus s2 = pack_weight(nullptr, raw, (size_t)words * 4u, n, k, true, &pl->w);
+    if (s2 != VXHIP_OK) return fail(s2);
+    TRY_OR_FAIL(hipDeviceSynchronize());
+#undef TRY_OR_FAIL
+    (void)hipFree(raw);
+    pl->resident = pl->w.bytes() + st.size() * sizeof(float) + n_pad * sizeof(float);
+    *out = pl;
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_packed_prepare_i8(VxHipContext* ctx, const float* input_dev, uint32_t rows, uint32_t k,
+                                    int8_t* prepared_dev, float* row_scales_dev) {
+    if (!ctx || !input_dev || !prepared_dev || !row_scales_dev || !k) return VXHIP_INVALID_ARGUMENT;
+    if (!rows) return VXHIP_OK;
+    if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
+    ctx->last_variant = "hip.packed-linear.prepare-i8";
+    return launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared_dev, k, row_scales_dev);
+}
+
+static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const int8_t* a8, uint32_t lda,
+                         const float* row_scales, float* y, int32_t* acc, const int32_t* zeros,
+                         uint32_t rows) {
+    LinearArgs a{};
+    a.mode = Epilogue::DequantF32;
+    a.x = a8;
+    a.ldx = lda;
+    a.rows = rows;
+    a.n = pl->w.n;
+    a.k = pl->w.k;
+    a.w = pl->w.data;
+    a.panels = pl->w.panels;
+    a.ksteps = pl->w.ksteps;
+    a.row_scale = row_scales;
+    a.scales_t = pl->scales_t;
+    a.bias_f32 = pl->bias;
+    a.group_size = pl->group_size;
+    a.groups = pl->groups;
+    a.n_pad = pl->w.panels * 32u;
+    a.y = y;
+    a.fault = ctx->fault_dev;
+    const char* id = nullptr;
+    if (y) {
+        id = run_linear(ctx, a);
+        if (!id) return -1;
+    }
+    if (acc) {
+        // exact full-K int32 sums: the same kernels in requantizing mode with the byte output
+        // off; unit scales and the zero array stand in for the unused per-channel inputs
+        LinearArgs b = a;
+        b.mode = Epilogue::RequantTensor;
+        b.y = nullptr;
+        b.acc_out = acc;
+        b.wscale = pl->bias;
+        b.bias_i32 = zeros;
+        b.wsum = zeros;
+        b.zw = nullptr;
+        b.input_scale = 1.0f;
+        b.input_zp = 0;
+        b.output_scale = 1.0f;
+        b.fault = ctx->fault_dev + 1;  // multipliers are meaningless here: keep them off the real word
+        b.out_lo = -128;
+        b.out_hi = 127;
+        const char* id2 = run_linear(ctx, b);
+        if (!id2) return -1;
+        if (!id) id = id2;
+    }
+    ctx->last_variant = id;
+    return 0;
+}
+
+int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* pl,
+                                   const int8_t* activation_dev, const float* row_scales_dev,
+                                   float* output_dev, int32_t* acc_dev, uint32_t rows) {
+    if (!ctx || !pl || !activation_dev || !row_scales_dev || (!output_dev && !acc_dev)) {
+        set_error("packed_linear_forward_a8: null handle or tensor");
+        return -1;
+    }
+    if (!rows) return 0;
+    if (!use_device(ctx->device)) return -1;
+    const uint32_t k = pl->w.k, n_pad = pl->w.panels * 32u;
+    if (acc_dev && (uint64_t)k * 127u * 128u > (uint64_t)INT32_MAX) {
+        set_error("packed_linear_forward_a8: full-K int32 sums are not provable for K=%u", k);
+        return -1;
+    }
+    const bool stage = (k % 16u) != 0u || ((uintptr_t)activation_dev % 16u) != 0u;
+    const uint32_t ld = stage ? (k + 15u) / 16u * 16u : k;
+    Carver sizes{nullptr};
+    sizes.take<int32_t>(acc_dev ? n_pad : 0);
+    sizes.take<int8_t>(stage ? (size_t)rows * ld : 0);
+    if (ensure_scratch(ctx, sizes.off + 256u) != VXHIP_OK) return -1;
+    Carver c{(char*)ctx->scratch};
+    int32_t* zeros = c.take<int32_t>(acc_dev ? n_pad : 0);
+    int8_t* staged = c.take<int8_t>(stage ? (size_t)rows * ld : 0);
+    // a fill kernel rather than a memset node, so the call stays graph-capturable
+    if (acc_dev && launch_fill_u32(ctx->stream, (uint32_t*)zeros, n_pad, 0u) != VXHIP_OK) return -1;
+    if (stage && launch_stage_activations(ctx->stream, activation_dev, rows, k, false, staged, ld, nullptr) !=
+                     VXHIP_OK)
+        return -1;
+    return packed_run_a8(ctx, pl, stage ? staged : activation_dev, ld, row_scales_dev, output_dev, acc_dev,
+                         zeros, rows);
+}
+
+int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,
+                                    float* output_dev, uint32_t rows) {
+    if (!ctx || !pl || !input_dev || !output_dev) {
+        set_error("packed_linear_forward_f32: null handle or tensor");
+        return -1;
+    }
+    if (!rows) return 0;
+    if (!use_device(ctx->device)) return -1;
+    const uint32_t k = pl->w.k;
+    const uint32_t ld = (k + 15u) / 16u * 16u;
+    Carver sizes{nullptr};
+    sizes.take<float>(rows);
+    sizes.take<int8_t>((size_t)rows * ld);
+    if (ensure_scratch(ctx, sizes.off + 256u) != VXHIP_OK) return -1;
+    Carver c{(char*)ctx->scratch};
+    float* row_scales = c.take<float>(rows);
+    int8_t* prepared = c.take<int8_t>((size_t)rows * ld);
+    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ld, row_scales) != VXHIP_OK) return -1;
+    return packed_run_a8(ctx, pl, prepared, ld, row_scales, output_dev, nullptr, nullptr, rows);
+}
+
+int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, const float* scale,
+                            const float* bias, float* output, uint64_t rows, int32_t key_dim,
+                            int32_t value_dim, int32_t rate, int32_t groups, int32_t normalize) {
+    // descriptor checks of vx_packed_linear_forward (packed_linear_ops.inc:1545-1554)
+    if (!input || !packed_weight || !scale || !output || key_dim <= 0 || value_dim <= 0 || !rows ||
+        rows > 0x7fffffffull)
+        return -1;
+    const uint32_t bits = groups ? (uint32_t)groups : 4u;
+    if (bits != 8u || normalize != 8) {
+        set_error("packed_linear_f32: this backend runs weight_bits=8 under DYNAMIC_I8 only");
+        return -1;
+    }
+    VxHipContext* ctx = default_context();
+    if (!ctx) return -1;
+    VxHipPackedLinear* pl = nullptr;
+    if (vxhip_packed_linear_create(packed_weight, scale, bias, (uint32_t)key_dim, (uint32_t)value_dim,
+                                   (uint32_t)rate, bits, &pl) != VXHIP_OK)
+        return -1;
+    const size_t in_bytes = (size_t)rows * key_dim * 4u, out_bytes = (size_t)rows * value_dim * 4u;
+    void *xd = nullptr, *yd = nullptr;
+    int st = -1;
+    if (hipMalloc(&xd, in_bytes) == hipSuccess && hipMalloc(&yd, out_bytes) == hipSuccess &&
+        vxhip_memcpy_to_device(ctx, xd, input, in_bytes) == VXHIP_OK) {
+        st = vxhip_packed_linear_forward_f32(ctx, pl, (const float*)xd, (float*)yd, (uint32_t)rows);
+        if (st == 0 && vxhip_memcpy_to_host(ctx, output, yd, out_bytes) != VXHIP_OK) st = -1;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (xd) (void)hipFree(xd);
+    if (yd) (void)hipFree(yd);
+    vxhip_packed_linear_destroy(pl);
+    return st;
+}
+
+// ---- boundaries -------------------------------------------------------------------
+
+int vxhip_quantize_forward(VxHipContext* ctx, const float* input_dev, uint32_t elements, void* output_dev,
+                           float scale, int32_t zp, uint32_t dtype) {
+    if (!ctx || !input_dev || !output_dev || !byte_dtype(dtype) || !scale_ok(scale) ||
+        !zero_point_ok(zp, dtype))
+        return 0;
+    if (!use_device(ctx->device)) return 0;
+    ctx->last_variant = "hip.quantize-linear.elementwise";
+    return launch_quantize(ctx->stream, input_dev, elements, output_dev, scale, zp,
+                           dtype == VXHIP_DTYPE_I8) == VXHIP_OK;
+}
+
+int vxhip_dequantize_forward(VxHipContext* ctx, const void* input_dev, uint32_t elements, float scale,
+                             int32_t zp, uint32_t dtype, float* output_dev) {
+    if (!ctx || !input_dev || !output_dev || !byte_dtype(dtype)) return 0;
+    if (!use_device(ctx->device)) return 0;
+    ctx->last_variant = "hip.dequantize-linear.elementwise";
+    return launch_dequantize(ctx->stream, input_dev, elements, scale, zp, dtype == VXHIP_DTYPE_I8,
+                             output_dev) == VXHIP_OK;
+}
+
+int vxhip_quantize_typed_f32_i8u8(const float* input, uint32_t elements, void* output, float scale,
+                                  int32_t zp, uint32_t dtype) {
+    if (!input || !output || !byte_dtype(dtype) || !scale_ok(scale) || !zero_point_ok(zp, dtype)) return 0;
+    if (!elements) return 1;
+    VxHipContext* ctx = default_context();
+    if (!ctx) return 0;
+    void *xd = nullptr, *yd = nullptr;
+    int ok = 0;
+    if (hipMalloc(&xd, (size_t)elements * 4u) == hipSuccess && hipMalloc(&yd, elements) == hipSuccess &&
+        vxhip_memcpy_to_device(ctx, xd, input, (size_t)elements * 4u) == VXHIP_OK) {
+        ok = vxhip_quantize_forward(ctx, (const float*)xd, elements, yd, scale, zp, dtype);
+        if (ok && vxhip_memcpy_to_host(ctx, output, yd, elements) != VXHIP_OK) ok = 0;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (xd) (void)hipFree(xd);
+    if (yd) (void)hipFree(yd);
+    return ok;
+}
+
+int vxhip_dequantize_typed_i8u8_f32(const void* input, uint32_t elements, float scale, int32_t zp,
+                                    uint32_t dtype, float* output) {
+    if (!input || !output || !byte_dtype(dtype)) return 0;
+    if (!elements) return 1;
+    VxHipContext* ctx = default_context();
+    if (!ctx) return 0;
+    void *xd = nullptr, *yd = nullptr;
+    int ok = 0;
+    if (hipMalloc(&xd, elements) == hipSuccess && hipMalloc(&yd, (size_t)elements * 4u) == hipSuccess &&
+        vxhip_memcpy_to_device(ctx, xd, input, elements) == VXHIP_OK) {
+        ok = vxhip_dequantize_forward(ctx, xd, elements, scale, zp, dtype, (float*)yd);
+        if (ok && vxhip_memcpy_to_host(ctx, output, yd, (size_t)elements * 4u) != VXHIP_OK) ok = 0;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (xd) (void)hipFree(xd);
+    if (yd) (void)hipFree(yd);
+    return ok;
+}
+
+}  // extern "C"

@@ -1,0 +1,152 @@
+// Kernels on either side of the linear: activation staging, PackedLinear's
+// dynamic activation quantization
+// and the QuantizeLinear / DequantizeLinear boundaries.  All HBM-bound
+// elementwise or per-row work.
+#include "common.h"
+#include "device_math.h"
+
+namespace vxhip {
+
+// ---- activation staging -----------------------------------------------------
+// Copies raw I8/U8 rows into a 16-byte aligned, zero padded signed buffer and
+// writes each row's sum of signed bytes (the operand-sum term of the
+// zero-point fold, cf. native/src/kernels/qlinear_vnni_kernel.inc:113-116).
+// One wavefront per row.
+__global__ __launch_bounds__(256) void stage_activations_kernel(
+        const uint8_t* __restrict__ x, uint32_t rows, uint32_t k, uint32_t flip,
+        int8_t* __restrict__ staged, uint32_t ld, int32_t* __restrict__ rowsum) {
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63u;
+    if (row >= rows) return;
+    const uint8_t* src = x + (size_t)row * k;
+    int32_t sum = 0;
+    for (uint32_t kk = lane; kk < ld; kk += 64u) {
+        int8_t v = 0;
+        if (kk < k) v = (int8_t)(src[kk] ^ (flip ? 0x80u : 0u));
+        sum += v;
+        if (staged) staged[(size_t)row * ld + kk] = v;
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+    if (lane == 0 && rowsum) rowsum[row] = sum;
+}
+
+VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows, uint32_t k,
+                                     bool flip, int8_t* staged, uint32_t ld, int32_t* rowsum) {
+    hipLaunchKernelGGL(stage_activations_kernel, dim3((rows + 3u) / 4u), dim3(256), 0, s,
+                       (const uint8_t*)x, rows, k, flip ? 1u : 0u, staged, ld, rowsum);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+// ---- PackedLinear activation preparation ------------------------------------
+// One workgroup per row (native/src/kernels/packed_linear_ops.inc:1574-1597):
+//   scale = max|x| / 127 (1.0 for an all-zero row, floored at 2^-126),
+//   code  = ties-to-even(x / scale) clamped to +-127, with a true f32 divide
+//   (multiplying by a reciprocal moves half-way values, ibid. :34-36).
+// A row holding NaN or Inf gets zero codes and a NaN scale, which makes every
+// output of that row NaN downstream as the reference requires (:1495).
+__global__ __launch_bounds__(256) void prepare_i8_kernel(
+        const float* __restrict__ x, uint32_t k, int8_t* __restrict__ prepared, uint32_t ld,
+        float* __restrict__ scales) {
+    __shared__ float wave_max[4];
+    __shared__ uint32_t wave_bad[4];
+    const uint32_t row = blockIdx.x;
+    const float* src = x + (size_t)row * k;
+    float maximum = 0.0f;
+    uint32_t bad = 0u;
+    for (uint32_t j = threadIdx.x; j < k; j += 256u) {
+        const float v = src[j];
+        bad |= finite_f32(v) ? 0u : 1u;
+        maximum = fmaxf(maximum, fabsf(v));  // fmaxf ignores a NaN operand; `bad` records it
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        maximum = fmaxf(maximum, __shfl_down(maximum, off, 64));
+        bad |= __shfl_down(bad, off, 64);
+    }
+    if ((threadIdx.x & 63u) == 0u) {
+        wave_max[threadIdx.x >> 6] = maximum;
+        wave_bad[threadIdx.x >> 6] = bad;
+    }
+    __syncthreads();
+    maximum = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    bad = wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3];
+    float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+    if (scale < 0x1p-126f) scale = 0x1p-126f;
+    int8_t* dst = prepared + (size_t)row * ld;
+    for (uint32_t j = threadIdx.x; j < ld; j += 256u) {
+        int32_t q = 0;
+        if (!bad && j < k) q = packed_round_i8(__fdiv_rn(src[j], scale));
+        dst[j] = (int8_t)q;
+    }
+    if (threadIdx.x == 0) scales[row] = bad ? __builtin_nanf("") : scale;
+}
+
+VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
+                              int8_t* prepared, uint32_t ld, float* scales) {
+    hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(256), 0, s, x, k, prepared, ld, scales);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* p, uint32_t count, uint32_t value) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) p[i] = value;
+}
+
+VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t value) {
+    if (!count) return VXHIP_OK;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, p, count, value);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+// ---- QuantizeLinear / DequantizeLinear --------------------------------------
+// q = saturate(ties-to-even(f32(x / s) + f32(zp))); NaN -> zp; +-Inf saturate
+// (native/src/kernels/quantize_linear_ops.inc:156-169).
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x, uint32_t n,
+                                                       uint8_t* __restrict__ y, float scale,
+                                                       int32_t zp, int32_t lo, int32_t hi) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    int32_t q;
+    if (v != v) {
+        q = zp;
+    } else {
+        const float t = __fadd_rn(__fdiv_rn(v, scale), (float)zp);
+        if (t <= (float)lo) q = lo;
+        else if (t >= (float)hi) q = hi;
+        else q = (int32_t)__builtin_rintf(t);
+    }
+    y[i] = (uint8_t)q;
+}
+
+// y = f32((double)(q - zp) * (double)s)   (quantize_linear_ops.inc:9-16)
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ x, uint32_t n,
+                                                         float scale, int32_t zp, uint32_t is_i8,
+                                                         float* __restrict__ y) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int32_t q = is_i8 ? (int32_t)(int8_t)x[i] : (int32_t)x[i];
+    y[i] = (float)((double)(q - zp) * (double)scale);
+}
+
+VxHipStatus launch_quantize(hipStream_t s, const float* x, uint32_t n, void* y, float scale,
+                            int32_t zp, bool is_i8) {
+    if (!n) return VXHIP_OK;
+    hipLaunchKernelGGL(quantize_kernel, dim3((n + 255u) / 256u), dim3(256), 0, s, x, n,
+                       (uint8_t*)y, scale, zp, is_i8 ? -128 : 0, is_i8 ? 127 : 255);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus launch_dequantize(hipStream_t s, const void* x, uint32_t n, float scale, int32_t zp,
+                              bool is_i8, float* y) {
+    if (!n) return VXHIP_OK;
+    hipLaunchKernelGGL(dequantize_kernel, dim3((n + 255u) / 256u), dim3(256), 0, s,
+                       (const uint8_t*)x, n, scale, zp, is_i8 ? 1u : 0u, y);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+}  // namespace vxhip

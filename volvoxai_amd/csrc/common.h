@@ -1,0 +1,147 @@
+// Internal declarations shared by the translation units of libvxhip_w8a8.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/vxhip_w8a8.h"
+
+namespace vxhip {
+
+// ---- error reporting ----------------------------------------------------
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+VxHipStatus hip_status(hipError_t e, const char* what);
+
+#define VXHIP_TRY(expr)                                            \
+    do {                                                           \
+        hipError_t vxhip_e_ = (expr);                              \
+        if (vxhip_e_ != hipSuccess) return hip_status(vxhip_e_, #expr); \
+    } while (0)
+
+// ---- prepacked weight layout --------------------------------------------
+// Signed int8 weights in MFMA operand order.  The matrix is cut into panels
+// of 32 output channels and steps of 32 input channels; block (panel, step)
+// is 1 KiB and holds, for lane l of a wavefront, the 16 bytes
+//     W[32*panel + l%32][32*step + 16*(l/32) + 0..15]
+// at byte offset 16*l.  One block is exactly one operand of
+// v_mfma_i32_32x32x32_i8, and half a block pair is one operand of
+// v_mfma_i32_16x16x64_i8.  Panels are padded to a multiple of 8 and steps to
+// a multiple of 4 with zero weights, so tiles never need a weight-side bound.
+struct PackedWeight {
+    int8_t* data = nullptr;
+    uint32_t n = 0, k = 0;
+    uint32_t panels = 0;   // padded
+    uint32_t ksteps = 0;   // padded
+    size_t bytes() const { return (size_t)panels * ksteps * 1024u; }
+};
+
+constexpr uint32_t kPanelRows = 32, kStepK = 32, kPanelPad = 8, kStepPad = 4;
+constexpr uint32_t kMaxGemvRows = 16;
+
+enum FaultBits : uint32_t {
+    kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive
+};
+
+}  // namespace vxhip
+
+struct VxHipContext {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    // grow-only scratch (activation staging, per-channel parameters, prepared rows)
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    uint32_t* fault_dev = nullptr;
+    const char* last_variant = "";
+    int cu_count = 0;
+};
+
+struct VxHipQLinear {
+    int device = 0;
+    vxhip::PackedWeight w;
+    uint32_t weight_dtype = 0;
+    float* scales = nullptr;       // [n_pad]
+    int32_t* zero_points = nullptr; // [n_pad], in the signed-byte domain
+    int32_t* bias = nullptr;        // [n_pad]
+    int32_t* weight_sums = nullptr; // [n_pad], sum over k of the signed bytes
+    bool any_zero_point = false;
+    float scale_min = 0.f, scale_max = 0.f;
+    int64_t weight_abs_max = 0;     // max |w - zero_point|
+    int64_t bias_abs_max = 0;
+    uint64_t resident = 0;
+};
+
+struct VxHipPackedLinear {
+    int device = 0;
+    vxhip::PackedWeight w;
+    uint32_t group_size = 0, groups = 0;
+    float* scales_t = nullptr;  // [groups][n_pad], transposed so 4 channels are contiguous
+    float* bias = nullptr;      // [n_pad] (zeros when the node has no bias)
+    uint64_t resident = 0;
+};
+
+namespace vxhip {
+
+VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes);
+
+// pack.hip ------------------------------------------------------------------
+// raw_dev: [n] rows of `row_stride` bytes holding k weight bytes each.
+// flip: XOR 0x80 (U8 or offset-binary source -> signed byte).
+VxHipStatus pack_weight(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
+                        uint32_t n, uint32_t k, bool flip, PackedWeight* out);
+VxHipStatus weight_row_stats(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
+                             uint32_t n, uint32_t k, bool flip, const int32_t* zero_points_signed,
+                             int32_t* sums_dev, int32_t* absmax_dev /* single word */);
+
+// boundary.hip ---------------------------------------------------------------
+VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows, uint32_t k,
+                                     bool flip, int8_t* staged, uint32_t ld, int32_t* rowsum);
+VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
+                              int8_t* prepared, uint32_t ld, float* scales);
+VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t value);
+VxHipStatus launch_quantize(hipStream_t s, const float* x, uint32_t n, void* y, float scale,
+                            int32_t zp, bool is_i8);
+VxHipStatus launch_dequantize(hipStream_t s, const void* x, uint32_t n, float scale, int32_t zp,
+                              bool is_i8, float* y);
+
+// One description for both the GEMM and the GEMV launchers.
+enum class Epilogue : int { RequantTensor = 0, RequantRow = 1, DequantF32 = 2 };
+
+struct LinearArgs {
+    Epilogue mode;
+    const int8_t* x;        // signed activations [rows][ldx]
+    uint32_t ldx;
+    uint32_t rows, n, k;
+    const int8_t* w;        // packed
+    uint32_t panels, ksteps;
+    // requant: per-channel arrays are padded to n_pad and 16-byte aligned
+    const float* wscale;    // [n_pad] weight scales
+    const int32_t* bias_i32;// [n_pad] accumulator-domain bias
+    const int32_t* wsum;    // [n_pad] sum over k of the signed weight bytes
+    const int32_t* zw;      // [n_pad] signed-domain weight zero points, null when all are zero
+    const int32_t* rowsum;  // [rows] sum of signed activations (read only with zw)
+    const float* row_scale; // [rows]  RequantRow / DequantF32: activation scales
+    const float* bias_row;  // [n_pad] RequantRow: optional real-valued bias
+    float input_scale;      // RequantTensor
+    int32_t input_zp;       // RequantTensor, signed-byte domain
+    float output_scale;
+    int32_t out_zp, out_lo, out_hi;
+    // dequant
+    const float* scales_t;  // [groups][n_pad]
+    const float* bias_f32;  // [n_pad]
+    uint32_t group_size, groups, n_pad;
+    // outputs
+    void* y;                // int8/uint8 [rows][n] or float [rows][n]; may be null with acc_out
+    int32_t* acc_out;       // optional int32 [rows][n]
+    uint32_t* fault;
+};
+
+// gemm_mfma.hip / gemv_stream.hip: return the variant id that ran, or null if
+// the shape is outside the kernel's domain (nothing launched).
+const char* launch_gemm_mfma(hipStream_t s, const LinearArgs& a, int cu_count, const char* force);
+const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force);
+
+const char* forced_variant();
+
+}  // namespace vxhip

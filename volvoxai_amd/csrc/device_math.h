@@ -1,0 +1,57 @@
+// Device-side scalar rules of the W8A8 contract.  Every f32 operation that the
+// reference rounds separately is written with an explicit round-to-nearest
+// intrinsic, so the compiler can neither contract a multiply-add into an FMA
+// nor reassociate: a fused value can cross a ties-to-even boundary and change
+// the output byte (reference: native/src/kernels/w8a8_affine.h:133-144).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vxhip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bool scale_valid(float v) {
+    // finite and strictly positive (w8a8_affine.h:63-65)
+    return v > 0.0f && v < __builtin_inff();
+}
+
+// multiplier = f32(f32(s_in * s_w) / s_out)   (w8a8_affine.h:155-181)
+__device__ __forceinline__ float requant_multiplier(float s_in, float s_w, float s_out) {
+    return __fdiv_rn(__fmul_rn(s_in, s_w), s_out);
+}
+
+// t = f32(f32(acc) * mult) + f32(zp)          (w8a8_affine.h:139-144)
+__device__ __forceinline__ float transform_accumulator(int32_t acc, float mult, float zp_f) {
+    return __fadd_rn(__fmul_rn((float)acc, mult), zp_f);
+}
+
+// Saturating ties-to-even round into [lo, hi]; NaN maps to the zero point
+// (w8a8_affine.h:114-131).  v_rndne_f32 is ties-to-even and equals the
+// reference's floor-based rule for every value strictly inside the range.
+__device__ __forceinline__ int32_t requantize(float t, float lo_f, float hi_f, int32_t zp) {
+    if (t != t) return zp;
+    float c = fminf(fmaxf(t, lo_f), hi_f);
+    return (int32_t)__builtin_rintf(c);
+}
+
+// PackedLinear activation code: ties-to-even, clamped to +-127
+// (packed_linear.h:108-116).
+__device__ __forceinline__ int32_t packed_round_i8(float v) {
+    float c = fminf(fmaxf(v, -127.0f), 127.0f);
+    return (int32_t)__builtin_rintf(c);
+}
+
+__device__ __forceinline__ bool finite_f32(float v) {
+    return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u;
+}
+
+__device__ __forceinline__ uint32_t pack4_bytes(int32_t a, int32_t b, int32_t c, int32_t d) {
+    return (uint32_t)(a & 255) | ((uint32_t)(b & 255) << 8) | ((uint32_t)(c & 255) << 16) |
+           ((uint32_t)(d & 255) << 24);
+}
+
+}  // namespace vxhip

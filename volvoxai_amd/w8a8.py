@@ -1,0 +1,275 @@
+"""Host-side mirror of the reference's W8A8 device-op interface over the C ABI.
+
+Names and argument order follow the reference slots they stand in for:
+``qlinear_i8u8`` is VxQLinearI8U8Fn (native/src/backends/w8a8_device_ops.h:15-17),
+``quantize_typed_f32_i8u8`` / ``dequantize_typed_i8u8_f32`` are :31-32, and
+``packed_linear_f32`` takes the PackedLinear fields of VxLLMOpArgs
+(native/src/kernels/llm_ops.h:22-32).  Resident classes (Context, QLinear,
+PackedLinear) take torch CUDA tensors, which only supply device addresses.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from ._lib import library
+
+DTYPE_U8 = 5
+DTYPE_I8 = 6
+
+
+class VxHipError(RuntimeError):
+    pass
+
+
+def _err() -> str:
+    return library().vxhip_last_error().decode(errors="replace")
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise VxHipError(f"{what} failed with status {status}: {_err()}")
+
+
+def _np(a, dtype=None):
+    a = np.ascontiguousarray(a if dtype is None else np.asarray(a, dtype=dtype))
+    return a
+
+
+def _hp(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _dp(t):
+    """Device address of a contiguous torch tensor."""
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "expected a contiguous device tensor"
+    return C.c_void_p(t.data_ptr())
+
+
+def _torch_dtype(code):
+    import torch
+    return torch.int8 if code == DTYPE_I8 else torch.uint8
+
+
+class Context:
+    """Context scope: one stream plus mutable scratch (one thread at a time)."""
+
+    def __init__(self, device: int = 0, stream=None):
+        self._h = C.c_void_p()
+        raw = None
+        if stream is not None:
+            raw = C.c_void_p(stream.cuda_stream)
+        self._stream = stream
+        _check(library().vxhip_context_create(device, raw, C.byref(self._h)), "vxhip_context_create")
+
+    def close(self):
+        if self._h:
+            library().vxhip_context_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def synchronize(self):
+        _check(library().vxhip_context_synchronize(self._h), "vxhip_context_synchronize")
+
+    @property
+    def last_variant(self) -> str:
+        return library().vxhip_context_last_variant(self._h).decode()
+
+    def fault_flags(self) -> int:
+        v = C.c_uint32(0)
+        _check(library().vxhip_context_fault_flags(self._h, C.byref(v)), "vxhip_context_fault_flags")
+        return v.value
+
+
+class QLinear:
+    """Compiled scope of one QLinear/QMatMul/QGemm node: prepacked weights."""
+
+    def __init__(self, weight, weight_scales, weight_zero_points, bias=None, weight_dtype=DTYPE_I8):
+        w = _np(weight)
+        assert w.ndim == 2 and w.dtype in (np.int8, np.uint8)
+        self.d_out, self.d_in = w.shape
+        s = _np(weight_scales, np.float32)
+        z = _np(weight_zero_points, np.int32)
+        b = None if bias is None else _np(bias, np.int32)
+        self._h = C.c_void_p()
+        _check(library().vxhip_qlinear_create(_hp(w), _hp(s), _hp(z), _hp(b), self.d_in, self.d_out,
+                                               weight_dtype, C.byref(self._h)), "vxhip_qlinear_create")
+
+    def close(self):
+        if self._h:
+            library().vxhip_qlinear_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def resident_bytes(self) -> int:
+        return int(library().vxhip_qlinear_resident_bytes(self._h))
+
+    def forward(self, ctx: Context, x, input_scale, input_zero_point, output_scale,
+                output_zero_point, input_dtype=DTYPE_I8, output_dtype=DTYPE_I8, out=None,
+                want_accumulators=False, accumulators=None):
+        import torch
+        rows = x.shape[0]
+        if out is None:
+            out = torch.empty((rows, self.d_out), dtype=_torch_dtype(output_dtype), device=x.device)
+        if want_accumulators and accumulators is None:
+            accumulators = torch.empty((rows, self.d_out), dtype=torch.int32, device=x.device)
+        ok = library().vxhip_qlinear_forward(
+            ctx._h, self._h, _dp(x), _dp(out), _dp(accumulators), rows, float(np.float32(input_scale)),
+            int(input_zero_point), float(np.float32(output_scale)), int(output_zero_point),
+            input_dtype, output_dtype)
+        return (ok, out, accumulators) if want_accumulators else (ok, out)
+
+    def forward_rowscale(self, ctx: Context, x, row_scales, output_scale, output_zero_point=0,
+                         output_dtype=DTYPE_I8, bias_f32=None, out=None, want_accumulators=False,
+                         accumulators=None):
+        import torch
+        rows = x.shape[0]
+        if out is None:
+            out = torch.empty((rows, self.d_out), dtype=_torch_dtype(output_dtype), device=x.device)
+        if want_accumulators and accumulators is None:
+            accumulators = torch.empty((rows, self.d_out), dtype=torch.int32, device=x.device)
+        ok = library().vxhip_qlinear_forward_rowscale(
+            ctx._h, self._h, _dp(x), _dp(row_scales), _dp(bias_f32), _dp(out), _dp(accumulators), rows,
+            float(np.float32(output_scale)), int(output_zero_point), output_dtype)
+        return (ok, out, accumulators) if want_accumulators else (ok, out)
+
+
+class PackedLinear:
+    """Compiled scope of one PackedLinear node (weight_bits=8, DYNAMIC_I8)."""
+
+    def __init__(self, packed_words, scales, bias, k, n, group_size, weight_bits=8):
+        pw = _np(packed_words, np.uint32)
+        sc = _np(scales, np.float32)
+        b = None if bias is None else _np(bias, np.float32)
+        self.k, self.n, self.group_size = int(k), int(n), int(group_size)
+        self._h = C.c_void_p()
+        _check(library().vxhip_packed_linear_create(_hp(pw), _hp(sc), _hp(b), self.k, self.n,
+                                                     self.group_size, weight_bits, C.byref(self._h)),
+               "vxhip_packed_linear_create")
+
+    def close(self):
+        if self._h:
+            library().vxhip_packed_linear_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def resident_bytes(self) -> int:
+        return int(library().vxhip_packed_linear_resident_bytes(self._h))
+
+    def forward_f32(self, ctx: Context, x, out=None):
+        import torch
+        rows = x.shape[0]
+        if out is None:
+            out = torch.empty((rows, self.n), dtype=torch.float32, device=x.device)
+        st = library().vxhip_packed_linear_forward_f32(ctx._h, self._h, _dp(x), _dp(out), rows)
+        return st, out
+
+    def forward_a8(self, ctx: Context, a8, row_scales, out=None, want_accumulators=False,
+                   accumulators=None):
+        import torch
+        rows = a8.shape[0]
+        if out is None:
+            out = torch.empty((rows, self.n), dtype=torch.float32, device=a8.device)
+        if want_accumulators and accumulators is None:
+            accumulators = torch.empty((rows, self.n), dtype=torch.int32, device=a8.device)
+        st = library().vxhip_packed_linear_forward_a8(ctx._h, self._h, _dp(a8), _dp(row_scales),
+                                                       _dp(out), _dp(accumulators), rows)
+        return (st, out, accumulators) if want_accumulators else (st, out)
+
+
+def packed_prepare_i8(ctx: Context, x):
+    import torch
+    rows, k = x.shape
+    a8 = torch.empty((rows, k), dtype=torch.int8, device=x.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    _check(library().vxhip_packed_prepare_i8(ctx._h, _dp(x), rows, k, _dp(a8), _dp(scales)),
+           "vxhip_packed_prepare_i8")
+    return a8, scales
+
+
+# ---- host-pointer drop-ins (numpy in, numpy out) -------------------------------
+
+def qlinear_i8u8(input, weight, weight_scales, weight_zero_points, bias, rows, d_in, d_out,
+                 input_scale, input_zero_point, output_scale, output_zero_point, input_dtype,
+                 weight_dtype, output_dtype):
+    """VxQLinearI8U8Fn with the output returned: (handled, output[rows, d_out])."""
+    x = _np(input)
+    w = _np(weight)
+    s = _np(weight_scales, np.float32)
+    z = _np(weight_zero_points, np.int32)
+    b = None if bias is None else _np(bias, np.int32)
+    out = np.zeros((rows, d_out), dtype=np.int8 if output_dtype == DTYPE_I8 else np.uint8)
+    ok = library().vxhip_qlinear_i8u8(_hp(x), _hp(w), _hp(s), _hp(z), _hp(b), _hp(out), rows, d_in,
+                                      d_out, float(np.float32(input_scale)), int(input_zero_point),
+                                      float(np.float32(output_scale)), int(output_zero_point),
+                                      input_dtype, weight_dtype, output_dtype)
+    return int(ok), out
+
+
+def packed_linear_f32(x, packed_weight, scale, bias, key_dim, value_dim, rate, groups=8, normalize=8):
+    """vx_llm_forward_f32 for a PackedLinear node: (status, out[rows, value_dim])."""
+    xx = _np(x, np.float32)
+    rows = xx.shape[0]
+    pw = _np(packed_weight, np.uint32)
+    sc = _np(scale, np.float32)
+    b = None if bias is None else _np(bias, np.float32)
+    out = np.zeros((rows, value_dim), dtype=np.float32)
+    st = library().vxhip_packed_linear_f32(_hp(xx), _hp(pw), _hp(sc), _hp(b), _hp(out), rows,
+                                           key_dim, value_dim, rate, groups, normalize)
+    return int(st), out
+
+
+def quantize_typed_f32_i8u8(input, scale, zero_point, output_dtype):
+    x = _np(input, np.float32)
+    out = np.zeros(x.shape, dtype=np.int8 if output_dtype == DTYPE_I8 else np.uint8)
+    ok = library().vxhip_quantize_typed_f32_i8u8(_hp(x), x.size, _hp(out), float(np.float32(scale)),
+                                                 int(zero_point), output_dtype)
+    return int(ok), out
+
+
+def dequantize_typed_i8u8_f32(input, scale, zero_point, input_dtype):
+    q = _np(input)
+    out = np.zeros(q.shape, dtype=np.float32)
+    ok = library().vxhip_dequantize_typed_i8u8_f32(_hp(q), q.size, float(np.float32(scale)),
+                                                   int(zero_point), input_dtype, _hp(out))
+    return int(ok), out
+
+
+class _Variant(C.Structure):
+    _fields_ = [("id", C.c_char_p), ("backend", C.c_int32), ("operator_kind", C.c_int32),
+                ("entrypoint_id", C.c_char_p), ("predicate_id", C.c_char_p),
+                ("required_features", C.c_char_p), ("priority", C.c_int32)]
+
+
+def kernel_variants():
+    n = C.c_size_t(0)
+    p = library().vxhip_kernel_variants(C.byref(n))
+    arr = C.cast(p, C.POINTER(_Variant))
+    return [dict(id=arr[i].id.decode(), backend=arr[i].backend, operator_kind=arr[i].operator_kind,
+                 entrypoint_id=arr[i].entrypoint_id.decode(), predicate_id=arr[i].predicate_id.decode(),
+                 required_features=arr[i].required_features.decode(), priority=arr[i].priority)
+            for i in range(n.value)]
+
+
+def force_variant(prefix: str | None):
+    library().vxhip_force_variant((prefix or "").encode())
