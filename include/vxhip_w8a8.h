@@ -62,9 +62,13 @@ const char* vxhip_last_error(void);
 
 /* ---- context scope ---------------------------------------------------- */
 
-/* stream: an existing hipStream_t passed as void* (work is enqueued there and
- * the caller owns synchronisation), or NULL for a context-owned stream. */
-VxHipStatus vxhip_context_create(int32_t device, void* stream,
+/* flags = VXHIP_CONTEXT_OWN_STREAM: the context creates and owns a stream
+ * (`stream` is ignored).  flags = VXHIP_CONTEXT_BORROW_STREAM: work is enqueued
+ * on the caller's hipStream_t passed as void* (NULL names the device's default
+ * stream) and the caller owns its lifetime. */
+#define VXHIP_CONTEXT_OWN_STREAM    0u
+#define VXHIP_CONTEXT_BORROW_STREAM 1u
+VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags,
                                  VxHipContext** out_context);
 void vxhip_context_destroy(VxHipContext* context);
 VxHipStatus vxhip_context_synchronize(VxHipContext* context);

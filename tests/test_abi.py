@@ -39,7 +39,7 @@ def _no_gpu():
 def test_without_device_entry_points_decline_and_say_why():
     lib = library()
     h = C.c_void_p()
-    assert lib.vxhip_context_create(0, None, C.byref(h)) == -6  # BACKEND_UNAVAILABLE
+    assert lib.vxhip_context_create(0, None, 0, C.byref(h)) == -6  # BACKEND_UNAVAILABLE
     assert not h and b"device" in lib.vxhip_last_error()
     x = np.zeros((2, 16), np.int8)
     w = np.zeros((4, 16), np.int8)

@@ -341,9 +341,9 @@ def test_declines_leave_output_untouched():
                   dict(bias=np.full(4, 2**31 - 1, np.int32)), dict(input_dtype=18)):
         ok, y = vx.qlinear_i8u8(**{**base, **patch})
         assert ok == 0 and not y.any(), patch
-    # K beyond the int32 proof: declined before launch
-    big = cases.qlinear_random_case(1, 40000, 4, 4, U8, U8, I8, False)
-    ok, _ = vx.qlinear_i8u8(big["x"], big["w"], big["scales"], big["zps"], big["bias"], 1, 40000, 4, big["s_in"],
+    # K beyond the int32 proof (K * max|x-zx| * max|w-zw| > INT32_MAX): declined before launch
+    big = cases.qlinear_random_case(1, 140000, 4, 4, U8, U8, I8, False)
+    ok, _ = vx.qlinear_i8u8(big["x"], big["w"], big["scales"], big["zps"], big["bias"], 1, 140000, 4, big["s_in"],
                             big["zp_in"], big["s_out"], big["zp_out"], U8, U8, I8)
     assert ok == 0 and b"int32" in vx.library().vxhip_last_error()
 

@@ -37,6 +37,13 @@ def library() -> C.CDLL:
             raise LibraryMissing(
                 f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C volvoxai_amd/csrc`. This package has no non-HIP path.")
+        # PyTorch bundles its own libamdhip64 under the same soname as /opt/rocm's.  Whichever
+        # is mapped first serves the whole process, and torch does not find the GPU when the
+        # system copy got there first -- so where torch exists, let it load its runtime first.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = C.CDLL(str(path))
         _declare(_lib)
     return _lib
@@ -50,7 +57,7 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_device_count": (i32, []),
         "vxhip_device_name": (i32, [i32, C.c_char_p, sz]),
         "vxhip_last_error": (C.c_char_p, []),
-        "vxhip_context_create": (i32, [i32, vp, pp]),
+        "vxhip_context_create": (i32, [i32, vp, u32, pp]),
         "vxhip_context_destroy": (None, [vp]),
         "vxhip_context_synchronize": (i32, [vp]),
         "vxhip_context_last_variant": (C.c_char_p, [vp]),

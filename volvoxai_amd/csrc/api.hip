@@ -78,7 +78,7 @@ struct Carver {
 
 static VxHipContext* default_context() {
     static thread_local VxHipContext* ctx = nullptr;
-    if (!ctx && vxhip_context_create(0, nullptr, &ctx) != VXHIP_OK) ctx = nullptr;
+    if (!ctx && vxhip_context_create(0, nullptr, VXHIP_CONTEXT_OWN_STREAM, &ctx) != VXHIP_OK) ctx = nullptr;
     return ctx;
 }
 
@@ -144,8 +144,8 @@ void vxhip_force_variant(const char* id_prefix) {
 
 // ---- context -----------------------------------------------------------------
 
-VxHipStatus vxhip_context_create(int32_t device, void* stream, VxHipContext** out) {
-    if (!out) return VXHIP_INVALID_ARGUMENT;
+VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags, VxHipContext** out) {
+    if (!out || flags > VXHIP_CONTEXT_BORROW_STREAM) return VXHIP_INVALID_ARGUMENT;
     *out = nullptr;
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) != hipSuccess) {
@@ -162,7 +162,7 @@ VxHipStatus vxhip_context_create(int32_t device, void* stream, VxHipContext** ou
     if (!ctx) return VXHIP_OUT_OF_MEMORY;
     ctx->device = device;
     ctx->cu_count = prop.multiProcessorCount;
-    if (stream) {
+    if (flags == VXHIP_CONTEXT_BORROW_STREAM) {
         ctx->stream = (hipStream_t)stream;
     } else {
         hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);

@@ -81,7 +81,9 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(const LinearArgs a) {
                 const uint32_t g = min(t * 2u, a.groups - 1u), g1 = min(t * 2u + 1u, a.groups - 1u);
                 sbuf[slot][0] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g * a.n_pad + nq);
                 sbuf[slot][1] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g1 * a.n_pad + nq);
-            } else if (slot % GK == 0) {
+            } else if (slot % GK == GK - 1 || t + 1 == t1) {
+                // the scale rides in the slot of the step that closes the group, which is
+                // not refilled until that step's fold has read it
                 const uint32_t g = min(t / GK, a.groups - 1u);
                 sbuf[slot][0] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g * a.n_pad + nq);
             }
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(const LinearArgs a) {
                     if constexpr (F) {
                         // group closes after GK steps (t0 is group aligned) or at the row end
                         if ((i + 1) % GK == 0 || t + i + 1 == t1) {
-                            fold(acc, sbuf[i - (i % GK)][0], (t + i) / GK);
+                            fold(acc, sbuf[i][0], (t + i) / GK);
                             acc = v4i{0, 0, 0, 0};
                         }
                     }

@@ -59,11 +59,12 @@ class Context:
 
     def __init__(self, device: int = 0, stream=None):
         self._h = C.c_void_p()
-        raw = None
-        if stream is not None:
-            raw = C.c_void_p(stream.cuda_stream)
         self._stream = stream
-        _check(library().vxhip_context_create(device, raw, C.byref(self._h)), "vxhip_context_create")
+        if stream is not None:  # borrow the caller's stream (handle 0 is the default stream)
+            raw, flags = C.c_void_p(stream.cuda_stream), 1
+        else:
+            raw, flags = None, 0
+        _check(library().vxhip_context_create(device, raw, flags, C.byref(self._h)), "vxhip_context_create")
 
     def close(self):
         if self._h:
