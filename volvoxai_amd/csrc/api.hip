@@ -413,6 +413,11 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     a.input_scale = input_scale;
     a.input_zp = input_zp - (flip ? 128 : 0);
     a.output_scale = output_scale;
+    // 1/s in double is within 2^-53 of the true quotient, which can never sit that close to
+    // an f32 rounding boundary, so the second rounding gives the correctly rounded f32
+    a.output_scale_recip = (float)(1.0 / (double)output_scale);
+    a.wscale_min = lin->scale_min;
+    a.wscale_max = lin->scale_max;
     a.out_zp = output_zp;
     a.out_lo = output_dtype == VXHIP_DTYPE_I8 ? -128 : 0;
     a.out_hi = output_dtype == VXHIP_DTYPE_I8 ? 127 : 255;
@@ -612,6 +617,8 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
         b.input_scale = 1.0f;
         b.input_zp = 0;
         b.output_scale = 1.0f;
+        b.output_scale_recip = 1.0f;
+        b.wscale_min = b.wscale_max = 1.0f;
         b.fault = ctx->fault_dev + 1;  // multipliers are meaningless here: keep them off the real word
         b.out_lo = -128;
         b.out_hi = 127;

@@ -126,6 +126,8 @@ struct LinearArgs {
     float input_scale;      // RequantTensor
     int32_t input_zp;       // RequantTensor, signed-byte domain
     float output_scale;
+    float output_scale_recip;  // RN(1 / output_scale), correctly rounded by the host
+    float wscale_min, wscale_max;  // extremes of wscale[0..n)
     int32_t out_zp, out_lo, out_hi;
     // dequant
     const float* scales_t;  // [groups][n_pad]
