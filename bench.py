@@ -34,6 +34,13 @@ sys.path.insert(0, str(ROOT / "tests"))
 METRIC = "W8A8 linear int8 TOPS (%MFMA peak) at 4096³; GB/s (%HBM) at M=1"
 PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0     # HBM3E, MI355X
+# HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under
+# profiles/ (each counter scaled by what it reads for a 512 MiB copy kernel).  A counter run
+# cannot share a process with the timed run, so the measured values are carried here.
+MEASURED_TRAFFIC_BYTES = {
+    "gemm_4096x4096x4096": 101_209_592 + 16_957_980,
+    "gemv_1x4096x14336": 62_639_417 + 57_344,
+}
 
 
 def gemv_algorithmic_bytes(m, k, n):
@@ -134,8 +141,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["gemm", "gemv"], default=None,
-                    help="run one leg only (for profiling a single kernel)")
+    ap.add_argument("--only", choices=["gemm", "gemv", "copy"], default=None,
+                    help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
+                         "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (one kernel on one GPU's share of the "
@@ -148,6 +156,15 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.only == "copy":
+        nbytes = 512 << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "launches": args.steps}))
+        return
     ctx = vx.Context(0, torch.cuda.current_stream())
     out = {"metric": METRIC, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
@@ -183,7 +200,7 @@ def main():
                            "M": M, "K": K, "N": N, "variant": ctx.last_variant})
         out["roofline"] = {"bound": "mfma", "achieved": ops / (mean_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS,
                            "unit": "TFLOP/s", "frac": ops / (mean_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
-                           "traffic": None, "kernel": ctx.last_variant, "ops_per_launch": ops,
+                           "traffic": MEASURED_TRAFFIC_BYTES["gemm_4096x4096x4096"], "kernel": ctx.last_variant, "ops_per_launch": ops,
                            "avg_kernel_ms": mean_ms, "median_kernel_ms": med_ms, "min_kernel_ms": min_ms,
                            "note": "int8 TOP/s against the 5.0 POP/s dense int8 MFMA peak"}
         # spot parity on the benchmarked output itself
@@ -233,7 +250,8 @@ def main():
                        "hot_in_cache_GBs": gb / (hmean * 1e-3) / 1e9,
                        "parity_bit_exact": bool((yg.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all())}
         out["roofline_gemv"] = {"bound": "hbm", "achieved": gb / (gmean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                                "unit": "GB/s", "frac": gb / (gmean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                                "unit": "GB/s", "frac": gb / (gmean * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                "traffic": MEASURED_TRAFFIC_BYTES["gemv_1x4096x14336"],
                                 "kernel": ctx.last_variant, "bytes_per_launch": gb, "avg_kernel_ms": gmean,
                                 "median_kernel_ms": gmed, "min_kernel_ms": gmin}
         if args.only == "gemv":

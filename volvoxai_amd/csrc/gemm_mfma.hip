@@ -42,8 +42,10 @@
 #ifndef VXHIP_PROBE_NO_EPILOGUE
 #define VXHIP_PROBE_NO_EPILOGUE 0
 #endif
+// The L2 prefetch of later k-blocks measured slower than leaving it out (the extra
+// requests compete with the real loads), so it is compiled out unless asked for.
 #ifndef VXHIP_PROBE_NO_PREFETCH
-#define VXHIP_PROBE_NO_PREFETCH 0
+#define VXHIP_PROBE_NO_PREFETCH 1
 #endif
 
 namespace vxhip {
