@@ -21,13 +21,13 @@ def test_library_exports_every_declared_symbol():
 def test_kernel_variant_table_shape():
     rows = vx.kernel_variants()
     ids = {r["id"] for r in rows}
-    assert {"hip.qlinear.mfma-i8", "hip.qlinear.gemv-mfma16", "hip.packed-linear.a8-mfma",
-            "hip.packed-linear.a8-gemv-mfma16"} <= ids
+    assert {"hip.qlinear.mfma-i8", "hip.qlinear.gemv-mfma", "hip.packed-linear.a8-mfma",
+            "hip.packed-linear.a8-gemv-mfma"} <= ids
     for r in rows:
         assert r["backend"] == 0 and r["id"].startswith("hip.") and r["priority"] > 0
         assert r["operator_kind"] in (1002, 1005, 1007, 1036)
     # QLinear, QGemm and QMatMul share one kernel family, as upstream's cuda.qlinear.* rows do
-    for fam in ("hip.qlinear.mfma-i8", "hip.qlinear.gemv-mfma16"):
+    for fam in ("hip.qlinear.mfma-i8", "hip.qlinear.gemv-mfma"):
         assert {r["operator_kind"] for r in rows if r["id"] == fam} == {1002, 1005, 1007}
 
 

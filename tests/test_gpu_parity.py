@@ -166,7 +166,7 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
                              c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
     seen = set()
     try:
-        for force in ("gemv.stream", "gemv.splitk", "mfma-i8.t128x128", "mfma-i8.t256x256"):
+        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128", "mfma-i8.t256x256"):
             vx.force_variant(force)
             (ok, y), variant = run_resident_qlinear(vx, ctx, c)
             assert ok == 1 and (y == want).all(), variant
@@ -187,7 +187,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.stream", "gemv.splitk", "a8-mfma.t128x128", "a8-mfma.t256x256"):
+        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -195,7 +195,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert len(seen) >= 3, seen  # split-K is skipped when its ordered-sum buffer would not fit LDS
+    assert len(seen) == 4, seen
     pl.close()
 
 

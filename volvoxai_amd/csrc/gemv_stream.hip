@@ -1,24 +1,26 @@
 // Bandwidth-bound W8A8 linear for decode-shaped M <= 16.  Every weight byte is
 // read exactly once, straight from HBM into MFMA operand registers with
 // coalesced dwordx4 loads (no LDS hop), and multiplied against all M rows at
-// once on v_mfma_i32_16x16x64_i8, whose internal reduction replaces the
+// once on v_mfma_i32_32x32x32_i8, whose internal reduction replaces the
 // cross-lane dot-product reduce.  The GPU counterpart of the reference's
 // single-row route vx_packed_linear_single_row_range
 // (native/src/kernels/packed_linear_ops.inc:1471-1535) and of its M=1 QLinear
 // route (native/src/kernels/qlinear_vnni_kernel.inc:41-127).
 //
-// Work unit: 16 output channels.  A wavefront streams a unit's weights over a
-// K range in steps of 64: lane l supplies the weight operand row l%16, k-chunk
-// l/16 (one dwordx4 from the packed layout) and the activation operand row
-// min(l%16, M-1), same k-chunk (one dwordx4 from the row-major activations,
-// L2-resident).  After a step the lane holds the partial dots of channels
-// 4*(l/16)+0..3 for row l%16.
+// Work split: one workgroup per panel of 32 output channels, split-K over its
+// wavefronts.  A wavefront owns a contiguous run of the panel's 1 KiB blocks
+// (the packed layout of common.h makes a panel's k-steps contiguous), requests
+// up to kDepth of them at once with non-temporal loads -- a plain read of the
+// same bytes is fastest in exactly this shape, 4-8 KiB per wave in flight -- and
+// feeds each block unchanged to the MFMA as the weight operand; the activation
+// operand (row min(l%32, M-1), k-chunk l/32) comes from the L2-resident
+// activation rows.
 //
-// Split-K: with few units (small N) the waves of a workgroup share one unit
-// and split K.  Integer partials add exactly; the f32 group terms of the
-// dequantizing epilogue are parked in LDS and summed in ascending group order
-// by one thread per output, which keeps the result bit-identical to the serial
-// order the reference uses (packed_linear_ops.inc:1498-1504).
+// Split-K reduction: the streaming phase is integer only.  Partial dots add
+// exactly; for the dequantizing epilogue the exact int32 dot of every storage
+// group is parked in LDS and one thread per output then applies the scales and
+// sums in ascending group order, which keeps the result bit-identical to the
+// serial order the reference uses (packed_linear_ops.inc:1498-1504).
 #include "common.h"
 #include "device_math.h"
 #include "epilogue.h"
@@ -26,181 +28,208 @@
 #include <stdio.h>
 #include <string.h>
 
+#ifndef VXHIP_GEMV_DEPTH
+#define VXHIP_GEMV_DEPTH 4
+#endif
+
 namespace vxhip {
 
 namespace {
 
 extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
-constexpr int kDepth = 8;  // k64 steps in flight per wave (8 KiB of weights)
+constexpr int kDepth = VXHIP_GEMV_DEPTH;  // 1 KiB blocks in flight per wave
 
-// MODE: Epilogue.  GK: k64 steps per scale group (1, 2, 4) or 0 for G=32 (two
-// groups per step).  SK: waves of the workgroup sharing one unit (1 or 4).
-template <int MODE, int GK, int SK>
-__global__ __launch_bounds__(256) void gemv_stream_kernel(const LinearArgs a) {
+__device__ __forceinline__ v4i load_stream(const int8_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+}
+
+// MODE: Epilogue.  GK: k-steps of 32 per scale group (1, 2, 4 or 8).  WAVES:
+// wavefronts of the workgroup, all sharing one panel.
+template <int MODE, int GK, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const uint32_t units = (a.n + 15u) / 16u;
-    const uint32_t unit = SK == 1 ? blockIdx.x * 4u + wave : blockIdx.x;
-    const bool active = unit < units;  // inactive waves still reach every barrier
+    const uint32_t panel = blockIdx.x;
+    const uint32_t rows = a.rows;
 
-    const uint32_t steps = (a.k + 63u) / 64u;  // k64 steps that hold real k
-    // K range of this wave, aligned to whole groups
-    uint32_t t0 = 0, t1 = steps;
-    if constexpr (SK > 1) {
-        constexpr uint32_t align = GK > 0 ? GK : 1;
-        const uint32_t chunks = (steps + align - 1) / align;
-        const uint32_t per = (chunks + SK - 1) / SK;
-        t0 = min(wave * per * align, steps);
-        t1 = min((wave + 1) * per * align, steps);
-    }
-    if (!active) t1 = t0;
+    // this wave's run of k-steps, aligned to whole groups
+    const uint32_t steps = (a.k + 31u) / 32u;
+    const uint32_t chunks = (steps + GK - 1) / GK;
+    const uint32_t per = (chunks + WAVES - 1) / WAVES;
+    const uint32_t t0 = min((uint32_t)wave * per * GK, steps);
+    const uint32_t t1 = min((uint32_t)(wave + 1) * per * GK, steps);
 
-    const uint32_t r16 = lane & 15, c = lane >> 4;
-    const uint32_t panel = unit >> 1, half = unit & 1u;
-    // weight operand: 32-row panel blocks of 1 KiB per 32 k; this lane's slot
-    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + (c >> 1)) * 1024u +
-                       (half * 16u + r16 + 32u * (c & 1u)) * 16u;
-    const uint32_t m = min(r16, a.rows - 1u);
+    const int8_t* wp = a.w + (size_t)panel * a.ksteps * 1024u + lane * 16u;
+    const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
     const int8_t* xp = a.x + (size_t)m * a.ldx;
+    const uint32_t half = lane >> 5;
     const uint32_t last_chunk = (a.k - 1u) / 16u;
-    const uint32_t nq = unit * 16u + c * 4u;  // first of the lane's four channels
 
-    float row_scale = 0.0f;
-    if constexpr (MODE != (int)Epilogue::RequantTensor) row_scale = a.row_scale[m];
+    // LDS: F: dots[group][row][32] exact int32 group dots   R: parts[wave][row][32]
+    int32_t* parts = reinterpret_cast<int32_t*>(gemv_lds);
+    const bool row_live = (uint32_t)(lane & 31) < rows;
 
     v4i wbuf[kDepth], xbuf[kDepth];
-    v4f sbuf[kDepth][GK == 0 ? 2 : 1];
     auto issue = [&](int slot, uint32_t t) {
-        wbuf[slot] = *reinterpret_cast<const v4i*>(wp + (size_t)t * 2048u);
-        const uint32_t chunk = min(t * 4u + c, last_chunk);
+        wbuf[slot] = load_stream(wp + (size_t)t * 1024u);
+        const uint32_t chunk = min(t * 2u + half, last_chunk);
         xbuf[slot] = *reinterpret_cast<const v4i*>(xp + chunk * 16u);
-        if constexpr (F) {
-            if constexpr (GK == 0) {
-                const uint32_t g = min(t * 2u, a.groups - 1u), g1 = min(t * 2u + 1u, a.groups - 1u);
-                sbuf[slot][0] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g * a.n_pad + nq);
-                sbuf[slot][1] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g1 * a.n_pad + nq);
-            } else if (slot % GK == GK - 1 || t + 1 == t1) {
-                // the scale rides in the slot of the step that closes the group, which is
-                // not refilled until that step's fold has read it
-                const uint32_t g = min(t / GK, a.groups - 1u);
-                sbuf[slot][0] = *reinterpret_cast<const v4f*>(a.scales_t + (size_t)g * a.n_pad + nq);
-            }
-        }
     };
 
-    v4i acc = {0, 0, 0, 0};
-    float fsum[4] = {0.f, 0.f, 0.f, 0.f};
-    float* terms = reinterpret_cast<float*>(gemv_lds);  // [groups][256], split-K dequant only
-
-    // sum += f32(dot) * (s_a * s_w[n][g])  -- or park the term for the ordered tail
-    auto fold = [&](const v4i& dots, const v4f& sw, uint32_t g) {
-        if constexpr (F) {
+    v16i acc;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float term = __fmul_rn((float)dots[e], __fmul_rn(row_scale, sw[e]));
-                if constexpr (SK == 1) fsum[e] = __fadd_rn(fsum[e], term);
-                else if (g < a.groups) terms[(size_t)g * 256u + lane * 4 + e] = term;
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+
+    // F: the panel's group scales [group][32] are fetched first (they are L2 hits and return
+    // ahead of the HBM stream) and kept in LDS for the tail.
+    constexpr int SCALE_SLOTS = 4;  // per thread; covers groups * 32 <= SCALE_SLOTS * threads
+    float* lds_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)a.groups * rows * 32u;
+    float sc[F ? SCALE_SLOTS : 1];
+    uint32_t sc_base = 0;
+    if constexpr (F) {
+        const uint32_t total = a.groups * 32u;
+        auto fetch = [&](uint32_t e) {
+            return e < total ? a.scales_t[(size_t)(e >> 5) * a.n_pad + panel * 32u + (e & 31u)] : 0.0f;
+        };
+        // many groups on few waves: copy all but the last pass before the stream starts
+        while (total - sc_base > (uint32_t)(SCALE_SLOTS * WAVES * 64)) {
+#pragma unroll
+            for (int u = 0; u < SCALE_SLOTS; u++) {
+                const uint32_t e = sc_base + threadIdx.x + u * WAVES * 64;
+                lds_scales[e] = fetch(e);
             }
+            sc_base += SCALE_SLOTS * WAVES * 64;
+        }
+#pragma unroll
+        for (int u = 0; u < SCALE_SLOTS; u++) sc[u] = fetch(sc_base + threadIdx.x + u * WAVES * 64);
+    }
+
+    // The streaming phase is integer only and the same for every epilogue: the exact dot of
+    // each closed group (F) or of the wave's whole run (R) is parked in LDS.
+    auto park = [&](uint32_t slab) {
+        if (row_live) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                *reinterpret_cast<v4i*>(parts + ((size_t)slab * rows + (lane & 31)) * 32u + q * 8 + half * 4) =
+                    v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
         }
     };
 
 #pragma unroll
     for (int i = 0; i < kDepth; i++)
         if (t0 + i < t1) issue(i, t0 + i);
+    if constexpr (F) {
+#pragma unroll
+        for (int u = 0; u < SCALE_SLOTS; u++) {
+            const uint32_t e = sc_base + threadIdx.x + u * WAVES * 64;
+            if (e < a.groups * 32u) lds_scales[e] = sc[u];
+        }
+    }
 
     for (uint32_t t = t0; t < t1; t += kDepth) {
 #pragma unroll
         for (int i = 0; i < kDepth; i++) {
             if (t + i < t1) {
-                if constexpr (F && GK == 0) {
-                    // two 32-wide groups per step: mask the other half of k
-                    v4i lo = xbuf[i], hi = xbuf[i];
-                    if (c >= 2) lo = v4i{0, 0, 0, 0}; else hi = v4i{0, 0, 0, 0};
-                    const v4i z = {0, 0, 0, 0};
-                    v4i d0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[i], lo, z, 0, 0, 0);
-                    v4i d1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[i], hi, z, 0, 0, 0);
-                    fold(d0, sbuf[i][0], (t + i) * 2u);
-                    fold(d1, sbuf[i][1], (t + i) * 2u + 1u);
-                } else {
-                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wbuf[i], xbuf[i], acc, 0, 0, 0);
-                    if constexpr (F) {
-                        // group closes after GK steps (t0 is group aligned) or at the row end
-                        if ((i + 1) % GK == 0 || t + i + 1 == t1) {
-                            fold(acc, sbuf[i][0], (t + i) / GK);
-                            acc = v4i{0, 0, 0, 0};
-                        }
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wbuf[i], xbuf[i], acc, 0, 0, 0);
+                if constexpr (F) {
+                    // a group closes after GK steps (t0 is group aligned) or at the row end
+                    if ((t + i + 1) % GK == 0 || t + i + 1 == t1) {
+                        park((t + i) / GK);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[r] = 0;
                     }
                 }
                 if (t + i + kDepth < t1) issue(i, t + i + kDepth);
             }
         }
     }
+    if constexpr (!F) park(wave);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
 
-    if constexpr (SK == 1) {
-        if (!active) return;
-        int32_t dot[4] = {acc[0], acc[1], acc[2], acc[3]};
-        int32_t rsum = 0;
-        if constexpr (MODE != (int)Epilogue::DequantF32) {
-            if (a.zw) rsum = a.rowsum[m];
-        }
-        ChannelConsts cc[4];
-        if constexpr (!F) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) cc[e] = channel_consts<MODE>(a, nq + e);
-        }
-        if (r16 < a.rows) store_quad<MODE>(a, r16, nq, dot, fsum, row_scale, rsum, cc);
-    } else {
-        // element e of lane l sits at index 4*l+e; thread tid finishes index tid
-        int32_t* parts = reinterpret_cast<int32_t*>(gemv_lds);  // [SK][256], requant only
-        if constexpr (!F) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) parts[wave * 256 + lane * 4 + e] = acc[e];
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (!active) return;
-        const uint32_t tid = threadIdx.x;
-        const uint32_t l = tid >> 2, e = tid & 3u;
-        const uint32_t om = l & 15u, on = unit * 16u + (l >> 4) * 4u + e;
+    // Tail: one thread per output, index o = row * 32 + channel.  F: sum += f32(dot_g) *
+    // (s_a * s_w[n][g]) in ascending group order with separate roundings
+    // (packed_linear_ops.inc:1498-1504); eight groups' operands are requested before the
+    // first add needs one.
+    for (uint32_t o = threadIdx.x; o < rows * 32u; o += WAVES * 64) {
+        const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
         float rs = 0.0f;
-        if constexpr (MODE != (int)Epilogue::RequantTensor) rs = a.row_scale[min(om, a.rows - 1u)];
+        if constexpr (MODE != (int)Epilogue::RequantTensor) rs = a.row_scale[om];
+        const size_t slab = (size_t)rows * 32u;
         if constexpr (F) {
             float sum = 0.0f;
-            for (uint32_t g = 0; g < a.groups; g++) sum = __fadd_rn(sum, terms[(size_t)g * 256u + tid]);
+            const int32_t* dp = parts + o;
+            const float* sp = lds_scales + (o & 31u);
+            uint32_t g = 0;
+            for (; g + 8u <= a.groups; g += 8u) {
+                int32_t d[8];
+                float sw[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    d[u] = dp[(size_t)(g + u) * slab];
+                    sw[u] = sp[(g + u) * 32u];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+                    sum = __fadd_rn(sum, __fmul_rn((float)d[u], __fmul_rn(rs, sw[u])));
+            }
+            for (; g < a.groups; g++)
+                sum = __fadd_rn(sum, __fmul_rn((float)dp[(size_t)g * slab], __fmul_rn(rs, sp[g * 32u])));
             store_element<MODE>(a, om, on, 0, sum, rs);
         } else {
             int32_t dot = 0;
 #pragma unroll
-            for (int w = 0; w < SK; w++) dot += parts[w * 256 + tid];
+            for (int w = 0; w < WAVES; w++) dot += parts[(size_t)w * slab + o];
             store_element<MODE>(a, om, on, dot, 0.0f, rs);
         }
     }
 }
 
+template <int MODE, int GK, int WAVES>
+bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
+    auto kern = gemv_panel_kernel<MODE, GK, WAVES>;
+    if (lds > 64u * 1024u) {
+        static bool configured = false;
+        if (!configured) {
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
+                hipSuccess)
+                return false;
+            configured = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
+    return hipGetLastError() == hipSuccess;
+}
+
 template <int MODE, int GK>
-const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
-    const uint32_t units = (a.n + 15u) / 16u;
-    bool split = units < (uint32_t)cu_count * 4u;  // fewer than four waves per CU otherwise
-    if (force && strstr(force, "splitk")) split = true;
-    if (force && strstr(force, "stream")) split = false;
-    size_t lds = 0;
-    if (split) {
-        lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * 1024u : 4u * 1024u;
-        if (lds > 64u * 1024u) split = false;
-    }
-    if (split) {
-        hipLaunchKernelGGL((gemv_stream_kernel<MODE, GK, 4>), dim3(units), dim3(256), lds, s, a);
-        return hipGetLastError() == hipSuccess ? "splitk4" : nullptr;
-    }
-    hipLaunchKernelGGL((gemv_stream_kernel<MODE, GK, 1>), dim3((units + 3u) / 4u), dim3(256), 0, s, a);
-    return hipGetLastError() == hipSuccess ? "stream" : nullptr;
+const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
+    const uint32_t steps = (a.k + 31u) / 32u;
+    // Measured at K=4096, N=14336: 4 blocks in flight per wave and 16 blocks per wave (two
+    // workgroups of 8 waves resident per CU) stream fastest; more waves or deeper queues cost
+    // occupancy, fewer leave the memory system short of requests.
+    int waves = steps >= 16u * 16u ? 16 : steps >= 8u * 16u ? 8 : steps >= 4u * 16u ? 4 : 2;
+    if (force && strstr(force, "w16")) waves = 16;
+    else if (force && strstr(force, "w8")) waves = 8;
+    else if (force && strstr(force, "w4")) waves = 4;
+    else if (force && strstr(force, "w2")) waves = 2;
+    const size_t lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * (a.rows + 1u) * 128u
+                                                          : (size_t)waves * a.rows * 128u;
+    // the MFMA GEMM takes shapes whose group dots or scales do not fit
+    if (lds > 156u * 1024u) return nullptr;
+    bool ok = false;
+    if (waves == 16) ok = launch_panel<MODE, GK, 16>(s, a, lds);
+    else if (waves == 8) ok = launch_panel<MODE, GK, 8>(s, a, lds);
+    else if (waves == 4) ok = launch_panel<MODE, GK, 4>(s, a, lds);
+    else ok = launch_panel<MODE, GK, 2>(s, a, lds);
+    return !ok ? nullptr : waves == 16 ? "w16" : waves == 8 ? "w8" : waves == 4 ? "w4" : "w2";
 }
 
 }  // namespace
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
+    (void)cu_count;
     if (a.rows == 0u || a.rows > kMaxGemvRows || a.ldx < 16u || (a.ldx % 16u) != 0u ||
         ((uintptr_t)a.x % 16u) != 0u)
         return nullptr;
@@ -208,20 +237,20 @@ const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count,
     const char* family = nullptr;
     switch (a.mode) {
         case Epilogue::RequantTensor:
-            family = "hip.qlinear.gemv-mfma16";
-            kind = launch_mode<(int)Epilogue::RequantTensor, 1>(s, a, cu_count, force);
+            family = "hip.qlinear.gemv-mfma";
+            kind = launch_mode<(int)Epilogue::RequantTensor, 1>(s, a, force);
             break;
         case Epilogue::RequantRow:
-            family = "hip.qlinear.gemv-mfma16-rowscale";
-            kind = launch_mode<(int)Epilogue::RequantRow, 1>(s, a, cu_count, force);
+            family = "hip.qlinear.gemv-mfma-rowscale";
+            kind = launch_mode<(int)Epilogue::RequantRow, 1>(s, a, force);
             break;
         case Epilogue::DequantF32:
-            family = "hip.packed-linear.a8-gemv-mfma16";
+            family = "hip.packed-linear.a8-gemv-mfma";
             switch (a.group_size) {
-                case 32: kind = launch_mode<(int)Epilogue::DequantF32, 0>(s, a, cu_count, force); break;
-                case 64: kind = launch_mode<(int)Epilogue::DequantF32, 1>(s, a, cu_count, force); break;
-                case 128: kind = launch_mode<(int)Epilogue::DequantF32, 2>(s, a, cu_count, force); break;
-                case 256: kind = launch_mode<(int)Epilogue::DequantF32, 4>(s, a, cu_count, force); break;
+                case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1>(s, a, force); break;
+                case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2>(s, a, force); break;
+                case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4>(s, a, force); break;
+                case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8>(s, a, force); break;
                 default: return nullptr;
             }
             break;
