@@ -273,6 +273,43 @@ def test_prefill_shape_config3_subblocks(ctx, oracle, rows):
     lin.close()
 
 
+@pytest.mark.parametrize("s_out_bits", [0x3D4CCCCD,   # 0.05
+                                        0x3FFFFFFF,   # mantissa all ones
+                                        0x3F800001,   # one ulp above 1
+                                        0x40400000,   # 3.0
+                                        0x3C49BA5E,   # 0.0123
+                                        0x3DE38E39])  # ~1/9
+@pytest.mark.parametrize("zp_out,int_bias", [(0, False), (0, True), (-3, False)])
+def test_rowscale_epilogue_levels_and_divisors(ctx, oracle, s_out_bits, zp_out, int_bias):
+    """The MFMA GEMM picks its requantizing epilogue from the call: no integer terms and a
+    zero output zero point take the shortest one (one-correction division, proved per divisor
+    on the device), otherwise the two-correction or the general one.  Every pick must give the
+    oracle's bytes, for divisors whose reciprocal rounds awkwardly too."""
+    import volvoxai_amd as vx
+    rows, k, n = 160, 384, 256
+    s_out = np.array([s_out_bits], np.uint32).view(np.float32)[0]
+    c = cases.rowscale_case(rows, k, n, 77)
+    # land the outputs inside the byte range whatever the divisor
+    scales = (c["scales"] * (s_out / np.float32(0.05))).astype(np.float32)
+    bias_f32 = (c["bias_f32"] * (s_out / np.float32(0.05))).astype(np.float32)
+    bias_i32 = np.random.default_rng(5).integers(-5000, 5000, n).astype(np.int32) if int_bias else None
+    lin = vx.QLinear(c["w"], scales, c["zps"], bias_i32, I8)
+    vx.force_variant("mfma-i8")
+    try:
+        ok, y = lin.forward_rowscale(ctx, dev(c["x"]), dev(c["row_scales"]), s_out, zp_out, bias_f32=dev(bias_f32))
+        ctx.synchronize()
+    finally:
+        vx.force_variant(None)
+    ok2, want, _ = oracle.qlinear_rowscale(c["x"], c["w"], scales, c["zps"], c["row_scales"], s_out, zp_out,
+                                           bias_i32=bias_i32, bias_f32=bias_f32)
+    assert ok == ok2 == 1 and "mfma-i8-rowscale" in ctx.last_variant
+    y = host(y)
+    assert (y == want).all()
+    assert ((y == 127) | (y == -128)).mean() < 0.5
+    assert ctx.fault_flags() == 0
+    lin.close()
+
+
 def test_outlier_large_k_config5_reduced_rows(ctx, oracle):
     """K=14336, N=4096 with 1% outlier channels scaled x20 before the dynamic
     per-row quantization; 96 rows here (the oracle is scalar), full K and N."""

@@ -174,6 +174,8 @@ VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags, V
     }
     hipError_t e = hipMalloc((void**)&ctx->fault_dev, 256);
     if (e == hipSuccess) e = hipMemset(ctx->fault_dev, 0, 256);
+    if (e == hipSuccess)
+        e = hipMalloc((void**)&ctx->div_proof_dev, VxHipContext::kDivisorSlots * 2 * sizeof(uint32_t));
     if (e != hipSuccess) {
         vxhip_context_destroy(ctx);
         return hip_status(e, "fault word");
@@ -188,6 +190,7 @@ void vxhip_context_destroy(VxHipContext* ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->fault_dev) (void)hipFree(ctx->fault_dev);
+    if (ctx->div_proof_dev) (void)hipFree(ctx->div_proof_dev);
     if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -338,6 +341,24 @@ VxHipStatus vxhip_qlinear_create(const void* weight, const float* weight_scales,
     return VXHIP_OK;
 }
 
+// Mismatch counters of the short divisions by `divisor`, proved on the context's stream the
+// first time the divisor is seen (a few microseconds; later calls find the slot).  The kernels
+// that read them are ordered after the proof by the stream.  Null if the launch failed.
+static const uint32_t* division_proof(VxHipContext* ctx, float divisor, float recip) {
+    uint32_t bits;
+    memcpy(&bits, &divisor, sizeof bits);
+    for (int i = 0; i < ctx->div_used; i++)
+        if (ctx->div_bits[i] == bits) return ctx->div_proof_dev + 2 * i;
+    const int slot = ctx->div_next;
+    uint32_t* counters = ctx->div_proof_dev + 2 * slot;
+    ctx->div_bits[slot] = 0;  // +0.0 is never a divisor: the slot matches nothing until the launch succeeded
+    if (launch_division_proof(ctx->stream, divisor, recip, counters) != VXHIP_OK) return nullptr;
+    ctx->div_bits[slot] = bits;
+    ctx->div_next = (slot + 1) % VxHipContext::kDivisorSlots;
+    if (ctx->div_used < VxHipContext::kDivisorSlots) ctx->div_used++;
+    return counters;
+}
+
 // Shared by the per-tensor and the per-row entry points.
 static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* input_dev,
                        const float* row_scales_dev, const float* bias_f32_dev, void* output_dev,
@@ -416,6 +437,8 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     // 1/s in double is within 2^-53 of the true quotient, which can never sit that close to
     // an f32 rounding boundary, so the second rounding gives the correctly rounded f32
     a.output_scale_recip = (float)(1.0 / (double)output_scale);
+    a.div_proof = per_row ? division_proof(ctx, output_scale, a.output_scale_recip) : nullptr;
+    a.int_bias_zero = lin->bias_abs_max == 0;
     a.wscale_min = lin->scale_min;
     a.wscale_max = lin->scale_max;
     a.out_zp = output_zp;

@@ -100,6 +100,33 @@ VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t
     return VXHIP_OK;
 }
 
+// ---- exactness proof of the short division ------------------------------------
+// Division by a fixed divisor scales exactly with the dividend's exponent (as long as nothing
+// leaves the normal range), so trying all 2^23 mantissas at one exponent decides it for every
+// dividend.  Thread t checks mantissas 4t .. 4t+3.
+__global__ __launch_bounds__(256) void division_proof_kernel(float s, float r, uint32_t* counters) {
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    uint32_t bad1 = 0, bad2 = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        const float p = __uint_as_float(0x3f800000u | (t * 4u + i));
+        const float want = __fdiv_rn(p, s);
+        bad1 += div_by_uniform_once(p, s, r) != want;
+        bad2 += div_by_uniform(p, s, r) != want;
+    }
+    if (bad1) atomicAdd(counters, bad1);
+    if (bad2) atomicAdd(counters + 1, bad2);
+}
+
+VxHipStatus launch_division_proof(hipStream_t s, float divisor, float recip, uint32_t* counters) {
+    VxHipStatus st = launch_fill_u32(s, counters, 2, 0);
+    if (st != VXHIP_OK) return st;
+    hipLaunchKernelGGL(division_proof_kernel, dim3((1u << 23) / 4u / 256u), dim3(256), 0, s, divisor, recip,
+                       counters);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
 // ---- QuantizeLinear / DequantizeLinear --------------------------------------
 // q = saturate(ties-to-even(f32(x / s) + f32(zp))); NaN -> zp; +-Inf saturate
 // (native/src/kernels/quantize_linear_ops.inc:156-169).

@@ -53,6 +53,12 @@ struct VxHipContext {
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
     uint32_t* fault_dev = nullptr;
+    // Exhaustive exactness proofs of the short division sequences, one pair of mismatch
+    // counters per divisor seen (the output scales of the calls made on this context).
+    static constexpr int kDivisorSlots = 16;
+    uint32_t* div_proof_dev = nullptr;          // [kDivisorSlots][2]
+    uint32_t div_bits[kDivisorSlots] = {};      // bit pattern of the divisor proved in each slot
+    int div_used = 0, div_next = 0;
     const char* last_variant = "";
     int cu_count = 0;
 };
@@ -100,6 +106,9 @@ VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows
 VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
                               int8_t* prepared, uint32_t ld, float* scales);
 VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t value);
+// Counts, over every f32 mantissa of the dividend, where the one- and the two-correction
+// division by `divisor` differ from IEEE division: counters[0] and counters[1].
+VxHipStatus launch_division_proof(hipStream_t s, float divisor, float recip, uint32_t* counters);
 VxHipStatus launch_quantize(hipStream_t s, const float* x, uint32_t n, void* y, float scale,
                             int32_t zp, bool is_i8);
 VxHipStatus launch_dequantize(hipStream_t s, const void* x, uint32_t n, float scale, int32_t zp,
@@ -127,6 +136,10 @@ struct LinearArgs {
     int32_t input_zp;       // RequantTensor, signed-byte domain
     float output_scale;
     float output_scale_recip;  // RN(1 / output_scale), correctly rounded by the host
+    // [2] mismatch counts of the one- / two-correction division by output_scale (zero = proved
+    // exact for every dividend mantissa); null = unproved, use IEEE division
+    const uint32_t* div_proof;
+    bool int_bias_zero;     // bias_i32 is all zeros
     float wscale_min, wscale_max;  // extremes of wscale[0..n)
     int32_t out_zp, out_lo, out_hi;
     // dequant

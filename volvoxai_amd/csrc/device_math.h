@@ -38,6 +38,15 @@ __device__ __forceinline__ float div_by_uniform(float p, float s, float r) {
     return __fmaf_rn(e, r, q);
 }
 
+// The same with one correction.  Markstein's theorem makes it exact whenever the first product
+// is already faithful; callers use it only for divisors where launch_division_proof counted no
+// mismatch over all dividend mantissas.
+__device__ __forceinline__ float div_by_uniform_once(float p, float s, float r) {
+    const float q = __fmul_rn(p, r);
+    const float e = __fmaf_rn(-q, s, p);
+    return __fmaf_rn(e, r, q);
+}
+
 // Operands between 2^-60 and 2^60 keep every intermediate of div_by_uniform a
 // normal number (quotient within 2^+-120, residuals 2^-24 below the operands).
 __device__ __forceinline__ bool fast_div_in_range(float v) {

@@ -30,6 +30,7 @@
 #include <string.h>
 
 #include <type_traits>
+#include <utility>
 
 // Compile-time probes used only when tuning (all off in the shipped build):
 // leave out one ingredient of the main loop to see what bounds it.
@@ -39,15 +40,18 @@
 #ifndef VXHIP_PROBE_NO_MFMA
 #define VXHIP_PROBE_NO_MFMA 0
 #endif
+#ifndef VXHIP_PROBE_SAME_KB
+#define VXHIP_PROBE_SAME_KB 0
+#endif
+#ifndef VXHIP_PROBE_CLOCK
+#define VXHIP_PROBE_CLOCK 0
+#endif
+#ifndef VXHIP_PROBE_NO_VMWAIT
+#define VXHIP_PROBE_NO_VMWAIT 0
+#endif
 #ifndef VXHIP_PROBE_NO_EPILOGUE
 #define VXHIP_PROBE_NO_EPILOGUE 0
 #endif
-// The L2 prefetch of later k-blocks measured slower than leaving it out (the extra
-// requests compete with the real loads), so it is compiled out unless asked for.
-#ifndef VXHIP_PROBE_NO_PREFETCH
-#define VXHIP_PROBE_NO_PREFETCH 1
-#endif
-
 namespace vxhip {
 
 namespace {
@@ -75,6 +79,18 @@ struct GemmParams {
     uint32_t tiles_n, tiles_m;
 };
 
+template <int V>
+using IC = std::integral_constant<int, V>;
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(IC<I>{}), ...);
+}
+// f(IC<0>{}), f(IC<1>{}), ... f(IC<N-1>{}): a loop whose index is a compile-time constant
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
 constexpr int KS = 4;  // k-steps of 32 per stage: 128 bytes of k, one cache line per activation row
 
 // WN x WM wavefronts, each owning TN x TM MFMA tiles of 32x32.  MODE is the
@@ -93,7 +109,8 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     const LinearArgs& a = p.a;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // wave-uniform, and known to the compiler as such: everything derived from it is scalar
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int wave_n = wave % WN, wave_m = wave / WN;
 
     // ---- workgroup -> tile, XCD aware ------------------------------------
@@ -101,6 +118,8 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // its own L2).  Give XCD x the x-th contiguous run of tiles, and order
     // tiles so a run is a compact block of the output: that block's operand
     // slices are then shared through one L2 instead of being fetched by all.
+    uint64_t probe_cycles = 0, probe_real = 0, probe_start = 0;
+    if (VXHIP_PROBE_CLOCK) probe_start = __builtin_amdgcn_s_memrealtime();
     const uint32_t total = p.tiles_n * p.tiles_m;
     const uint32_t per_xcd = (total + 7u) / 8u;
     const uint32_t lin = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
@@ -115,43 +134,45 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- per-lane load sources ---------------------------------------------
-    const int8_t* wsrc[WLOADS];
-    uint32_t xoff[XLOADS];
-#pragma unroll
-    for (int i = 0; i < WLOADS; i++) {
-        const int b = wave + i * NWAVES;  // block index inside the weight part: panel-major
-        const int pn = b / KS, s = b % KS;
-        wsrc[i] = a.w + ((size_t)(n0 / 32 + pn) * a.ksteps + s) * 1024u + lane * 16;
-    }
+    // Weights: block b = wave + t*NWAVES of the stage is (panel b/KS, step b%KS); its address is
+    // a uniform base plus the lane's 16*lane.  Activations: a per-lane row offset plus a chunk
+    // offset that is the same for all of a lane's loads of one k-block.
+    const uint32_t w_lane = lane * 16u;
+    const uint32_t panel_bytes = a.ksteps * 1024u;
+    const int8_t* const w_tile = a.w + (size_t)(n0 / 32u) * panel_bytes;
     const uint32_t last_chunk = (a.k - 1u) / 16u;  // rows are readable up to here
     const uint32_t my_chunk = (lane & 7) ^ ((lane >> 3) & 7);  // slot l%8 of row l/8 holds this chunk
+    uint32_t xrow[XLOADS];
 #pragma unroll
     for (int i = 0; i < XLOADS; i++) {
         const int b = wave + i * NWAVES;  // rows 8b .. 8b+7 of the tile
         uint32_t row = m0 + b * 8 + (lane >> 3);
         row = min(row, a.rows - 1u);  // rows past the end compute values nobody stores
-        xoff[i] = row * a.ldx;
+        xrow[i] = row * a.ldx;
     }
     const uint32_t ksteps_real = (a.k + 31u) / 32u;
     const uint32_t nkb = (ksteps_real + KS - 1) / KS;
 
-    auto issue_stage = [&](uint32_t kb, int stage) {
+    // Load t of the NLOADS that make up this wave's share of a stage (weights first).
+    // Blocks past the end are clamped to the last one: such a load refills a stage nobody reads.
+    constexpr int NLOADS = WLOADS + XLOADS;
+    auto issue_one = [&](auto t_tag, uint32_t kb, int stage) {
+        constexpr int t = decltype(t_tag)::value;
         if (VXHIP_PROBE_NO_LOADS && kb > 0) return;
+        kb = min(kb, nkb - 1u);
+        if (VXHIP_PROBE_SAME_KB) kb = kb & 1u;  // same two k-blocks over and over: cache hits only
         char* base = lds_raw + stage * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < WLOADS; i++) {
-            const int b = wave + i * NWAVES;
-            load_to_lds16(wsrc[i] + (size_t)kb * KS * 1024u, base + b * 1024);
-        }
-        // k-chunks past the row end pair with zero weights: clamp the address
-        const uint32_t chunk = min(kb * 8u + my_chunk, last_chunk);
-#pragma unroll
-        for (int i = 0; i < XLOADS; i++) {
-            const int b = wave + i * NWAVES;
-            load_to_lds16(a.x + xoff[i] + chunk * 16u, base + (WBLK + b) * 1024);
+        if constexpr (t < WLOADS) {
+            const uint32_t b = wave + t * NWAVES;
+            const int8_t* src = w_tile + (size_t)(b / KS) * panel_bytes + (size_t)(kb * KS + b % KS) * 1024u;
+            load_to_lds16(src + w_lane, base + b * 1024);
+        } else {
+            // k-chunks past the row end pair with zero weights: clamp the address
+            const uint32_t chunk16 = min(kb * 8u + my_chunk, last_chunk) * 16u;
+            const uint32_t b = wave + (t - WLOADS) * NWAVES;
+            load_to_lds16(a.x + (xrow[t - WLOADS] + chunk16), base + (WBLK + b) * 1024);
         }
     };
-
     // ---- accumulators --------------------------------------------------------
     v16i acc[TN][TM];
     v16i fsum[F32OUT ? TN : 1][F32OUT ? TM : 1];
@@ -219,13 +240,17 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
 #pragma unroll
     for (int s = 0; s < KS; s++) x_slot[s] = (((2u * s + (lane >> 5)) ^ (lane & 7u)) << 4);
 
-    auto read_frags = [&](const char* stage, int s, v4i (&wf)[TN], v4i (&xf)[TM]) {
-#pragma unroll
-        for (int i = 0; i < TN; i++)
+    // fragment r of a k-step, in the order the MFMAs want them: w0, x0 .. x(TM-1), w1 .. w(TN-1)
+    constexpr int READS = TN + TM, MF = TN * TM;
+    auto read_one = [&](auto r_tag, const char* stage, int s, v4i (&wf)[TN], v4i (&xf)[TM]) {
+        constexpr int r = decltype(r_tag)::value;
+        if constexpr (r == 0 || r > TM) {
+            constexpr int i = r == 0 ? 0 : r - TM;
             wf[i] = *reinterpret_cast<const v4i*>(stage + w_frag + (i * KS + s) * 1024);
-#pragma unroll
-        for (int j = 0; j < TM; j++)
+        } else {
+            constexpr int j = r - 1;
             xf[j] = *reinterpret_cast<const v4i*>(stage + x_row + j * 32 * 128 + x_slot[s]);
+        }
     };
 
     // ---- main loop -------------------------------------------------------------
@@ -234,14 +259,17 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // step ahead of the MFMAs that use them), so after the barrier the stage can be refilled
     // for block kb+2 and the first fragments of block kb+1 can be requested while the last
     // MFMAs of block kb still run.  MFMA issue therefore never waits on LDS latency.
-    issue_stage(0, 0);
+    //
+    // The instruction order inside a k-step is written out and fenced (sched_barrier) rather
+    // than left to the scheduler: MFMA m is preceded by the fragment reads and operand loads
+    // whose turn it is, so LDS reads, global->LDS loads and MFMAs issue evenly mixed.
+    static_for<NLOADS>([&](auto t) { issue_one(t, 0, 0); });
     // per-channel epilogue constants of this tile (structure of arrays, so a lane's four
     // consecutive channels are one ds_read_b128 each), computed while the first stage is in flight
     float* lds_f0 = reinterpret_cast<float*>(lds_raw + 2 * STAGE_BYTES);
     int32_t* lds_cb = reinterpret_cast<int32_t*>(lds_f0 + BN);
     float* lds_bo = reinterpret_cast<float*>(lds_cb + BN);
     int32_t* lds_zw = reinterpret_cast<int32_t*>(lds_bo + BN);
-    char* lds_sink = reinterpret_cast<char*>(lds_zw + BN);  // 1 KiB landing pad of the L2 prefetches
     if constexpr (!F32OUT) {
         for (int t = threadIdx.x; t < BN; t += NWAVES * 64) {
             const ChannelConsts c = channel_consts<MODE>(a, n0 + t);
@@ -251,91 +279,90 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             lds_zw[t] = c.zw;
         }
     }
-    // L2 prefetch: the operand slices of a k-block are shared by the workgroups of an XCD, but
-    // the first one to touch a line waits for the fabric.  Touch the lines of block kb+PF_AHEAD
-    // early (one 16-byte piece per 128-byte line, dumped into a scratch pad) so that the real
-    // loads, issued two blocks later, hit in L2.
-    constexpr uint32_t PF_AHEAD = 3;
-    constexpr int PF_LINES = (WBLK * 8 + BM);           // 128-byte lines per stage
-    constexpr int PF_LOADS = (PF_LINES + NWAVES * 64 - 1) / (NWAVES * 64);  // per wave
-    auto prefetch_l2 = [&](uint32_t kb) {
-        if (VXHIP_PROBE_NO_LOADS || VXHIP_PROBE_NO_PREFETCH) return;
-        kb = min(kb, nkb - 1u);
-#pragma unroll
-        for (int i = 0; i < PF_LOADS; i++) {
-            const uint32_t line = min((uint32_t)(i * NWAVES + wave) * 64u + lane, (uint32_t)PF_LINES - 1u);
-            const int8_t* src;
-            if (line < (uint32_t)WBLK * 8u) {  // weight lines: panel-major blocks of 8 lines
-                const uint32_t blk = line >> 3, pn = blk / KS, st = blk % KS;
-                src = a.w + ((size_t)(n0 / 32 + pn) * a.ksteps + kb * KS + st) * 1024u + (line & 7u) * 128u;
+
+    v4i wf[2][TN], xf[2][TM];
+    // One k-step: the MFMAs on fragment buffer S%2; mixed in, the reads of step RS of `rstage`
+    // into the other buffer (if READ) and the first NL operand loads of block load_kb into
+    // load_stage.  (All of a stage's loads go out in the step after the barrier: issuing part
+    // of them a step or two later measured slower, they then land too late.)
+    auto step = [&](auto s_tag, auto read_tag, auto rs_tag, const char* rstage, auto nl_tag, uint32_t load_kb,
+                    int load_stage, uint32_t kb) {
+        constexpr int S = decltype(s_tag)::value, RS = decltype(rs_tag)::value;
+        constexpr bool READ = decltype(read_tag)::value;
+        constexpr int NL = decltype(nl_tag)::value;
+        constexpr int CB = S & 1, NB = CB ^ 1;
+        static_for<MF>([&](auto m_tag) {
+            constexpr int m = decltype(m_tag)::value;
+            constexpr int i = m / TM, j = m % TM;
+            if constexpr (VXHIP_PROBE_NO_MFMA) {
+                acc[i][j][0] += wf[CB][i][0] ^ xf[CB][j][1];
             } else {
-                const uint32_t row = min(m0 + (line - WBLK * 8u), a.rows - 1u);
-                src = a.x + (size_t)row * a.ldx + min(kb * 8u, last_chunk) * 16u;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], acc[i][j], 0, 0, 0);
             }
-            load_to_lds16(src, lds_sink);
-        }
-    };
-    auto mfma_step = [&](int s, uint32_t kb, v4i (&wf)[TN], v4i (&xf)[TM]) {
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int j = 0; j < TM; j++) {
-                if (VXHIP_PROBE_NO_MFMA) {
-                    acc[i][j][0] += wf[i][0] ^ xf[j][1];
-                    continue;
-                }
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i], xf[j], acc[i][j], 0, 0, 0);
+            // after MFMA m: the reads and loads whose slot it is.  Reads keep clear of the
+            // step's last MFMAs, which cover the latency of the final read.
+            if constexpr (READ) {
+                static_for<READS>([&](auto r_tag) {
+                    constexpr int r = decltype(r_tag)::value;
+                    if constexpr ((r * (MF - 1)) / READS == m) read_one(r_tag, rstage, RS, wf[NB], xf[NB]);
+                });
             }
+            if constexpr (NL > 0) {
+                static_for<NL>([&](auto l_tag) {
+                    constexpr int l = decltype(l_tag)::value;
+                    if constexpr ((l * MF) / NL == m) issue_one(l_tag, load_kb, load_stage);
+                });
+            }
+            if constexpr (!F32OUT) __builtin_amdgcn_sched_barrier(0);
+        });
         if constexpr (F32OUT) {
             if constexpr (GK <= KS) {
-                if ((s + 1) % GK == 0) fold_group((kb * KS + s) / GK);
+                if ((S + 1) % GK == 0) fold_group((kb * KS + S) / GK);
             }
         }
     };
-    // interleave the next step's fragment reads with this step's MFMAs
-    auto interleave = [&]() {
-        constexpr int READS = TN + TM, MF = TN * TM, PER = MF / READS;
-#pragma unroll
-        for (int r = 0; r < READS; r++) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // one LDS read
-            __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);  // PER MFMAs
-        }
-        if constexpr (MF - PER * READS > 0) __builtin_amdgcn_sched_group_barrier(0x008, MF - PER * READS, 0);
-    };
 
-    prefetch_l2(1);
-    prefetch_l2(2);
     wait_vmcnt<0>();
     wg_barrier();
-    if (nkb > 1) issue_stage(1, 1);
-    prefetch_l2(PF_AHEAD);
-    v4i wf[2][TN], xf[2][TM];
-    read_frags(lds_raw, 0, wf[0], xf[0]);
-    for (uint32_t kb = 0; kb < nkb; kb++) {
+    if (VXHIP_PROBE_CLOCK) {
+        probe_cycles = __builtin_readcyclecounter();
+        probe_real = __builtin_amdgcn_s_memrealtime();
+    }
+    if (nkb > 1) static_for<NLOADS>([&](auto t) { issue_one(t, 1, 1); });
+    static_for<READS>([&](auto r) { read_one(r, lds_raw, 0, wf[0], xf[0]); });
+    auto k_block = [&](uint32_t kb, auto last_tag) {
+        constexpr bool LAST = decltype(last_tag)::value;
         const int cur = kb & 1;
         const char* stage = lds_raw + cur * STAGE_BYTES;
-#pragma unroll
-        for (int s = 0; s < KS - 1; s++) {
-            read_frags(stage, s + 1, wf[(s + 1) & 1], xf[(s + 1) & 1]);
-            mfma_step(s, kb, wf[s & 1], xf[s & 1]);
-            if constexpr (!F32OUT) interleave();
-        }
-        if (kb + 1 < nkb) {
-            wait_lgkm0();  // my reads of this stage have landed in registers
-            // my loads of the next stage have landed (the prefetches issued after them may still fly)
-            if (VXHIP_PROBE_NO_LOADS || VXHIP_PROBE_NO_PREFETCH) wait_vmcnt<0>(); else wait_vmcnt<PF_LOADS>();
+        static_for<KS - 1>([&](auto s_tag) {
+            constexpr int S = decltype(s_tag)::value;
+            step(s_tag, std::true_type{}, IC<S + 1>{}, stage, IC<0>{}, 0u, 0, kb);
+        });
+        if constexpr (!LAST) {
+            wait_lgkm0();     // my reads of this stage have landed in registers
+            if (!VXHIP_PROBE_NO_VMWAIT) wait_vmcnt<0>();  // my loads of the next stage have landed
             wg_barrier();
-            if (kb + 2 < nkb) issue_stage(kb + 2, cur);
-            prefetch_l2(kb + 1 + PF_AHEAD);
-            read_frags(lds_raw + (cur ^ 1) * STAGE_BYTES, 0, wf[0], xf[0]);
+            step(IC<KS - 1>{}, std::true_type{}, IC<0>{}, lds_raw + (cur ^ 1) * STAGE_BYTES, IC<NLOADS>{},
+                 kb + 2, cur, kb);
+        } else {
+            step(IC<KS - 1>{}, std::false_type{}, IC<0>{}, stage, IC<0>{}, 0u, 0, kb);
         }
-        mfma_step(KS - 1, kb, wf[(KS - 1) & 1], xf[(KS - 1) & 1]);
-        if constexpr (!F32OUT) interleave();
         if constexpr (F32OUT && (GK > KS)) {
             if (((kb + 1) * KS) % GK == 0 || kb + 1 == nkb) fold_group((kb * KS) / GK);
         }
-    }
+    };
+    for (uint32_t kb = 0; kb + 1 < nkb; kb++) k_block(kb, std::false_type{});
+    k_block(nkb - 1u, std::true_type{});
     wait_vmcnt<0>();  // nothing of this workgroup may still be writing LDS when the epilogue reuses it
+    uint64_t probe_loop_end = 0;
+    if (VXHIP_PROBE_CLOCK) {
+        probe_loop_end = __builtin_amdgcn_s_memrealtime();
+        if (blockIdx.x == 8 && threadIdx.x == 0) {
+            // shader cycles and 100 MHz ticks this workgroup's main loop took
+            ((uint64_t*)a.fault)[2] = __builtin_readcyclecounter() - probe_cycles;
+            ((uint64_t*)a.fault)[3] = probe_loop_end - probe_real;
+        }
+    }
     if (VXHIP_PROBE_NO_EPILOGUE) {
         int fold = 0;
 #pragma unroll
@@ -358,7 +385,19 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         const float so = a.output_scale, sr = a.output_scale_recip;
         uint32_t mrow[TM];
         int32_t rsum[TM];
-        bool lean = fast_div_in_range(so) && a.zw == nullptr;
+        // mismatch counts of the one- and two-correction division by the output scale
+        uint32_t miss1 = 1, miss2 = 1;
+        if (MODE == (int)Epilogue::RequantRow && a.div_proof) {
+            miss1 = a.div_proof[0];
+            miss2 = a.div_proof[1];
+        }
+        bool lean = a.zw == nullptr;
+        if constexpr (MODE == (int)Epilogue::RequantRow) lean = lean && fast_div_in_range(so) && miss2 == 0;
+        // BARE on top of LEAN: nothing to add to the accumulator or to the product (an output zero
+        // point of 0 adds +0.0, which changes no value that is rounded afterwards), and for
+        // per-row scales the one-correction division is proved as well
+        const bool no_int_terms = a.int_bias_zero && (MODE == (int)Epilogue::RequantRow || a.input_zp == 0);
+        const bool bare_ok = no_int_terms && a.out_zp == 0 && (MODE != (int)Epilogue::RequantRow || miss1 == 0);
         bool bad = false;
 #pragma unroll
         for (int j = 0; j < TM; j++) {
@@ -376,9 +415,11 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         }
         if (bad) atomicOr(a.fault, (uint32_t)kFaultBadMultiplier);
         const bool wave_lean = __builtin_amdgcn_ballot_w64(!lean) == 0ull;
-        // LEAN: no weight zero points and every quotient in the range of div_by_uniform
-        auto run = [&](auto lean_tag) {
-            constexpr bool LEAN = decltype(lean_tag)::value;
+        // LEVEL 0: general.  1 (LEAN): no weight zero points, every quotient in the range of the
+        // proved short division.  2 (BARE): see above.
+        auto run = [&](auto level_tag) {
+            constexpr int LEVEL = decltype(level_tag)::value;
+            constexpr bool LEAN = LEVEL >= 1, BARE = LEVEL == 2;
 #pragma unroll
             for (int i = 0; i < TN; i++) {
                 uint32_t packed[TM][4];
@@ -389,22 +430,27 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                     const v4i cb = *reinterpret_cast<const v4i*>(lds_cb + c0);
                     v4f bo = {0.f, 0.f, 0.f, 0.f};
                     v4i zw = {0, 0, 0, 0};
-                    if (MODE == (int)Epilogue::RequantRow && a.bias_row) bo = *reinterpret_cast<const v4f*>(lds_bo + c0);
+                    if (MODE == (int)Epilogue::RequantRow && (BARE || a.bias_row)) bo = *reinterpret_cast<const v4f*>(lds_bo + c0);
                     if (!LEAN && a.zw) zw = *reinterpret_cast<const v4i*>(lds_zw + c0);
 #pragma unroll
                     for (int j = 0; j < TM; j++) {
                         uint32_t u[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            uint32_t total = (uint32_t)acc[i][j][q * 4 + e] + (uint32_t)cb[e];
+                            uint32_t total = (uint32_t)acc[i][j][q * 4 + e];
+                            if (!BARE) total += (uint32_t)cb[e];
                             if (!LEAN) total -= (uint32_t)zw[e] * (uint32_t)rsum[j];
                             float mu = f0[e];
                             if constexpr (MODE == (int)Epilogue::RequantRow) {
                                 const float prod = __fmul_rn(row_scale[j], f0[e]);
-                                mu = LEAN ? div_by_uniform(prod, so, sr) : __fdiv_rn(prod, so);
+                                mu = BARE   ? div_by_uniform_once(prod, so, sr)
+                                     : LEAN ? div_by_uniform(prod, so, sr)
+                                            : __fdiv_rn(prod, so);
                             }
-                            float t = __fadd_rn(__fmul_rn((float)(int32_t)total, mu), zp_f);
-                            if (MODE == (int)Epilogue::RequantRow && a.bias_row) t = __fadd_rn(t, bo[e]);
+                            float t = __fmul_rn((float)(int32_t)total, mu);
+                            if (!BARE) t = __fadd_rn(t, zp_f);
+                            // BARE adds the bias term unconditionally: it is +0.0 when there is none
+                            if (MODE == (int)Epilogue::RequantRow && (BARE || a.bias_row)) t = __fadd_rn(t, bo[e]);
                             // A valid multiplier cannot produce NaN here and an invalid one was flagged
                             // above.  Clamp, then round to nearest even by adding 1.5 * 2^23: the sum's
                             // low mantissa bits are the two's-complement integer.
@@ -430,7 +476,9 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                 }
             }
         };
-        if (wave_lean) run(std::true_type{}); else run(std::false_type{});
+        if (wave_lean && bare_ok) run(IC<2>{});
+        else if (wave_lean) run(IC<1>{});
+        else run(IC<0>{});
     } else {
 #pragma unroll
         for (int j = 0; j < TM; j++) {
@@ -465,12 +513,21 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             }
         }
     }
+    if (VXHIP_PROBE_CLOCK && threadIdx.x == 0) {
+        // per workgroup: start, loop begin, loop end, end (100 MHz ticks); the probe build borrows bias_f32
+        __builtin_amdgcn_s_waitcnt(0);
+        uint64_t* o = (uint64_t*)a.bias_f32 + 4 * (size_t)blockIdx.x;
+        o[0] = probe_start;
+        o[1] = probe_real;
+        o[2] = probe_loop_end;
+        o[3] = __builtin_amdgcn_s_memrealtime();
+    }
 }
 
 template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
-    constexpr int LDS = 2 * ((BN / 32) * KS + BM / 8) * 1024 + BN * 16 + 1024;
+    constexpr int LDS = 2 * ((BN / 32) * KS + BM / 8) * 1024 + BN * 16;
     static bool configured = false;
     auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST>;
     if (!configured) {
