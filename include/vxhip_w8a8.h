@@ -80,6 +80,17 @@ const char* vxhip_context_last_variant(const VxHipContext* context);
  * ...); reading it synchronises the stream.  0 = clean. */
 VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
 
+/* Measurement aid with no counterpart in the reference: runs a register-only
+ * v_mfma_i32_32x32x32_i8 loop (16 accumulators per wave, one wave per SIMD,
+ * `rounds` x 16 MFMAs per wave) and reports the int8 rate it reached, the
+ * shader clock it ran at and the launch time.  random_operands != 0 feeds
+ * random 8-bit operand bytes instead of constants; the clock the device then
+ * sustains is the ceiling of any int8 GEMM on such data.  Synchronises the
+ * context's stream. */
+VxHipStatus vxhip_probe_mfma_rate(VxHipContext* context, uint32_t rounds,
+                                  uint32_t random_operands, double* tops,
+                                  double* shader_mhz, double* microseconds);
+
 /* Device memory for hosts without HIP headers. */
 VxHipStatus vxhip_device_malloc(size_t bytes, void** out_device_pointer);
 void vxhip_device_free(void* device_pointer);
@@ -103,6 +114,16 @@ VxHipStatus vxhip_qlinear_create(const void* weight, const float* weight_scales,
 void vxhip_qlinear_destroy(VxHipQLinear* linear);
 /* Bytes of device memory held by the compiled weight (attestation input). */
 uint64_t vxhip_qlinear_resident_bytes(const VxHipQLinear* linear);
+/* 1 if vxhip_qlinear_forward would accept these call scalars for this weight
+ * (dtypes, scales, zero points, every requantization multiplier, and the int32
+ * accumulator proof K*max|x-zx|*max|w-zw| + max|bias| <= INT32_MAX of
+ * src/kernels/qlinear_w8a8_x86.c:80,92-99), else 0 with vxhip_last_error set.
+ * Lets a provider refuse a graph at compile time, where the reference rejects
+ * an unprovable fused operator (docs/w8a8-safetensors.md:158-175, item 8). */
+int vxhip_qlinear_admits(const VxHipQLinear* linear, float input_scale,
+                         int32_t input_zero_point, float output_scale,
+                         int32_t output_zero_point, uint32_t input_dtype,
+                         uint32_t output_dtype);
 
 /* Canonical QLinear on resident buffers (the resident half of
  * cuda_graph_qlinear_i8u8, src/backends/cuda/host/

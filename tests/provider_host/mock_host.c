@@ -1,0 +1,232 @@
+/* Test double of the runtime side of the provider SPI
+ * (native/include/volvoxai_backend.h): accepts a registration under the same
+ * descriptor checks as the reference (native/src/runtime/backend_sdk.c:96-139),
+ * then drives one package through runtime_create -> compile -> context_create
+ * -> context_execute -> destroy the way the reference's lifecycle does, holding
+ * the provider to the contract: identities echoed, route attested, every
+ * declared output written exactly once with the exact name, dtype and shape.
+ * Test infrastructure only. */
+#include "volvoxai_backend.h"
+
+#include <stdio.h>
+#include <string.h>
+
+static VxBackendProvider g_provider;
+static char g_name[VX_BACKEND_NAME_CAPACITY];
+static int g_registered;
+
+static int name_valid(const char* name) {
+    size_t length;
+    if (!name || !name[0]) return 0;
+    length = strlen(name);
+    if (length >= VX_BACKEND_NAME_CAPACITY || name[0] < 'a' || name[0] > 'z') return 0;
+    for (size_t i = 1; i < length; i++) {
+        unsigned char c = (unsigned char)name[i];
+        if (!((c >= 'a' && c <= 'z') || (c >= '0' && c <= '9') || c == '.' || c == '_' || c == '-')) return 0;
+    }
+    return strcmp(name, "cpu") && strcmp(name, "cuda") && strcmp(name, "vulkan") && strcmp(name, "metal");
+}
+
+VX_API VxStatus vx_backend_register_provider(const VxBackendProvider* p, VxReport* report) {
+    if (!report || report->struct_size != sizeof(*report)) return VX_STATUS_INVALID_ARGUMENT;
+    if (p && p->struct_size == sizeof(*p) && p->abi_version != VX_BACKEND_ABI_VERSION) return VX_STATUS_ABI_UNSUPPORTED;
+    if (!p || p->struct_size != sizeof(*p) || p->exact_contract_marker != VX_BACKEND_PROVIDER_EXACT_CONTRACT_MARKER ||
+        p->exact_contract_extent != sizeof(*p) || !name_valid(p->name) || p->flags != 0 ||
+        p->shape_domain.struct_size != sizeof(p->shape_domain) || !p->shape_domain.proof_protocol ||
+        !p->shape_domain.resource_protocol ||
+        strcmp(p->shape_domain.proof_protocol, VX_BACKEND_SHAPE_PROOF_PROTOCOL) ||
+        strcmp(p->shape_domain.resource_protocol, VX_BACKEND_RESOURCE_PROTOCOL) ||
+        (p->shape_domain.support != VX_BACKEND_SHAPE_DOMAIN_FULL &&
+         p->shape_domain.support != VX_BACKEND_SHAPE_DOMAIN_UNSUPPORTED) ||
+        !p->runtime_create || !p->runtime_destroy || !p->compile || !p->compiled_destroy ||
+        (!!p->compiled_batch_contract != !!p->context_execute_batch) || !p->context_create || !p->context_execute ||
+        !p->context_destroy)
+        return VX_STATUS_INVALID_ARGUMENT;
+    if (g_registered && !strcmp(g_name, p->name)) return VX_STATUS_INVALID_ARGUMENT; /* duplicate */
+    g_provider = *p;
+    snprintf(g_name, sizeof(g_name), "%s", p->name);
+    g_provider.name = g_name;
+    g_registered = 1;
+    report->status = VX_STATUS_OK;
+    return VX_STATUS_OK;
+}
+
+/* Calls a provider's registration function with a report of the right layout. */
+int32_t mock_host_register(VxStatus (*register_provider)(VxReport*)) {
+    VxReport report = VX_REPORT_INIT;
+    return register_provider ? (int32_t)register_provider(&report) : (int32_t)VX_STATUS_INVALID_ARGUMENT;
+}
+
+const char* mock_host_registered_name(void) { return g_registered ? g_name : ""; }
+uint32_t mock_host_shape_domain_support(void) { return g_registered ? g_provider.shape_domain.support : 0u; }
+
+typedef struct MockRun {
+    /* in */
+    const char* graph_path;
+    const char* weight_path;
+    int32_t packed_arithmetic;
+    const char* input_name;
+    int32_t input_dtype;
+    uint32_t rank;
+    int64_t input_shape[VX_MAX_TENSOR_RANK];
+    int64_t lead_max[VX_MAX_TENSOR_RANK]; /* > 0: that leading axis is symbolic, bounded 1..lead_max */
+    const void* input;
+    uint64_t input_bytes;
+    const char* output_name;
+    int32_t output_dtype;
+    int64_t output_last;
+    void* output;
+    uint64_t output_capacity;
+    int32_t executions;
+    /* out */
+    int32_t status;
+    int32_t failed_stage; /* VxStage of the callback that failed */
+    uint64_t output_bytes;
+    int32_t writes;
+    int32_t sink_mismatch;
+    int32_t compile_attested, execute_attested, identities_echoed, attested_arithmetic;
+    uint64_t maximum_tensor_bytes, maximum_resident_bytes;
+    char message[VX_REPORT_MESSAGE_CAPACITY];
+    char compile_route[VX_REPORT_ROUTE_CAPACITY];
+    char execute_route[VX_REPORT_ROUTE_CAPACITY];
+    char device[VX_REPORT_DEVICE_CAPACITY];
+} MockRun;
+
+static VxStatus sink_write(void* user, const char* name, VxDataType dtype, const int64_t* shape, uint32_t rank,
+                           const void* data, size_t bytes) {
+    MockRun* run = (MockRun*)user;
+    run->writes++;
+    if (!name || strcmp(name, run->output_name) || (int32_t)dtype != run->output_dtype || rank != run->rank || !data ||
+        bytes > run->output_capacity || shape[rank - 1] != run->output_last) {
+        run->sink_mismatch = 1;
+        return VX_STATUS_INVALID_ARGUMENT;
+    }
+    for (uint32_t a = 0; a + 1 < rank; a++)
+        if (shape[a] != run->input_shape[a]) {
+            run->sink_mismatch = 1;
+            return VX_STATUS_INVALID_ARGUMENT;
+        }
+    memcpy(run->output, data, bytes); /* the sink copies before write returns */
+    run->output_bytes = bytes;
+    return VX_STATUS_OK;
+}
+
+static void spec_from(VxTensorSpec* spec, const char* name, int32_t dtype, const MockRun* run, int64_t last) {
+    memset(spec, 0, sizeof(*spec));
+    spec->struct_size = sizeof(*spec);
+    spec->name = name;
+    spec->dtype = (VxDataType)dtype;
+    spec->rank = run->rank;
+    spec->location = VX_MEMORY_HOST;
+    for (uint32_t a = 0; a < run->rank; a++) {
+        VxDimensionConstraint* d = &spec->dimensions[a];
+        d->struct_size = sizeof(*d);
+        d->multiple_of = 1;
+        if (a + 1 < run->rank && run->lead_max[a] > 0) {
+            d->kind = VX_DIMENSION_SYMBOLIC;
+            d->symbol = "rows";
+            d->min = 1;
+            d->max = run->lead_max[a];
+        } else {
+            d->kind = VX_DIMENSION_FIXED;
+            d->symbol = NULL;
+            d->min = d->max = a + 1 < run->rank ? run->input_shape[a] : last;
+        }
+    }
+}
+
+int32_t mock_host_run(MockRun* run) {
+    static const char fingerprint[] = "sha256:mock-graph-fingerprint";
+    static const char proof[] = "sha256:mock-shape-domain-proof";
+    VxRuntimeOptions runtime_options = VX_RUNTIME_OPTIONS_INIT;
+    VxContextOptions context_options = VX_CONTEXT_OPTIONS_INIT;
+    VxReport report = VX_REPORT_INIT;
+    VxModelSource source = VX_MODEL_SOURCE_INIT;
+    VxBackendCompileInput input = VX_BACKEND_COMPILE_INPUT_INIT;
+    VxBackendShapeDomainAttestation attestation = VX_BACKEND_SHAPE_DOMAIN_ATTESTATION_INIT;
+    VxBackendPolicy policy = VX_BACKEND_POLICY_INIT;
+    VxTensorSpec in_spec, out_spec;
+    VxTensorBinding binding = VX_TENSOR_BINDING_INIT;
+    VxBackendOutputSink sink = {sizeof(VxBackendOutputSink), run, sink_write};
+    const char* weights[1];
+    const char* wanted[1];
+    void *runtime = NULL, *compiled = NULL, *context = NULL;
+    VxStatus status;
+    if (!g_registered) return run->status = VX_STATUS_NOT_FOUND;
+    run->writes = 0;
+    run->sink_mismatch = 0;
+
+    status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
+    run->failed_stage = VX_STAGE_RUNTIME_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+
+    weights[0] = run->weight_path;
+    source.graph_path = run->graph_path;
+    source.weight_paths = weights;
+    source.weight_path_count = 1;
+    spec_from(&in_spec, run->input_name, run->input_dtype, run, run->input_shape[run->rank - 1]);
+    spec_from(&out_spec, run->output_name, run->output_dtype, run, run->output_last);
+    input.source = &source;
+    input.graph_fingerprint = fingerprint;
+    input.shape_domain_proof_identity = proof;
+    input.inputs = &in_spec;
+    input.input_count = 1;
+    input.outputs = &out_spec;
+    input.output_count = 1;
+    input.packed_arithmetic = (VxPackedArithmetic)run->packed_arithmetic;
+    wanted[0] = g_name;
+    policy.mode = VX_BACKEND_REQUIRE;
+    policy.operator_fallback = VX_OPERATOR_FALLBACK_FORBID;
+    policy.backends = wanted;
+    policy.backend_count = 1;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.compile(runtime, &input, &policy, &compiled, &attestation, &report);
+    run->failed_stage = VX_STAGE_COMPILE;
+    if (status != VX_STATUS_OK) {
+        if (compiled) status = VX_STATUS_INTERNAL; /* a failed compile must not leave an instance */
+        goto done;
+    }
+    run->compile_attested = report.route_attested && !report.operator_fallback_used && report.route_evidence[0] &&
+                            report.device[0];
+    snprintf(run->compile_route, sizeof(run->compile_route), "%s", report.route_evidence);
+    snprintf(run->device, sizeof(run->device), "%s", report.device);
+    run->identities_echoed = attestation.graph_fingerprint && attestation.shape_domain_proof_identity &&
+                             !strcmp(attestation.graph_fingerprint, fingerprint) &&
+                             !strcmp(attestation.shape_domain_proof_identity, proof);
+    run->attested_arithmetic = attestation.packed_arithmetic;
+    run->maximum_tensor_bytes = attestation.maximum_tensor_bytes;
+    run->maximum_resident_bytes = attestation.maximum_resident_bytes;
+
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_create(compiled, &context_options, &context, &report);
+    run->failed_stage = VX_STAGE_CONTEXT_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+
+    binding.name = run->input_name;
+    binding.dtype = (VxDataType)run->input_dtype;
+    binding.rank = run->rank;
+    memcpy(binding.shape, run->input_shape, sizeof(binding.shape));
+    binding.data = run->input;
+    binding.byte_size = (size_t)run->input_bytes;
+    binding.location = VX_MEMORY_HOST;
+    run->failed_stage = VX_STAGE_EXECUTE;
+    for (int32_t i = 0; i < (run->executions > 0 ? run->executions : 1) && status == VX_STATUS_OK; i++) {
+        const int32_t before = run->writes;
+        report = (VxReport)VX_REPORT_INIT;
+        status = g_provider.context_execute(context, &binding, 1, &sink, &report);
+        if (status == VX_STATUS_OK && (run->writes != before + 1 || run->sink_mismatch)) status = VX_STATUS_EXECUTION_FAILED;
+        run->execute_attested = report.route_attested && report.route_evidence[0];
+        snprintf(run->execute_route, sizeof(run->execute_route), "%s", report.route_evidence);
+    }
+    if (status == VX_STATUS_OK) run->failed_stage = VX_STAGE_NONE;
+
+done:
+    snprintf(run->message, sizeof(run->message), "%s", report.message);
+    if (context) {
+        if (g_provider.context_close) (void)g_provider.context_close(context, &report);
+        g_provider.context_destroy(context);
+    }
+    if (compiled) g_provider.compiled_destroy(compiled);
+    if (runtime) g_provider.runtime_destroy(runtime);
+    return run->status = status;
+}

@@ -1,0 +1,373 @@
+"""The backend provider (volvoxai_amd/provider) driven through a test double of the
+runtime side of the reference's provider SPI (tests/provider_host/mock_host.c).
+
+Without a GPU: registration, package reading and every refusal.  With a GPU: whole
+packages from graph.json + SafeTensors to output bytes, against the literal KAT of
+tests/parity/external/quantized_oracle.py:34-41,89-103 and against the oracle.
+"""
+import ctypes as C
+import json
+import struct
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import _cases as cases
+
+ROOT = Path(__file__).resolve().parent.parent
+PROVIDER = ROOT / "volvoxai_amd" / "lib" / "libvxhip_provider.so"
+MOCK = ROOT / "tests" / "provider_host" / "libvx_mock_host.so"
+
+pytestmark = pytest.mark.skipif(not (PROVIDER.exists() and MOCK.exists()),
+                                reason="provider and mock host are built where the reference's headers are present")
+
+DT = {"u8": 5, "i8": 6, "i32": 16, "f32": 18}
+ARITH = {"dynamic_i8": 1, "f16": 2, "f32": 3, "f32_fast": 4, "dynamic_i4": 5}
+ST = {-1: "INVALID_ARGUMENT", -4: "IO_ERROR", -5: "INVALID_GRAPH", -6: "BACKEND_UNAVAILABLE", -7: "BACKEND_UNSUPPORTED"}
+
+
+class MockRun(C.Structure):
+    _fields_ = [("graph_path", C.c_char_p), ("weight_path", C.c_char_p), ("packed_arithmetic", C.c_int32),
+                ("input_name", C.c_char_p), ("input_dtype", C.c_int32), ("rank", C.c_uint32),
+                ("input_shape", C.c_int64 * 8), ("lead_max", C.c_int64 * 8), ("input", C.c_void_p),
+                ("input_bytes", C.c_uint64), ("output_name", C.c_char_p), ("output_dtype", C.c_int32),
+                ("output_last", C.c_int64), ("output", C.c_void_p), ("output_capacity", C.c_uint64),
+                ("executions", C.c_int32),
+                ("status", C.c_int32), ("failed_stage", C.c_int32), ("output_bytes", C.c_uint64),
+                ("writes", C.c_int32), ("sink_mismatch", C.c_int32), ("compile_attested", C.c_int32),
+                ("execute_attested", C.c_int32), ("identities_echoed", C.c_int32),
+                ("attested_arithmetic", C.c_int32), ("maximum_tensor_bytes", C.c_uint64),
+                ("maximum_resident_bytes", C.c_uint64), ("message", C.c_char * 256),
+                ("compile_route", C.c_char * 512), ("execute_route", C.c_char * 512), ("device", C.c_char * 128)]
+
+
+class ModelSource(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("graph_path", C.c_char_p), ("weight_paths", C.POINTER(C.c_char_p)),
+                ("weight_path_count", C.c_size_t), ("bank_residency", C.c_void_p), ("bank_residency_count", C.c_size_t)]
+
+
+@pytest.fixture(scope="module")
+def host():
+    import volvoxai_amd as vx
+    vx.library()  # brings in the HIP runtime in the right order
+    mock = C.CDLL(str(MOCK), mode=C.RTLD_GLOBAL)
+    provider = C.CDLL(str(PROVIDER))
+    mock.mock_host_registered_name.restype = C.c_char_p
+    mock.mock_host_run.argtypes = [C.POINTER(MockRun)]
+    provider.volvoxai_hip_gfx950_inspect_package.argtypes = [
+        C.POINTER(ModelSource), C.c_int32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_int32),
+        C.c_char_p, C.c_size_t]
+    return mock, provider, None
+
+
+def write_safetensors(path, tensors):
+    names = {np.dtype(np.int8): "I8", np.dtype(np.uint8): "U8", np.dtype(np.int32): "I32",
+             np.dtype(np.uint32): "U32", np.dtype(np.float32): "F32"}
+    header, blobs, offset = {}, [], 0
+    for name, arr in tensors.items():
+        arr = np.ascontiguousarray(arr)
+        dtype = names[arr.dtype]
+        if name.endswith("#as_i32"):  # packed words are stored as I32
+            name, dtype = name[:-7], "I32"
+        raw = arr.tobytes()
+        header[name] = {"dtype": dtype, "shape": list(arr.shape), "data_offsets": [offset, offset + len(raw)]}
+        blobs.append(raw)
+        offset += len(raw)
+    text = json.dumps(header, separators=(",", ":")).encode()
+    text += b" " * (-len(text) % 8)
+    Path(path).write_bytes(struct.pack("<Q", len(text)) + text + b"".join(blobs))
+
+
+def qlinear_package(tmp, x_shape, w, scales, zps, bias, s_in, zp_in, s_out, zp_out, in_dtype="int8", out_dtype="int8",
+                    mutate=None, op="QLinear", rows_symbol=False):
+    d_out, d_in = w.shape
+    np_of = {"int8": np.int8, "uint8": np.uint8}
+    graph = {
+        "format": "volvox-graph/v1", "dimensions": {},
+        "inputs": {"hidden_q": {"shape": list(x_shape), "dtype": in_dtype}},
+        "nodes": [{"id": "projection", "opType": op,
+                   "inputs": {"input": "hidden_q", "weight": "projection.weight", "bias": "projection.bias"},
+                   "outputs": {"out": {"tensor": "projected_q", "shape": list(x_shape[:-1]) + [d_out], "dtype": out_dtype}},
+                   "params": {}}],
+        "outputs": ["projected_q"],
+        "quantization": {"format": "volvox-affine-safetensors/v1", "tensors": {
+            "hidden_q": {"scheme": "per_tensor", "scale_tensor": "__quant__.hidden.scale",
+                         "zero_point_tensor": "__quant__.hidden.zero_point"},
+            "projection.weight": {"scheme": "per_axis", "axis": 0, "scale_tensor": "__quant__.projection.weight.scale",
+                                  "zero_point_tensor": "__quant__.projection.weight.zero_point"},
+            "projected_q": {"scheme": "per_tensor", "scale_tensor": "__quant__.projected.scale",
+                            "zero_point_tensor": "__quant__.projected.zero_point"}}},
+        "execution": {"stateless": {}, "entrypoints": [{"name": "evaluate", "effect": 1, "allowed_ranges": [1],
+                                                         "inputs": ["hidden_q"], "outputs": ["projected_q"]}]}}
+    tensors = {
+        "projection.weight": w, "projection.bias": np.asarray(bias, np.int32),
+        "__quant__.hidden.scale": np.array([s_in], np.float32),
+        "__quant__.hidden.zero_point": np.array([zp_in], np_of[in_dtype]),
+        "__quant__.projection.weight.scale": np.asarray(scales, np.float32),
+        "__quant__.projection.weight.zero_point": np.asarray(zps).astype(w.dtype),
+        "__quant__.projected.scale": np.array([s_out], np.float32),
+        "__quant__.projected.zero_point": np.array([zp_out], np_of[out_dtype])}
+    if rows_symbol:
+        graph["dimensions"] = {"rows": {"min": 1, "max": 64}}
+        graph["inputs"]["hidden_q"]["shape"][0] = "rows"
+        graph["nodes"][0]["outputs"]["out"]["shape"][0] = "rows"
+    if mutate:
+        mutate(graph, tensors)
+    tmp.mkdir(parents=True, exist_ok=True)
+    (tmp / "graph.json").write_text(json.dumps(graph, separators=(",", ":")) + "\n")
+    write_safetensors(tmp / "model.safetensors", tensors)
+    return tmp / "graph.json", tmp / "model.safetensors"
+
+
+def packed_package(tmp, x_shape, words, scales, bias, group, bits=8, mutate=None):
+    n = words.shape[0]
+    graph = {
+        "format": "volvox-graph/v1", "dimensions": {},
+        "inputs": {"x": {"shape": list(x_shape), "dtype": "float32"}},
+        "nodes": [{"id": "packed", "opType": "PackedLinear",
+                   "inputs": {"input": "x", "weight": "w", "scale": "s", "bias": "b"},
+                   "outputs": {"out": {"tensor": "logits", "shape": list(x_shape[:-1]) + [n], "dtype": "float32"}},
+                   "params": {"group_size": group, "weight_bits": bits}}],
+        "outputs": ["logits"],
+        "execution": {"stateless": {}, "entrypoints": [{"name": "evaluate", "effect": 1, "allowed_ranges": [1],
+                                                         "inputs": ["x"], "outputs": ["logits"]}]}}
+    tensors = {"w#as_i32": words.astype(np.uint32), "s": scales.astype(np.float32), "b": bias.astype(np.float32)}
+    if mutate:
+        mutate(graph, tensors)
+    tmp.mkdir(parents=True, exist_ok=True)
+    (tmp / "graph.json").write_text(json.dumps(graph, separators=(",", ":")))
+    write_safetensors(tmp / "model.safetensors", tensors)
+    return tmp / "graph.json", tmp / "model.safetensors"
+
+
+def inspect(host, graph, weights, arithmetic="f32"):
+    _, provider, _ = host
+    paths = (C.c_char_p * 1)(str(weights).encode())
+    src = ModelSource(C.sizeof(ModelSource), str(graph).encode(), paths, 1, None, 0)
+    d_in, d_out, packed = C.c_uint32(0), C.c_uint32(0), C.c_int32(0)
+    msg = C.create_string_buffer(256)
+    st = provider.volvoxai_hip_gfx950_inspect_package(C.byref(src), ARITH[arithmetic], C.byref(d_in), C.byref(d_out),
+                                                      C.byref(packed), msg, 256)
+    return st, d_in.value, d_out.value, packed.value, msg.value.decode()
+
+
+def run(host, graph, weights, x, in_name, in_dtype, out_name, out_dtype, d_out, arithmetic="f32", lead_max=None,
+        executions=1):
+    mock, _, _ = host
+    x = np.ascontiguousarray(x)
+    out_np = {"i8": np.int8, "u8": np.uint8, "f32": np.float32}[out_dtype]
+    y = np.zeros(x.shape[:-1] + (d_out,), out_np)
+    r = MockRun()
+    r.graph_path, r.weight_path = str(graph).encode(), str(weights).encode()
+    r.packed_arithmetic = ARITH[arithmetic]
+    r.input_name, r.input_dtype, r.rank = in_name.encode(), DT[in_dtype], x.ndim
+    for i, e in enumerate(x.shape):
+        r.input_shape[i] = e
+    for i, e in enumerate(lead_max or []):
+        r.lead_max[i] = e
+    r.input, r.input_bytes = x.ctypes.data, x.nbytes
+    r.output_name, r.output_dtype, r.output_last = out_name.encode(), DT[out_dtype], d_out
+    r.output, r.output_capacity, r.executions = y.ctypes.data, y.nbytes, executions
+    mock.mock_host_run(C.byref(r))
+    return r, y
+
+
+@pytest.fixture(scope="module")
+def registered(host):
+    mock, provider, _ = host
+    if not mock.mock_host_registered_name():
+        register = C.cast(provider.volvoxai_hip_gfx950_backend_register, C.c_void_p)
+        mock.mock_host_register.argtypes = [C.c_void_p]
+        assert mock.mock_host_register(register) == 0, "registration was refused"
+        assert mock.mock_host_register(register) == -1, "a second registration under the same name must be refused"
+    return host
+
+
+KAT = dict(x=np.array([[-1, -1, -1], [-3, -3, -3]], np.int8),
+           w=np.array([[2, 1, 1], [-3, -2, -3], [127] * 3, [-128] * 3], np.int8),
+           zps=[1, -3, 2, -1], scales=[.5, .5, 1, 1], bias=[0, 0, 0, 0], s_in=1.0, zp_in=-2, s_out=1.0, zp_out=3,
+           want=np.array([[4, 4, 127, -128], [2, 2, -128, 127]], np.int8))
+
+
+# ---- no GPU needed ---------------------------------------------------------------------------------
+
+def test_registration_passes_the_descriptor_checks(registered):
+    mock, _, _ = registered
+    assert mock.mock_host_registered_name() == b"hip-gfx950"
+    assert mock.mock_host_shape_domain_support() == 1  # FULL
+
+
+def test_reads_qlinear_and_packed_packages(registered, tmp_path):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"])
+    assert inspect(registered, g, w)[:4] == (0, 3, 4, 0)
+    for op in ("QGemm", "QMatMul"):
+        g, w = qlinear_package(tmp_path / op, k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"],
+                               k["zp_in"], k["s_out"], k["zp_out"], op=op)
+        assert inspect(registered, g, w)[0] == 0
+    c = cases.packed_case(3, 96, 5, 32, 1)
+    from oracle.pyoracle import Oracle
+    words = Oracle().pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "p", c["x"].shape, words, c["scales"], c["bias"], 32)
+    assert inspect(registered, g, w, "dynamic_i8")[:4] == (0, 96, 5, 1)
+
+
+def _drop(path):
+    def f(graph, tensors):
+        node = graph
+        for key in path[:-1]:
+            node = node[key]
+        del node[path[-1]]
+    return f
+
+
+@pytest.mark.parametrize("name,mutate,status", [
+    ("format", lambda g, t: g.__setitem__("format", "volvox-graph/v0"), -5),
+    ("two nodes", lambda g, t: g["nodes"].append(dict(g["nodes"][0], id="again")), -7),
+    ("other op", lambda g, t: g["nodes"][0].__setitem__("opType", "Linear"), -7),
+    ("no table", _drop(["quantization"]), -5),
+    ("table extra field", lambda g, t: g["quantization"].__setitem__("scales", [1.0]), -5),
+    ("descriptor extra field", lambda g, t: g["quantization"]["tensors"]["hidden_q"].__setitem__("scale", 0.5), -5),
+    ("missing zero point", _drop(["quantization", "tensors", "projected_q", "zero_point_tensor"]), -5),
+    ("weight per_tensor", lambda g, t: g["quantization"]["tensors"]["projection.weight"].update(scheme="per_tensor"), -5),
+    ("weight axis 1", lambda g, t: g["quantization"]["tensors"]["projection.weight"].update(axis=1), -7),
+    ("negative axis spelling", lambda g, t: g["quantization"]["tensors"]["projection.weight"].update(axis=-2), 0),
+    ("scale not positive", lambda g, t: t.__setitem__("__quant__.projected.scale", np.array([0.0], np.float32)), -5),
+    ("scale nan", lambda g, t: t.__setitem__("__quant__.hidden.scale", np.array([np.nan], np.float32)), -5),
+    ("zero point dtype", lambda g, t: t.__setitem__("__quant__.hidden.zero_point", np.array([0], np.uint8)), -5),
+    ("scale count", lambda g, t: t.__setitem__("__quant__.projection.weight.scale", np.ones(3, np.float32)), -5),
+    ("same tensor twice", lambda g, t: g["quantization"]["tensors"]["hidden_q"].update(
+        zero_point_tensor="__quant__.hidden.scale"), -5),
+    ("weight shape", lambda g, t: t.__setitem__("projection.weight", np.zeros((4, 5), np.int8)), -5),
+    ("bias dtype", lambda g, t: t.__setitem__("projection.bias", np.zeros(4, np.float32)), -5),
+    ("dangling weight", lambda g, t: t.pop("projection.weight"), -5),
+])
+def test_qlinear_package_refusals(registered, tmp_path, name, mutate, status):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"], mutate=mutate)
+    st, *_, msg = inspect(registered, g, w)
+    assert st == status, f"{name}: {ST.get(st, st)} {msg!r}"
+    assert (st == 0) == (msg == "")
+
+
+def test_packed_package_refusals(registered, tmp_path):
+    from oracle.pyoracle import Oracle
+    c = cases.packed_case(3, 96, 5, 32, 1)
+    words = Oracle().pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "a", c["x"].shape, words, c["scales"], c["bias"], 32)
+    for arithmetic in ("f32", "f16", "f32_fast", "dynamic_i4"):
+        assert inspect(registered, g, w, arithmetic)[0] == -7  # only DYNAMIC_I8 is this arithmetic
+    g, w = packed_package(tmp_path / "b", c["x"].shape, words, c["scales"], c["bias"], 32, bits=4)
+    assert inspect(registered, g, w, "dynamic_i8")[0] == -7
+    g, w = packed_package(tmp_path / "c", c["x"].shape, words, c["scales"], c["bias"], 48)
+    assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+    g, w = packed_package(tmp_path / "d", c["x"].shape, words[:, :-1], c["scales"], c["bias"], 32)
+    assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+    g, w = packed_package(tmp_path / "e", c["x"].shape, words, c["scales"][:, :-1], c["bias"], 32)
+    assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+
+
+def test_malformed_documents_are_refused(registered, tmp_path):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"])
+    good = g.read_text()
+    for bad in (good[:-3], good.replace('"nodes"', '"format"', 1), good + "{}", "[1,2", '{"a":1,"a":2}'):
+        g.write_text(bad)
+        assert inspect(registered, g, w)[0] == -5
+    g.write_text(good)
+    w.write_bytes(w.read_bytes()[:20])
+    assert inspect(registered, g, w)[0] == -4
+    assert inspect(registered, tmp_path / "nothing.json", w)[0] == -4
+
+
+@pytest.mark.skipif(__import__("torch").cuda.is_available(), reason="covers the box without a GPU")
+def test_without_a_device_the_provider_is_unavailable(registered, tmp_path):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"])
+    r, _ = run(registered, g, w, k["x"], "hidden_q", "i8", "projected_q", "i8", 4)
+    assert r.status == -6 and r.failed_stage == 1 and r.writes == 0
+
+
+# ---- on the GPU ---------------------------------------------------------------------------------------
+
+@pytest.mark.gpu
+def test_literal_kat_package_end_to_end(registered, tmp_path):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"])
+    r, y = run(registered, g, w, k["x"], "hidden_q", "i8", "projected_q", "i8", 4, executions=2)
+    assert r.status == 0, r.message
+    assert (y == k["want"]).all()
+    assert r.writes == 2 and r.compile_attested and r.execute_attested and r.identities_echoed
+    assert b"provider=hip-gfx950" in r.compile_route and b"hip.qlinear" in r.execute_route
+    assert b"gfx950" in r.device and r.maximum_resident_bytes >= 1024 and r.maximum_tensor_bytes == 8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,k,n,in_dtype,w_dtype", [(1, 64, 48, "int8", np.int8), (33, 200, 72, "uint8", np.int8),
+                                                        (300, 512, 256, "int8", np.uint8)])
+def test_qlinear_package_matches_oracle(registered, oracle, tmp_path, rows, k, n, in_dtype, w_dtype):
+    rng = np.random.default_rng(rows)
+    lo, hi = (-128, 128) if in_dtype == "int8" else (0, 256)
+    x = rng.integers(lo, hi, (2, rows, k)).astype(np.int8 if in_dtype == "int8" else np.uint8)
+    wlo, whi = (-127, 128) if w_dtype == np.int8 else (0, 256)
+    wt = rng.integers(wlo, whi, (n, k)).astype(w_dtype)
+    scales = (rng.uniform(0.002, 0.01, n) / np.sqrt(k) * 8).astype(np.float32)
+    zps = rng.integers(-3, 4, n) if w_dtype == np.int8 else rng.integers(120, 136, n)
+    bias = rng.integers(-2000, 2000, n).astype(np.int32)
+    zp_in = 3 if in_dtype == "int8" else 131
+    g, w = qlinear_package(tmp_path / "q", x.shape, wt, scales, zps, bias, 0.04, zp_in, 0.05, -5, in_dtype=in_dtype,
+                           rows_symbol=True)
+    r, y = run(registered, g, w, x, "hidden_q", "i8" if in_dtype == "int8" else "u8", "projected_q", "i8", n,
+               lead_max=[64, 0])
+    assert r.status == 0, r.message
+    dt = {np.int8: 6, np.uint8: 5}
+    ok, want = oracle.qlinear(x.reshape(-1, k), wt, bias, scales, np.asarray(zps, np.int32), 0.04, zp_in, 0.05, -5,
+                              6 if in_dtype == "int8" else 5, dt[w_dtype], 6)[:2]
+    assert ok == 1 and (y.reshape(-1, n) == want).all()
+
+
+@pytest.mark.gpu
+def test_qlinear_package_with_unprovable_accumulator_is_refused_at_compile(registered, tmp_path):
+    k = 40000  # 40000 * 255 * 255 > INT32_MAX
+    x = np.zeros((1, k), np.uint8)
+    wt = np.full((8, k), 255, np.uint8)
+    g, w = qlinear_package(tmp_path / "q", x.shape, wt, np.full(8, 0.01, np.float32), np.zeros(8), np.zeros(8), 0.04, 0,
+                           0.05, 0, in_dtype="uint8")
+    r, _ = run(registered, g, w, x, "hidden_q", "u8", "projected_q", "i8", 8)
+    assert r.status == -5 and r.failed_stage == 3 and r.writes == 0 and b"int32" in r.message
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,k,n,group", [(3, 96, 5, 32), (1, 4096, 512, 128), (40, 1000, 264, 64)])
+def test_packed_linear_package_matches_oracle(registered, oracle, tmp_path, rows, k, n, group):
+    c = cases.packed_case(rows, k, n, group, rows + k)
+    words = oracle.pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "p", c["x"].shape, words, c["scales"], c["bias"], group)
+    r, y = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", n, arithmetic="dynamic_i8")
+    assert r.status == 0, r.message
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
+    assert r.attested_arithmetic == ARITH["dynamic_i8"] and b"hip.packed-linear" in r.execute_route
+    # the same package under another arithmetic is refused before anything is allocated
+    r2, _ = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", n, arithmetic="f32")
+    assert r2.status == -7 and r2.failed_stage == 3 and r2.writes == 0
+
+
+@pytest.mark.gpu
+def test_bindings_are_validated_before_anything_runs(registered, tmp_path):
+    k = KAT
+    g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
+                           k["s_out"], k["zp_out"])
+    r, _ = run(registered, g, w, k["x"], "hidden_q", "i8", "projected_q", "i8", 4)
+    assert r.status == 0
+    wrong = np.zeros((2, 3), np.uint8)
+    r, _ = run(registered, g, w, wrong, "hidden_q", "u8", "projected_q", "i8", 4)  # dtype differs from the graph's
+    assert r.status == -1 and r.writes == 0
+    r, _ = run(registered, g, w, k["x"], "other", "i8", "projected_q", "i8", 4)
+    assert r.status == -1 and r.writes == 0

@@ -62,6 +62,8 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_context_synchronize": (i32, [vp]),
         "vxhip_context_last_variant": (C.c_char_p, [vp]),
         "vxhip_context_fault_flags": (i32, [vp, C.POINTER(u32)]),
+        "vxhip_probe_mfma_rate": (i32, [vp, u32, u32, C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double)]),
         "vxhip_device_malloc": (i32, [sz, pp]),
         "vxhip_device_free": (None, [vp]),
         "vxhip_memcpy_to_device": (i32, [vp, vp, vp, sz]),
@@ -69,6 +71,7 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_qlinear_create": (i32, [vp, vp, vp, vp, u32, u32, u32, pp]),
         "vxhip_qlinear_destroy": (None, [vp]),
         "vxhip_qlinear_resident_bytes": (u64, [vp]),
+        "vxhip_qlinear_admits": (C.c_int, [vp, f32, i32, f32, i32, u32, u32]),
         "vxhip_qlinear_forward": (C.c_int, [vp, vp, vp, vp, vp, u32, f32, i32, f32, i32, u32, u32]),
         "vxhip_qlinear_forward_rowscale": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u32, f32, i32, u32]),
         "vxhip_qlinear_i8u8": (C.c_int, [vp, vp, vp, vp, vp, vp, u32, u32, u32, f32, i32, f32, i32,

@@ -359,6 +359,54 @@ static const uint32_t* division_proof(VxHipContext* ctx, float divisor, float re
     return counters;
 }
 
+// Everything a QLinear call must satisfy before anything is launched; shared by the forward
+// entry points and by vxhip_qlinear_admits.
+static bool qlinear_admission(const VxHipQLinear* lin, bool per_row, float input_scale, int32_t input_zp,
+                              float output_scale, int32_t output_zp, uint32_t input_dtype,
+                              uint32_t output_dtype) {
+    if (!byte_dtype(input_dtype) || !byte_dtype(output_dtype) || !scale_ok(output_scale) ||
+        !zero_point_ok(input_zp, input_dtype) || !zero_point_ok(output_zp, output_dtype)) {
+        set_error("qlinear_forward: invalid dtype, scale or zero point");
+        return false;
+    }
+    const uint32_t k = lin->w.k;
+    if (!per_row) {
+        // product and quotient are monotone in s_w, so the extremes decide for every channel
+        if (!scale_ok(input_scale) || !multiplier_ok(input_scale, lin->scale_min, output_scale) ||
+            !multiplier_ok(input_scale, lin->scale_max, output_scale)) {
+            set_error("qlinear_forward: a requantization multiplier is not a positive finite f32");
+            return false;
+        }
+    }
+    // int32 admission: no partial sum can leave int32 when
+    //   K * max|x - zx| * max|w - zw| + max|bias| <= INT32_MAX
+    // (the proof the reference's vector route demands, native/src/kernels/qlinear_w8a8_x86.c:80,92-99)
+    const int64_t lo = input_dtype == VXHIP_DTYPE_I8 ? -128 : 0, hi = input_dtype == VXHIP_DTYPE_I8 ? 127 : 255;
+    const int64_t xmax = llabs(lo - input_zp) > llabs(hi - input_zp) ? llabs(lo - input_zp) : llabs(hi - input_zp);
+    if ((int64_t)k * xmax * lin->weight_abs_max + lin->bias_abs_max > (int64_t)INT32_MAX) {
+        set_error("qlinear_forward: int32 accumulator bound not provable for K=%u", k);
+        return false;
+    }
+    return true;
+}
+
+static bool per_row_ok(bool per_row, const float* row_scales_dev) {
+    if (per_row && !row_scales_dev) {
+        set_error("qlinear_forward_rowscale: row scales are required");
+        return false;
+    }
+    return true;
+}
+
+int vxhip_qlinear_admits(const VxHipQLinear* lin, float input_scale, int32_t input_zp, float output_scale,
+                         int32_t output_zp, uint32_t input_dtype, uint32_t output_dtype) {
+    if (!lin) {
+        set_error("qlinear_admits: null handle");
+        return 0;
+    }
+    return qlinear_admission(lin, false, input_scale, input_zp, output_scale, output_zp, input_dtype, output_dtype) ? 1 : 0;
+}
+
 // Shared by the per-tensor and the per-row entry points.
 static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* input_dev,
                        const float* row_scales_dev, const float* bias_f32_dev, void* output_dev,
@@ -369,32 +417,10 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
         set_error("qlinear_forward: null handle/tensor or zero rows");
         return 0;
     }
-    if (!byte_dtype(input_dtype) || !byte_dtype(output_dtype) || !scale_ok(output_scale) ||
-        !zero_point_ok(input_zp, input_dtype) || !zero_point_ok(output_zp, output_dtype)) {
-        set_error("qlinear_forward: invalid dtype, scale or zero point");
+    if (!per_row_ok(per_row, row_scales_dev) ||
+        !qlinear_admission(lin, per_row, input_scale, input_zp, output_scale, output_zp, input_dtype, output_dtype))
         return 0;
-    }
     const uint32_t k = lin->w.k, n = lin->w.n;
-    if (!per_row) {
-        // product and quotient are monotone in s_w, so the extremes decide for every channel
-        if (!scale_ok(input_scale) || !multiplier_ok(input_scale, lin->scale_min, output_scale) ||
-            !multiplier_ok(input_scale, lin->scale_max, output_scale)) {
-            set_error("qlinear_forward: a requantization multiplier is not a positive finite f32");
-            return 0;
-        }
-    } else if (!row_scales_dev) {
-        set_error("qlinear_forward_rowscale: row scales are required");
-        return 0;
-    }
-    // int32 admission: no partial sum can leave int32 when
-    //   K * max|x - zx| * max|w - zw| + max|bias| <= INT32_MAX
-    // (the proof the reference's vector route demands, native/src/kernels/qlinear_w8a8_x86.c:80,92-99)
-    const int64_t lo = input_dtype == VXHIP_DTYPE_I8 ? -128 : 0, hi = input_dtype == VXHIP_DTYPE_I8 ? 127 : 255;
-    const int64_t xmax = llabs(lo - input_zp) > llabs(hi - input_zp) ? llabs(lo - input_zp) : llabs(hi - input_zp);
-    if ((int64_t)k * xmax * lin->weight_abs_max + lin->bias_abs_max > (int64_t)INT32_MAX) {
-        set_error("qlinear_forward: int32 accumulator bound not provable for K=%u", k);
-        return 0;
-    }
     if (!use_device(ctx->device)) return 0;
 
     const bool flip = input_dtype == VXHIP_DTYPE_U8;

@@ -28,6 +28,10 @@
 #include <stdio.h>
 #include <string.h>
 
+// tuning probe: per-workgroup phase timestamps (100 MHz ticks) through the unused bias_row pointer
+#ifndef VXHIP_GEMV_PROBE
+#define VXHIP_GEMV_PROBE 0
+#endif
 #ifndef VXHIP_GEMV_DEPTH
 #define VXHIP_GEMV_DEPTH 4
 #endif
@@ -49,6 +53,8 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 template <int MODE, int GK, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
+    uint64_t probe[4] = {0, 0, 0, 0};
+    if (VXHIP_GEMV_PROBE) probe[0] = __builtin_amdgcn_s_memrealtime();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const uint32_t panel = blockIdx.x;
@@ -81,6 +87,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
+
+    // The tail's per-output operands (activation scale, bias) are requested now, so that their
+    // latency hides behind the stream instead of following it.
+    constexpr int TAIL_ITERS = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);
+    float tail_rs[F ? TAIL_ITERS : 1], tail_bias[F ? TAIL_ITERS : 1];
+    if constexpr (F) {
+#pragma unroll
+        for (int it = 0; it < TAIL_ITERS; it++) {
+            const uint32_t o = threadIdx.x + it * WAVES * 64;
+            tail_rs[it] = a.row_scale[min(o >> 5, rows - 1u)];
+            tail_bias[it] = a.bias_f32[panel * 32u + (o & 31u)];  // padded to whole panels
+        }
+    }
 
     // F: the panel's group scales [group][32] are fetched first (they are L2 hits and return
     // ahead of the HBM stream) and kept in LDS for the tail.
@@ -147,18 +166,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     }
     if constexpr (!F) park(wave);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (VXHIP_GEMV_PROBE) probe[1] = __builtin_amdgcn_s_memrealtime();
     __syncthreads();
+    if (VXHIP_GEMV_PROBE) probe[2] = __builtin_amdgcn_s_memrealtime();
 
     // Tail: one thread per output, index o = row * 32 + channel.  F: sum += f32(dot_g) *
     // (s_a * s_w[n][g]) in ascending group order with separate roundings
     // (packed_linear_ops.inc:1498-1504); eight groups' operands are requested before the
     // first add needs one.
-    for (uint32_t o = threadIdx.x; o < rows * 32u; o += WAVES * 64) {
-        const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
-        float rs = 0.0f;
-        if constexpr (MODE != (int)Epilogue::RequantTensor) rs = a.row_scale[om];
-        const size_t slab = (size_t)rows * 32u;
-        if constexpr (F) {
+    const size_t slab = (size_t)rows * 32u;
+    if constexpr (F) {
+#pragma unroll
+        for (int it = 0; it < TAIL_ITERS; it++) {
+            const uint32_t o = threadIdx.x + it * WAVES * 64;
+            if (o >= rows * 32u) break;
+            const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
+            const float rs = tail_rs[it];
             float sum = 0.0f;
             const int32_t* dp = parts + o;
             const float* sp = lds_scales + (o & 31u);
@@ -177,13 +200,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
             }
             for (; g < a.groups; g++)
                 sum = __fadd_rn(sum, __fmul_rn((float)dp[(size_t)g * slab], __fmul_rn(rs, sp[g * 32u])));
-            store_element<MODE>(a, om, on, 0, sum, rs);
-        } else {
+            if (on < a.n) ((float*)a.y)[(size_t)om * a.n + on] = __fadd_rn(sum, tail_bias[it]);
+        }
+    } else {
+        for (uint32_t o = threadIdx.x; o < rows * 32u; o += WAVES * 64) {
+            const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
+            float rs = 0.0f;
+            if constexpr (MODE == (int)Epilogue::RequantRow) rs = a.row_scale[om];
             int32_t dot = 0;
 #pragma unroll
             for (int w = 0; w < WAVES; w++) dot += parts[(size_t)w * slab + o];
             store_element<MODE>(a, om, on, dot, 0.0f, rs);
         }
+    }
+    if (VXHIP_GEMV_PROBE && threadIdx.x == 0) {
+        __builtin_amdgcn_s_waitcnt(0);
+        uint64_t* o = (uint64_t*)a.bias_row + 4 * (size_t)blockIdx.x;
+        o[0] = probe[0];
+        o[1] = probe[1];
+        o[2] = probe[2];
+        o[3] = __builtin_amdgcn_s_memrealtime();
     }
 }
 

@@ -1,0 +1,826 @@
+/* Backend provider "hip-gfx950": plugs libvxhip_w8a8 into the unchanged
+ * VolvoxAI runtime through its provider SPI (native/include/volvoxai_backend.h:168-259).
+ *
+ * The provider compiles single-node W8A8 packages:
+ *   - one QLinear / QGemm / QMatMul node in the volvox-affine-safetensors/v1
+ *     representation (docs/w8a8-safetensors.md:13-59, validation list :158-175);
+ *   - one PackedLinear node with weight_bits 8 under DYNAMIC_I8 packed
+ *     arithmetic (node form: native/tests/test_packed_arithmetic.inc:35-37).
+ * Anything else is refused with BACKEND_UNSUPPORTED before a compiled instance
+ * exists, which is what shape_domain.support = FULL promises
+ * (native/include/volvoxai_backend.h:112-118).
+ *
+ * Ownership follows docs/backend-sdk.md:77-95: the runtime instance names the
+ * device, the compiled instance holds the immutable prepacked weights, every
+ * context instance owns its stream, staging buffers and scratch, so contexts of
+ * one compiled model may execute concurrently
+ * (native/tests/test_packed_arithmetic.inc:128-147).
+ */
+#include "hip_gfx950_provider.h"
+
+#include "json_min.h"
+#include "safetensors_min.h"
+#include "vxhip_w8a8.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define PROVIDER_NAME "hip-gfx950"
+#define NAME_CAPACITY 256u
+
+typedef struct HipRuntime {
+    int32_t device;
+    char device_name[VX_REPORT_DEVICE_CAPACITY];
+} HipRuntime;
+
+typedef enum PlanKind { PLAN_QLINEAR = 1, PLAN_PACKED_LINEAR = 2 } PlanKind;
+
+/* Host-side result of reading a package; tensor pointers borrow the mapped weight files. */
+typedef struct PackagePlan {
+    PlanKind kind;
+    char node_id[NAME_CAPACITY];
+    char input_name[NAME_CAPACITY];
+    char output_name[NAME_CAPACITY];
+    uint32_t d_in, d_out;
+    VxDataType input_dtype, output_dtype;
+    /* QLinear */
+    const void* weight;
+    uint32_t weight_dtype;
+    const float* weight_scales;
+    int32_t* weight_zero_points; /* owned */
+    const int32_t* bias_i32;
+    float input_scale, output_scale;
+    int32_t input_zero_point, output_zero_point;
+    /* PackedLinear */
+    const uint32_t* packed_words;
+    const float* group_scales;
+    const float* bias_f32;
+    uint32_t group_size;
+    /* mapped files */
+    VxstFile** files;
+    size_t file_count;
+} PackagePlan;
+
+typedef struct HipCompiled {
+    HipRuntime* runtime;
+    PlanKind kind;
+    char input_name[NAME_CAPACITY];
+    char output_name[NAME_CAPACITY];
+    uint32_t d_in, d_out;
+    VxDataType input_dtype, output_dtype;
+    size_t input_element_bytes, output_element_bytes;
+    uint32_t rank;                        /* of input and output alike */
+    int64_t lead_min[VX_MAX_TENSOR_RANK]; /* bounds of the leading dimensions */
+    int64_t lead_max[VX_MAX_TENSOR_RANK];
+    int64_t lead_multiple[VX_MAX_TENSOR_RANK];
+    VxHipQLinear* qlinear;
+    VxHipPackedLinear* packed;
+    float input_scale, output_scale;
+    int32_t input_zero_point, output_zero_point;
+    char route[128];
+} HipCompiled;
+
+typedef struct HipContext {
+    HipCompiled* compiled;
+    VxHipContext* ctx;
+    void* input_dev;
+    void* output_dev;
+    void* output_host;
+    size_t input_capacity, output_capacity, host_capacity;
+    int closed;
+} HipContext;
+
+/* ---- reports ---------------------------------------------------------------- */
+
+static int report_writable(const VxReport* report) {
+    return report && report->struct_size == sizeof(*report);
+}
+
+static void fill_report(VxReport* report, const HipRuntime* runtime, VxStatus status, VxStage stage,
+                        VxOperationCode code, const char* message) {
+    if (!report_writable(report)) return;
+    memset(report, 0, sizeof(*report));
+    report->struct_size = sizeof(*report);
+    report->status = status;
+    report->stage = stage;
+    report->code = code;
+    snprintf(report->backend, sizeof(report->backend), "%s", PROVIDER_NAME);
+    snprintf(report->device, sizeof(report->device), "%s",
+             runtime && runtime->device_name[0] ? runtime->device_name : "gfx950");
+    snprintf(report->message, sizeof(report->message), "%s", message ? message : "");
+}
+
+static VxOperationCode code_for(VxStatus status) {
+    switch (status) {
+        case VX_STATUS_OK: return VX_CODE_NONE;
+        case VX_STATUS_OUT_OF_MEMORY: return VX_CODE_OUT_OF_MEMORY;
+        case VX_STATUS_BACKEND_UNSUPPORTED: return VX_CODE_BACKEND_UNSUPPORTED;
+        case VX_STATUS_BACKEND_UNAVAILABLE: return VX_CODE_BACKEND_UNAVAILABLE;
+        case VX_STATUS_DEVICE_LOST: return VX_CODE_DEVICE_LOST;
+        case VX_STATUS_INVALID_GRAPH: return VX_CODE_INVALID_GRAPH;
+        case VX_STATUS_EXECUTION_FAILED: return VX_CODE_DEVICE_EXECUTION_FAILED;
+        default: return VX_CODE_INVALID_ARGUMENT;
+    }
+}
+
+static void attest(VxReport* report, const char* route) {
+    if (!report_writable(report)) return;
+    report->route_attested = 1;
+    report->operator_fallback_used = 0;
+    snprintf(report->route_evidence, sizeof(report->route_evidence), "provider=%s;nodes=1;route=%s", PROVIDER_NAME,
+             route);
+    snprintf(report->fallback_evidence, sizeof(report->fallback_evidence), "%s", "operator=none");
+}
+
+/* ---- package reading ------------------------------------------------------------ */
+
+typedef struct Failure {
+    VxStatus status;
+    char message[VX_REPORT_MESSAGE_CAPACITY];
+} Failure;
+
+static VxStatus refuse(Failure* failure, VxStatus status, const char* format, const char* detail) {
+    failure->status = status;
+    snprintf(failure->message, sizeof(failure->message), format, detail ? detail : "");
+    return status;
+}
+
+static void plan_release(PackagePlan* plan) {
+    for (size_t i = 0; i < plan->file_count; i++) vxst_close(plan->files[i]);
+    free(plan->files);
+    free(plan->weight_zero_points);
+    memset(plan, 0, sizeof(*plan));
+}
+
+static char* read_text_file(const char* path, size_t* length) {
+    FILE* file = path ? fopen(path, "rb") : NULL;
+    long size;
+    char* bytes;
+    if (!file) return NULL;
+    if (fseek(file, 0, SEEK_END) != 0 || (size = ftell(file)) < 0 || fseek(file, 0, SEEK_SET) != 0) {
+        fclose(file);
+        return NULL;
+    }
+    bytes = (char*)malloc((size_t)size + 1u);
+    if (bytes && fread(bytes, 1, (size_t)size, file) != (size_t)size) {
+        free(bytes);
+        bytes = NULL;
+    }
+    fclose(file);
+    if (bytes) {
+        bytes[size] = '\0';
+        *length = (size_t)size;
+    }
+    return bytes;
+}
+
+/* A tensor name must resolve in exactly one of the bound weight files
+ * (docs/w8a8-safetensors.md:103-108). */
+static int find_tensor(const PackagePlan* plan, const char* name, VxstTensor* out) {
+    int found = 0;
+    for (size_t i = 0; i < plan->file_count; i++) {
+        VxstTensor t;
+        if (vxst_find(plan->files[i], name, &t)) {
+            if (found) return -1;
+            *out = t;
+            found = 1;
+        }
+    }
+    return found;
+}
+
+static int copy_name(char* dst, const char* src) {
+    if (!src || !src[0] || strlen(src) >= NAME_CAPACITY) return 0;
+    memcpy(dst, src, strlen(src) + 1u);
+    return 1;
+}
+
+static int graph_dtype(const char* text, VxDataType* out) {
+    if (!text) return 0;
+    if (!strcmp(text, "int8")) *out = VX_DTYPE_I8;
+    else if (!strcmp(text, "uint8")) *out = VX_DTYPE_U8;
+    else if (!strcmp(text, "float32")) *out = VX_DTYPE_F32;
+    else return 0;
+    return 1;
+}
+
+static int object_has_only(const VxjValue* object, const char* const* allowed, size_t allowed_count) {
+    if (!object || object->kind != VXJ_OBJECT) return 0;
+    for (const VxjValue* m = object->first; m; m = m->next) {
+        size_t i = 0;
+        while (i < allowed_count && strcmp(allowed[i], m->key)) i++;
+        if (i == allowed_count) return 0;
+    }
+    return 1;
+}
+
+/* One descriptor of the central quantization table, resolved to its parameter tensors.
+ * per_axis_extent = 0 asks for the per_tensor form. */
+static VxStatus resolve_affine(const PackagePlan* plan, const VxjValue* table, const char* target,
+                               VxDataType target_dtype, uint32_t target_rank, int64_t per_axis_extent,
+                               VxstTensor* scale, VxstTensor* zero_point, Failure* failure) {
+    static const char* const tensor_fields[] = {"scheme", "scale_tensor", "zero_point_tensor"};
+    static const char* const axis_fields[] = {"scheme", "axis", "scale_tensor", "zero_point_tensor"};
+    const VxjValue* d = vxj_member(table, target);
+    const char* scheme = vxj_member_string(d, "scheme");
+    const char* scale_name = vxj_member_string(d, "scale_tensor");
+    const char* zp_name = vxj_member_string(d, "zero_point_tensor");
+    if (!d || !scheme || !scale_name || !zp_name)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "no complete affine descriptor for tensor '%s'", target);
+    if (per_axis_extent) {
+        const VxjValue* axis = vxj_member(d, "axis");
+        int64_t a;
+        if (strcmp(scheme, "per_axis") || !object_has_only(d, axis_fields, 4) || !axis || axis->kind != VXJ_NUMBER ||
+            !axis->is_integer)
+            return refuse(failure, VX_STATUS_INVALID_GRAPH, "tensor '%s' needs a per_axis descriptor", target);
+        a = axis->integer < 0 ? axis->integer + (int64_t)target_rank : axis->integer;
+        if (a != 0)
+            return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
+                          "weight '%s' must be quantized per output channel (axis 0)", target);
+    } else if (strcmp(scheme, "per_tensor") || !object_has_only(d, tensor_fields, 3)) {
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "tensor '%s' needs a per_tensor descriptor", target);
+    }
+    if (!strcmp(scale_name, zp_name))
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "scale and zero point of '%s' name the same tensor", target);
+    if (vxj_member(table, scale_name) || vxj_member(table, zp_name))
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "a quantization parameter of '%s' is itself quantized", target);
+    if (find_tensor(plan, scale_name, scale) != 1 || find_tensor(plan, zp_name, zero_point) != 1)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "quantization parameters of '%s' do not resolve uniquely",
+                      target);
+    const int64_t want = per_axis_extent ? per_axis_extent : 1;
+    const char* zp_dtype = target_dtype == VX_DTYPE_I8 ? "I8" : "U8";
+    if (strcmp(scale->dtype, "F32") || scale->rank != 1 || scale->shape[0] != want || strcmp(zero_point->dtype, zp_dtype) ||
+        zero_point->rank != 1 || zero_point->shape[0] != want)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "quantization parameters of '%s' have the wrong dtype or shape",
+                      target);
+    for (int64_t i = 0; i < want; i++) {
+        float s;
+        memcpy(&s, scale->data + 4 * i, 4);
+        if (!(s > 0.0f) || !isfinite(s))
+            return refuse(failure, VX_STATUS_INVALID_GRAPH, "a scale of '%s' is not finite and positive", target);
+    }
+    return VX_STATUS_OK;
+}
+
+static int32_t typed_zero_point(const VxstTensor* t, int64_t index) {
+    return !strcmp(t->dtype, "I8") ? (int32_t)((const int8_t*)t->data)[index] : (int32_t)t->data[index];
+}
+
+static VxStatus plan_qlinear(PackagePlan* plan, const VxjValue* root, const VxjValue* node, const VxjValue* out,
+                             Failure* failure) {
+    static const char* const table_fields[] = {"format", "tensors"};
+    const VxjValue* node_inputs = vxj_member(node, "inputs");
+    const char* weight_name = vxj_member_string(node_inputs, "weight");
+    const char* bias_name = vxj_member_string(node_inputs, "bias");
+    const VxjValue* quantization = vxj_member(root, "quantization");
+    const VxjValue* table = vxj_member(quantization, "tensors");
+    const char* table_format = vxj_member_string(quantization, "format");
+    VxstTensor weight, bias, scale, zero_point;
+    VxStatus status;
+    (void)out;
+    if (!weight_name) return refuse(failure, VX_STATUS_INVALID_GRAPH, "QLinear node '%s' names no weight", plan->node_id);
+    if (!quantization || !object_has_only(quantization, table_fields, 2) || !table_format ||
+        strcmp(table_format, "volvox-affine-safetensors/v1") || !table || table->kind != VXJ_OBJECT || !table->count)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH,
+                      "graph has no volvox-affine-safetensors/v1 quantization table%s", "");
+    if (plan->input_dtype == VX_DTYPE_F32 || plan->output_dtype == VX_DTYPE_F32)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "QLinear node '%s' needs int8/uint8 input and output",
+                      plan->node_id);
+    if (find_tensor(plan, weight_name, &weight) != 1)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "weight '%s' does not resolve uniquely", weight_name);
+    if ((strcmp(weight.dtype, "I8") && strcmp(weight.dtype, "U8")) || weight.rank != 2 ||
+        weight.shape[0] != (int64_t)plan->d_out || weight.shape[1] != (int64_t)plan->d_in)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "weight '%s' is not I8/U8 [d_out, d_in]", weight_name);
+    plan->weight = weight.data;
+    plan->weight_dtype = !strcmp(weight.dtype, "I8") ? VXHIP_DTYPE_I8 : VXHIP_DTYPE_U8;
+
+    status = resolve_affine(plan, table, plan->input_name, plan->input_dtype, 2, 0, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    memcpy(&plan->input_scale, scale.data, 4);
+    plan->input_zero_point = typed_zero_point(&zero_point, 0);
+
+    status = resolve_affine(plan, table, plan->output_name, plan->output_dtype, 2, 0, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    memcpy(&plan->output_scale, scale.data, 4);
+    plan->output_zero_point = typed_zero_point(&zero_point, 0);
+
+    status = resolve_affine(plan, table, weight_name, plan->weight_dtype == VXHIP_DTYPE_I8 ? VX_DTYPE_I8 : VX_DTYPE_U8,
+                            2, plan->d_out, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    plan->weight_scales = (const float*)(const void*)scale.data;
+    plan->weight_zero_points = (int32_t*)malloc(sizeof(int32_t) * plan->d_out);
+    if (!plan->weight_zero_points) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
+    for (uint32_t n = 0; n < plan->d_out; n++) plan->weight_zero_points[n] = typed_zero_point(&zero_point, n);
+
+    if (bias_name) {
+        if (find_tensor(plan, bias_name, &bias) != 1 || strcmp(bias.dtype, "I32") || bias.rank != 1 ||
+            bias.shape[0] != (int64_t)plan->d_out)
+            return refuse(failure, VX_STATUS_INVALID_GRAPH, "bias '%s' is not a unique I32 [d_out] tensor", bias_name);
+        plan->bias_i32 = (const int32_t*)(const void*)bias.data;
+    }
+    plan->kind = PLAN_QLINEAR;
+    return VX_STATUS_OK;
+}
+
+static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedArithmetic arithmetic,
+                            Failure* failure) {
+    const VxjValue* node_inputs = vxj_member(node, "inputs");
+    const VxjValue* params = vxj_member(node, "params");
+    const VxjValue* group = vxj_member(params, "group_size");
+    const VxjValue* bits = vxj_member(params, "weight_bits");
+    const char* weight_name = vxj_member_string(node_inputs, "weight");
+    const char* scale_name = vxj_member_string(node_inputs, "scale");
+    const char* bias_name = vxj_member_string(node_inputs, "bias");
+    VxstTensor weight, scale, bias;
+    if (arithmetic != VX_PACKED_ARITHMETIC_DYNAMIC_I8)
+        return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
+                      "PackedLinear is offered under DYNAMIC_I8 packed arithmetic only%s", "");
+    if (!group || group->kind != VXJ_NUMBER || !group->is_integer || !bits || bits->kind != VXJ_NUMBER ||
+        !bits->is_integer || !weight_name || !scale_name)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s' lacks weight, scale or parameters",
+                      plan->node_id);
+    if (bits->integer != 8)
+        return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "PackedLinear node '%s': only weight_bits 8 is offered",
+                      plan->node_id);
+    if (group->integer != 32 && group->integer != 64 && group->integer != 128 && group->integer != 256)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s': group_size must be 32, 64, 128 or 256",
+                      plan->node_id);
+    if (plan->input_dtype != VX_DTYPE_F32 || plan->output_dtype != VX_DTYPE_F32)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s' needs float32 input and output",
+                      plan->node_id);
+    plan->group_size = (uint32_t)group->integer;
+    const int64_t words = ((int64_t)plan->d_in + 3) / 4;
+    const int64_t groups = ((int64_t)plan->d_in + plan->group_size - 1) / plan->group_size;
+    if (find_tensor(plan, weight_name, &weight) != 1 || (strcmp(weight.dtype, "I32") && strcmp(weight.dtype, "U32")) ||
+        weight.rank != 2 || weight.shape[0] != (int64_t)plan->d_out || weight.shape[1] != words)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "packed weight '%s' is not I32 [d_out, ceil(d_in/4)]",
+                      weight_name);
+    if (find_tensor(plan, scale_name, &scale) != 1 || strcmp(scale.dtype, "F32") || scale.rank != 2 ||
+        scale.shape[0] != (int64_t)plan->d_out || scale.shape[1] != groups)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "group scales '%s' are not F32 [d_out, groups]", scale_name);
+    plan->packed_words = (const uint32_t*)(const void*)weight.data;
+    plan->group_scales = (const float*)(const void*)scale.data;
+    if (bias_name) {
+        if (find_tensor(plan, bias_name, &bias) != 1 || strcmp(bias.dtype, "F32") || bias.rank != 1 ||
+            bias.shape[0] != (int64_t)plan->d_out)
+            return refuse(failure, VX_STATUS_INVALID_GRAPH, "bias '%s' is not a unique F32 [d_out] tensor", bias_name);
+        plan->bias_f32 = (const float*)(const void*)bias.data;
+    }
+    plan->kind = PLAN_PACKED_LINEAR;
+    return VX_STATUS_OK;
+}
+
+/* Reads graph.json and the weight files named by the model source into a plan. */
+static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic arithmetic, PackagePlan* plan,
+                             Failure* failure) {
+    size_t length = 0;
+    const char* json_error = NULL;
+    char* text;
+    VxjValue* root;
+    VxStatus status = VX_STATUS_OK;
+    memset(plan, 0, sizeof(*plan));
+    text = read_text_file(source->graph_path, &length);
+    if (!text) return refuse(failure, VX_STATUS_IO_ERROR, "cannot read graph document '%s'", source->graph_path);
+    root = vxj_parse(text, length, &json_error);
+    free(text);
+    if (!root) return refuse(failure, VX_STATUS_INVALID_GRAPH, "graph document is not valid JSON: %s", json_error);
+
+    do {
+        const char* format = vxj_member_string(root, "format");
+        const VxjValue* inputs = vxj_member(root, "inputs");
+        const VxjValue* nodes = vxj_member(root, "nodes");
+        const VxjValue* outputs = vxj_member(root, "outputs");
+        const VxjValue* node = vxj_item(nodes, 0);
+        const char* op = vxj_member_string(node, "opType");
+        const VxjValue* out = vxj_member(vxj_member(node, "outputs"), "out");
+        const VxjValue* out_shape = vxj_member(out, "shape");
+        const VxjValue* graph_input = inputs && inputs->kind == VXJ_OBJECT ? inputs->first : NULL;
+        const VxjValue* in_shape = vxj_member(graph_input, "shape");
+        const VxjValue* last;
+        if (!format || strcmp(format, "volvox-graph/v1")) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph format is not volvox-graph/v1%s", "");
+            break;
+        }
+        if (!nodes || nodes->kind != VXJ_ARRAY || nodes->count != 1 || !inputs || inputs->count != 1 || !outputs ||
+            outputs->kind != VXJ_ARRAY || outputs->count != 1) {
+            status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
+                            "this provider compiles graphs of one node, one input and one output%s", "");
+            break;
+        }
+        if (!op || !out || !copy_name(plan->node_id, vxj_member_string(node, "id")) ||
+            !copy_name(plan->input_name, graph_input->key) ||
+            !copy_name(plan->output_name, vxj_member_string(out, "tensor")) ||
+            !graph_dtype(vxj_member_string(graph_input, "dtype"), &plan->input_dtype) ||
+            !graph_dtype(vxj_member_string(out, "dtype"), &plan->output_dtype) || !in_shape ||
+            in_shape->kind != VXJ_ARRAY || !in_shape->count || !out_shape || out_shape->kind != VXJ_ARRAY ||
+            out_shape->count != in_shape->count) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "node or tensor declaration is incomplete%s", "");
+            break;
+        }
+        {
+            const char* fed = vxj_member_string(vxj_member(node, "inputs"), "input");
+            const VxjValue* declared = vxj_item(outputs, 0);
+            if (!fed || strcmp(fed, plan->input_name) || declared->kind != VXJ_STRING ||
+                strcmp(declared->string, plan->output_name)) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                "the node must read the graph input and feed the graph output%s", "");
+                break;
+            }
+        }
+        /* dense on the last axis: that extent is a number in both declarations */
+        last = vxj_item(in_shape, in_shape->count - 1);
+        if (last->kind != VXJ_NUMBER || !last->is_integer || last->integer <= 0 || last->integer > INT32_MAX) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the input's last extent must be a fixed d_in%s", "");
+            break;
+        }
+        plan->d_in = (uint32_t)last->integer;
+        last = vxj_item(out_shape, out_shape->count - 1);
+        if (last->kind != VXJ_NUMBER || !last->is_integer || last->integer <= 0 || last->integer > INT32_MAX) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the output's last extent must be a fixed d_out%s", "");
+            break;
+        }
+        plan->d_out = (uint32_t)last->integer;
+
+        plan->files = (VxstFile**)calloc(source->weight_path_count ? source->weight_path_count : 1, sizeof(VxstFile*));
+        if (!plan->files) {
+            status = refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
+            break;
+        }
+        for (size_t i = 0; i < source->weight_path_count && status == VX_STATUS_OK; i++) {
+            char error[VX_REPORT_MESSAGE_CAPACITY];
+            if (vxst_open(source->weight_paths[i], &plan->files[plan->file_count], error, sizeof(error)) != 0)
+                status = refuse(failure, VX_STATUS_IO_ERROR, "%s", error);
+            else
+                plan->file_count++;
+        }
+        if (status != VX_STATUS_OK) break;
+
+        if (!strcmp(op, "QLinear") || !strcmp(op, "QGemm") || !strcmp(op, "QMatMul"))
+            status = plan_qlinear(plan, root, node, out, failure);
+        else if (!strcmp(op, "PackedLinear"))
+            status = plan_packed(plan, node, arithmetic, failure);
+        else
+            status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "operator '%s' is not offered by this provider", op);
+    } while (0);
+    vxj_free(root);
+    if (status != VX_STATUS_OK) plan_release(plan);
+    return status;
+}
+
+/* ---- SPI callbacks ---------------------------------------------------------------- */
+
+static VxStatus hip_runtime_create(void* user_data, const VxRuntimeOptions* options, void** out_runtime,
+                                   VxReport* report) {
+    HipRuntime* runtime;
+    (void)user_data;
+    if (!out_runtime) return VX_STATUS_INVALID_ARGUMENT;
+    *out_runtime = NULL;
+    if (!options || options->struct_size != sizeof(*options)) return VX_STATUS_INVALID_ARGUMENT;
+    if (vxhip_device_count() <= 0) {
+        /* optional hardware absent: the runtime omits this provider (runtime/backend_sdk.c:206-213) */
+        fill_report(report, NULL, VX_STATUS_BACKEND_UNAVAILABLE, VX_STAGE_RUNTIME_CREATE, VX_CODE_BACKEND_UNAVAILABLE,
+                    "no gfx950 device is visible");
+        return VX_STATUS_BACKEND_UNAVAILABLE;
+    }
+    runtime = (HipRuntime*)calloc(1, sizeof(*runtime));
+    if (!runtime) return VX_STATUS_OUT_OF_MEMORY;
+    runtime->device = 0;
+    if (vxhip_device_name(0, runtime->device_name, sizeof(runtime->device_name)) != VXHIP_OK)
+        snprintf(runtime->device_name, sizeof(runtime->device_name), "%s", "gfx950");
+    *out_runtime = runtime;
+    fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_RUNTIME_CREATE, VX_CODE_NONE, "hip-gfx950 runtime created");
+    return VX_STATUS_OK;
+}
+
+static void hip_runtime_destroy(void* runtime_instance) {
+    free(runtime_instance);
+}
+
+static int policy_names(const VxBackendPolicy* policy, const char* name) {
+    if (!policy || policy->struct_size != sizeof(*policy) || !policy->backends) return 0;
+    for (size_t i = 0; i < policy->backend_count; i++)
+        if (policy->backends[i] && !strcmp(policy->backends[i], name)) return 1;
+    return 0;
+}
+
+static void hip_compiled_destroy(void* compiled_instance) {
+    HipCompiled* compiled = (HipCompiled*)compiled_instance;
+    if (!compiled) return;
+    if (compiled->qlinear) vxhip_qlinear_destroy(compiled->qlinear);
+    if (compiled->packed) vxhip_packed_linear_destroy(compiled->packed);
+    free(compiled);
+}
+
+/* The logical specifications the core hands over must describe the same tensors as the graph. */
+static int specs_match(const VxBackendCompileInput* input, const PackagePlan* plan, HipCompiled* compiled) {
+    const VxTensorSpec* in = &input->inputs[0];
+    const VxTensorSpec* out = &input->outputs[0];
+    if (in->struct_size != sizeof(*in) || out->struct_size != sizeof(*out) || !in->name || !out->name ||
+        strcmp(in->name, plan->input_name) || strcmp(out->name, plan->output_name) || in->dtype != plan->input_dtype ||
+        out->dtype != plan->output_dtype || in->rank != out->rank || in->rank < 1 || in->rank > VX_MAX_TENSOR_RANK ||
+        in->location != VX_MEMORY_HOST || out->location != VX_MEMORY_HOST)
+        return 0;
+    const VxDimensionConstraint* last_in = &in->dimensions[in->rank - 1];
+    const VxDimensionConstraint* last_out = &out->dimensions[out->rank - 1];
+    if (last_in->kind != VX_DIMENSION_FIXED || last_in->min != (int64_t)plan->d_in || last_in->max != last_in->min ||
+        last_out->kind != VX_DIMENSION_FIXED || last_out->min != (int64_t)plan->d_out || last_out->max != last_out->min)
+        return 0;
+    compiled->rank = in->rank;
+    for (uint32_t axis = 0; axis + 1 < in->rank; axis++) {
+        const VxDimensionConstraint* a = &in->dimensions[axis];
+        const VxDimensionConstraint* b = &out->dimensions[axis];
+        if (a->min < 1 || a->max < a->min || a->multiple_of < 1 || a->min != b->min || a->max != b->max ||
+            a->multiple_of != b->multiple_of)
+            return 0;
+        compiled->lead_min[axis] = a->min;
+        compiled->lead_max[axis] = a->max;
+        compiled->lead_multiple[axis] = a->multiple_of;
+    }
+    return 1;
+}
+
+static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput* input, const VxBackendPolicy* policy,
+                            void** out_compiled, VxBackendShapeDomainAttestation* attestation, VxReport* report) {
+    HipRuntime* runtime = (HipRuntime*)runtime_instance;
+    PackagePlan plan;
+    Failure failure = {VX_STATUS_OK, {0}};
+    HipCompiled* compiled;
+    VxStatus status;
+    uint64_t rows_max = 1, resident, tensor_bytes;
+    if (!runtime || !input || input->struct_size != sizeof(*input) || !input->source ||
+        input->source->struct_size != sizeof(*input->source) || !input->graph_fingerprint ||
+        !input->shape_domain_proof_identity || !out_compiled || !attestation ||
+        attestation->struct_size != sizeof(*attestation) || !policy_names(policy, PROVIDER_NAME))
+        return VX_STATUS_INVALID_ARGUMENT;
+    *out_compiled = NULL;
+    if (input->packed_arithmetic == VX_PACKED_ARITHMETIC_DYNAMIC_I4) {
+        /* a known option this provider has no executable for: refuse before allocating anything
+         * (native/tests/test_packed_arithmetic.inc:111-123) */
+        fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
+                    "DYNAMIC_I4 packed arithmetic is not offered");
+        return VX_STATUS_BACKEND_UNSUPPORTED;
+    }
+    if (input->input_count != 1 || input->output_count != 1 || !input->inputs || !input->outputs) {
+        fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
+                    "this provider compiles graphs of one node, one input and one output");
+        return VX_STATUS_BACKEND_UNSUPPORTED;
+    }
+    status = plan_package(input->source, input->packed_arithmetic, &plan, &failure);
+    if (status != VX_STATUS_OK) {
+        fill_report(report, runtime, status, VX_STAGE_COMPILE, code_for(status), failure.message);
+        return status;
+    }
+    compiled = (HipCompiled*)calloc(1, sizeof(*compiled));
+    if (!compiled) {
+        plan_release(&plan);
+        return VX_STATUS_OUT_OF_MEMORY;
+    }
+    if (!specs_match(input, &plan, compiled)) {
+        plan_release(&plan);
+        free(compiled);
+        fill_report(report, runtime, VX_STATUS_INVALID_ARGUMENT, VX_STAGE_COMPILE, VX_CODE_INVALID_ARGUMENT,
+                    "logical tensor specifications do not describe the graph's input and output");
+        return VX_STATUS_INVALID_ARGUMENT;
+    }
+    compiled->runtime = runtime;
+    compiled->kind = plan.kind;
+    memcpy(compiled->input_name, plan.input_name, sizeof(compiled->input_name));
+    memcpy(compiled->output_name, plan.output_name, sizeof(compiled->output_name));
+    compiled->d_in = plan.d_in;
+    compiled->d_out = plan.d_out;
+    compiled->input_dtype = plan.input_dtype;
+    compiled->output_dtype = plan.output_dtype;
+    compiled->input_element_bytes = plan.input_dtype == VX_DTYPE_F32 ? 4u : 1u;
+    compiled->output_element_bytes = plan.output_dtype == VX_DTYPE_F32 ? 4u : 1u;
+    compiled->input_scale = plan.input_scale;
+    compiled->output_scale = plan.output_scale;
+    compiled->input_zero_point = plan.input_zero_point;
+    compiled->output_zero_point = plan.output_zero_point;
+
+    if (plan.kind == PLAN_QLINEAR) {
+        status = (VxStatus)vxhip_qlinear_create(plan.weight, plan.weight_scales, plan.weight_zero_points, plan.bias_i32,
+                                                plan.d_in, plan.d_out, plan.weight_dtype, &compiled->qlinear);
+        /* a fused integer operator is published only with its multiplier and accumulator-range
+         * contract satisfied (docs/w8a8-safetensors.md:158-175, item 8) */
+        if (status == VX_STATUS_OK &&
+            !vxhip_qlinear_admits(compiled->qlinear, plan.input_scale, plan.input_zero_point, plan.output_scale,
+                                  plan.output_zero_point, (uint32_t)plan.input_dtype, (uint32_t)plan.output_dtype))
+            status = VX_STATUS_INVALID_GRAPH;
+        snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.qlinear");
+    } else {
+        status = (VxStatus)vxhip_packed_linear_create(plan.packed_words, plan.group_scales, plan.bias_f32, plan.d_in,
+                                                      plan.d_out, plan.group_size, 8, &compiled->packed);
+        snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.packed-linear");
+    }
+    plan_release(&plan);
+    if (status != VX_STATUS_OK) {
+        fill_report(report, runtime, status, VX_STAGE_COMPILE, code_for(status), vxhip_last_error());
+        hip_compiled_destroy(compiled);
+        return status;
+    }
+
+    for (uint32_t axis = 0; axis + 1 < compiled->rank; axis++) {
+        if (rows_max > (UINT64_C(1) << 31) / (uint64_t)compiled->lead_max[axis]) {
+            fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
+                        "the bounded domain allows more than 2^31 rows");
+            hip_compiled_destroy(compiled);
+            return VX_STATUS_BACKEND_UNSUPPORTED;
+        }
+        rows_max *= (uint64_t)compiled->lead_max[axis];
+    }
+    resident = compiled->qlinear ? vxhip_qlinear_resident_bytes(compiled->qlinear)
+                                 : vxhip_packed_linear_resident_bytes(compiled->packed);
+    tensor_bytes = rows_max * compiled->d_in * compiled->input_element_bytes;
+    if (rows_max * compiled->d_out * compiled->output_element_bytes > tensor_bytes)
+        tensor_bytes = rows_max * compiled->d_out * compiled->output_element_bytes;
+    attestation->graph_fingerprint = input->graph_fingerprint;
+    attestation->shape_domain_proof_identity = input->shape_domain_proof_identity;
+    attestation->maximum_tensor_bytes = tensor_bytes;
+    /* weights plus, per context, staged input, output and the int8 staging of a PackedLinear call */
+    attestation->maximum_resident_bytes =
+        resident + rows_max * ((uint64_t)compiled->d_in * (compiled->input_element_bytes + 1u) +
+                               (uint64_t)compiled->d_out * compiled->output_element_bytes + 8u);
+    attestation->resource_limit_bytes = 0;
+    attestation->has_resource_limit = 0;
+    attestation->packed_arithmetic =
+        compiled->packed ? VX_PACKED_ARITHMETIC_DYNAMIC_I8 : input->packed_arithmetic;
+    *out_compiled = compiled;
+    fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE, "single-node W8A8 package compiled");
+    attest(report, compiled->route);
+    return VX_STATUS_OK;
+}
+
+static void hip_context_destroy(void* context_instance) {
+    HipContext* context = (HipContext*)context_instance;
+    if (!context) return;
+    if (context->input_dev) vxhip_device_free(context->input_dev);
+    if (context->output_dev) vxhip_device_free(context->output_dev);
+    free(context->output_host);
+    if (context->ctx) vxhip_context_destroy(context->ctx);
+    free(context);
+}
+
+static VxStatus hip_context_create(void* compiled_instance, const VxContextOptions* options, void** out_context,
+                                   VxReport* report) {
+    HipCompiled* compiled = (HipCompiled*)compiled_instance;
+    HipContext* context;
+    VxStatus status;
+    if (!out_context) return VX_STATUS_INVALID_ARGUMENT;
+    *out_context = NULL;
+    if (!compiled || !options || options->struct_size != sizeof(*options)) return VX_STATUS_INVALID_ARGUMENT;
+    if (options->decode_row_mode != VX_DECODE_ROW_DISABLED) return VX_STATUS_BACKEND_UNSUPPORTED;
+    context = (HipContext*)calloc(1, sizeof(*context));
+    if (!context) return VX_STATUS_OUT_OF_MEMORY;
+    context->compiled = compiled;
+    status = (VxStatus)vxhip_context_create(compiled->runtime->device, NULL, VXHIP_CONTEXT_OWN_STREAM, &context->ctx);
+    if (status != VX_STATUS_OK) {
+        fill_report(report, compiled->runtime, status, VX_STAGE_CONTEXT_CREATE, VX_CODE_BACKEND_CONTEXT_CREATE_FAILED,
+                    vxhip_last_error());
+        hip_context_destroy(context);
+        return status;
+    }
+    *out_context = context;
+    fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_CONTEXT_CREATE, VX_CODE_NONE, "context created");
+    return VX_STATUS_OK;
+}
+
+static VxStatus grow_device(void** buffer, size_t* capacity, size_t bytes) {
+    void* fresh = NULL;
+    VxStatus status;
+    if (bytes <= *capacity) return VX_STATUS_OK;
+    status = (VxStatus)vxhip_device_malloc(bytes, &fresh);
+    if (status != VX_STATUS_OK) return status;
+    if (*buffer) vxhip_device_free(*buffer);
+    *buffer = fresh;
+    *capacity = bytes;
+    return VX_STATUS_OK;
+}
+
+static VxStatus hip_context_execute(void* context_instance, const VxTensorBinding* inputs, size_t input_count,
+                                    const VxBackendOutputSink* sink, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    const HipCompiled* compiled;
+    const VxTensorBinding* binding;
+    int64_t shape[VX_MAX_TENSOR_RANK];
+    uint64_t rows = 1;
+    size_t input_bytes, output_bytes;
+    VxStatus status;
+    int handled;
+    if (!context || context->closed || !inputs || input_count != 1 || !sink || sink->struct_size != sizeof(*sink) ||
+        !sink->write)
+        return VX_STATUS_INVALID_ARGUMENT;
+    compiled = context->compiled;
+    binding = &inputs[0];
+    /* the complete batch is validated before anything is mutated */
+    if (binding->struct_size != sizeof(*binding) || !binding->name || strcmp(binding->name, compiled->input_name) ||
+        binding->dtype != compiled->input_dtype || binding->rank != compiled->rank ||
+        binding->location != VX_MEMORY_HOST || !binding->data ||
+        binding->shape[compiled->rank - 1] != (int64_t)compiled->d_in)
+        return VX_STATUS_INVALID_ARGUMENT;
+    for (uint32_t axis = 0; axis + 1 < compiled->rank; axis++) {
+        const int64_t extent = binding->shape[axis];
+        if (extent < compiled->lead_min[axis] || extent > compiled->lead_max[axis] ||
+            extent % compiled->lead_multiple[axis] != 0)
+            return VX_STATUS_INVALID_ARGUMENT;
+        rows *= (uint64_t)extent;
+        shape[axis] = extent;
+    }
+    shape[compiled->rank - 1] = (int64_t)compiled->d_out;
+    input_bytes = (size_t)rows * compiled->d_in * compiled->input_element_bytes;
+    output_bytes = (size_t)rows * compiled->d_out * compiled->output_element_bytes;
+    if (binding->byte_size != input_bytes) return VX_STATUS_INVALID_ARGUMENT;
+
+    status = grow_device(&context->input_dev, &context->input_capacity, input_bytes);
+    if (status == VX_STATUS_OK) status = grow_device(&context->output_dev, &context->output_capacity, output_bytes);
+    if (status == VX_STATUS_OK && output_bytes > context->host_capacity) {
+        void* fresh = realloc(context->output_host, output_bytes);
+        if (!fresh) status = VX_STATUS_OUT_OF_MEMORY;
+        else {
+            context->output_host = fresh;
+            context->host_capacity = output_bytes;
+        }
+    }
+    if (status != VX_STATUS_OK) {
+        fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
+        return status;
+    }
+    status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->input_dev, binding->data, input_bytes);
+    if (status == VX_STATUS_OK) {
+        if (compiled->qlinear)
+            handled = vxhip_qlinear_forward(context->ctx, compiled->qlinear, context->input_dev, context->output_dev, NULL,
+                                            (uint32_t)rows, compiled->input_scale, compiled->input_zero_point,
+                                            compiled->output_scale, compiled->output_zero_point,
+                                            (uint32_t)compiled->input_dtype, (uint32_t)compiled->output_dtype);
+        else
+            handled = vxhip_packed_linear_forward_f32(context->ctx, compiled->packed, (const float*)context->input_dev,
+                                                      (float*)context->output_dev, (uint32_t)rows) == 0;
+        if (!handled) status = VX_STATUS_EXECUTION_FAILED;
+    }
+    if (status == VX_STATUS_OK)
+        status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host, context->output_dev, output_bytes);
+    if (status != VX_STATUS_OK) {
+        fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
+        return status;
+    }
+    status = sink->write(sink->user_data, compiled->output_name, compiled->output_dtype, shape, compiled->rank,
+                         context->output_host, output_bytes);
+    if (status != VX_STATUS_OK) return status;
+    fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear executed");
+    attest(report, vxhip_context_last_variant(context->ctx));
+    return VX_STATUS_OK;
+}
+
+static VxStatus hip_context_close(void* context_instance, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    (void)report;
+    if (!context) return VX_STATUS_INVALID_ARGUMENT;
+    context->closed = 1;
+    return VX_STATUS_OK;
+}
+
+VxStatus volvoxai_hip_gfx950_backend_register(VxReport* report) {
+    const VxBackendProvider provider = {
+        .struct_size = sizeof(VxBackendProvider),
+        .abi_version = VX_BACKEND_ABI_VERSION,
+        .name = PROVIDER_NAME,
+        .shape_domain = {
+            .struct_size = sizeof(VxBackendShapeDomainCapability),
+            .proof_protocol = VX_BACKEND_SHAPE_PROOF_PROTOCOL,
+            .resource_protocol = VX_BACKEND_RESOURCE_PROTOCOL,
+            .support = VX_BACKEND_SHAPE_DOMAIN_FULL,
+        },
+        .runtime_create = hip_runtime_create,
+        .runtime_destroy = hip_runtime_destroy,
+        .compile = hip_compile,
+        .compiled_destroy = hip_compiled_destroy,
+        .context_create = hip_context_create,
+        .context_execute = hip_context_execute,
+        .context_close = hip_context_close,
+        .context_destroy = hip_context_destroy,
+        .exact_contract_marker = VX_BACKEND_PROVIDER_EXACT_CONTRACT_MARKER,
+        .exact_contract_extent = sizeof(VxBackendProvider),
+    };
+    return vx_backend_register_provider(&provider, report);
+}
+
+/* Reads a package exactly as compile does, without a device: lets a build without a GPU check
+ * what the provider would accept.  Returns the compile status and the refusal text. */
+VxStatus volvoxai_hip_gfx950_inspect_package(const VxModelSource* source, VxPackedArithmetic arithmetic,
+                                             uint32_t* d_in, uint32_t* d_out, int32_t* is_packed_linear,
+                                             char* message, size_t message_capacity) {
+    PackagePlan plan;
+    Failure failure = {VX_STATUS_OK, {0}};
+    VxStatus status;
+    if (!source || source->struct_size != sizeof(*source)) return VX_STATUS_INVALID_ARGUMENT;
+    status = plan_package(source, arithmetic, &plan, &failure);
+    if (message && message_capacity) snprintf(message, message_capacity, "%s", failure.message);
+    if (status == VX_STATUS_OK) {
+        if (d_in) *d_in = plan.d_in;
+        if (d_out) *d_out = plan.d_out;
+        if (is_packed_linear) *is_packed_linear = plan.kind == PLAN_PACKED_LINEAR;
+        plan_release(&plan);
+    }
+    return status;
+}

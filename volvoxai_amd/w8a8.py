@@ -89,6 +89,13 @@ class Context:
         _check(library().vxhip_context_fault_flags(self._h, C.byref(v)), "vxhip_context_fault_flags")
         return v.value
 
+    def probe_mfma_rate(self, rounds=128, random_operands=True) -> dict:
+        """Register-only MFMA loop: the int8 rate, shader clock and time it reached."""
+        tops, mhz, us = C.c_double(0), C.c_double(0), C.c_double(0)
+        _check(library().vxhip_probe_mfma_rate(self._h, int(rounds), 1 if random_operands else 0, C.byref(tops),
+                                               C.byref(mhz), C.byref(us)), "vxhip_probe_mfma_rate")
+        return {"tops": tops.value, "shader_mhz": mhz.value, "microseconds": us.value}
+
 
 class QLinear:
     """Compiled scope of one QLinear/QMatMul/QGemm node: prepacked weights."""
