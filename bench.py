@@ -144,13 +144,61 @@ def cpu_baseline_gemv(k, n, seed):
             "kind": kind, "sample": f"{route}, M=1 K={k} N={n} full size, {dt * 1e3:.2f} ms per call"}
 
 
+def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
+    """BASELINE config 4: random-init W8A8 decoder, every linear on the PackedLinear kernels,
+    greedy decode of 32 concurrent rows, 128-token prompts, 128 new tokens each."""
+    from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
+    cfg = DecoderConfig()
+    dec = W8A8Decoder(cfg, init_weights(cfg, 2024), rows)
+    prompt = torch.from_numpy(np.random.default_rng(7).integers(0, cfg.vocab, (rows, prompt_len))).cuda()
+    torch.cuda.synchronize()
+    dec.prefill(prompt)  # warm-up of the prefill shapes
+    dec.stream.synchronize()
+    t0 = time.perf_counter()
+    dec.prefill(prompt)
+    dec.stream.synchronize()
+    prefill_s = time.perf_counter() - t0
+    prefill_variant = dec.ctx.last_variant
+    dec.capture()
+    t0 = time.perf_counter()
+    tokens = dec.decode(new_tokens - 1)
+    decode_s = time.perf_counter() - t0
+    step_variant = dec.ctx.last_variant
+    # the same decode without the graph, for the launch-overhead comparison
+    dec.prefill(prompt)
+    dec.stream.synchronize()
+    graph, dec.graph = dec.graph, None
+    t0 = time.perf_counter()
+    eager_tokens = dec.decode(new_tokens - 1)
+    eager_s = time.perf_counter() - t0
+    same = bool((tokens == eager_tokens).all().item())
+    weight_bytes = sum(L[k].resident_bytes for L in dec.layers for k in ("qkv", "o", "gate_up", "down")) + \
+        dec.lm_head.resident_bytes
+    dec.graph = graph
+    dec.close()
+    total_s = prefill_s + decode_s
+    return {"workload": "configs[3]: 28-layer W8A8 decoder (hidden 1024, 16q/8kv x128, SwiGLU 3072, vocab 32000), "
+                        "32 rows, prompt 128, 128 new tokens, greedy",
+            "value": rows * new_tokens / total_s, "unit": "tokens/s",
+            "decode_tokens_per_s": rows * (new_tokens - 1) / decode_s,
+            "prefill_tokens_per_s": rows * prompt_len / prefill_s,
+            "ms_per_decode_step": decode_s * 1e3 / (new_tokens - 1),
+            "ms_per_decode_step_without_graph": eager_s * 1e3 / (new_tokens - 1),
+            "prefill_ms": prefill_s * 1e3, "graph_and_eager_tokens_equal": same,
+            "decode_linear_variant": step_variant, "prefill_linear_variant": prefill_variant,
+            "weight_bytes_read_per_step": weight_bytes,
+            "decode_hbm_GBs": weight_bytes / (decode_s / (new_tokens - 1)) / 1e9,
+            "glue": "PyTorch-ROCm f32 ops (RMSNorm, RoPE, GQA attention over a KV cache, SwiGLU); one HIP graph per "
+                    "decode step"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["gemm", "gemv", "copy"], default=None,
+    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "copy"], default=None,
                     help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
                          "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
@@ -278,6 +326,13 @@ def main():
                        config={"workload": out["gemv"]["workload"]}, roofline=out["roofline_gemv"])
         for p in pls:
             p.close()
+
+    # ---- config 4: 28-layer decoder, 32 rows, greedy decode ------------------------
+    if args.only in (None, "decoder"):
+        out["decoder"] = bench_decoder(torch)
+        if args.only == "decoder":
+            out.update(value=out["decoder"]["value"], unit="tokens/s", ms_per_step=out["decoder"]["ms_per_decode_step"],
+                       config={"workload": out["decoder"]["workload"]})
 
     if not args.no_cpu_baseline:
         if args.only in (None, "gemm"):

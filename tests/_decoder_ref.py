@@ -1,0 +1,76 @@
+"""CPU restatement of the config-4 decoder for the parity test: the oracle's PackedLinear
+(DYNAMIC_I8) for every linear, numpy for the glue, same definitions as
+volvoxai_amd/decoder.py (RMSNorm in double: native/src/kernels/softmax_rmsnorm.inc:3-17;
+non-interleaved rotary embedding: native/src/kernels/llm_math.h:256-274).  Test
+infrastructure only."""
+import numpy as np
+
+
+class DecoderRef:
+    def __init__(self, cfg, weights, oracle, rope_tables):
+        self.cfg, self.w, self.orc = cfg, weights, oracle
+        self.cos, self.sin = rope_tables(cfg)
+        self.packed = {}
+
+    def linear(self, key, lin, x2d):
+        if key not in self.packed:
+            self.packed[key] = self.orc.pack_w8_words(lin["w"])
+        _, y = self.orc.packed_linear(np.ascontiguousarray(x2d, np.float32), self.packed[key], lin["scales"], None,
+                                      lin["w"].shape[0], self.cfg.group)
+        return y
+
+    def rmsnorm(self, x, gain):
+        xd = x.astype(np.float64)
+        inv = 1.0 / np.sqrt((xd * xd).mean(-1, keepdims=True) + self.cfg.eps)
+        return (xd * inv * gain.astype(np.float64)).astype(np.float32)
+
+    def rope(self, x, cos, sin):
+        half = self.cfg.head_dim // 2
+        partner = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
+        return (x * cos[None, :, None, :] + partner * sin[None, :, None, :]).astype(np.float32)
+
+    def forward(self, tokens, start, k_cache, v_cache):
+        """tokens [rows, t] at positions start..start+t-1; caches [layers][rows, kvh, seq, d] lists
+        grown in place.  Returns the logits of the last position."""
+        cfg = self.cfg
+        rows, t = tokens.shape
+        x = self.w["embedding"][tokens]
+        cos, sin = self.cos[start:start + t], self.sin[start:start + t]
+        rep = cfg.q_heads // cfg.kv_heads
+        for li, L in enumerate(self.w["layers"]):
+            h = self.rmsnorm(x, L["norm1"])
+            qkv = self.linear((li, "qkv"), L["qkv"], h.reshape(rows * t, -1)).reshape(rows, t, -1)
+            q = self.rope(qkv[..., :cfg.q_dim].reshape(rows, t, cfg.q_heads, cfg.head_dim), cos, sin)
+            k = self.rope(qkv[..., cfg.q_dim:cfg.q_dim + cfg.kv_dim].reshape(rows, t, cfg.kv_heads, cfg.head_dim), cos, sin)
+            v = qkv[..., cfg.q_dim + cfg.kv_dim:].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
+            k_cache[li] = np.concatenate([k_cache[li], k.transpose(0, 2, 1, 3)], axis=2)
+            v_cache[li] = np.concatenate([v_cache[li], v.transpose(0, 2, 1, 3)], axis=2)
+            seq = k_cache[li].shape[2]
+            qg = q.transpose(0, 2, 1, 3).reshape(rows, cfg.kv_heads, rep, t, cfg.head_dim)
+            scores = np.einsum("bgrtd,bgsd->bgrts", qg, k_cache[li]).astype(np.float32) * np.float32(1.0 / np.sqrt(cfg.head_dim))
+            visible = np.arange(seq)[None, :] <= (start + np.arange(t))[:, None]
+            scores = np.where(visible[None, None, None], scores, -np.inf)
+            scores = scores - scores.max(-1, keepdims=True)
+            p = np.exp(scores).astype(np.float32)
+            p = p / p.sum(-1, keepdims=True)
+            ctxv = np.einsum("bgrts,bgsd->bgrtd", p, v_cache[li]).astype(np.float32)
+            attn = ctxv.reshape(rows, cfg.q_heads, t, cfg.head_dim).transpose(0, 2, 1, 3).reshape(rows * t, cfg.q_dim)
+            x = x + self.linear((li, "o"), L["o"], attn).reshape(rows, t, -1)
+            h = self.rmsnorm(x, L["norm2"])
+            gu = self.linear((li, "gu"), L["gate_up"], h.reshape(rows * t, -1))
+            gate, up = gu[:, :cfg.inter], gu[:, cfg.inter:]
+            act = (gate / (1.0 + np.exp(-gate.astype(np.float64)))).astype(np.float32) * up
+            x = x + self.linear((li, "down"), L["down"], act).reshape(rows, t, -1)
+        return self.linear("head", self.w["lm_head"], self.rmsnorm(x[:, -1, :], self.w["norm_f"]))
+
+    def generate(self, prompt, new_tokens):
+        cfg = self.cfg
+        rows = prompt.shape[0]
+        kc = [np.zeros((rows, cfg.kv_heads, 0, cfg.head_dim), np.float32) for _ in range(cfg.layers)]
+        vc = [np.zeros((rows, cfg.kv_heads, 0, cfg.head_dim), np.float32) for _ in range(cfg.layers)]
+        logits = [self.forward(prompt, 0, kc, vc)]
+        out = [logits[-1].argmax(-1)]
+        for i in range(new_tokens - 1):
+            logits.append(self.forward(out[-1][:, None], prompt.shape[1] + i, kc, vc))
+            out.append(logits[-1].argmax(-1))
+        return np.stack(out), logits

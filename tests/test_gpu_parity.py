@@ -158,7 +158,8 @@ def test_packed_reference_vectors(ctx, oracle, entry):
 
 # ---- both kernel families give the same bits ------------------------------------------
 
-@pytest.mark.parametrize("rows,k,n", [(1, 256, 64), (7, 640, 100), (16, 4096, 96), (16, 48, 40)])
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 64), (7, 640, 100), (16, 4096, 96), (16, 48, 40), (32, 1024, 72),
+                                      (23, 300, 33)])
 def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(rows, k, n, 77, I8, U8, I8, False)
@@ -177,7 +178,7 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
 
 
 @pytest.mark.parametrize("group", [32, 64, 128, 256])
-@pytest.mark.parametrize("rows,k,n", [(1, 4096, 48), (5, 1000, 36), (16, 1536, 130)])
+@pytest.mark.parametrize("rows,k,n", [(1, 4096, 48), (5, 1000, 36), (16, 1536, 130), (32, 1024, 40), (27, 1024, 96)])
 def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     import volvoxai_amd as vx
     c = cases.packed_case(rows, k, n, group, 5 + group, True, special_rows=(rows >= 5))

@@ -37,7 +37,7 @@ struct PackedWeight {
 };
 
 constexpr uint32_t kPanelRows = 32, kStepK = 32, kPanelPad = 8, kStepPad = 4;
-constexpr uint32_t kMaxGemvRows = 16;
+constexpr uint32_t kMaxGemvRows = 32;  // the MFMA operand has 32 row slots
 
 enum FaultBits : uint32_t {
     kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive

@@ -1,4 +1,4 @@
-// Bandwidth-bound W8A8 linear for decode-shaped M <= 16.  Every weight byte is
+// Bandwidth-bound W8A8 linear for decode-shaped M <= 32.  Every weight byte is
 // read exactly once, straight from HBM into MFMA operand registers with
 // coalesced dwordx4 loads (no LDS hop), and multiplied against all M rows at
 // once on v_mfma_i32_32x32x32_i8, whose internal reduction replaces the

@@ -1,0 +1,248 @@
+"""Decoder-only transformer with every linear routed to the W8A8 PackedLinear
+kernels (BASELINE config 4): RMSNorm, rotary embedding, grouped-query attention
+over a KV cache, SwiGLU, residual adds and greedy selection run as PyTorch-ROCm
+f32 ops around them; the linears are `vxhip_packed_linear_forward_f32`
+(DYNAMIC_I8: per-row activation quantization, int8 x int8 MFMA, dequant to f32).
+
+The glue follows the reference's definitions: RMSNorm accumulates and scales in
+double (native/src/kernels/softmax_rmsnorm.inc:3-17); the rotary embedding is the
+non-interleaved form y[d] = x[d]*cos + sign*x[partner]*sin with partner d +- width/2
+(native/src/kernels/llm_math.h:256-274).
+
+A decode step has fixed shapes (position and tokens live on the device), so it can
+be captured once in a HIP graph and replayed; the launches of the linears are
+captured with it because the context runs on the capture stream.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import w8a8 as vx
+
+
+@dataclass(frozen=True)
+class DecoderConfig:
+    layers: int = 28
+    hidden: int = 1024
+    q_heads: int = 16
+    kv_heads: int = 8
+    head_dim: int = 128
+    inter: int = 3072
+    vocab: int = 32000
+    group: int = 128
+    rope_theta: float = 10000.0
+    eps: float = 1e-6
+    max_seq: int = 256
+
+    @property
+    def q_dim(self):
+        return self.q_heads * self.head_dim
+
+    @property
+    def kv_dim(self):
+        return self.kv_heads * self.head_dim
+
+
+def pack_w8_words(w: np.ndarray) -> np.ndarray:
+    """int8 [n, k] -> offset-binary W8 words [n, ceil(k/4)]: code = w + 128, element 4i+j in
+    byte j of word i, absent elements as the zero code 0x80 (docs/packed-linear-design.md:24-32)."""
+    n, k = w.shape
+    words = (k + 3) // 4
+    codes = np.full((n, words * 4), 0x80, np.uint8)
+    codes[:, :k] = (w.astype(np.int16) + 128).astype(np.uint8)
+    return codes.view("<u4").reshape(n, words)
+
+
+def init_weights(cfg: DecoderConfig, seed: int) -> dict:
+    """Random-init weights of the architecture: int8 uniform +-127 with per-channel scales
+    ~U(0.002, 0.01) for every linear, f32 embedding and norm gains."""
+    rng = np.random.default_rng(seed)
+
+    def linear(n, k):
+        w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+        chan = rng.uniform(0.002, 0.01, n).astype(np.float32)
+        groups = (k + cfg.group - 1) // cfg.group
+        return {"w": w, "scales": np.repeat(chan[:, None], groups, axis=1).copy()}
+
+    layers = []
+    for _ in range(cfg.layers):
+        layers.append({
+            "norm1": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+            "qkv": linear(cfg.q_dim + 2 * cfg.kv_dim, cfg.hidden),
+            "o": linear(cfg.hidden, cfg.q_dim),
+            "norm2": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+            "gate_up": linear(2 * cfg.inter, cfg.hidden),
+            "down": linear(cfg.hidden, cfg.inter),
+        })
+    return {"embedding": rng.normal(0, 1, (cfg.vocab, cfg.hidden)).astype(np.float32),
+            "layers": layers,
+            "norm_f": rng.uniform(0.5, 1.5, cfg.hidden).astype(np.float32),
+            "lm_head": linear(cfg.vocab, cfg.hidden)}
+
+
+def rope_tables(cfg: DecoderConfig):
+    """cos/sin [max_seq, head_dim]: entry d and d + head_dim/2 share frequency d % (head_dim/2)."""
+    half = cfg.head_dim // 2
+    inv = cfg.rope_theta ** (-np.arange(half, dtype=np.float64) * 2.0 / cfg.head_dim)
+    angle = np.arange(cfg.max_seq, dtype=np.float64)[:, None] * inv[None, :]
+    angle = np.concatenate([angle, angle], axis=1)
+    return np.cos(angle).astype(np.float32), np.sin(angle).astype(np.float32)
+
+
+class W8A8Decoder:
+    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None):
+        import torch
+        self.torch, self.cfg, self.rows = torch, cfg, rows
+        self.stream = stream if stream is not None else torch.cuda.Stream()
+        self.ctx = vx.Context(0, self.stream)
+        dev = "cuda"
+
+        def make(lin):
+            k = lin["w"].shape[1]
+            return vx.PackedLinear(pack_w8_words(lin["w"]), lin["scales"], None, k, lin["w"].shape[0], cfg.group)
+
+        self.embedding = torch.from_numpy(weights["embedding"]).to(dev)
+        self.layers = []
+        for lw in weights["layers"]:
+            self.layers.append({"norm1": torch.from_numpy(lw["norm1"]).to(dev).double(),
+                                "norm2": torch.from_numpy(lw["norm2"]).to(dev).double(),
+                                "qkv": make(lw["qkv"]), "o": make(lw["o"]),
+                                "gate_up": make(lw["gate_up"]), "down": make(lw["down"])})
+        self.norm_f = torch.from_numpy(weights["norm_f"]).to(dev).double()
+        self.lm_head = make(weights["lm_head"])
+        cos, sin = rope_tables(cfg)
+        self.cos, self.sin = torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev)
+        shape = (cfg.layers, rows, cfg.kv_heads, cfg.max_seq, cfg.head_dim)
+        self.k_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
+        self.v_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
+        # state of the decode loop, on the device so a captured step advances by itself
+        self.tokens = torch.zeros(rows, dtype=torch.int64, device=dev)
+        self.position = torch.zeros(1, dtype=torch.int64, device=dev)
+        self.history = torch.zeros((cfg.max_seq, rows), dtype=torch.int64, device=dev)
+        self.slots = torch.arange(cfg.max_seq, device=dev)
+        self.graph = None
+
+    # ---- pieces ---------------------------------------------------------------------------
+    def _linear(self, pl, x2d):
+        torch = self.torch
+        x2d = x2d.contiguous()
+        out = torch.empty((x2d.shape[0], pl.n), dtype=torch.float32, device=x2d.device)
+        st, _ = pl.forward_f32(self.ctx, x2d, out=out)
+        if st != 0:
+            raise RuntimeError(vx.library().vxhip_last_error().decode())
+        return out
+
+    def _rmsnorm(self, x, gain):
+        xd = x.double()
+        inv = 1.0 / self.torch.sqrt((xd * xd).mean(-1, keepdim=True) + self.cfg.eps)
+        return (xd * inv * gain).float()
+
+    def _rope(self, x, cos, sin):
+        # x [rows, t, heads, d]; cos/sin [t, d]
+        half = self.cfg.head_dim // 2
+        partner = self.torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+        return x * cos[None, :, None, :] + partner * sin[None, :, None, :]
+
+    def _layer(self, li, x, cos, sin, write_slots, visible):
+        """x [rows, t, hidden]; write_slots [t] cache positions of these tokens; visible
+        [t, max_seq] bool: which cache slots each of them may attend to."""
+        torch, cfg, L = self.torch, self.cfg, self.layers[li]
+        rows, t, _ = x.shape
+        h = self._rmsnorm(x, L["norm1"])
+        qkv = self._linear(L["qkv"], h.reshape(rows * t, cfg.hidden)).reshape(rows, t, -1)
+        q = qkv[..., :cfg.q_dim].reshape(rows, t, cfg.q_heads, cfg.head_dim)
+        k = qkv[..., cfg.q_dim:cfg.q_dim + cfg.kv_dim].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
+        v = qkv[..., cfg.q_dim + cfg.kv_dim:].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
+        q, k = self._rope(q, cos, sin), self._rope(k, cos, sin)
+        self.k_cache[li].index_copy_(2, write_slots, k.permute(0, 2, 1, 3))
+        self.v_cache[li].index_copy_(2, write_slots, v.permute(0, 2, 1, 3))
+        rep = cfg.q_heads // cfg.kv_heads
+        qg = q.permute(0, 2, 1, 3).reshape(rows, cfg.kv_heads, rep * t, cfg.head_dim)
+        scores = torch.matmul(qg, self.k_cache[li].transpose(-1, -2)) * (1.0 / np.sqrt(cfg.head_dim))
+        scores = scores.reshape(rows, cfg.kv_heads, rep, t, cfg.max_seq)
+        scores = scores.masked_fill(~visible[None, None, None], float("-inf"))
+        probs = torch.softmax(scores, dim=-1).reshape(rows, cfg.kv_heads, rep * t, cfg.max_seq)
+        ctxv = torch.matmul(probs, self.v_cache[li]).reshape(rows, cfg.q_heads, t, cfg.head_dim)
+        attn = ctxv.permute(0, 2, 1, 3).reshape(rows * t, cfg.q_dim)
+        x = x + self._linear(L["o"], attn).reshape(rows, t, cfg.hidden)
+        h = self._rmsnorm(x, L["norm2"])
+        gu = self._linear(L["gate_up"], h.reshape(rows * t, cfg.hidden))
+        act = torch.nn.functional.silu(gu[:, :cfg.inter]) * gu[:, cfg.inter:]
+        return x + self._linear(L["down"], act).reshape(rows, t, cfg.hidden)
+
+    def _head(self, x_last):
+        logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
+        return logits, logits.argmax(dim=-1)
+
+    # ---- prefill and decode -----------------------------------------------------------------
+    def prefill(self, prompt):
+        """prompt int64 [rows, t] on the device; fills the cache and returns the first new tokens."""
+        torch, cfg = self.torch, self.cfg
+        with torch.cuda.stream(self.stream):
+            t = prompt.shape[1]
+            slots = self.slots[:t]
+            visible = self.slots[None, :] <= slots[:, None]
+            x = self.embedding[prompt]
+            for li in range(cfg.layers):
+                x = self._layer(li, x, self.cos[:t], self.sin[:t], slots, visible)
+            self.last_logits, nxt = self._head(x[:, -1, :])
+            self.tokens.copy_(nxt)
+            self.position.fill_(t)
+            self.history.zero_()
+            self.history[0].copy_(nxt)
+            self.emitted = 1
+        return nxt
+
+    def _step(self):
+        torch, cfg = self.torch, self.cfg
+        pos = self.position
+        visible = self.slots[None, :] <= pos[:, None]
+        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
+        x = self.embedding[self.tokens][:, None, :]
+        for li in range(cfg.layers):
+            x = self._layer(li, x, cos, sin, pos, visible)
+        self.last_logits, nxt = self._head(x[:, 0, :])
+        self.tokens.copy_(nxt)
+        self.position.add_(1)
+        return nxt
+
+    def capture(self):
+        """Capture one decode step in a HIP graph (after a warm-up step has sized every scratch)."""
+        torch = self.torch
+        keep = (self.tokens.clone(), self.position.clone(), self.k_cache.clone(), self.v_cache.clone())
+        with torch.cuda.stream(self.stream):
+            self._step()  # warm-up: allocations and one-time kernel attributes happen here
+        self.stream.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=self.stream):
+            self.step_out = self._step()
+        self.stream.synchronize()
+        self.tokens.copy_(keep[0])
+        self.position.copy_(keep[1])
+        self.k_cache.copy_(keep[2])
+        self.v_cache.copy_(keep[3])
+        torch.cuda.synchronize()
+
+    def decode(self, steps):
+        """Greedy decode of `steps` further tokens per row; returns int64 [emitted, rows]."""
+        torch = self.torch
+        with torch.cuda.stream(self.stream):
+            for _ in range(steps):
+                if self.graph is not None:
+                    self.graph.replay()
+                    nxt = self.step_out
+                else:
+                    nxt = self._step()
+                self.history[self.emitted].copy_(nxt)
+                self.emitted += 1
+        self.stream.synchronize()
+        return self.history[:self.emitted]
+
+    def close(self):
+        for L in self.layers:
+            for name in ("qkv", "o", "gate_up", "down"):
+                L[name].close()
+        self.lm_head.close()
+        self.ctx.close()
