@@ -80,6 +80,45 @@ const char* vxhip_context_last_variant(const VxHipContext* context);
  * ...); reading it synchronises the stream.  0 = clean. */
 VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
 
+/* ---- decoder glue around the PackedLinear calls ------------------------- */
+/* The steps either side of the linears of a decoder layer (the components the
+ * reference runs through src/kernels/softmax_rmsnorm.inc, src/kernels/llm_math.h
+ * and src/kernels/attention_f32_core.h; its CUDA backend fuses the same pairs,
+ * src/backends/cuda/kernels/cuda_forward_gemv_pair_kernels.inc:408,672).
+ * Device pointers, asynchronous on the context's stream, f32 row-major. */
+
+/* RMSNorm of rows [rows, d] (double accumulation and scaling, one rounding to
+ * f32: softmax_rmsnorm.inc:3-17) followed by the activation preparation of
+ * vxhip_packed_prepare_i8 on the normalized row.  normalized_dev may be NULL. */
+VxHipStatus vxhip_rmsnorm_prepare_i8(VxHipContext* context, const float* input_dev,
+                                     const float* gain_dev, uint32_t rows, uint32_t d,
+                                     double eps, int8_t* prepared_dev,
+                                     float* row_scales_dev, float* normalized_dev);
+/* silu(gate) * up of gate_up [rows, 2*inter] (gate first), then the same
+ * preparation.  activated_dev [rows, inter] may be NULL. */
+VxHipStatus vxhip_swiglu_prepare_i8(VxHipContext* context, const float* gate_up_dev,
+                                    uint32_t rows, uint32_t inter, int8_t* prepared_dev,
+                                    float* row_scales_dev, float* activated_dev);
+/* Non-interleaved rotary embedding (llm_math.h:256-274) of the q and k heads of
+ * qkv [rows, t, (q_heads + 2*kv_heads) * head_dim] with cos/sin tables
+ * [max_seq, head_dim], token i of every row at cache slot positions_dev[i];
+ * rotated q to q_out [rows, t, q_heads, head_dim], rotated k and plain v into the
+ * caches [rows, kv_heads, max_seq, head_dim]. */
+VxHipStatus vxhip_rope_append_kv(VxHipContext* context, const float* qkv_dev,
+                                 const float* cos_dev, const float* sin_dev,
+                                 const int64_t* positions_dev, uint32_t rows, uint32_t t,
+                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                 uint32_t max_seq, float* q_out_dev, float* k_cache_dev,
+                                 float* v_cache_dev);
+/* Grouped-query attention of q [rows, t, q_heads, head_dim] over the caches:
+ * scores q.k * f32(1/sqrt(head_dim)), slots 0..positions_dev[i] visible to
+ * token i, softmax, P.V; out [rows, t, q_heads * head_dim]. */
+VxHipStatus vxhip_gqa_attention(VxHipContext* context, const float* q_dev,
+                                const float* k_cache_dev, const float* v_cache_dev,
+                                const int64_t* positions_dev, uint32_t rows, uint32_t t,
+                                uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                uint32_t max_seq, float* out_dev);
+
 /* Measurement aid with no counterpart in the reference: runs a register-only
  * v_mfma_i32_32x32x32_i8 loop (16 accumulators per wave, one wave per SIMD,
  * `rounds` x 16 MFMAs per wave) and reports the int8 rate it reached, the

@@ -29,9 +29,103 @@ def test_rope_tables_are_rotations():
     assert (cos[:, :cfg.head_dim // 2] == cos[:, cfg.head_dim // 2:]).all()
 
 
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,d", [(1, 64), (5, 1024), (33, 3000)])
+def test_rmsnorm_prepare_kernel(ctx, oracle, rows, d):
+    """Normalized rows against the double-precision definition; codes and scales must be exactly
+    what the oracle's preparation makes of the kernel's own normalized rows."""
+    import volvoxai_amd.w8a8 as vx
+    rng = np.random.default_rng(d)
+    x = (rng.normal(0, 3, (rows, d)) * rng.uniform(0.01, 100, (rows, 1))).astype(np.float32)
+    if rows >= 5:
+        x[1] = 0.0
+        x[2, 3] = np.inf
+    gain = rng.uniform(0.5, 1.5, d).astype(np.float32)
+    a8, sc, normalized = vx.rmsnorm_prepare_i8(ctx, _dev(x), _dev(gain), 1e-6, want_normalized=True)
+    ctx.synchronize()
+    a8, sc, normalized = a8.cpu().numpy(), sc.cpu().numpy(), normalized.cpu().numpy()
+    xd = x.astype(np.float64)
+    with np.errstate(all="ignore"):
+        want = (xd * (1.0 / np.sqrt((xd * xd).mean(-1, keepdims=True) + 1e-6)) * gain.astype(np.float64)).astype(np.float32)
+    finite = np.isfinite(want).all(-1)
+    assert np.allclose(normalized[finite], want[finite], rtol=3e-7, atol=0)
+    want_codes, want_scales, fin = oracle.packed_prepare(normalized)
+    good = fin == 1
+    assert (np.isnan(sc) == ~good).all() and (good == finite).all() and not a8[~good].any()
+    assert (a8[good] == want_codes[good]).all() and (sc[good].view(np.uint32) == want_scales[good].view(np.uint32)).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,inter", [(1, 32), (7, 3072), (32, 1000)])
+def test_swiglu_prepare_kernel(ctx, oracle, rows, inter):
+    import volvoxai_amd.w8a8 as vx
+    rng = np.random.default_rng(inter)
+    gu = rng.normal(0, 4, (rows, 2 * inter)).astype(np.float32)
+    a8, sc, act = vx.swiglu_prepare_i8(ctx, _dev(gu), want_activated=True)
+    ctx.synchronize()
+    a8, sc, act = a8.cpu().numpy(), sc.cpu().numpy(), act.cpu().numpy()
+    gate, up = gu[:, :inter].astype(np.float64), gu[:, inter:].astype(np.float64)
+    want = gate / (1.0 + np.exp(-gate)) * up
+    assert np.allclose(act, want, rtol=1e-6, atol=1e-30)
+    want_codes, want_scales, fin = oracle.packed_prepare(act)
+    assert fin.all() and (a8 == want_codes).all() and (sc.view(np.uint32) == want_scales.view(np.uint32)).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,t,start", [(2, 1, 7), (3, 5, 0)])
+def test_rope_append_and_attention_kernels(ctx, rows, t, start):
+    import torch
+    import volvoxai_amd.w8a8 as vx
+    from volvoxai_amd.decoder import DecoderConfig, rope_tables
+    cfg = DecoderConfig(layers=1, hidden=64, q_heads=4, kv_heads=2, head_dim=32, inter=64, vocab=10, max_seq=16)
+    rng = np.random.default_rng(rows * 10 + t)
+    cos, sin = rope_tables(cfg)
+    width = cfg.q_dim + 2 * cfg.kv_dim
+    qkv = rng.normal(0, 1, (rows, t, width)).astype(np.float32)
+    k_cache = rng.normal(0, 1, (rows, cfg.kv_heads, cfg.max_seq, cfg.head_dim)).astype(np.float32)
+    v_cache = rng.normal(0, 1, (rows, cfg.kv_heads, cfg.max_seq, cfg.head_dim)).astype(np.float32)
+    positions = np.arange(start, start + t, dtype=np.int64)
+    kd, vd = _dev(k_cache), _dev(v_cache)
+    q = vx.rope_append_kv(ctx, _dev(qkv), _dev(cos), _dev(sin), _dev(positions), cfg.q_heads, cfg.kv_heads,
+                          cfg.head_dim, kd, vd)
+    out = vx.gqa_attention(ctx, q, kd, vd, _dev(positions))
+    ctx.synchronize()
+    half = cfg.head_dim // 2
+
+    def rope(x):  # [rows, t, heads, d]
+        partner = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
+        c, s = cos[positions][None, :, None, :], sin[positions][None, :, None, :]
+        return (x * c + partner * s).astype(np.float32)
+
+    wq = rope(qkv[..., :cfg.q_dim].reshape(rows, t, cfg.q_heads, cfg.head_dim))
+    wk = rope(qkv[..., cfg.q_dim:cfg.q_dim + cfg.kv_dim].reshape(rows, t, cfg.kv_heads, cfg.head_dim))
+    wv = qkv[..., cfg.q_dim + cfg.kv_dim:].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
+    k_cache[:, :, positions] = wk.transpose(0, 2, 1, 3)
+    v_cache[:, :, positions] = wv.transpose(0, 2, 1, 3)
+    assert (q.cpu().numpy() == wq).all()                 # two products and one sum: same bits
+    assert (kd.cpu().numpy() == k_cache).all() and (vd.cpu().numpy() == v_cache).all()
+    rep = cfg.q_heads // cfg.kv_heads
+    want = np.zeros((rows, t, cfg.q_heads, cfg.head_dim))
+    for h in range(cfg.q_heads):
+        for i in range(t):
+            vis = positions[i] + 1
+            kk, vv = k_cache[:, h // rep, :vis].astype(np.float64), v_cache[:, h // rep, :vis].astype(np.float64)
+            sc = np.einsum("bd,bsd->bs", wq[:, i, h].astype(np.float64), kk) / np.sqrt(cfg.head_dim)
+            p = np.exp(sc - sc.max(-1, keepdims=True))
+            p /= p.sum(-1, keepdims=True)
+            want[:, i, h] = np.einsum("bs,bsd->bd", p, vv)
+    assert np.allclose(out.cpu().numpy().reshape(want.shape), want, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("use_graph", [False, True])
-def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph):
+def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
     import torch
     from volvoxai_amd.decoder import W8A8Decoder, init_weights, rope_tables
     cfg = small_config()
@@ -40,7 +134,7 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph):
     prompt = np.random.default_rng(2).integers(0, cfg.vocab, (rows, prompt_len))
     want_tokens, want_logits = DecoderRef(cfg, weights, oracle, rope_tables).generate(prompt, new)
 
-    dec = W8A8Decoder(cfg, weights, rows)
+    dec = W8A8Decoder(cfg, weights, rows, fused=fused)
     pd = torch.from_numpy(prompt).cuda()
     torch.cuda.synchronize()
     dec.prefill(pd)

@@ -62,6 +62,10 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_context_synchronize": (i32, [vp]),
         "vxhip_context_last_variant": (C.c_char_p, [vp]),
         "vxhip_context_fault_flags": (i32, [vp, C.POINTER(u32)]),
+        "vxhip_rmsnorm_prepare_i8": (i32, [vp, vp, vp, u32, u32, C.c_double, vp, vp, vp]),
+        "vxhip_swiglu_prepare_i8": (i32, [vp, vp, u32, u32, vp, vp, vp]),
+        "vxhip_rope_append_kv": (i32, [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
+        "vxhip_gqa_attention": (i32, [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]),
         "vxhip_probe_mfma_rate": (i32, [vp, u32, u32, C.POINTER(C.c_double), C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]),
         "vxhip_device_malloc": (i32, [sz, pp]),

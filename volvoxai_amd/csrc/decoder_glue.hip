@@ -1,0 +1,277 @@
+// The steps either side of the W8A8 linears in a decoder layer, fused so that a decode step
+// is a dozen launches per layer instead of several dozen elementwise ones:
+//
+//   rmsnorm_prepare   RMSNorm (native/src/kernels/softmax_rmsnorm.inc:3-17: double accumulation,
+//                     x * inv_std * gain in double, one rounding to f32) followed by the
+//                     PackedLinear activation preparation of that row
+//                     (native/src/kernels/packed_linear_ops.inc:97-217)
+//   swiglu_prepare    silu(gate) * up, then the same preparation
+//   rope_append       non-interleaved rotary embedding of q and k
+//                     (native/src/kernels/llm_math.h:256-274) and the KV-cache append
+//   gqa_attention     grouped-query attention of the new tokens over the cache: f32 scores
+//                     scaled by 1/sqrt(d), causal visibility slot <= position, softmax, P.V
+//
+// All are row-sized, latency-bound kernels; none of them is on the int8 roofline.
+#include "common.h"
+#include "device_math.h"
+
+#include <math.h>
+
+namespace vxhip {
+namespace {
+
+extern __shared__ __attribute__((aligned(16))) char glue_lds[];
+
+__device__ __forceinline__ float block_max(float v, float* slots) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off, 64));
+    if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float m = slots[0];
+    for (uint32_t w = 1; w < blockDim.x / 64u; w++) m = fmaxf(m, slots[w]);
+    __syncthreads();
+    return m;
+}
+
+__device__ __forceinline__ float block_sum(float v, float* slots) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = slots[0];
+    for (uint32_t w = 1; w < blockDim.x / 64u; w++) s += slots[w];
+    __syncthreads();
+    return s;
+}
+
+// Shared tail of the two *_prepare kernels: the row's f32 values are in `vals` (LDS).
+// scale = max|v| / 127 (1.0 for an all-zero row, floored at 2^-126), code = ties-to-even(v / scale)
+// clamped to +-127 with a true f32 divide; a non-finite row gets zero codes and a NaN scale.
+__device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_t* codes, float* scale_out,
+                                            float* slots) {
+    float maximum = 0.0f, bad = 0.0f;
+    for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) {
+        const float v = vals[j];
+        if (!finite_f32(v)) bad = 1.0f;
+        maximum = fmaxf(maximum, fabsf(v));
+    }
+    maximum = block_max(maximum, slots);
+    bad = block_max(bad, slots);
+    float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+    if (scale < 0x1p-126f) scale = 0x1p-126f;
+    for (uint32_t j = threadIdx.x; j < d; j += blockDim.x)
+        codes[j] = bad != 0.0f ? (int8_t)0 : (int8_t)packed_round_i8(__fdiv_rn(vals[j], scale));
+    if (threadIdx.x == 0) *scale_out = bad != 0.0f ? __builtin_nanf("") : scale;
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_prepare_kernel(const float* __restrict__ x,
+                                                              const float* __restrict__ gain, uint32_t d, double eps,
+                                                              int8_t* __restrict__ prepared,
+                                                              float* __restrict__ row_scales,
+                                                              float* __restrict__ normalized) {
+    float* vals = reinterpret_cast<float*>(glue_lds);
+    __shared__ double dslots[4];
+    __shared__ float slots[4];
+    const uint32_t row = blockIdx.x;
+    const float* src = x + (size_t)row * d;
+    double sum = 0.0;
+    for (uint32_t j = threadIdx.x; j < d; j += 256u) {
+        const float v = src[j];
+        vals[j] = v;
+        sum += (double)v * (double)v;
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+    if ((threadIdx.x & 63u) == 0u) dslots[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    const double var = (dslots[0] + dslots[1] + dslots[2] + dslots[3]) / (double)d;
+    const double inv_std = 1.0 / sqrt(var + eps);
+    for (uint32_t j = threadIdx.x; j < d; j += 256u) {
+        const float y = (float)((double)vals[j] * inv_std * (double)gain[j]);
+        vals[j] = y;
+        if (normalized) normalized[(size_t)row * d + j] = y;
+    }
+    __syncthreads();
+    prepare_row(vals, d, prepared + (size_t)row * d, row_scales + row, slots);
+}
+
+__global__ __launch_bounds__(256) void swiglu_prepare_kernel(const float* __restrict__ gate_up, uint32_t inter,
+                                                             int8_t* __restrict__ prepared,
+                                                             float* __restrict__ row_scales,
+                                                             float* __restrict__ activated) {
+    float* vals = reinterpret_cast<float*>(glue_lds);
+    __shared__ float slots[4];
+    const uint32_t row = blockIdx.x;
+    const float* gate = gate_up + (size_t)row * 2u * inter;
+    const float* up = gate + inter;
+    for (uint32_t j = threadIdx.x; j < inter; j += 256u) {
+        const float g = gate[j];
+        const float s = __fdiv_rn(g, __fadd_rn(1.0f, expf(-g)));
+        const float y = __fmul_rn(s, up[j]);
+        vals[j] = y;
+        if (activated) activated[(size_t)row * inter + j] = y;
+    }
+    __syncthreads();
+    prepare_row(vals, inter, prepared + (size_t)row * inter, row_scales + row, slots);
+}
+
+// grid (rows * t, q_heads + 2 * kv_heads), block head_dim.  Token (row, i) sits at cache slot
+// positions[i]; cos/sin are [max_seq][head_dim] tables indexed by that slot.
+__global__ void rope_append_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_table,
+                                   const float* __restrict__ sin_table, const int64_t* __restrict__ positions,
+                                   uint32_t t, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                   uint32_t max_seq, float* __restrict__ q_out, float* __restrict__ k_cache,
+                                   float* __restrict__ v_cache) {
+    const uint32_t token = blockIdx.x, head = blockIdx.y, dd = threadIdx.x;
+    const uint32_t row = token / t, i = token % t;
+    const uint32_t width = (q_heads + 2u * kv_heads) * head_dim;
+    const float* src = qkv + (size_t)token * width + (size_t)head * head_dim;
+    const uint32_t slot = (uint32_t)positions[i];
+    const uint32_t half = head_dim / 2u;
+    const float v = src[dd];
+    if (head >= q_heads + kv_heads) {  // value head: plain append
+        const uint32_t h = head - q_heads - kv_heads;
+        v_cache[(((size_t)row * kv_heads + h) * max_seq + slot) * head_dim + dd] = v;
+        return;
+    }
+    const float partner = dd < half ? -src[dd + half] : src[dd - half];
+    const float c = cos_table[(size_t)slot * head_dim + dd], s = sin_table[(size_t)slot * head_dim + dd];
+    const float y = __fadd_rn(__fmul_rn(v, c), __fmul_rn(partner, s));
+    if (head < q_heads) q_out[((size_t)token * q_heads + head) * head_dim + dd] = y;
+    else k_cache[(((size_t)row * kv_heads + (head - q_heads)) * max_seq + slot) * head_dim + dd] = y;
+}
+
+// grid (rows * t, q_heads), block 256.  LDS: q[head_dim] + scores[max_seq] + partial[2][head_dim]
+// floats.  Scores: one thread per visible slot (its whole dot product, 16-byte loads, all
+// independent); P.V: the slots split over the two halves of the block, one thread per channel.
+__global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restrict__ q,
+                                                            const float* __restrict__ k_cache,
+                                                            const float* __restrict__ v_cache,
+                                                            const int64_t* __restrict__ positions, uint32_t t,
+                                                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                                            uint32_t max_seq, float scale, float* __restrict__ out) {
+    float* qs = reinterpret_cast<float*>(glue_lds);
+    float* scores = qs + head_dim;
+    float* partial = scores + max_seq;
+    __shared__ float slots[4];
+    const uint32_t token = blockIdx.x, head = blockIdx.y;
+    const uint32_t row = token / t, i = token % t;
+    const uint32_t kvh = head / (q_heads / kv_heads);
+    const uint32_t visible = (uint32_t)positions[i] + 1u;  // slots 0 .. position
+    const float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    const float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
+        qs[dd] = q[((size_t)token * q_heads + head) * head_dim + dd];
+    __syncthreads();
+    float m = -INFINITY;
+    for (uint32_t s = threadIdx.x; s < visible; s += 256u) {
+        const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)s * head_dim);
+        float dot = 0.0f;
+#pragma unroll 8
+        for (uint32_t c = 0; c < head_dim / 4u; c++) {
+            const float4 kv = kr[c];
+            dot += qs[4 * c] * kv.x + qs[4 * c + 1] * kv.y + qs[4 * c + 2] * kv.z + qs[4 * c + 3] * kv.w;
+        }
+        dot = __fmul_rn(dot, scale);
+        scores[s] = dot;
+        m = fmaxf(m, dot);
+    }
+    m = block_max(m, slots);
+    float sum = 0.0f;
+    for (uint32_t s = threadIdx.x; s < visible; s += 256u) {
+        const float e = expf(scores[s] - m);
+        scores[s] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, slots);
+    for (uint32_t s = threadIdx.x; s < visible; s += 256u) scores[s] = __fdiv_rn(scores[s], sum);
+    __syncthreads();
+    // half 0 takes the even slots, half 1 the odd ones
+    const uint32_t part = threadIdx.x >> 7, lane_d = threadIdx.x & 127u;
+    for (uint32_t dd = lane_d; dd < head_dim; dd += 128u) {
+        float acc = 0.0f;
+#pragma unroll 8
+        for (uint32_t s = part; s < visible; s += 2u) acc += scores[s] * vbase[(size_t)s * head_dim + dd];
+        partial[part * head_dim + dd] = acc;
+    }
+    __syncthreads();
+    for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
+        out[((size_t)token * q_heads + head) * head_dim + dd] = partial[dd] + partial[head_dim + dd];
+}
+
+bool device_ready(VxHipContext* ctx) {
+    return ctx && hipSetDevice(ctx->device) == hipSuccess;
+}
+
+}  // namespace
+}  // namespace vxhip
+
+using namespace vxhip;
+
+extern "C" {
+
+VxHipStatus vxhip_rmsnorm_prepare_i8(VxHipContext* ctx, const float* input_dev, const float* gain_dev, uint32_t rows,
+                                     uint32_t d, double eps, int8_t* prepared_dev, float* row_scales_dev,
+                                     float* normalized_dev) {
+    if (!ctx || !input_dev || !gain_dev || !prepared_dev || !row_scales_dev || !d || d > 15360u) {
+        set_error("rmsnorm_prepare_i8: null argument or row length outside 1..15360");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(256), d * sizeof(float), ctx->stream, input_dev,
+                       gain_dev, d, eps, prepared_dev, row_scales_dev, normalized_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_swiglu_prepare_i8(VxHipContext* ctx, const float* gate_up_dev, uint32_t rows, uint32_t inter,
+                                    int8_t* prepared_dev, float* row_scales_dev, float* activated_dev) {
+    if (!ctx || !gate_up_dev || !prepared_dev || !row_scales_dev || !inter || inter > 15360u) {
+        set_error("swiglu_prepare_i8: null argument or row length outside 1..15360");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    hipLaunchKernelGGL(swiglu_prepare_kernel, dim3(rows), dim3(256), inter * sizeof(float), ctx->stream,
+                       gate_up_dev, inter, prepared_dev, row_scales_dev, activated_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_rope_append_kv(VxHipContext* ctx, const float* qkv_dev, const float* cos_dev, const float* sin_dev,
+                                 const int64_t* positions_dev, uint32_t rows, uint32_t t, uint32_t q_heads,
+                                 uint32_t kv_heads, uint32_t head_dim, uint32_t max_seq, float* q_out_dev,
+                                 float* k_cache_dev, float* v_cache_dev) {
+    if (!ctx || !qkv_dev || !cos_dev || !sin_dev || !positions_dev || !q_out_dev || !k_cache_dev || !v_cache_dev ||
+        !q_heads || !kv_heads || q_heads % kv_heads || !head_dim || head_dim % 2u || head_dim > 1024u || !max_seq) {
+        set_error("rope_append_kv: null argument or unsupported head geometry");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows || !t) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    hipLaunchKernelGGL(rope_append_kernel, dim3(rows * t, q_heads + 2u * kv_heads), dim3(head_dim), 0, ctx->stream,
+                       qkv_dev, cos_dev, sin_dev, positions_dev, t, q_heads, kv_heads, head_dim, max_seq, q_out_dev,
+                       k_cache_dev, v_cache_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const float* k_cache_dev,
+                                const float* v_cache_dev, const int64_t* positions_dev, uint32_t rows, uint32_t t,
+                                uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, uint32_t max_seq,
+                                float* out_dev) {
+    if (!ctx || !q_dev || !k_cache_dev || !v_cache_dev || !positions_dev || !out_dev || !q_heads || !kv_heads ||
+        q_heads % kv_heads || !head_dim || head_dim % 4u || !max_seq ||
+        (3u * head_dim + max_seq) * sizeof(float) > 60u * 1024u) {
+        set_error("gqa_attention: null argument or unsupported geometry");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows || !t) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    const float scale = (float)(1.0 / sqrt((double)head_dim));
+    hipLaunchKernelGGL(gqa_attention_kernel, dim3(rows * t, q_heads), dim3(256),
+                       (3u * head_dim + max_seq) * sizeof(float), ctx->stream, q_dev, k_cache_dev, v_cache_dev,
+                       positions_dev, t, q_heads, kv_heads, head_dim, max_seq, scale, out_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+}  // extern "C"

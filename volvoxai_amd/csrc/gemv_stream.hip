@@ -246,6 +246,12 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
     // workgroups of 8 waves resident per CU) stream fastest; more waves or deeper queues cost
     // occupancy, fewer leave the memory system short of requests.
     int waves = steps >= 16u * 16u ? 16 : steps >= 8u * 16u ? 8 : steps >= 4u * 16u ? 4 : 2;
+    // Few panels (small N) leave most of the device idle and every wave latency bound on its
+    // own short run: then split K further, down to one scale group per wave, until about 4096
+    // waves are in flight.
+    const uint32_t panels = (a.n + 31u) / 32u, chunks = (steps + GK - 1) / GK;
+    for (int more = waves * 2; more <= 16 && (uint32_t)more <= chunks && panels * (uint32_t)more <= 4096u; more *= 2)
+        waves = more;
     if (force && strstr(force, "w16")) waves = 16;
     else if (force && strstr(force, "w8")) waves = 8;
     else if (force && strstr(force, "w4")) waves = 4;

@@ -20,6 +20,7 @@ from dataclasses import dataclass
 import numpy as np
 
 from . import w8a8 as vx
+from ._lib import library as _library
 
 
 @dataclass(frozen=True)
@@ -92,9 +93,11 @@ def rope_tables(cfg: DecoderConfig):
 
 
 class W8A8Decoder:
-    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None):
+    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None, fused=True):
+        """fused=True runs the glue through the library's fused kernels (RMSNorm+prepare,
+        rotary+cache append, attention, SwiGLU+prepare); fused=False through PyTorch ops."""
         import torch
-        self.torch, self.cfg, self.rows = torch, cfg, rows
+        self.torch, self.cfg, self.rows, self.fused = torch, cfg, rows, fused
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
         dev = "cuda"
@@ -108,9 +111,12 @@ class W8A8Decoder:
         for lw in weights["layers"]:
             self.layers.append({"norm1": torch.from_numpy(lw["norm1"]).to(dev).double(),
                                 "norm2": torch.from_numpy(lw["norm2"]).to(dev).double(),
+                                "gain1": torch.from_numpy(lw["norm1"]).to(dev),
+                                "gain2": torch.from_numpy(lw["norm2"]).to(dev),
                                 "qkv": make(lw["qkv"]), "o": make(lw["o"]),
                                 "gate_up": make(lw["gate_up"]), "down": make(lw["down"])})
         self.norm_f = torch.from_numpy(weights["norm_f"]).to(dev).double()
+        self.gain_f = torch.from_numpy(weights["norm_f"]).to(dev)
         self.lm_head = make(weights["lm_head"])
         cos, sin = rope_tables(cfg)
         self.cos, self.sin = torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev)
@@ -131,8 +137,33 @@ class W8A8Decoder:
         out = torch.empty((x2d.shape[0], pl.n), dtype=torch.float32, device=x2d.device)
         st, _ = pl.forward_f32(self.ctx, x2d, out=out)
         if st != 0:
-            raise RuntimeError(vx.library().vxhip_last_error().decode())
+            raise RuntimeError(_library().vxhip_last_error().decode())
         return out
+
+    def _linear_a8(self, pl, a8, scales):
+        torch = self.torch
+        out = torch.empty((a8.shape[0], pl.n), dtype=torch.float32, device=a8.device)
+        st, _ = pl.forward_a8(self.ctx, a8, scales, out=out)
+        if st != 0:
+            raise RuntimeError(_library().vxhip_last_error().decode())
+        return out
+
+    def _layer_fused(self, li, x, positions):
+        """The same layer through the fused glue kernels; x [rows, t, hidden], positions int64 [t]."""
+        cfg, L = self.cfg, self.layers[li]
+        rows, t, _ = x.shape
+        x2 = x.reshape(rows * t, cfg.hidden)
+        a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, L["gain1"], cfg.eps)
+        qkv = self._linear_a8(L["qkv"], a8, sc).reshape(rows, t, -1)
+        q = vx.rope_append_kv(self.ctx, qkv, self.cos, self.sin, positions, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
+                              self.k_cache[li], self.v_cache[li])
+        attn = vx.gqa_attention(self.ctx, q, self.k_cache[li], self.v_cache[li], positions)
+        x2 = x2 + self._linear(L["o"], attn.reshape(rows * t, cfg.q_dim))
+        a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, L["gain2"], cfg.eps)
+        gu = self._linear_a8(L["gate_up"], a8, sc)
+        a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
+        x2 = x2 + self._linear_a8(L["down"], a8, sc)
+        return x2.reshape(rows, t, cfg.hidden)
 
     def _rmsnorm(self, x, gain):
         xd = x.double()
@@ -173,7 +204,11 @@ class W8A8Decoder:
         return x + self._linear(L["down"], act).reshape(rows, t, cfg.hidden)
 
     def _head(self, x_last):
-        logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
+        if self.fused:
+            a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x_last.contiguous(), self.gain_f, self.cfg.eps)
+            logits = self._linear_a8(self.lm_head, a8, sc)
+        else:
+            logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
         return logits, logits.argmax(dim=-1)
 
     # ---- prefill and decode -----------------------------------------------------------------
@@ -186,7 +221,10 @@ class W8A8Decoder:
             visible = self.slots[None, :] <= slots[:, None]
             x = self.embedding[prompt]
             for li in range(cfg.layers):
-                x = self._layer(li, x, self.cos[:t], self.sin[:t], slots, visible)
+                if self.fused:
+                    x = self._layer_fused(li, x, slots)
+                else:
+                    x = self._layer(li, x, self.cos[:t], self.sin[:t], slots, visible)
             self.last_logits, nxt = self._head(x[:, -1, :])
             self.tokens.copy_(nxt)
             self.position.fill_(t)
@@ -202,7 +240,10 @@ class W8A8Decoder:
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
         x = self.embedding[self.tokens][:, None, :]
         for li in range(cfg.layers):
-            x = self._layer(li, x, cos, sin, pos, visible)
+            if self.fused:
+                x = self._layer_fused(li, x, pos)
+            else:
+                x = self._layer(li, x, cos, sin, pos, visible)
         self.last_logits, nxt = self._head(x[:, 0, :])
         self.tokens.copy_(nxt)
         self.position.add_(1)

@@ -205,6 +205,53 @@ class PackedLinear:
         return (st, out, accumulators) if want_accumulators else (st, out)
 
 
+def rmsnorm_prepare_i8(ctx: Context, x, gain, eps, want_normalized=False):
+    """RMSNorm then activation preparation of x [rows, d]; returns (codes int8, row scales[, normalized f32])."""
+    import torch
+    rows, d = x.shape
+    a8 = torch.empty((rows, d), dtype=torch.int8, device=x.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    normalized = torch.empty((rows, d), dtype=torch.float32, device=x.device) if want_normalized else None
+    _check(library().vxhip_rmsnorm_prepare_i8(ctx._h, _dp(x), _dp(gain), rows, d, float(eps), _dp(a8), _dp(scales),
+                                              _dp(normalized)), "vxhip_rmsnorm_prepare_i8")
+    return (a8, scales, normalized) if want_normalized else (a8, scales)
+
+
+def swiglu_prepare_i8(ctx: Context, gate_up, want_activated=False):
+    """silu(gate) * up of gate_up [rows, 2*inter], then activation preparation."""
+    import torch
+    rows, two = gate_up.shape
+    inter = two // 2
+    a8 = torch.empty((rows, inter), dtype=torch.int8, device=gate_up.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=gate_up.device)
+    act = torch.empty((rows, inter), dtype=torch.float32, device=gate_up.device) if want_activated else None
+    _check(library().vxhip_swiglu_prepare_i8(ctx._h, _dp(gate_up), rows, inter, _dp(a8), _dp(scales), _dp(act)),
+           "vxhip_swiglu_prepare_i8")
+    return (a8, scales, act) if want_activated else (a8, scales)
+
+
+def rope_append_kv(ctx: Context, qkv, cos, sin, positions, q_heads, kv_heads, head_dim, k_cache, v_cache):
+    """qkv [rows, t, (q+2kv)*d]; caches [rows, kv_heads, max_seq, d] updated in place; returns rotated q."""
+    import torch
+    rows, t, _ = qkv.shape
+    q = torch.empty((rows, t, q_heads, head_dim), dtype=torch.float32, device=qkv.device)
+    _check(library().vxhip_rope_append_kv(ctx._h, _dp(qkv), _dp(cos), _dp(sin), _dp(positions), rows, t, q_heads,
+                                          kv_heads, head_dim, k_cache.shape[2], _dp(q), _dp(k_cache), _dp(v_cache)),
+           "vxhip_rope_append_kv")
+    return q
+
+
+def gqa_attention(ctx: Context, q, k_cache, v_cache, positions):
+    """q [rows, t, q_heads, d] over caches [rows, kv_heads, max_seq, d]; returns [rows, t, q_heads*d]."""
+    import torch
+    rows, t, q_heads, head_dim = q.shape
+    out = torch.empty((rows, t, q_heads * head_dim), dtype=torch.float32, device=q.device)
+    _check(library().vxhip_gqa_attention(ctx._h, _dp(q), _dp(k_cache), _dp(v_cache), _dp(positions), rows, t, q_heads,
+                                         k_cache.shape[1], head_dim, k_cache.shape[2], _dp(out)),
+           "vxhip_gqa_attention")
+    return out
+
+
 def packed_prepare_i8(ctx: Context, x):
     import torch
     rows, k = x.shape
