@@ -144,6 +144,71 @@ def cpu_baseline_gemv(k, n, seed):
             "kind": kind, "sample": f"{route}, M=1 K={k} N={n} full size, {dt * 1e3:.2f} ms per call"}
 
 
+def region_ms(fn, steps, torch, warmup=5):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def bench_other_configs(torch, vx, cases, ctx):
+    """configs[1] at M=4,16, configs[2] at M=512,2048 and configs[4] (M=2048, K=14336, N=4096,
+    dynamic per-token scales, f32 dequant+bias): time per call with inputs resident."""
+    from volvoxai_amd.decoder import pack_w8_words
+    res = {}
+    # decode GEMV, M = 4 and 16 (rotating weight copies as for M = 1)
+    Kg, Ng, G, copies = 4096, 14336, 128, 6
+    d = cases.decode_case(16, Kg, Ng, G, 14336)
+    words = pack_w8_words(d["w"])
+    pls = [vx.PackedLinear(words, d["scales"], d["bias"], Kg, Ng, G) for _ in range(copies)]
+    for m in (4, 16):
+        a8 = torch.from_numpy(d["a8"][:m]).cuda()
+        ars = torch.from_numpy(d["row_scales"][:m]).cuda()
+        y = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
+        ms = region_ms(lambda i: pls[i % copies].forward_a8(ctx, a8, ars, out=y), 100, torch)
+        gb = gemv_algorithmic_bytes(m, Kg, Ng)
+        res[f"gemv_M{m}_K4096_N14336"] = {"ms": ms, "GBs": gb / (ms * 1e-3) / 1e9, "frac_hbm": gb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                           "variant": ctx.last_variant}
+    for p in pls:
+        p.close()
+    # prefill GEMM, M = 512 and 2048
+    c = cases.rowscale_case(2048, 4096, 4096, 4096)
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, vx.DTYPE_I8)
+    bd = torch.from_numpy(c["bias_f32"]).cuda()
+    for m in (512, 2048):
+        xd = torch.from_numpy(c["x"][:m]).cuda()
+        rs = torch.from_numpy(c["row_scales"][:m]).cuda()
+        yd = torch.empty((m, 4096), dtype=torch.int8, device="cuda")
+        ms = region_ms(lambda i: lin.forward_rowscale(ctx, xd, rs, c["s_out"], 0, bias_f32=bd, out=yd), 100, torch)
+        ops = 2.0 * m * 4096 * 4096
+        res[f"gemm_M{m}_K4096_N4096"] = {"ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12, "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                                          "variant": ctx.last_variant}
+    lin.close()
+    # outlier-heavy large-K GEMM: f32 activations, dynamic per-token quantization, f32 out
+    rows, k, n = 2048, 14336, 4096
+    rng = np.random.default_rng(55)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[:, rng.choice(k, k // 100, replace=False)] *= 20.0
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    chan = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    pl = vx.PackedLinear(pack_w8_words(w), np.repeat(chan[:, None], k // G, axis=1).copy(),
+                         rng.normal(0, 0.1, n).astype(np.float32), k, n, G)
+    xd = torch.from_numpy(x).cuda()
+    y = torch.empty((rows, n), dtype=torch.float32, device="cuda")
+    ms = region_ms(lambda i: pl.forward_f32(ctx, xd, out=y), 20, torch)
+    ops = 2.0 * rows * k * n
+    res["gemm_f32out_M2048_K14336_N4096"] = {"ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12,
+                                             "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                                             "variant": ctx.last_variant,
+                                             "includes": "activation preparation (f32 -> int8 codes + per-token scales)"}
+    pl.close()
+    return res
+
+
 def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
     """BASELINE config 4: random-init W8A8 decoder, every linear on the PackedLinear kernels,
     greedy decode of 32 concurrent rows, 128-token prompts, 128 new tokens each."""
@@ -326,6 +391,10 @@ def main():
                        config={"workload": out["gemv"]["workload"]}, roofline=out["roofline_gemv"])
         for p in pls:
             p.close()
+
+    # ---- the other sizes BASELINE names, timed only (their parity is in tests/) -----
+    if args.only is None:
+        out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
 
     # ---- config 4: 28-layer decoder, 32 rows, greedy decode ------------------------
     if args.only in (None, "decoder"):

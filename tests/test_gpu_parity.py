@@ -167,14 +167,15 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
                              c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128", "mfma-i8.t256x256"):
+        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128", "mfma-i8.t256x256", "mfma-i8.t256x128",
+                      "mfma-i8.t128x64", "mfma-i8.t256x128w4"):
             vx.force_variant(force)
             (ok, y), variant = run_resident_qlinear(vx, ctx, c)
             assert ok == 1 and (y == want).all(), variant
             seen.add(variant)
     finally:
         vx.force_variant(None)
-    assert len(seen) == 4, seen
+    assert len(seen) == 7, seen
 
 
 @pytest.mark.parametrize("group", [32, 64, 128, 256])

@@ -567,9 +567,22 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (big) return launch_cfg<2, 4, 2, 2, MODE, GK>(s, a) ? "t128x256" : nullptr;
         return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
     } else {
-        if (big && forced("w4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256w4" : nullptr;
-        if (big) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
-        return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
+        // Largest tile (channels x rows) that still gives every compute unit work; names are BNxBM.
+        const auto tiles = [&](uint32_t bn, uint32_t bm) {
+            return (uint64_t)((a.n + bn - 1) / bn) * ((a.rows + bm - 1) / bm);
+        };
+        const uint64_t enough = (uint64_t)cu_count * 3 / 4;
+        int pick = tiles(256, 256) >= enough ? 0 : tiles(256, 128) >= enough ? 1 : tiles(128, 128) >= enough ? 2 : 3;
+        if (forced("t256x256")) pick = 0;
+        if (forced("t256x128")) pick = 1;
+        if (forced("t128x128")) pick = 2;
+        if (forced("t128x64")) pick = 3;
+        if (pick == 0 && forced("w4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256w4" : nullptr;
+        if (pick == 0) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
+        if (pick == 1 && forced("w4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128w4" : nullptr;
+        if (pick == 1) return launch_cfg<2, 4, 4, 1, MODE, GK>(s, a) ? "t256x128" : nullptr;
+        if (pick == 2) return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
+        return launch_cfg<2, 2, 2, 1, MODE, GK>(s, a) ? "t128x64" : nullptr;
     }
 }
 
