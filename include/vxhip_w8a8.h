@@ -94,6 +94,12 @@ VxHipStatus vxhip_rmsnorm_prepare_i8(VxHipContext* context, const float* input_d
                                      const float* gain_dev, uint32_t rows, uint32_t d,
                                      double eps, int8_t* prepared_dev,
                                      float* row_scales_dev, float* normalized_dev);
+/* The same after the residual add: residual_dev [rows, d] += delta_dev in place
+ * (one f32 add per element), then RMSNorm and preparation of the updated rows. */
+VxHipStatus vxhip_add_rmsnorm_prepare_i8(VxHipContext* context, float* residual_dev,
+                                         const float* delta_dev, const float* gain_dev,
+                                         uint32_t rows, uint32_t d, double eps,
+                                         int8_t* prepared_dev, float* row_scales_dev);
 /* silu(gate) * up of gate_up [rows, 2*inter] (gate first), then the same
  * preparation.  activated_dev [rows, inter] may be NULL. */
 VxHipStatus vxhip_swiglu_prepare_i8(VxHipContext* context, const float* gate_up_dev,

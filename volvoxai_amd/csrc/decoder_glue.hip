@@ -62,7 +62,9 @@ __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_
     if (threadIdx.x == 0) *scale_out = bad != 0.0f ? __builtin_nanf("") : scale;
 }
 
-__global__ __launch_bounds__(256) void rmsnorm_prepare_kernel(const float* __restrict__ x,
+// delta (may be null): the row is first updated in place, x += delta (the residual add), and the
+// updated row is what gets normalized.
+__global__ __launch_bounds__(256) void rmsnorm_prepare_kernel(float* __restrict__ x, const float* __restrict__ delta,
                                                               const float* __restrict__ gain, uint32_t d, double eps,
                                                               int8_t* __restrict__ prepared,
                                                               float* __restrict__ row_scales,
@@ -71,10 +73,14 @@ __global__ __launch_bounds__(256) void rmsnorm_prepare_kernel(const float* __res
     __shared__ double dslots[4];
     __shared__ float slots[4];
     const uint32_t row = blockIdx.x;
-    const float* src = x + (size_t)row * d;
+    float* src = x + (size_t)row * d;
     double sum = 0.0;
     for (uint32_t j = threadIdx.x; j < d; j += 256u) {
-        const float v = src[j];
+        float v = src[j];
+        if (delta) {
+            v = __fadd_rn(v, delta[(size_t)row * d + j]);
+            src[j] = v;
+        }
         vals[j] = v;
         sum += (double)v * (double)v;
     }
@@ -138,9 +144,9 @@ __global__ void rope_append_kernel(const float* __restrict__ qkv, const float* _
     else k_cache[(((size_t)row * kv_heads + (head - q_heads)) * max_seq + slot) * head_dim + dd] = y;
 }
 
-// grid (rows * t, q_heads), block 256.  LDS: q[head_dim] + scores[max_seq] + partial[2][head_dim]
+// grid (rows * t, q_heads), block 256.  LDS: q[head_dim] + scores[max_seq] + partial[8][head_dim]
 // floats.  Scores: one thread per visible slot (its whole dot product, 16-byte loads, all
-// independent); P.V: the slots split over the two halves of the block, one thread per channel.
+// independent); P.V: the slots split over eight groups of threads.
 __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restrict__ q,
                                                             const float* __restrict__ k_cache,
                                                             const float* __restrict__ v_cache,
@@ -164,7 +170,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     for (uint32_t s = threadIdx.x; s < visible; s += 256u) {
         const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)s * head_dim);
         float dot = 0.0f;
-#pragma unroll 8
+#pragma unroll 16
         for (uint32_t c = 0; c < head_dim / 4u; c++) {
             const float4 kv = kr[c];
             dot += qs[4 * c] * kv.x + qs[4 * c + 1] * kv.y + qs[4 * c + 2] * kv.z + qs[4 * c + 3] * kv.w;
@@ -183,17 +189,29 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     sum = block_sum(sum, slots);
     for (uint32_t s = threadIdx.x; s < visible; s += 256u) scores[s] = __fdiv_rn(scores[s], sum);
     __syncthreads();
-    // half 0 takes the even slots, half 1 the odd ones
-    const uint32_t part = threadIdx.x >> 7, lane_d = threadIdx.x & 127u;
-    for (uint32_t dd = lane_d; dd < head_dim; dd += 128u) {
-        float acc = 0.0f;
+    // P.V: eight groups of 32 threads; group g takes the slots s = g (mod 8), a thread four
+    // channels of them (16-byte loads, eight in flight); the eight partial rows meet in LDS.
+    const uint32_t group = threadIdx.x >> 5, chunk = threadIdx.x & 31u;
+    for (uint32_t c4 = chunk * 4u; c4 < head_dim; c4 += 128u) {
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 8
-        for (uint32_t s = part; s < visible; s += 2u) acc += scores[s] * vbase[(size_t)s * head_dim + dd];
-        partial[part * head_dim + dd] = acc;
+        for (uint32_t s = group; s < visible; s += 8u) {
+            const float4 vv = *reinterpret_cast<const float4*>(vbase + (size_t)s * head_dim + c4);
+            const float p = scores[s];
+            acc.x += p * vv.x;
+            acc.y += p * vv.y;
+            acc.z += p * vv.z;
+            acc.w += p * vv.w;
+        }
+        *reinterpret_cast<float4*>(partial + group * head_dim + c4) = acc;
     }
     __syncthreads();
-    for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
-        out[((size_t)token * q_heads + head) * head_dim + dd] = partial[dd] + partial[head_dim + dd];
+    for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u) {
+        float total = 0.0f;
+#pragma unroll
+        for (uint32_t g = 0; g < 8u; g++) total += partial[g * head_dim + dd];
+        out[((size_t)token * q_heads + head) * head_dim + dd] = total;
+    }
 }
 
 bool device_ready(VxHipContext* ctx) {
@@ -216,8 +234,24 @@ VxHipStatus vxhip_rmsnorm_prepare_i8(VxHipContext* ctx, const float* input_dev, 
     }
     if (!rows) return VXHIP_OK;
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
-    hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(256), d * sizeof(float), ctx->stream, input_dev,
-                       gain_dev, d, eps, prepared_dev, row_scales_dev, normalized_dev);
+    hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(256), d * sizeof(float), ctx->stream,
+                       const_cast<float*>(input_dev), (const float*)nullptr, gain_dev, d, eps, prepared_dev,
+                       row_scales_dev, normalized_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_add_rmsnorm_prepare_i8(VxHipContext* ctx, float* residual_dev, const float* delta_dev,
+                                         const float* gain_dev, uint32_t rows, uint32_t d, double eps,
+                                         int8_t* prepared_dev, float* row_scales_dev) {
+    if (!ctx || !residual_dev || !delta_dev || !gain_dev || !prepared_dev || !row_scales_dev || !d || d > 15360u) {
+        set_error("add_rmsnorm_prepare_i8: null argument or row length outside 1..15360");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(256), d * sizeof(float), ctx->stream, residual_dev,
+                       delta_dev, gain_dev, d, eps, prepared_dev, row_scales_dev, (float*)nullptr);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -260,7 +294,7 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
                                 float* out_dev) {
     if (!ctx || !q_dev || !k_cache_dev || !v_cache_dev || !positions_dev || !out_dev || !q_heads || !kv_heads ||
         q_heads % kv_heads || !head_dim || head_dim % 4u || !max_seq ||
-        (3u * head_dim + max_seq) * sizeof(float) > 60u * 1024u) {
+        (9u * head_dim + max_seq) * sizeof(float) > 60u * 1024u) {
         set_error("gqa_attention: null argument or unsupported geometry");
         return VXHIP_INVALID_ARGUMENT;
     }
@@ -268,7 +302,7 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     const float scale = (float)(1.0 / sqrt((double)head_dim));
     hipLaunchKernelGGL(gqa_attention_kernel, dim3(rows * t, q_heads), dim3(256),
-                       (3u * head_dim + max_seq) * sizeof(float), ctx->stream, q_dev, k_cache_dev, v_cache_dev,
+                       (9u * head_dim + max_seq) * sizeof(float), ctx->stream, q_dev, k_cache_dev, v_cache_dev,
                        positions_dev, t, q_heads, kv_heads, head_dim, max_seq, scale, out_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;

@@ -148,22 +148,39 @@ class W8A8Decoder:
             raise RuntimeError(_library().vxhip_last_error().decode())
         return out
 
-    def _layer_fused(self, li, x, positions):
-        """The same layer through the fused glue kernels; x [rows, t, hidden], positions int64 [t]."""
+    def _layer_fused(self, li, x2, delta, positions, rows, t):
+        """The same layer through the fused glue kernels.  x2 [rows*t, hidden] is the residual
+        stream, updated in place; delta is the previous layer's MLP output still to be added to it
+        (the add rides in the next RMSNorm kernel).  Returns this layer's pending delta."""
         cfg, L = self.cfg, self.layers[li]
-        rows, t, _ = x.shape
-        x2 = x.reshape(rows * t, cfg.hidden)
-        a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, L["gain1"], cfg.eps)
+        if delta is None:
+            a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, L["gain1"], cfg.eps)
+        else:
+            a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, delta, L["gain1"], cfg.eps)
         qkv = self._linear_a8(L["qkv"], a8, sc).reshape(rows, t, -1)
         q = vx.rope_append_kv(self.ctx, qkv, self.cos, self.sin, positions, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
                               self.k_cache[li], self.v_cache[li])
         attn = vx.gqa_attention(self.ctx, q, self.k_cache[li], self.v_cache[li], positions)
-        x2 = x2 + self._linear(L["o"], attn.reshape(rows * t, cfg.q_dim))
-        a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, L["gain2"], cfg.eps)
+        o = self._linear(L["o"], attn.reshape(rows * t, cfg.q_dim))
+        a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, o, L["gain2"], cfg.eps)
         gu = self._linear_a8(L["gate_up"], a8, sc)
         a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
-        x2 = x2 + self._linear_a8(L["down"], a8, sc)
-        return x2.reshape(rows, t, cfg.hidden)
+        return self._linear_a8(L["down"], a8, sc)
+
+    def _forward_fused(self, tokens, positions):
+        """tokens int64 [rows, t] -> logits of the last position and their argmax."""
+        cfg = self.cfg
+        rows, t = tokens.shape
+        x2 = self.embedding[tokens].reshape(rows * t, cfg.hidden)
+        delta = None
+        for li in range(cfg.layers):
+            delta = self._layer_fused(li, x2, delta, positions, rows, t)
+        if t > 1:
+            x2 = x2.reshape(rows, t, cfg.hidden)[:, -1, :].contiguous()
+            delta = delta.reshape(rows, t, cfg.hidden)[:, -1, :].contiguous()
+        a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, delta, self.gain_f, cfg.eps)
+        logits = self._linear_a8(self.lm_head, a8, sc)
+        return logits, logits.argmax(dim=-1)
 
     def _rmsnorm(self, x, gain):
         xd = x.double()
@@ -204,11 +221,7 @@ class W8A8Decoder:
         return x + self._linear(L["down"], act).reshape(rows, t, cfg.hidden)
 
     def _head(self, x_last):
-        if self.fused:
-            a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x_last.contiguous(), self.gain_f, self.cfg.eps)
-            logits = self._linear_a8(self.lm_head, a8, sc)
-        else:
-            logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
+        logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
         return logits, logits.argmax(dim=-1)
 
     # ---- prefill and decode -----------------------------------------------------------------
@@ -219,13 +232,13 @@ class W8A8Decoder:
             t = prompt.shape[1]
             slots = self.slots[:t]
             visible = self.slots[None, :] <= slots[:, None]
-            x = self.embedding[prompt]
-            for li in range(cfg.layers):
-                if self.fused:
-                    x = self._layer_fused(li, x, slots)
-                else:
+            if self.fused:
+                self.last_logits, nxt = self._forward_fused(prompt, slots)
+            else:
+                x = self.embedding[prompt]
+                for li in range(cfg.layers):
                     x = self._layer(li, x, self.cos[:t], self.sin[:t], slots, visible)
-            self.last_logits, nxt = self._head(x[:, -1, :])
+                self.last_logits, nxt = self._head(x[:, -1, :])
             self.tokens.copy_(nxt)
             self.position.fill_(t)
             self.history.zero_()
@@ -238,13 +251,13 @@ class W8A8Decoder:
         pos = self.position
         visible = self.slots[None, :] <= pos[:, None]
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        x = self.embedding[self.tokens][:, None, :]
-        for li in range(cfg.layers):
-            if self.fused:
-                x = self._layer_fused(li, x, pos)
-            else:
+        if self.fused:
+            self.last_logits, nxt = self._forward_fused(self.tokens[:, None], pos)
+        else:
+            x = self.embedding[self.tokens][:, None, :]
+            for li in range(cfg.layers):
                 x = self._layer(li, x, cos, sin, pos, visible)
-        self.last_logits, nxt = self._head(x[:, 0, :])
+            self.last_logits, nxt = self._head(x[:, 0, :])
         self.tokens.copy_(nxt)
         self.position.add_(1)
         return nxt

@@ -217,6 +217,17 @@ def rmsnorm_prepare_i8(ctx: Context, x, gain, eps, want_normalized=False):
     return (a8, scales, normalized) if want_normalized else (a8, scales)
 
 
+def add_rmsnorm_prepare_i8(ctx: Context, residual, delta, gain, eps):
+    """residual += delta in place, then RMSNorm and preparation of the updated rows."""
+    import torch
+    rows, d = residual.shape
+    a8 = torch.empty((rows, d), dtype=torch.int8, device=residual.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=residual.device)
+    _check(library().vxhip_add_rmsnorm_prepare_i8(ctx._h, _dp(residual), _dp(delta), _dp(gain), rows, d, float(eps),
+                                                  _dp(a8), _dp(scales)), "vxhip_add_rmsnorm_prepare_i8")
+    return a8, scales
+
+
 def swiglu_prepare_i8(ctx: Context, gate_up, want_activated=False):
     """silu(gate) * up of gate_up [rows, 2*inter], then activation preparation."""
     import torch
