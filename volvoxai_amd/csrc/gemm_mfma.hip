@@ -563,8 +563,9 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
     if (forced("t256x256")) big = true;
     if (forced("t128x128")) big = false;
     if constexpr (MODE == (int)Epilogue::DequantF32) {
-        // int32 tile accumulators plus f32 running sums: keep the wave tile at 64x64
-        if (big) return launch_cfg<2, 4, 2, 2, MODE, GK>(s, a) ? "t128x256" : nullptr;
+        // int32 tile accumulators plus f32 running sums: keep the wave tile at 64x64.  With a
+        // scale group per k-step the eight-wave tile runs out of registers, so it stays with four.
+        if (big && GK > 1) return launch_cfg<2, 4, 2, 2, MODE, GK>(s, a) ? "t128x256" : nullptr;
         return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
     } else {
         // Largest tile (channels x rows) that still gives every compute unit work; names are BNxBM.

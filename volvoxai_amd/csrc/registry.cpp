@@ -15,22 +15,22 @@ constexpr int kQuantizeLinear = 0, kDequantizeLinear = 0;  // boundary ops carry
 
 const VxHipKernelVariant kVariants[] = {
     QROWS("hip.qlinear.mfma-i8", "gemm_mfma_kernel<RequantTensor>",
-          "hip.qlinear.canonical-resident-int32-bound-rows-gt16-any-k-tail",
+          "hip.qlinear.canonical-resident-int32-bound-rows-gt32-any-k-tail",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300),
     QROWS("hip.qlinear.mfma-i8-rowscale", "gemm_mfma_kernel<RequantRow>",
-          "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-gt16",
+          "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-gt32",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300),
     QROWS("hip.qlinear.gemv-mfma", "gemv_panel_kernel<RequantTensor>",
-          "hip.qlinear.canonical-resident-int32-bound-rows-le16",
+          "hip.qlinear.canonical-resident-int32-bound-rows-le32",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400),
     QROWS("hip.qlinear.gemv-mfma-rowscale", "gemv_panel_kernel<RequantRow>",
-          "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-le16",
+          "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-le32",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400),
     {"hip.packed-linear.a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32>",
-     "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-gt16",
+     "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-gt32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300},
     {"hip.packed-linear.a8-gemv-mfma", 0, kPackedLinear, "gemv_panel_kernel<DequantF32>",
-     "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-le16",
+     "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-le32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400},
     {"hip.packed-linear.prepare-i8", 0, kPackedLinear, "prepare_i8_kernel",
      "hip.packed-linear.dynamic-i8-row-absmax", "", 100},
