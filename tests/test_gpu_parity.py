@@ -197,7 +197,8 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert len(seen) == 4, seen
+    # one scale group per k-step has no eight-wave tile: both GEMM requests run the same one
+    assert len(seen) == (3 if group == 32 else 4), seen
     pl.close()
 
 
