@@ -8,7 +8,9 @@
  * Test infrastructure only. */
 #include "volvoxai_backend.h"
 
+#include <pthread.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 static VxBackendProvider g_provider;
@@ -228,5 +230,115 @@ done:
     }
     if (compiled) g_provider.compiled_destroy(compiled);
     if (runtime) g_provider.runtime_destroy(runtime);
+    return run->status = status;
+}
+
+/* Several contexts of ONE compiled instance executing at the same time on their own threads
+ * (native/tests/test_packed_arithmetic.inc:128-147): every thread must deliver the bytes a
+ * single-threaded run delivers.  run->output receives thread 0's result. */
+typedef struct Worker {
+    MockRun run; /* private copy: own sink state and output buffer */
+    void* compiled;
+    VxStatus status;
+} Worker;
+
+static void* worker_main(void* opaque) {
+    Worker* w = (Worker*)opaque;
+    VxContextOptions context_options = VX_CONTEXT_OPTIONS_INIT;
+    VxTensorBinding binding = VX_TENSOR_BINDING_INIT;
+    VxBackendOutputSink sink = {sizeof(VxBackendOutputSink), &w->run, sink_write};
+    VxReport report = VX_REPORT_INIT;
+    void* context = NULL;
+    w->status = g_provider.context_create(w->compiled, &context_options, &context, &report);
+    if (w->status != VX_STATUS_OK) return NULL;
+    binding.name = w->run.input_name;
+    binding.dtype = (VxDataType)w->run.input_dtype;
+    binding.rank = w->run.rank;
+    memcpy(binding.shape, w->run.input_shape, sizeof(binding.shape));
+    binding.data = w->run.input;
+    binding.byte_size = (size_t)w->run.input_bytes;
+    binding.location = VX_MEMORY_HOST;
+    for (int32_t i = 0; i < w->run.executions && w->status == VX_STATUS_OK; i++) {
+        report = (VxReport)VX_REPORT_INIT;
+        w->status = g_provider.context_execute(context, &binding, 1, &sink, &report);
+        if (w->status == VX_STATUS_OK && (w->run.writes != i + 1 || w->run.sink_mismatch))
+            w->status = VX_STATUS_EXECUTION_FAILED;
+    }
+    g_provider.context_destroy(context);
+    return NULL;
+}
+
+int32_t mock_host_run_concurrent(MockRun* run, int32_t threads) {
+    static const char fingerprint[] = "sha256:mock-graph-fingerprint";
+    static const char proof[] = "sha256:mock-shape-domain-proof";
+    VxRuntimeOptions runtime_options = VX_RUNTIME_OPTIONS_INIT;
+    VxReport report = VX_REPORT_INIT;
+    VxModelSource source = VX_MODEL_SOURCE_INIT;
+    VxBackendCompileInput input = VX_BACKEND_COMPILE_INPUT_INIT;
+    VxBackendShapeDomainAttestation attestation = VX_BACKEND_SHAPE_DOMAIN_ATTESTATION_INIT;
+    VxBackendPolicy policy = VX_BACKEND_POLICY_INIT;
+    VxTensorSpec in_spec, out_spec;
+    const char* weights[1];
+    const char* wanted[1];
+    void *runtime = NULL, *compiled = NULL;
+    Worker* workers;
+    pthread_t* ids;
+    VxStatus status;
+    if (!g_registered || threads < 1 || threads > 16) return run->status = VX_STATUS_INVALID_ARGUMENT;
+    status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
+    if (status != VX_STATUS_OK) return run->status = status;
+    weights[0] = run->weight_path;
+    source.graph_path = run->graph_path;
+    source.weight_paths = weights;
+    source.weight_path_count = 1;
+    spec_from(&in_spec, run->input_name, run->input_dtype, run, run->input_shape[run->rank - 1]);
+    spec_from(&out_spec, run->output_name, run->output_dtype, run, run->output_last);
+    input.source = &source;
+    input.graph_fingerprint = fingerprint;
+    input.shape_domain_proof_identity = proof;
+    input.inputs = &in_spec;
+    input.input_count = 1;
+    input.outputs = &out_spec;
+    input.output_count = 1;
+    input.packed_arithmetic = (VxPackedArithmetic)run->packed_arithmetic;
+    wanted[0] = g_name;
+    policy.mode = VX_BACKEND_REQUIRE;
+    policy.operator_fallback = VX_OPERATOR_FALLBACK_FORBID;
+    policy.backends = wanted;
+    policy.backend_count = 1;
+    status = g_provider.compile(runtime, &input, &policy, &compiled, &attestation, &report);
+    if (status != VX_STATUS_OK) {
+        g_provider.runtime_destroy(runtime);
+        return run->status = status;
+    }
+    workers = (Worker*)calloc((size_t)threads, sizeof(*workers));
+    ids = (pthread_t*)calloc((size_t)threads, sizeof(*ids));
+    for (int32_t t = 0; t < threads; t++) {
+        workers[t].run = *run;
+        workers[t].run.writes = 0;
+        workers[t].run.sink_mismatch = 0;
+        workers[t].run.executions = run->executions > 0 ? run->executions : 1;
+        workers[t].run.output = malloc((size_t)run->output_capacity);
+        workers[t].compiled = compiled;
+        pthread_create(&ids[t], NULL, worker_main, &workers[t]);
+    }
+    for (int32_t t = 0; t < threads; t++) {
+        pthread_join(ids[t], NULL);
+        if (status == VX_STATUS_OK) status = workers[t].status;
+        if (status == VX_STATUS_OK && (workers[t].run.output_bytes != workers[0].run.output_bytes ||
+                                       memcmp(workers[t].run.output, workers[0].run.output,
+                                              (size_t)workers[0].run.output_bytes) != 0))
+            status = VX_STATUS_EXECUTION_FAILED;
+    }
+    if (status == VX_STATUS_OK) {
+        memcpy(run->output, workers[0].run.output, (size_t)workers[0].run.output_bytes);
+        run->output_bytes = workers[0].run.output_bytes;
+        run->writes = workers[0].run.writes;
+    }
+    for (int32_t t = 0; t < threads; t++) free(workers[t].run.output);
+    free(workers);
+    free(ids);
+    g_provider.compiled_destroy(compiled);
+    g_provider.runtime_destroy(runtime);
     return run->status = status;
 }

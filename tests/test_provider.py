@@ -153,7 +153,7 @@ def inspect(host, graph, weights, arithmetic="f32"):
 
 
 def run(host, graph, weights, x, in_name, in_dtype, out_name, out_dtype, d_out, arithmetic="f32", lead_max=None,
-        executions=1):
+        executions=1, threads=0):
     mock, _, _ = host
     x = np.ascontiguousarray(x)
     out_np = {"i8": np.int8, "u8": np.uint8, "f32": np.float32}[out_dtype]
@@ -169,7 +169,11 @@ def run(host, graph, weights, x, in_name, in_dtype, out_name, out_dtype, d_out, 
     r.input, r.input_bytes = x.ctypes.data, x.nbytes
     r.output_name, r.output_dtype, r.output_last = out_name.encode(), DT[out_dtype], d_out
     r.output, r.output_capacity, r.executions = y.ctypes.data, y.nbytes, executions
-    mock.mock_host_run(C.byref(r))
+    if threads:
+        mock.mock_host_run_concurrent.argtypes = [C.POINTER(MockRun), C.c_int32]
+        mock.mock_host_run_concurrent(C.byref(r), threads)
+    else:
+        mock.mock_host_run(C.byref(r))
     return r, y
 
 
@@ -333,6 +337,36 @@ def test_qlinear_package_matches_oracle(registered, oracle, tmp_path, rows, k, n
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("case", ["q-dense-rank2", "q-dense-rank3"])
+def test_reference_shape_contract_cases(registered, oracle, tmp_path, case):
+    """The two q-dense success cases of the reference's shape-contract vectors
+    (tests/contracts/shape_vectors/quantized_vectors.json): shapes, dtypes and quantization
+    parameters as given there, tensor contents seeded here, bytes against the oracle."""
+    spec = {"q-dense-rank2": dict(x_shape=(2, 4), in_dtype="int8", w_shape=(3, 4), w_dtype=np.int8,
+                                  scales=[0.02, 0.03, 0.04], zps=[0, 0, 0], s_in=0.1, zp_in=0, out_dtype="uint8",
+                                  s_out=0.05, zp_out=128),
+            "q-dense-rank3": dict(x_shape=(2, 5, 4), in_dtype="uint8", w_shape=(2, 4), w_dtype=np.uint8,
+                                  scales=[0.01, 0.02], zps=[127, 127], s_in=0.1, zp_in=128, out_dtype="int8",
+                                  s_out=0.05, zp_out=0)}[case]
+    rng = np.random.default_rng(len(case))
+    signed_in = spec["in_dtype"] == "int8"
+    x = rng.integers(-128 if signed_in else 0, 128 if signed_in else 256, spec["x_shape"]).astype(
+        np.int8 if signed_in else np.uint8)
+    signed_w = spec["w_dtype"] == np.int8
+    wt = rng.integers(-127 if signed_w else 0, 128 if signed_w else 256, spec["w_shape"]).astype(spec["w_dtype"])
+    bias = rng.integers(-50, 50, spec["w_shape"][0]).astype(np.int32)
+    g, w = qlinear_package(tmp_path / "q", x.shape, wt, spec["scales"], spec["zps"], bias, spec["s_in"], spec["zp_in"],
+                           spec["s_out"], spec["zp_out"], in_dtype=spec["in_dtype"], out_dtype=spec["out_dtype"])
+    out_code = "u8" if spec["out_dtype"] == "uint8" else "i8"
+    r, y = run(registered, g, w, x, "hidden_q", "i8" if signed_in else "u8", "projected_q", out_code, wt.shape[0])
+    assert r.status == 0, r.message
+    ok, want = oracle.qlinear(x.reshape(-1, x.shape[-1]), wt, bias, np.asarray(spec["scales"], np.float32),
+                              np.asarray(spec["zps"], np.int32), spec["s_in"], spec["zp_in"], spec["s_out"],
+                              spec["zp_out"], 6 if signed_in else 5, 6 if signed_w else 5, DT[out_code])[:2]
+    assert ok == 1 and (y.reshape(want.shape) == want).all()
+
+
+@pytest.mark.gpu
 def test_qlinear_package_with_unprovable_accumulator_is_refused_at_compile(registered, tmp_path):
     k = 40000  # 40000 * 255 * 255 > INT32_MAX
     x = np.zeros((1, k), np.uint8)
@@ -357,6 +391,19 @@ def test_packed_linear_package_matches_oracle(registered, oracle, tmp_path, rows
     # the same package under another arithmetic is refused before anything is allocated
     r2, _ = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", n, arithmetic="f32")
     assert r2.status == -7 and r2.failed_stage == 3 and r2.writes == 0
+
+
+@pytest.mark.gpu
+def test_contexts_of_one_compiled_model_run_concurrently(registered, oracle, tmp_path):
+    """Four threads, each with its own context on the same compiled instance, eight executions each."""
+    c = cases.packed_case(24, 1024, 520, 128, 9)
+    words = oracle.pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "p", c["x"].shape, words, c["scales"], c["bias"], 128)
+    r, y = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", 520, arithmetic="dynamic_i8", executions=8,
+               threads=4)
+    assert r.status == 0 and r.writes == 8
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], 520, 128)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
 
 
 @pytest.mark.gpu
