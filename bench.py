@@ -3,11 +3,11 @@
 
 A "step" is one W8A8 linear over one batch of synthetic, HBM-resident input:
 
-  headline  M=K=N=4096 prefill GEMM (BASELINE config 3): int8 A x prepacked
+  headline  M=K=N=4096 prefill GEMM (the prefill benchmark shape): int8 A x prepacked
             int8 B, int32 accumulation, per-token x per-channel scale, f32
             bias, requantization to int8 at output scale 0.05 (ties to even).
             Reported as int8 TOPS and as a fraction of the int8 MFMA peak.
-  gemv      M=1, K=4096, N=14336 decode GEMV (BASELINE config 2): dequant +
+  gemv      M=1, K=4096, N=14336 decode GEMV (the decode benchmark shape): dequant +
             bias to f32.  Reported as GB/s of algorithmic bytes and as a
             fraction of HBM peak, rotating over enough weight copies that the
             256 MB Infinity Cache cannot serve them.
@@ -210,7 +210,7 @@ def bench_other_configs(torch, vx, cases, ctx):
 
 
 def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
-    """BASELINE config 4: random-init W8A8 decoder, every linear on the PackedLinear kernels,
+    """The decoder benchmark: random-init W8A8 decoder, every linear on the PackedLinear kernels,
     greedy decode of 32 concurrent rows, 128-token prompts, 128 new tokens each."""
     from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
     cfg = DecoderConfig()
@@ -392,7 +392,7 @@ def main():
         for p in pls:
             p.close()
 
-    # ---- the other sizes BASELINE names, timed only (their parity is in tests/) -----
+    # ---- the other benchmark sizes, timed only (their parity is in tests/) -----
     if args.only is None:
         out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
 

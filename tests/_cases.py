@@ -105,7 +105,7 @@ def quant_gemm_case(weight_case, input_dtype, weight_dtype, output_dtype, rows, 
 
 def qlinear_random_case(rows, d_in, d_out, seed, input_dtype=DTYPE_I8, weight_dtype=DTYPE_I8,
                         output_dtype=DTYPE_I8, zero_weight_zp=True, s_out=0.05):
-    """BASELINE-style QLinear inputs: weights uniform in [-127,127], per-channel
+    """Benchmark-style QLinear inputs: weights uniform in [-127,127], per-channel
     scales ~U(0.005,0.02), activations clip(round(N(0,30)))."""
     rng = np.random.default_rng(seed)
     if input_dtype == DTYPE_I8:
@@ -128,7 +128,7 @@ def qlinear_random_case(rows, d_in, d_out, seed, input_dtype=DTYPE_I8, weight_dt
 
 
 def rowscale_case(rows, d_in, d_out, seed, with_bias=True):
-    """BASELINE config 3: A, B uniform in [-127,127], per-token scales
+    """Prefill benchmark inputs: A, B uniform in [-127,127], per-token scales
     ~U(0.01,0.05), per-channel ~U(0.002,0.01), output scale 0.05."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-127, 128, (rows, d_in)).astype(np.int8)
@@ -158,7 +158,7 @@ def packed_case(rows, k, n, group, seed, with_bias=True, special_rows=False):
 
 
 def decode_case(rows, k, n, group, seed):
-    """BASELINE config 2: int8 activations clip(round(N(0,30))), per-token scales
+    """Decode benchmark inputs: int8 activations clip(round(N(0,30))), per-token scales
     ~U(0.01,0.05), weights uniform +-127, per-channel scales ~U(0.002,0.01)
     replicated over the K/G groups (PackedLinear has no whole-row group)."""
     rng = np.random.default_rng(seed)

@@ -51,7 +51,7 @@ QLINEAR_CASES = (
     + [("random", dict(rows=r, d_in=k, d_out=n, seed=s, input_dtype=i, weight_dtype=w, output_dtype=o,
                        zero_weight_zp=z))
        for (r, k, n, s, i, w, o, z) in [
-           (8, 256, 256, 1, I8, I8, I8, True),       # BASELINE config 1 shape
+           (8, 256, 256, 1, I8, I8, I8, True),       # the CPU-runnable benchmark shape
            (1, 4096, 512, 2, I8, I8, I8, True),      # decode shaped
            (16, 4096, 256, 3, I8, I8, I8, True),
            (16, 1000, 130, 4, U8, U8, U8, False),

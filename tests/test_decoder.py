@@ -1,4 +1,4 @@
-"""BASELINE config 4 glue: the decoder built on the W8A8 linears against its CPU restatement."""
+"""Decoder glue: the decoder built on the W8A8 linears against its CPU restatement."""
 import numpy as np
 import pytest
 

@@ -202,7 +202,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     pl.close()
 
 
-# ---- BASELINE shapes --------------------------------------------------------------------
+# ---- benchmark shapes ---------------------------------------------------------------------
 
 @pytest.mark.parametrize("rows", [1, 4, 16])
 def test_decode_shape_config2(ctx, oracle, rows):

@@ -1,5 +1,5 @@
 """Decoder-only transformer with every linear routed to the W8A8 PackedLinear
-kernels (BASELINE config 4): RMSNorm, rotary embedding, grouped-query attention
+kernels (28 layers, hidden 1024, 16 query / 8 KV heads of 128, SwiGLU 3072 by default): RMSNorm, rotary embedding, grouped-query attention
 over a KV cache, SwiGLU, residual adds and greedy selection run as PyTorch-ROCm
 f32 ops around them; the linears are `vxhip_packed_linear_forward_f32`
 (DYNAMIC_I8: per-row activation quantization, int8 x int8 MFMA, dequant to f32).
