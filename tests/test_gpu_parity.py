@@ -395,3 +395,57 @@ def test_context_reports_variant_and_clean_fault_word(ctx):
     assert ok == 1 and variant.startswith("hip.qlinear.mfma-i8")
     assert variant.split(".t")[0] in {r["id"] for r in vx.kernel_variants()}
     assert ctx.fault_flags() == 0
+
+
+# ---- seeded sweep over ragged shapes ----------------------------------------------------------
+
+def test_random_shape_sweep_qlinear(ctx, oracle):
+    """Forty seeded shapes with ragged rows/K/N, every byte-dtype combination, weight zero points
+    and both output scales' regimes; each through the default dispatch and the other kernel family."""
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(2025)
+    for trial in range(40):
+        rows = int(rng.choice([1, 2, 3, 7, 16, 17, 31, 32, 33, 64, 100, 257]))
+        k = int(rng.choice([1, 5, 16, 31, 32, 33, 100, 127, 128, 129, 255, 640, 1000]))
+        n = int(rng.choice([1, 3, 16, 31, 32, 33, 48, 100, 255, 256, 300]))
+        in_dt, w_dt, out_dt = (int(rng.choice([I8, U8])) for _ in range(3))
+        c = cases.qlinear_random_case(rows, k, n, 9000 + trial, in_dt, w_dt, out_dt, zero_weight_zp=bool(trial % 2),
+                                      s_out=float(rng.choice([0.05, 0.5, 3.0])))
+        ok_w, want = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
+                                    c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+        assert ok_w == 1
+        for force in (None, "mfma-i8" if rows <= 32 else None):
+            if force is None and rows > 32 and trial % 3 == 0:
+                force = "mfma-i8.t128x64"
+            vx.force_variant(force)
+            try:
+                (ok, y), variant = run_resident_qlinear(vx, ctx, c)
+            finally:
+                vx.force_variant(None)
+            assert ok == 1 and (y == want).all(), (trial, rows, k, n, in_dt, w_dt, out_dt, variant)
+    assert ctx.fault_flags() == 0
+
+
+def test_random_shape_sweep_packed(ctx, oracle):
+    """Thirty seeded PackedLinear shapes: ragged K (partial last group and word), every group size,
+    with and without bias, rows on both sides of the GEMV/GEMM boundary."""
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(77)
+    for trial in range(30):
+        rows = int(rng.choice([1, 2, 5, 16, 31, 32, 33, 40, 130]))
+        k = int(rng.choice([1, 7, 32, 33, 95, 128, 130, 257, 512, 1000]))
+        n = int(rng.choice([1, 2, 31, 32, 33, 70, 129, 264]))
+        group = int(rng.choice([32, 64, 128, 256]))
+        c = cases.packed_case(rows, k, n, group, 500 + trial, with_bias=bool(trial % 2), special_rows=(trial % 5 == 0))
+        words = oracle.pack_w8_words(c["w"])
+        _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group)
+        pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+        for force in (None, "a8-mfma" if rows <= 32 else None):
+            vx.force_variant(force)
+            try:
+                st, y = pl.forward_f32(ctx, dev(c["x"]))
+                ctx.synchronize()
+            finally:
+                vx.force_variant(None)
+            assert st == 0 and same_f32(host(y), want), (trial, rows, k, n, group, ctx.last_variant)
+        pl.close()
