@@ -45,16 +45,16 @@ VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows
 //   (multiplying by a reciprocal moves half-way values, ibid. :34-36).
 // A row holding NaN or Inf gets zero codes and a NaN scale, which makes every
 // output of that row NaN downstream as the reference requires (:1495).
-__global__ __launch_bounds__(256) void prepare_i8_kernel(
+__global__ __launch_bounds__(1024) void prepare_i8_kernel(
         const float* __restrict__ x, uint32_t k, int8_t* __restrict__ prepared, uint32_t ld,
         float* __restrict__ scales) {
-    __shared__ float wave_max[4];
-    __shared__ uint32_t wave_bad[4];
+    __shared__ float wave_max[16];
+    __shared__ uint32_t wave_bad[16];
     const uint32_t row = blockIdx.x;
     const float* src = x + (size_t)row * k;
     float maximum = 0.0f;
     uint32_t bad = 0u;
-    for (uint32_t j = threadIdx.x; j < k; j += 256u) {
+    for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) {
         const float v = src[j];
         bad |= finite_f32(v) ? 0u : 1u;
         maximum = fmaxf(maximum, fabsf(v));  // fmaxf ignores a NaN operand; `bad` records it
@@ -68,12 +68,16 @@ __global__ __launch_bounds__(256) void prepare_i8_kernel(
         wave_bad[threadIdx.x >> 6] = bad;
     }
     __syncthreads();
-    maximum = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-    bad = wave_bad[0] | wave_bad[1] | wave_bad[2] | wave_bad[3];
+    maximum = wave_max[0];
+    bad = wave_bad[0];
+    for (uint32_t w = 1; w < blockDim.x / 64u; w++) {
+        maximum = fmaxf(maximum, wave_max[w]);
+        bad |= wave_bad[w];
+    }
     float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
     int8_t* dst = prepared + (size_t)row * ld;
-    for (uint32_t j = threadIdx.x; j < ld; j += 256u) {
+    for (uint32_t j = threadIdx.x; j < ld; j += blockDim.x) {
         int32_t q = 0;
         if (!bad && j < k) q = packed_round_i8(__fdiv_rn(src[j], scale));
         dst[j] = (int8_t)q;
@@ -83,7 +87,9 @@ __global__ __launch_bounds__(256) void prepare_i8_kernel(
 
 VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
                               int8_t* prepared, uint32_t ld, float* scales) {
-    hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(256), 0, s, x, k, prepared, ld, scales);
+    // few long rows: latency bound, give each row a full workgroup
+    const uint32_t block = rows <= 256u && k >= 1024u ? 1024u : 256u;
+    hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(block), 0, s, x, k, prepared, ld, scales);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
