@@ -342,3 +342,159 @@ int32_t mock_host_run_concurrent(MockRun* run, int32_t threads) {
     g_provider.runtime_destroy(runtime);
     return run->status = status;
 }
+
+/* Scheduler-style batch: the provider freezes a batch contract at compile and then receives ONE
+ * invocation with the requests stacked along the batch axis, one output sink per lane
+ * (native/include/volvoxai_backend.h:39-92; contract checks as in
+ * native/src/runtime/public_api_model_lifecycle.inc:790-849).  run->input is the stacked input
+ * [batch, ..., d_in] (input_shape[0] == batch, lead_max[0] the symbolic bound); lane i's output
+ * lands at run->output + i * lane_bytes. */
+typedef struct Lane {
+    MockRun* run;
+    unsigned char* dst;
+    size_t capacity;
+    int32_t writes;
+    int32_t mismatch;
+    size_t bytes;
+} Lane;
+
+static VxStatus lane_write(void* user, const char* name, VxDataType dtype, const int64_t* shape, uint32_t rank,
+                           const void* data, size_t bytes) {
+    Lane* lane = (Lane*)user;
+    const MockRun* run = lane->run;
+    lane->writes++;
+    if (!name || strcmp(name, run->output_name) || (int32_t)dtype != run->output_dtype || rank != run->rank || !data ||
+        bytes > lane->capacity || shape[0] != 1 || shape[rank - 1] != run->output_last) {
+        lane->mismatch = 1;
+        return VX_STATUS_INVALID_ARGUMENT;
+    }
+    for (uint32_t a = 1; a + 1 < rank; a++)
+        if (shape[a] != run->input_shape[a]) lane->mismatch = 1;
+    memcpy(lane->dst, data, bytes);
+    lane->bytes = bytes;
+    return lane->mismatch ? VX_STATUS_INVALID_ARGUMENT : VX_STATUS_OK;
+}
+
+int32_t mock_host_run_batch(MockRun* run, int32_t with_proof) {
+    static const char fingerprint[] = "sha256:mock-graph-fingerprint";
+    static const char proof[] = "sha256:mock-shape-domain-proof";
+    static const char batch_proof[] = "sha256:mock-independent-batch-proof";
+    VxRuntimeOptions runtime_options = VX_RUNTIME_OPTIONS_INIT;
+    VxContextOptions context_options = VX_CONTEXT_OPTIONS_INIT;
+    VxReport report = VX_REPORT_INIT;
+    VxModelSource source = VX_MODEL_SOURCE_INIT;
+    VxBackendCompileInput input = VX_BACKEND_COMPILE_INPUT_INIT;
+    VxBackendShapeDomainAttestation attestation = VX_BACKEND_SHAPE_DOMAIN_ATTESTATION_INIT;
+    VxBackendBatchContract contract = VX_BACKEND_BATCH_CONTRACT_INIT;
+    VxBackendBatchInvocation invocation = VX_BACKEND_BATCH_INVOCATION_INIT;
+    VxBackendPolicy policy = VX_BACKEND_POLICY_INIT;
+    VxTensorSpec in_spec, out_spec;
+    VxTensorBinding binding = VX_TENSOR_BINDING_INIT;
+    const char* weights[1];
+    const char* wanted[1];
+    void *runtime = NULL, *compiled = NULL, *context = NULL;
+    const uint32_t batch = (uint32_t)run->input_shape[0];
+    VxBackendOutputSink* sinks = NULL;
+    Lane* lanes = NULL;
+    uint64_t* ids = NULL;
+    VxStatus status;
+    if (!g_registered || !g_provider.compiled_batch_contract || !g_provider.context_execute_batch || !batch)
+        return run->status = VX_STATUS_BACKEND_UNSUPPORTED;
+    status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
+    run->failed_stage = VX_STAGE_RUNTIME_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+    weights[0] = run->weight_path;
+    source.graph_path = run->graph_path;
+    source.weight_paths = weights;
+    source.weight_path_count = 1;
+    spec_from(&in_spec, run->input_name, run->input_dtype, run, run->input_shape[run->rank - 1]);
+    spec_from(&out_spec, run->output_name, run->output_dtype, run, run->output_last);
+    input.source = &source;
+    input.graph_fingerprint = fingerprint;
+    input.shape_domain_proof_identity = proof;
+    input.inputs = &in_spec;
+    input.input_count = 1;
+    input.outputs = &out_spec;
+    input.output_count = 1;
+    input.packed_arithmetic = (VxPackedArithmetic)run->packed_arithmetic;
+    if (with_proof) {
+        input.independent_batch_proof_protocol = VX_BACKEND_INDEPENDENT_BATCH_PROOF_PROTOCOL;
+        input.independent_batch_proof_identity = batch_proof;
+    }
+    wanted[0] = g_name;
+    policy.mode = VX_BACKEND_REQUIRE;
+    policy.operator_fallback = VX_OPERATOR_FALLBACK_FORBID;
+    policy.backends = wanted;
+    policy.backend_count = 1;
+    status = g_provider.compile(runtime, &input, &policy, &compiled, &attestation, &report);
+    run->failed_stage = VX_STAGE_COMPILE;
+    if (status != VX_STATUS_OK) goto done;
+    status = g_provider.compiled_batch_contract(compiled, &contract, &report);
+    if (status == VX_STATUS_OK &&
+        (contract.struct_size != sizeof(contract) || !contract.protocol ||
+         strcmp(contract.protocol, VX_BACKEND_BATCH_PROTOCOL) || !contract.resource_domain ||
+         !contract.compatibility_token || !contract.min_batch || contract.max_batch < contract.min_batch ||
+         !contract.multiple_of || contract.min_batch % contract.multiple_of || contract.batch_axis < 0 ||
+         (contract.device_resident != 0 && contract.device_resident != 1)))
+        status = VX_STATUS_ABI_UNSUPPORTED;
+    if (status == VX_STATUS_OK && contract.max_batch > 1u &&
+        (!with_proof || !contract.graph_fingerprint || strcmp(contract.graph_fingerprint, fingerprint) ||
+         !contract.independent_batch_proof_identity || strcmp(contract.independent_batch_proof_identity, batch_proof) ||
+         contract.batch_axis != 0 || (int64_t)contract.max_batch > run->lead_max[0]))
+        status = VX_STATUS_ABI_UNSUPPORTED;
+    run->attested_arithmetic = (int32_t)contract.max_batch; /* reported back: the frozen maximum */
+    if (status != VX_STATUS_OK) goto done;
+    if (batch > contract.max_batch) {
+        status = VX_STATUS_BACKEND_UNSUPPORTED; /* the scheduler would not coalesce beyond the contract */
+        goto done;
+    }
+    status = g_provider.context_create(compiled, &context_options, &context, &report);
+    run->failed_stage = VX_STAGE_CONTEXT_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+
+    sinks = (VxBackendOutputSink*)calloc(batch, sizeof(*sinks));
+    lanes = (Lane*)calloc(batch, sizeof(*lanes));
+    ids = (uint64_t*)calloc(batch, sizeof(*ids));
+    for (uint32_t i = 0; i < batch; i++) {
+        lanes[i].run = run;
+        lanes[i].capacity = (size_t)(run->output_capacity / batch);
+        lanes[i].dst = (unsigned char*)run->output + (size_t)i * lanes[i].capacity;
+        sinks[i].struct_size = sizeof(sinks[i]);
+        sinks[i].user_data = &lanes[i];
+        sinks[i].write = lane_write;
+        ids[i] = 1000u + i;
+    }
+    binding.name = run->input_name;
+    binding.dtype = (VxDataType)run->input_dtype;
+    binding.rank = run->rank;
+    memcpy(binding.shape, run->input_shape, sizeof(binding.shape));
+    binding.data = run->input;
+    binding.byte_size = (size_t)run->input_bytes;
+    binding.location = VX_MEMORY_HOST;
+    invocation.stacked_inputs = &binding;
+    invocation.stacked_input_count = 1;
+    invocation.batch_size = batch;
+    invocation.request_ids = ids;
+    invocation.lane_output_sinks = sinks;
+    invocation.lane_output_sink_count = batch;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_execute_batch(context, &invocation, &report);
+    run->failed_stage = VX_STAGE_EXECUTE;
+    run->writes = 0;
+    for (uint32_t i = 0; i < batch && status == VX_STATUS_OK; i++) {
+        if (lanes[i].writes != 1 || lanes[i].mismatch || lanes[i].bytes != lanes[i].capacity) status = VX_STATUS_EXECUTION_FAILED;
+        run->writes += lanes[i].writes;
+    }
+    run->execute_attested = report.route_attested && report.route_evidence[0];
+    snprintf(run->execute_route, sizeof(run->execute_route), "%s", report.route_evidence);
+    if (status == VX_STATUS_OK) run->failed_stage = VX_STAGE_NONE;
+done:
+    snprintf(run->message, sizeof(run->message), "%s", report.message);
+    free(sinks);
+    free(lanes);
+    free(ids);
+    if (context) g_provider.context_destroy(context);
+    if (compiled) g_provider.compiled_destroy(compiled);
+    if (runtime) g_provider.runtime_destroy(runtime);
+    return run->status = status;
+}

@@ -153,7 +153,7 @@ def inspect(host, graph, weights, arithmetic="f32"):
 
 
 def run(host, graph, weights, x, in_name, in_dtype, out_name, out_dtype, d_out, arithmetic="f32", lead_max=None,
-        executions=1, threads=0):
+        executions=1, threads=0, batch_proof=None):
     mock, _, _ = host
     x = np.ascontiguousarray(x)
     out_np = {"i8": np.int8, "u8": np.uint8, "f32": np.float32}[out_dtype]
@@ -169,7 +169,10 @@ def run(host, graph, weights, x, in_name, in_dtype, out_name, out_dtype, d_out, 
     r.input, r.input_bytes = x.ctypes.data, x.nbytes
     r.output_name, r.output_dtype, r.output_last = out_name.encode(), DT[out_dtype], d_out
     r.output, r.output_capacity, r.executions = y.ctypes.data, y.nbytes, executions
-    if threads:
+    if batch_proof is not None:
+        mock.mock_host_run_batch.argtypes = [C.POINTER(MockRun), C.c_int32]
+        mock.mock_host_run_batch(C.byref(r), 1 if batch_proof else 0)
+    elif threads:
         mock.mock_host_run_concurrent.argtypes = [C.POINTER(MockRun), C.c_int32]
         mock.mock_host_run_concurrent(C.byref(r), threads)
     else:
@@ -404,6 +407,27 @@ def test_contexts_of_one_compiled_model_run_concurrently(registered, oracle, tmp
     assert r.status == 0 and r.writes == 8
     _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], 520, 128)
     assert (y.view(np.uint32) == want.view(np.uint32)).all()
+
+
+@pytest.mark.gpu
+def test_scheduler_batch_runs_as_one_invocation(registered, oracle, tmp_path):
+    """Six requests of [1, 3, K] stacked along a symbolic axis 0: one provider invocation, six lane
+    sinks, every lane the slice the oracle computes; without the core's independence proof the
+    frozen contract stays at B = 1."""
+    batch, inner, k, n, group = 6, 3, 384, 200, 128
+    c = cases.packed_case(batch * inner, k, n, group, 21)
+    x = c["x"].reshape(batch, inner, k)
+    words = oracle.pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "p", (1, inner, k), words, c["scales"], c["bias"], group)
+    r, y = run(registered, g, w, x, "x", "f32", "logits", "f32", n, arithmetic="dynamic_i8", lead_max=[16, 0],
+               batch_proof=True)
+    assert r.status == 0, r.message
+    assert r.writes == batch and r.execute_attested and r.attested_arithmetic == 16  # frozen max_batch
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group)
+    assert (y.reshape(-1, n).view(np.uint32) == want.view(np.uint32)).all()
+    r2, _ = run(registered, g, w, x, "x", "f32", "logits", "f32", n, arithmetic="dynamic_i8", lead_max=[16, 0],
+                batch_proof=False)
+    assert r2.status == -7 and r2.attested_arithmetic == 1 and r2.writes == 0
 
 
 @pytest.mark.gpu

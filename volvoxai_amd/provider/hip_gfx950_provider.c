@@ -75,6 +75,11 @@ typedef struct HipCompiled {
     int64_t lead_min[VX_MAX_TENSOR_RANK]; /* bounds of the leading dimensions */
     int64_t lead_max[VX_MAX_TENSOR_RANK];
     int64_t lead_multiple[VX_MAX_TENSOR_RANK];
+    /* Scheduler batching: possible when axis 0 is a symbolic axis that admits extent 1 and the
+     * core proved the requests independent along it; the identities are echoed in the contract. */
+    int batch_capable;
+    char graph_fingerprint[256];
+    char batch_proof_identity[256];
     VxHipQLinear* qlinear;
     VxHipPackedLinear* packed;
     float input_scale, output_scale;
@@ -538,6 +543,19 @@ static int specs_match(const VxBackendCompileInput* input, const PackagePlan* pl
         compiled->lead_max[axis] = a->max;
         compiled->lead_multiple[axis] = a->multiple_of;
     }
+    compiled->batch_capable = in->rank >= 2 && in->dimensions[0].kind == VX_DIMENSION_SYMBOLIC &&
+                              out->dimensions[0].kind == VX_DIMENSION_SYMBOLIC && in->dimensions[0].min <= 1 &&
+                              in->dimensions[0].multiple_of == 1 && input->independent_batch_proof_protocol &&
+                              !strcmp(input->independent_batch_proof_protocol,
+                                      VX_BACKEND_INDEPENDENT_BATCH_PROOF_PROTOCOL) &&
+                              input->independent_batch_proof_identity &&
+                              strlen(input->independent_batch_proof_identity) < sizeof(compiled->batch_proof_identity) &&
+                              strlen(input->graph_fingerprint) < sizeof(compiled->graph_fingerprint);
+    if (compiled->batch_capable) {
+        snprintf(compiled->graph_fingerprint, sizeof(compiled->graph_fingerprint), "%s", input->graph_fingerprint);
+        snprintf(compiled->batch_proof_identity, sizeof(compiled->batch_proof_identity), "%s",
+                 input->independent_batch_proof_identity);
+    }
     return 1;
 }
 
@@ -698,40 +716,34 @@ static VxStatus grow_device(void** buffer, size_t* capacity, size_t bytes) {
     return VX_STATUS_OK;
 }
 
-static VxStatus hip_context_execute(void* context_instance, const VxTensorBinding* inputs, size_t input_count,
-                                    const VxBackendOutputSink* sink, VxReport* report) {
-    HipContext* context = (HipContext*)context_instance;
-    const HipCompiled* compiled;
-    const VxTensorBinding* binding;
-    int64_t shape[VX_MAX_TENSOR_RANK];
-    uint64_t rows = 1;
-    size_t input_bytes, output_bytes;
-    VxStatus status;
-    int handled;
-    if (!context || context->closed || !inputs || input_count != 1 || !sink || sink->struct_size != sizeof(*sink) ||
-        !sink->write)
-        return VX_STATUS_INVALID_ARGUMENT;
-    compiled = context->compiled;
-    binding = &inputs[0];
-    /* the complete batch is validated before anything is mutated */
+/* Checks one binding against the compiled contract; on success the row count and output shape. */
+static int binding_admitted(const HipCompiled* compiled, const VxTensorBinding* binding, uint64_t* rows,
+                            int64_t* shape) {
+    *rows = 1;
     if (binding->struct_size != sizeof(*binding) || !binding->name || strcmp(binding->name, compiled->input_name) ||
         binding->dtype != compiled->input_dtype || binding->rank != compiled->rank ||
         binding->location != VX_MEMORY_HOST || !binding->data ||
         binding->shape[compiled->rank - 1] != (int64_t)compiled->d_in)
-        return VX_STATUS_INVALID_ARGUMENT;
+        return 0;
     for (uint32_t axis = 0; axis + 1 < compiled->rank; axis++) {
         const int64_t extent = binding->shape[axis];
         if (extent < compiled->lead_min[axis] || extent > compiled->lead_max[axis] ||
             extent % compiled->lead_multiple[axis] != 0)
-            return VX_STATUS_INVALID_ARGUMENT;
-        rows *= (uint64_t)extent;
+            return 0;
+        *rows *= (uint64_t)extent;
         shape[axis] = extent;
     }
     shape[compiled->rank - 1] = (int64_t)compiled->d_out;
-    input_bytes = (size_t)rows * compiled->d_in * compiled->input_element_bytes;
-    output_bytes = (size_t)rows * compiled->d_out * compiled->output_element_bytes;
-    if (binding->byte_size != input_bytes) return VX_STATUS_INVALID_ARGUMENT;
+    return binding->byte_size == (size_t)*rows * compiled->d_in * compiled->input_element_bytes;
+}
 
+/* Upload, one linear over all rows, download into the context's host buffer. */
+static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, VxReport* report) {
+    const HipCompiled* compiled = context->compiled;
+    const size_t input_bytes = (size_t)rows * compiled->d_in * compiled->input_element_bytes;
+    const size_t output_bytes = (size_t)rows * compiled->d_out * compiled->output_element_bytes;
+    VxStatus status;
+    int handled;
     status = grow_device(&context->input_dev, &context->input_capacity, input_bytes);
     if (status == VX_STATUS_OK) status = grow_device(&context->output_dev, &context->output_capacity, output_bytes);
     if (status == VX_STATUS_OK && output_bytes > context->host_capacity) {
@@ -742,11 +754,8 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
             context->host_capacity = output_bytes;
         }
     }
-    if (status != VX_STATUS_OK) {
-        fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
-        return status;
-    }
-    status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->input_dev, binding->data, input_bytes);
+    if (status == VX_STATUS_OK)
+        status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->input_dev, input, input_bytes);
     if (status == VX_STATUS_OK) {
         if (compiled->qlinear)
             handled = vxhip_qlinear_forward(context->ctx, compiled->qlinear, context->input_dev, context->output_dev, NULL,
@@ -760,14 +769,94 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
     }
     if (status == VX_STATUS_OK)
         status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host, context->output_dev, output_bytes);
-    if (status != VX_STATUS_OK) {
+    if (status != VX_STATUS_OK)
         fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
-        return status;
-    }
+    return status;
+}
+
+static VxStatus hip_context_execute(void* context_instance, const VxTensorBinding* inputs, size_t input_count,
+                                    const VxBackendOutputSink* sink, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    const HipCompiled* compiled;
+    int64_t shape[VX_MAX_TENSOR_RANK];
+    uint64_t rows;
+    VxStatus status;
+    if (!context || context->closed || !inputs || input_count != 1 || !sink || sink->struct_size != sizeof(*sink) ||
+        !sink->write)
+        return VX_STATUS_INVALID_ARGUMENT;
+    compiled = context->compiled;
+    /* the complete batch is validated before anything is mutated */
+    if (!binding_admitted(compiled, &inputs[0], &rows, shape)) return VX_STATUS_INVALID_ARGUMENT;
+    status = run_rows(context, inputs[0].data, rows, report);
+    if (status != VX_STATUS_OK) return status;
     status = sink->write(sink->user_data, compiled->output_name, compiled->output_dtype, shape, compiled->rank,
-                         context->output_host, output_bytes);
+                         context->output_host, (size_t)rows * compiled->d_out * compiled->output_element_bytes);
     if (status != VX_STATUS_OK) return status;
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear executed");
+    attest(report, vxhip_context_last_variant(context->ctx));
+    return VX_STATUS_OK;
+}
+
+/* Frozen batch contract (native/include/volvoxai_backend.h:39-73).  B > 1 is offered along
+ * axis 0 only, inside the symbolic range the core handed over and only with its proof identity. */
+static VxStatus hip_compiled_batch_contract(void* compiled_instance, VxBackendBatchContract* contract,
+                                            VxReport* report) {
+    HipCompiled* compiled = (HipCompiled*)compiled_instance;
+    if (!compiled || !contract || contract->struct_size != sizeof(*contract)) return VX_STATUS_INVALID_ARGUMENT;
+    contract->protocol = VX_BACKEND_BATCH_PROTOCOL;
+    contract->resource_domain = compiled;
+    contract->compatibility_token = compiled;
+    contract->min_batch = 1;
+    contract->max_batch = 1;
+    contract->multiple_of = 1;
+    contract->batch_axis = 0;
+    contract->device_resident = 0;
+    contract->device_epoch = 0;
+    contract->graph_fingerprint = NULL;
+    contract->independent_batch_proof_identity = NULL;
+    if (compiled->batch_capable) {
+        contract->graph_fingerprint = compiled->graph_fingerprint;
+        contract->independent_batch_proof_identity = compiled->batch_proof_identity;
+        contract->max_batch = compiled->lead_max[0] > 65536 ? 65536u : (uint32_t)compiled->lead_max[0];
+    }
+    fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE, "batch contract frozen");
+    return VX_STATUS_OK;
+}
+
+/* One entry into the device for the whole invocation: the stacked rows run as one linear and lane
+ * i is the i-th slice along axis 0 (native/include/volvoxai_backend.h:75-92). */
+static VxStatus hip_context_execute_batch(void* context_instance, const VxBackendBatchInvocation* invocation,
+                                          VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    const HipCompiled* compiled;
+    int64_t shape[VX_MAX_TENSOR_RANK];
+    uint64_t rows;
+    size_t lane_bytes;
+    VxStatus status;
+    if (!context || context->closed || !invocation || invocation->struct_size != sizeof(*invocation) ||
+        !invocation->stacked_inputs || invocation->stacked_input_count != 1 || !invocation->batch_size ||
+        !invocation->lane_output_sinks || invocation->lane_output_sink_count != invocation->batch_size)
+        return VX_STATUS_INVALID_ARGUMENT;
+    compiled = context->compiled;
+    if (invocation->batch_size > 1 && !compiled->batch_capable) return VX_STATUS_BACKEND_UNSUPPORTED;
+    if (!binding_admitted(compiled, &invocation->stacked_inputs[0], &rows, shape) ||
+        shape[0] != (int64_t)invocation->batch_size)
+        return VX_STATUS_INVALID_ARGUMENT;
+    for (uint32_t lane = 0; lane < invocation->batch_size; lane++) {
+        const VxBackendOutputSink* sink = &invocation->lane_output_sinks[lane];
+        if (sink->struct_size != sizeof(*sink) || !sink->write) return VX_STATUS_INVALID_ARGUMENT;
+    }
+    status = run_rows(context, invocation->stacked_inputs[0].data, rows, report);
+    if (status != VX_STATUS_OK) return status;
+    lane_bytes = (size_t)(rows / invocation->batch_size) * compiled->d_out * compiled->output_element_bytes;
+    shape[0] = 1;
+    for (uint32_t lane = 0; lane < invocation->batch_size; lane++) {
+        const VxBackendOutputSink* sink = &invocation->lane_output_sinks[lane];
+        status = sink->write(sink->user_data, compiled->output_name, compiled->output_dtype, shape, compiled->rank,
+                             (const unsigned char*)context->output_host + (size_t)lane * lane_bytes, lane_bytes);
+        if (status != VX_STATUS_OK) return status;
+    }
+    fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear batch executed");
     attest(report, vxhip_context_last_variant(context->ctx));
     return VX_STATUS_OK;
 }
@@ -795,6 +884,8 @@ VxStatus volvoxai_hip_gfx950_backend_register(VxReport* report) {
         .runtime_destroy = hip_runtime_destroy,
         .compile = hip_compile,
         .compiled_destroy = hip_compiled_destroy,
+        .compiled_batch_contract = hip_compiled_batch_contract,
+        .context_execute_batch = hip_context_execute_batch,
         .context_create = hip_context_create,
         .context_execute = hip_context_execute,
         .context_close = hip_context_close,
