@@ -12,6 +12,9 @@ A "step" is one W8A8 linear over one batch of synthetic, HBM-resident input:
             fraction of HBM peak, rotating over enough weight copies that the
             256 MB Infinity Cache cannot serve them.
 
+The timed region is exactly K steps, recorded once into a HIP graph and replayed
+(`ms_per_step_launched_singly` gives the same K steps launched one by one).
+
 Prints ONE JSON line.  The CPU column times the reference's own native CPU
 route (oracle/_ref, compiled from the reference sources) on the host cores
 with a bounded sample; it is a reported baseline, never part of the GPU path.
@@ -50,11 +53,45 @@ def gemv_algorithmic_bytes(m, k, n):
 
 def kernel_ms(per_launch_mean_ms, region_ms_per_step):
     """Average kernel duration.  Both measurements bound it from above: an event pair around one
-    launch adds the events' own cost (about 2 us, visible on a 12 us kernel), and the timed
-    region divided by its launches adds the gaps between launches (about 4 us, visible on the
-    GEMM).  The smaller of the two is the estimate; it is the one rocprofv3's kernel trace
-    agrees with."""
+    launch adds the events' own cost (about 2 us, visible on a 12 us kernel), and a region of
+    single launches divided by their number adds the gaps between launches (about 4 us, visible
+    on the GEMM).  The smaller of the two is the estimate; it is the one rocprofv3's kernel
+    trace agrees with.  (The graph-replayed region is not used here: consecutive kernels of a
+    graph overlap their ramp-down and ramp-up, so its per-step time can undercut the duration
+    of a kernel on its own.)"""
     return min(per_launch_mean_ms, region_ms_per_step)
+
+
+def timed_region(fn, steps, torch, stream):
+    """ms per step over exactly `steps` calls fn(0..steps-1), two ways: launched one by one, and
+    the same launches recorded once into a HIP graph and replayed (the recording is not timed;
+    the first replay, which uploads the graph, is not either).  The replay is how a serving loop
+    would issue a fixed sequence of launches; it takes the 4-5 us idle gaps between consecutive
+    launches away.  Returns (singly_ms, graph_ms or None)."""
+    with torch.cuda.stream(stream):
+        stream.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i)
+        stream.synchronize()
+        singly = (time.perf_counter() - t0) * 1e3 / steps
+    graph_ms = None
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(steps):
+                fn(i)
+        stream.synchronize()
+        with torch.cuda.stream(stream):
+            graph.replay()
+            stream.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            stream.synchronize()
+            graph_ms = (time.perf_counter() - t0) * 1e3 / steps
+    except RuntimeError as e:  # capture refused: report the singly launched figure only
+        print(f"bench.py: HIP graph capture failed ({e}); timing single launches", file=sys.stderr)
+    return singly, graph_ms
 
 
 def time_events(fn, steps, torch):
@@ -287,7 +324,8 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "launches": args.steps}))
         return
-    ctx = vx.Context(0, torch.cuda.current_stream())
+    stream = torch.cuda.Stream()
+    ctx = vx.Context(0, stream)
     out = {"metric": METRIC, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
            "data": "synthetic (seeded; random-init weights)"}
@@ -306,18 +344,18 @@ def main():
             ok, _ = lin.forward_rowscale(ctx, xd, rs, c["s_out"], 0, bias_f32=bd, out=yd)
             assert ok == 1, vx.library().vxhip_last_error()
 
-        for _ in range(args.warmup):
-            step()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        mean_ms, med_ms, min_ms = time_events(step, args.steps, torch)
+        with torch.cuda.stream(stream):
+            for _ in range(args.warmup):
+                step()
+        singly_ms, graph_ms = timed_region(step, args.steps, torch, stream)
+        wall_ms = graph_ms if graph_ms is not None else singly_ms
+        with torch.cuda.stream(stream):
+            mean_ms, med_ms, min_ms = time_events(step, args.steps, torch)
         ops = 2.0 * M * K * N
-        mean_ms = kernel_ms(mean_ms, wall_ms)
-        out.update(value=ops / (wall_ms * 1e-3) / 1e12, ms_per_step=wall_ms,
+        mean_ms = kernel_ms(mean_ms, singly_ms)
+        out.update(value=ops / (wall_ms * 1e-3) / 1e12, ms_per_step=wall_ms, ms_per_step_launched_singly=singly_ms,
+                   launch="the K steps replayed from one HIP graph" if graph_ms is not None else "K single launches",
                    config={"workload": "configs[2]: prefill GEMM M=K=N=4096, int8 x int8 -> int32, per-token x "
                                        "per-channel scale + f32 bias, requant to int8 (scale 0.05, ties-even)",
                            "M": M, "K": K, "N": N, "variant": ctx.last_variant})
@@ -363,21 +401,21 @@ def main():
         def gstep_hot(_i=0):
             gstep(0)
 
-        for i in range(args.warmup):
-            gstep(i)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            gstep(i)
-        torch.cuda.synchronize()
-        gwall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        gmean, gmed, gmin = time_events(gstep, args.steps, torch)
-        hmean, hmed, hmin = time_events(gstep_hot, args.steps, torch)
+        with torch.cuda.stream(stream):
+            for i in range(args.warmup):
+                gstep(i)
+        gsingly_ms, ggraph_ms = timed_region(gstep, args.steps, torch, stream)
+        gwall_ms = ggraph_ms if ggraph_ms is not None else gsingly_ms
+        with torch.cuda.stream(stream):
+            gmean, gmed, gmin = time_events(gstep, args.steps, torch)
+            hmean, hmed, hmin = time_events(gstep_hot, args.steps, torch)
         gb = gemv_algorithmic_bytes(Mg, Kg, Ng)
-        gmean = kernel_ms(gmean, gwall_ms)
+        gmean = kernel_ms(gmean, gsingly_ms)
         _, want, _ = orc.packed_linear_a8(d["a8"], d["row_scales"], words, d["scales"], d["bias"], Ng, G)
         out["gemv"] = {"workload": "configs[1]: decode GEMV M=1, K=4096, N=14336, dequant + bias to f32",
                        "value": gb / (gwall_ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": gwall_ms,
+                       "ms_per_step_launched_singly": gsingly_ms,
                        "variant": ctx.last_variant, "weight_copies_rotated": copies,
                        "hot_in_cache_GBs": gb / (hmean * 1e-3) / 1e9,
                        "parity_bit_exact": bool((yg.cpu().numpy().view(np.uint32) == want.view(np.uint32)).all())}
@@ -394,7 +432,8 @@ def main():
 
     # ---- the other benchmark sizes, timed only (their parity is in tests/) -----
     if args.only is None:
-        out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
+        with torch.cuda.stream(stream):
+            out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
 
     # ---- config 4: 28-layer decoder, 32 rows, greedy decode ------------------------
     if args.only in (None, "decoder"):
