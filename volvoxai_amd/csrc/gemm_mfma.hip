@@ -206,14 +206,27 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // Per-group scale-accumulate of PackedLinear/DYNAMIC_I8: complete the exact
     // int32 dot of one storage group, then sum += f32(dot) * (s_a * s_w[n][g]) in
     // ascending group order (packed_linear_ops.inc:1498-1504).
-    auto fold_group = [&](uint32_t g) {
+    // The group's weight scales are requested one group ahead (right after the previous fold),
+    // so the fold never waits on their L2 latency (that wait was 15 % of the large-K GEMM).
+    v4f sw_next[F32OUT ? TN : 1][4];
+    auto load_scales = [&](uint32_t g) {
         if constexpr (F32OUT) {
             const float* srow = a.scales_t + (size_t)min(g, a.groups - 1u) * a.n_pad;
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    sw_next[i][q] = *reinterpret_cast<const v4f*>(srow + nbase + i * 32 + q * 8);
+        }
+    };
+    load_scales(0);
+    auto fold_group = [&](uint32_t g) {
+        if constexpr (F32OUT) {
 #pragma unroll
             for (int i = 0; i < TN; i++) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const v4f sw = *reinterpret_cast<const v4f*>(srow + nbase + i * 32 + q * 8);
+                    const v4f sw = sw_next[i][q];
 #pragma unroll
                     for (int j = 0; j < TM; j++) {
 #pragma unroll
@@ -223,11 +236,13 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                             const float term = __fmul_rn((float)acc[i][j][r], gs);
                             fsum[i][j][r] = __float_as_int(
                                 __fadd_rn(__int_as_float(fsum[i][j][r]), term));
-                            acc[i][j][r] = 0;
+                            // groups that end inside a k-block restart from the MFMA's zero C operand
+                            if constexpr (GK > KS) acc[i][j][r] = 0;
                         }
                     }
                 }
             }
+            load_scales(g + 1u);
         }
     };
 
@@ -297,7 +312,10 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             if constexpr (VXHIP_PROBE_NO_MFMA) {
                 acc[i][j][0] += wf[CB][i][0] ^ xf[CB][j][1];
             } else {
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], acc[i][j], 0, 0, 0);
+                // first k-step of a scale group: accumulate onto zero instead of clearing registers
+                constexpr bool FRESH = F32OUT && GK <= KS && (S % GK) == 0;
+                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], FRESH ? zero : acc[i][j], 0, 0, 0);
             }
             // after MFMA m: the reads and loads whose slot it is.  Reads keep clear of the
             // step's last MFMAs, which cover the latency of the final read.
@@ -563,6 +581,8 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
     if (forced("t256x256")) big = true;
     if (forced("t128x128")) big = false;
     if constexpr (MODE == (int)Epilogue::DequantF32) {
+        if (!forced("t256x256") && !forced("t128x128"))
+            big = (uint64_t)((a.n + 127) / 128) * ((a.rows + 255) / 256) >= (uint64_t)cu_count * 3 / 4;
         // int32 tile accumulators plus f32 running sums: keep the wave tile at 64x64.  With a
         // scale group per k-step the eight-wave tile runs out of registers, so it stays with four.
         if (big && GK > 1) return launch_cfg<2, 4, 2, 2, MODE, GK>(s, a) ? "t128x256" : nullptr;
