@@ -182,14 +182,12 @@ def cpu_baseline_gemv(k, n, seed):
 
 
 def region_ms(fn, steps, torch, warmup=5):
+    """ms per call over `steps` calls replayed from one HIP graph on the current stream (launched
+    one by one if capture is refused); see timed_region."""
     for i in range(warmup):
         fn(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        fn(i)
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    singly, graph = timed_region(fn, steps, torch, torch.cuda.current_stream())
+    return graph if graph is not None else singly
 
 
 def bench_other_configs(torch, vx, cases, ctx):
@@ -210,6 +208,29 @@ def bench_other_configs(torch, vx, cases, ctx):
         gb = gemv_algorithmic_bytes(m, Kg, Ng)
         res[f"gemv_M{m}_K4096_N14336"] = {"ms": ms, "GBs": gb / (ms * 1e-3) / 1e9, "frac_hbm": gb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                            "variant": ctx.last_variant}
+    for p in pls:
+        p.close()
+    # the same decode shape with four-bit weights: half the weight bytes, same scales and output
+    from volvoxai_amd.decoder import pack_w4_words
+    w4words = pack_w4_words((d["w"] >> 4).astype(np.int8))
+    pls = [vx.PackedLinear(w4words, d["scales"], d["bias"], Kg, Ng, G, weight_bits=4) for _ in range(copies)]
+    for m in (1, 16):
+        a8 = torch.from_numpy(d["a8"][:m]).cuda()
+        ars = torch.from_numpy(d["row_scales"][:m]).cuda()
+        y = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
+        ms = region_ms(lambda i: pls[i % copies].forward_a8(ctx, a8, ars, out=y), 100, torch)
+        gb = gemv_algorithmic_bytes(m, Kg, Ng) - Kg * Ng // 2
+        res[f"w4a8_gemv_M{m}_K4096_N14336"] = {"ms": ms, "GBs": gb / (ms * 1e-3) / 1e9,
+                                                "frac_hbm": gb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                                "variant": ctx.last_variant}
+    a8 = torch.from_numpy(np.tile(d["a8"], (128, 1))).cuda()
+    ars = torch.from_numpy(np.tile(d["row_scales"], 128)).cuda()
+    y = torch.empty((2048, Ng), dtype=torch.float32, device="cuda")
+    ms = region_ms(lambda i: pls[0].forward_a8(ctx, a8, ars, out=y), 30, torch)
+    ops = 2.0 * 2048 * Kg * Ng
+    res["w4a8_gemm_f32out_M2048_K4096_N14336"] = {"ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12,
+                                                   "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                                                   "variant": ctx.last_variant}
     for p in pls:
         p.close()
     # prefill GEMM, M = 512 and 2048
@@ -300,7 +321,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "copy"], default=None,
+    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "copy", "other"], default=None,
                     help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
                          "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
@@ -431,7 +452,7 @@ def main():
             p.close()
 
     # ---- the other benchmark sizes, timed only (their parity is in tests/) -----
-    if args.only is None:
+    if args.only in (None, "other"):
         with torch.cuda.stream(stream):
             out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
 

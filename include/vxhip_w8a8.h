@@ -213,12 +213,16 @@ int vxhip_qlinear_i8u8(const void* input, const void* weight,
                        int32_t output_zero_point, uint32_t input_dtype,
                        uint32_t weight_dtype, uint32_t output_dtype);
 
-/* ---- PackedLinear W8 under DYNAMIC_I8: dequant + bias to f32 ----------- */
+/* ---- PackedLinear W8/W4 under DYNAMIC_I8: dequant + bias to f32 -------- */
 
-/* packed_words [n, ceil(k/4)] offset-binary I32 words, scales [n, ceil(k/G)],
- * bias [n] or NULL, group_size in {32,64,128,256}, weight_bits must be 8
- * (docs/packed-linear-design.md:24-32; physical shapes as checked at
- * src/runtime/engine_runtime_llm.inc:94-99).  HOST pointers, not retained. */
+/* packed_words [n, vx_packed_words(k, bits)] I32 words
+ * (src/kernels/packed_linear_ops.inc:246-248): weight_bits 8 = offset-binary
+ * bytes (code - 128), four per word; weight_bits 4 = nibbles (code - 8),
+ * eight per word, lowest first (:474-480).  scales [n, ceil(k/G)], bias [n] or
+ * NULL, group_size in {32,64,128,256} (docs/packed-linear-design.md:24-32;
+ * physical shapes as checked at src/runtime/engine_runtime_llm.inc:94-99).
+ * Other widths return VXHIP_BACKEND_UNSUPPORTED.  HOST pointers, not retained.
+ * Four-bit weights stay four-bit in device memory. */
 VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words,
                                        const float* scales, const float* bias,
                                        uint32_t k, uint32_t n,
@@ -238,7 +242,7 @@ VxHipStatus vxhip_packed_prepare_i8(VxHipContext* context,
                                     uint32_t k, int8_t* prepared_dev,
                                     float* row_scales_dev);
 
-/* vx_packed_linear_forward with normalize==8, groups==8
+/* vx_packed_linear_forward with normalize==8, groups==8 or 4
  * (src/kernels/packed_linear_ops.inc:1545-1621) on resident f32 rows.
  * Returns 0 on success, -1 on a rejected descriptor (reference convention). */
 int vxhip_packed_linear_forward_f32(VxHipContext* context,
@@ -249,7 +253,8 @@ int vxhip_packed_linear_forward_f32(VxHipContext* context,
 /* Same arithmetic from already prepared activations (the x[4]/x[5] form of
  * src/kernels/llm_ops.h:30-32): int8 codes [rows,k] and one f32 scale per
  * row; a NaN scale marks a non-finite row (whole output row NaN).
- * accumulators_dev optional int32 [rows,n] = full-K sum of the group dots. */
+ * accumulators_dev optional int32 [rows,n] = full-K sum of the group dots
+ * (8-bit weights only). */
 int vxhip_packed_linear_forward_a8(VxHipContext* context,
                                    const VxHipPackedLinear* linear,
                                    const int8_t* activation_dev,
@@ -261,7 +266,8 @@ int vxhip_packed_linear_forward_a8(VxHipContext* context,
  * (src/kernels/llm_ops.h:38-53) is not reproduced here; this one-shot HOST
  * entry takes the same values as plain arguments: x=input f32 [rows,k],
  * packed_weight, scale, bias (optional), y=out [rows,n], key_dim=k,
- * value_dim=n, rate=group_size, groups=weight_bits, normalize=8.
+ * value_dim=n, rate=group_size, groups=weight_bits (8 or 4; 0 means 4 as in
+ * the reference), normalize=8.
  * Returns 0 / -1 like vx_llm_forward_f32 (src/kernels/llm_ops.inc:41-56). */
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
                             const float* scale, const float* bias,

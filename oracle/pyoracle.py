@@ -103,6 +103,14 @@ class Oracle:
         L.vxo_ptq_pack_bias_i32.argtypes = [_f32p, C.c_int32, C.c_float, _f32p, _i32p]
         L.vxo_pack_w8_words.restype = None
         L.vxo_pack_w8_words.argtypes = [_i8p, C.c_uint32, C.c_uint32, _u32p]
+        L.vxo_pack_w4_words.restype = None
+        L.vxo_pack_w4_words.argtypes = [_i8p, C.c_uint32, C.c_uint32, _u32p]
+        L.vxo_packed_linear_forward_bits.restype = C.c_int
+        L.vxo_packed_linear_forward_bits.argtypes = (
+            list(L.vxo_packed_linear_forward.argtypes) + [C.c_uint32])
+        L.vxo_packed_linear_a8_bits.restype = C.c_int
+        L.vxo_packed_linear_a8_bits.argtypes = (
+            list(L.vxo_packed_linear_a8.argtypes) + [C.c_uint32])
 
     # -- scalar helpers ---------------------------------------------------
     def round_ties_even(self, v):
@@ -161,24 +169,31 @@ class Oracle:
             s[r] = sc.value
         return a, s, fin
 
-    def packed_linear(self, x, packed, scales, bias, n, group):
+    def packed_linear(self, x, packed, scales, bias, n, group, bits=8):
         rows, k = x.shape
         y = np.zeros((rows, n), dtype=np.float32)
-        st = self.lib.vxo_packed_linear_forward(
+        st = self.lib.vxo_packed_linear_forward_bits(
             _ptr(x, _f32p), _ptr(packed, _u32p), _ptr(scales, _f32p),
-            _ptr(bias, _f32p), _ptr(y, _f32p), rows, k, n, group)
+            _ptr(bias, _f32p), _ptr(y, _f32p), rows, k, n, group, bits)
         return st, y
 
     def packed_linear_a8(self, a, row_scales, packed, scales, bias, n, group,
-                         row_finite=None):
+                         row_finite=None, bits=8):
         rows, k = a.shape
         y = np.zeros((rows, n), dtype=np.float32)
         acc = np.zeros((rows, n), dtype=np.int32)
-        st = self.lib.vxo_packed_linear_a8(
+        st = self.lib.vxo_packed_linear_a8_bits(
             _ptr(a, _i8p), _ptr(row_scales, _f32p), _ptr(row_finite, _u8p),
             _ptr(packed, _u32p), _ptr(scales, _f32p), _ptr(bias, _f32p),
-            _ptr(y, _f32p), _ptr(acc, _i32p), rows, k, n, group)
+            _ptr(y, _f32p), _ptr(acc, _i32p), rows, k, n, group, bits)
         return st, y, acc
+
+    def pack_w4_words(self, w):
+        n, k = w.shape
+        words = (k // 32) * 4 + ((k % 32) * 4 + 31) // 32
+        out = np.zeros((n, words), dtype=np.uint32)
+        self.lib.vxo_pack_w4_words(_ptr(w, _i8p), n, k, _ptr(out, _u32p))
+        return out
 
     def pack_w8_words(self, w):
         n, k = w.shape
@@ -338,14 +353,14 @@ class Reference:
             rows, k, n, w_dtype, int(zero_zp)))
 
     # PackedLinear -----------------------------------------------------------
-    def packed_linear(self, x, packed, scales, bias, n, group):
+    def packed_linear(self, x, packed, scales, bias, n, group, bits=8):
         rows, k = x.shape
         y = np.zeros((rows, n), dtype=np.float32)
         a = _LLMOpArgs()
         a.kind = OP_PACKED_LINEAR
         a.batch, a.sequence = 1, rows
         a.key_dim, a.value_dim = k, n
-        a.groups, a.rate, a.normalize = 8, group, 8
+        a.groups, a.rate, a.normalize = bits, group, 8
         a.x[0] = x.ctypes.data
         a.x[1] = packed.ctypes.data
         a.x[2] = scales.ctypes.data

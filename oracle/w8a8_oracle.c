@@ -226,19 +226,30 @@ static int group_size_ok(uint32_t g) {
     return g == 32u || g == 64u || g == 128u || g == 256u;
 }
 
-static int32_t w8_code(const uint32_t* row_words, uint32_t k) {
+/* src/kernels/packed_linear_ops.inc:474-480: W8 codes are offset by 128, W4
+ * codes by 8; both little-endian within their I32 word. */
+static int32_t packed_code(const uint32_t* row_words, uint32_t k, uint32_t bits) {
+    if (bits == 4u)
+        return (int32_t)((row_words[k / 8u] >> ((k % 8u) * 4u)) & 15u) - 8;
     return (int32_t)((row_words[k / 4u] >> ((k % 4u) * 8u)) & 255u) - 128;
 }
 
-int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
-                         const uint8_t* row_finite, const uint32_t* packed,
-                         const float* scales, const float* bias, float* output,
-                         int32_t* accumulators, uint64_t rows, uint32_t k,
-                         uint32_t n, uint32_t group_size) {
+/* src/kernels/packed_linear_ops.inc:246-248 */
+static uint32_t packed_words(uint32_t k, uint32_t bits) {
+    return (k / 32u) * bits + ((k % 32u) * bits + 31u) / 32u;
+}
+
+int vxo_packed_linear_a8_bits(const int8_t* activation, const float* row_scales,
+                              const uint8_t* row_finite, const uint32_t* packed,
+                              const float* scales, const float* bias,
+                              float* output, int32_t* accumulators,
+                              uint64_t rows, uint32_t k, uint32_t n,
+                              uint32_t group_size, uint32_t weight_bits) {
     if (!activation || !row_scales || !packed || !scales || !output || !k ||
-        !n || !group_size_ok(group_size))
+        !n || !group_size_ok(group_size) ||
+        (weight_bits != 4u && weight_bits != 8u))
         return -1;
-    const uint32_t words = (k + 3u) / 4u;
+    const uint32_t words = packed_words(k, weight_bits);
     const uint32_t groups = (k + group_size - 1u) / group_size;
     for (uint64_t r = 0; r < rows; r++) {
         const int8_t* a = activation + r * k;
@@ -257,7 +268,7 @@ int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
                 const uint32_t end = begin + group_size < k ? begin + group_size : k;
                 int32_t dot = 0;
                 for (uint32_t j = begin; j < end; j++)
-                    dot += (int32_t)a[j] * w8_code(w, j);
+                    dot += (int32_t)a[j] * packed_code(w, j, weight_bits);
                 total += dot;
                 const float group_scale = as * scales[(uint64_t)o * groups + g];
                 const float term = (float)dot * group_scale;
@@ -270,10 +281,21 @@ int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
     return 0;
 }
 
-int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
-                              const float* scales, const float* bias,
-                              float* output, uint64_t rows, uint32_t k,
-                              uint32_t n, uint32_t group_size) {
+int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
+                         const uint8_t* row_finite, const uint32_t* packed,
+                         const float* scales, const float* bias, float* output,
+                         int32_t* accumulators, uint64_t rows, uint32_t k,
+                         uint32_t n, uint32_t group_size) {
+    return vxo_packed_linear_a8_bits(activation, row_scales, row_finite, packed,
+                                     scales, bias, output, accumulators, rows,
+                                     k, n, group_size, 8u);
+}
+
+int vxo_packed_linear_forward_bits(const float* input, const uint32_t* packed,
+                                   const float* scales, const float* bias,
+                                   float* output, uint64_t rows, uint32_t k,
+                                   uint32_t n, uint32_t group_size,
+                                   uint32_t weight_bits) {
     if (!input || !k || !n || !group_size_ok(group_size)) return -1;
     int8_t* prepared = (int8_t*)malloc(k);
     if (!prepared) return -1;
@@ -282,12 +304,20 @@ int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
         float as;
         const uint8_t finite =
             (uint8_t)vxo_packed_prepare_i8(input + r * k, k, prepared, &as);
-        status = vxo_packed_linear_a8(prepared, &as, &finite, packed, scales,
-                                      bias, output + r * n, NULL, 1u, k, n,
-                                      group_size);
+        status = vxo_packed_linear_a8_bits(prepared, &as, &finite, packed,
+                                           scales, bias, output + r * n, NULL,
+                                           1u, k, n, group_size, weight_bits);
     }
     free(prepared);
     return status;
+}
+
+int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
+                              const float* scales, const float* bias,
+                              float* output, uint64_t rows, uint32_t k,
+                              uint32_t n, uint32_t group_size) {
+    return vxo_packed_linear_forward_bits(input, packed, scales, bias, output,
+                                          rows, k, n, group_size, 8u);
 }
 
 /* ---- Quantize / Dequantize boundaries --------------------------------- */
@@ -400,6 +430,24 @@ void vxo_pack_w8_words(const int8_t* weight, uint32_t n, uint32_t k,
                 const uint32_t code =
                     j < k ? (uint32_t)((int32_t)weight[(uint64_t)o * k + j] + 128) : 128u;
                 word |= code << (8u * b);
+            }
+            packed[(uint64_t)o * words + w] = word;
+        }
+    }
+}
+
+void vxo_pack_w4_words(const int8_t* weight, uint32_t n, uint32_t k,
+                       uint32_t* packed) {
+    const uint32_t words = packed_words(k, 4u);
+    for (uint32_t o = 0; o < n; o++) {
+        for (uint32_t w = 0; w < words; w++) {
+            uint32_t word = 0;
+            for (uint32_t b = 0; b < 8u; b++) {
+                const uint32_t j = w * 8u + b;
+                /* a code of 8 is the value zero, which pads the tail */
+                const uint32_t code =
+                    j < k ? (uint32_t)((int32_t)weight[(uint64_t)o * k + j] + 8) & 15u : 8u;
+                word |= code << (4u * b);
             }
             packed[(uint64_t)o * words + w] = word;
         }

@@ -100,6 +100,22 @@ int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
                          int32_t* accumulators, uint64_t rows, uint32_t k,
                          uint32_t n, uint32_t group_size);
 
+/* The same two routines for 4-bit weights as well (weight_bits 4 or 8):
+ * I32 words [n, vx_packed_words(k, bits)] (src/kernels/packed_linear_ops.inc:
+ * 246-248), W4 codes offset by 8, eight per word, lowest nibble first (integer
+ * dot :474-477; single-row body :1493-1504). */
+int vxo_packed_linear_forward_bits(const float* input, const uint32_t* packed,
+                                   const float* scales, const float* bias,
+                                   float* output, uint64_t rows, uint32_t k,
+                                   uint32_t n, uint32_t group_size,
+                                   uint32_t weight_bits);
+int vxo_packed_linear_a8_bits(const int8_t* activation, const float* row_scales,
+                              const uint8_t* row_finite, const uint32_t* packed,
+                              const float* scales, const float* bias,
+                              float* output, int32_t* accumulators,
+                              uint64_t rows, uint32_t k, uint32_t n,
+                              uint32_t group_size, uint32_t weight_bits);
+
 /* src/kernels/quantize_linear_ops.inc:156-169 (scalar rule), :234-254 */
 int vxo_quantize_linear(const float* input, uint32_t elements, void* output,
                         float scale, int32_t zero_point, uint32_t dtype);
@@ -120,6 +136,10 @@ int vxo_ptq_pack_bias_i32(const float* values, int32_t count,
 
 /* docs/packed-linear-design.md:24-28: offset-binary W8 codes, LSB first. */
 void vxo_pack_w8_words(const int8_t* weight, uint32_t n, uint32_t k,
+                       uint32_t* packed);
+/* W4 codes (values -8..7, stored +8), eight per word, lowest nibble first
+ * (src/kernels/packed_linear_ops.inc:476-477). */
+void vxo_pack_w4_words(const int8_t* weight, uint32_t n, uint32_t k,
                        uint32_t* packed);
 
 #ifdef __cplusplus

@@ -157,6 +157,12 @@ def packed_case(rows, k, n, group, seed, with_bias=True, special_rows=False):
     return dict(x=x, w=w, scales=scales, bias=bias, group=group, k=k, n=n)
 
 
+def four_bit(w):
+    """int8 weights reduced to the W4 value range -8..7 (arithmetic shift, so signs and the
+    rough distribution are kept)."""
+    return (w.astype(np.int8) >> 4).astype(np.int8)
+
+
 def decode_case(rows, k, n, group, seed):
     """Decode benchmark inputs: int8 activations clip(round(N(0,30))), per-token scales
     ~U(0.01,0.05), weights uniform +-127, per-channel scales ~U(0.002,0.01)

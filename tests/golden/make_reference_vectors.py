@@ -89,7 +89,7 @@ def main():
     orc = Oracle()
     out = {"_comment": "Outputs of the reference's C kernels on the seeded inputs of tests/_cases.py; "
                        "written by tests/golden/make_reference_vectors.py.",
-           "qlinear": [], "rowscale": [], "packed": []}
+           "qlinear": [], "rowscale": [], "packed": [], "packed_w4": []}
     for kind, params in QLINEAR_CASES:
         c = build_case(kind, params)
         args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
@@ -118,6 +118,12 @@ def main():
         st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"])
         assert st == 0
         out["packed"].append({"params": params, "expected": digest(y)})
+    for params in PACKED_CASES:  # the same inputs with the weights reduced to four bits
+        c = cases.packed_case(**params)
+        words = orc.pack_w4_words(cases.four_bit(c["w"]))
+        st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=4)
+        assert st == 0
+        out["packed_w4"].append({"params": params, "expected": digest(y)})
     path = Path(__file__).with_name("reference_vectors.json")
     path.write_text(json.dumps(out, indent=1) + "\n")
     print("wrote", path, path.stat().st_size, "bytes")

@@ -202,6 +202,98 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     pl.close()
 
 
+# ---- four-bit weights ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("entry", VECTORS["packed_w4"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_packed_w4_reference_vectors(ctx, oracle, entry):
+    import volvoxai_amd as vx
+    c = cases.packed_case(**entry["params"])
+    words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], c["k"], c["n"], c["group"], weight_bits=4)
+    st, y = pl.forward_f32(ctx, dev(c["x"]))
+    ctx.synchronize()
+    y = host(y)
+    assert st == 0 and "w4a8" in ctx.last_variant
+    if not np.isnan(y).any():
+        assert sha(y) == entry["expected"]["sha256"], f"f32 bits differ from the reference ({ctx.last_variant})"
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=4)
+    assert same_f32(y, want), ctx.last_variant
+    pl.close()
+
+
+@pytest.mark.parametrize("group", [32, 64, 128, 256])
+@pytest.mark.parametrize("rows,k,n", [(1, 4096, 48), (5, 1000, 36), (16, 1536, 130), (32, 1024, 40), (27, 1056, 96),
+                                      (3, 40, 7)])
+def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
+    import volvoxai_amd as vx
+    c = cases.packed_case(rows, k, n, group, 9 + group, True, special_rows=(rows >= 5))
+    words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, bits=4)
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=4)
+    xd = dev(c["x"])
+    seen = set()
+    try:
+        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256"):
+            vx.force_variant(force)
+            st, y = pl.forward_f32(ctx, xd)
+            ctx.synchronize()
+            assert st == 0 and same_f32(host(y), want), ctx.last_variant
+            seen.add(ctx.last_variant)
+    finally:
+        vx.force_variant(None)
+    assert all("w4a8" in v for v in seen) and len(seen) == (3 if group == 32 else 4), seen
+    pl.close()
+
+
+def test_random_shape_sweep_packed_w4(ctx, oracle):
+    """Thirty seeded W4 shapes: ragged K (partial last word, block and group), every group size,
+    rows on both sides of the GEMV/GEMM boundary."""
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(78)
+    for trial in range(30):
+        rows = int(rng.choice([1, 2, 5, 16, 31, 32, 33, 40, 130, 300]))
+        k = int(rng.choice([1, 7, 32, 33, 64, 95, 128, 130, 257, 512, 1000]))
+        n = int(rng.choice([1, 2, 31, 32, 33, 70, 129, 264]))
+        group = int(rng.choice([32, 64, 128, 256]))
+        c = cases.packed_case(rows, k, n, group, 700 + trial, with_bias=bool(trial % 2), special_rows=(trial % 5 == 0))
+        words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+        _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, bits=4)
+        pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=4)
+        for force in (None, "a8-mfma" if rows <= 32 else None):
+            vx.force_variant(force)
+            try:
+                st, y = pl.forward_f32(ctx, dev(c["x"]))
+                ctx.synchronize()
+            finally:
+                vx.force_variant(None)
+            assert st == 0 and same_f32(host(y), want), (trial, rows, k, n, group, ctx.last_variant)
+        pl.close()
+
+
+def test_packed_w4_large_shapes_against_w8(ctx, oracle):
+    """Full-size shapes, too big for the CPU oracle in a test: four-bit weights must give exactly
+    what the same values stored as eight-bit codes give (already pinned), at M=1 (streaming kernel)
+    and M=512 (MFMA GEMM)."""
+    import volvoxai_amd as vx
+    k, n, group = 4096, 14336, 128
+    rng = np.random.default_rng(4)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    scales = rng.uniform(0.002, 0.01, (n, k // group)).astype(np.float32)
+    bias = rng.normal(0, 0.1, n).astype(np.float32)
+    p4 = vx.PackedLinear(oracle.pack_w4_words(w), scales, bias, k, n, group, weight_bits=4)
+    p8 = vx.PackedLinear(oracle.pack_w8_words(w), scales, bias, k, n, group)
+    assert p4.resident_bytes < 0.56 * p8.resident_bytes
+    for rows in (1, 512):
+        x = dev(rng.normal(0, 1, (rows, k)).astype(np.float32))
+        st4, y4 = p4.forward_f32(ctx, x)
+        v4 = ctx.last_variant
+        st8, y8 = p8.forward_f32(ctx, x)
+        ctx.synchronize()
+        assert st4 == st8 == 0 and "w4a8" in v4
+        assert same_f32(host(y4), host(y8)), (rows, v4)
+    p4.close(); p8.close()
+
+
 # ---- benchmark shapes ---------------------------------------------------------------------
 
 @pytest.mark.parametrize("rows", [1, 4, 16])

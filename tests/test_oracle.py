@@ -154,6 +154,37 @@ def test_packed_matches_reference_vectors(oracle, entry):
     check_digest(y, entry["expected"])
 
 
+@pytest.mark.parametrize("entry", VECTORS["packed_w4"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_packed_w4_matches_reference_vectors(oracle, entry):
+    c = cases.packed_case(**entry["params"])
+    words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+    st, y = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=4)
+    assert st == 0
+    check_digest(y, entry["expected"])
+
+
+def test_packed_w4_codes_and_group_dots(oracle):
+    """Nibble j of word j//8 holds value+8, lowest nibble first; a one-hot activation reads one
+    weight back, and the group dots are the plain integer products."""
+    k, n, g = 75, 3, 32
+    rng = np.random.default_rng(3)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    words = oracle.pack_w4_words(w)
+    assert words.shape == (n, 10)  # (75 // 32) * 4 + ceil(11 * 4 / 32)
+    for j in (0, 7, 8, 31, 32, 74):
+        assert int((words[1, j // 8] >> (4 * (j % 8))) & 15) - 8 == int(w[1, j])
+    assert int(words[0, 9] >> 12) == 0x88888  # the unused tail holds the code of zero
+    scales = np.ones((n, 3), np.float32)
+    for j in (0, 33, 74):
+        a8 = np.zeros((1, k), np.int8); a8[0, j] = 1
+        st, y, _ = oracle.packed_linear_a8(a8, np.ones(1, np.float32), words, scales, None, n, g, bits=4)
+        assert st == 0 and y[0].tolist() == w[:, j].astype(np.float32).tolist()
+    a8 = rng.integers(-127, 128, (4, k)).astype(np.int8)
+    st, y, acc = oracle.packed_linear_a8(a8, np.ones(4, np.float32), words, scales, None, n, g, bits=4)
+    assert st == 0 and (acc == a8.astype(np.int64) @ w.astype(np.int64).T).all()
+    assert (y == acc.astype(np.float32)).all()  # sums of three small integers are exact in f32
+
+
 # ---- live comparison with the reference build ------------------------------------
 
 def test_live_reference_qlinear(oracle, reference):
@@ -193,6 +224,13 @@ def test_live_reference_packed_and_bias_rule(oracle, reference):
             x[5, 3] = np.inf
         a = oracle.packed_linear(x, words, c["scales"], c["bias"], c["n"], c["group"])
         b = reference.packed_linear(x, words, c["scales"], c["bias"], c["n"], c["group"])
+        assert a[0] == b[0] == 0
+        nan = np.isnan(b[1])
+        assert (np.isnan(a[1]) == nan).all()
+        assert (a[1].view(np.uint32)[~nan] == b[1].view(np.uint32)[~nan]).all()
+        w4 = oracle.pack_w4_words(cases.four_bit(c["w"]))
+        a = oracle.packed_linear(x, w4, c["scales"], c["bias"], c["n"], c["group"], bits=4)
+        b = reference.packed_linear(x, w4, c["scales"], c["bias"], c["n"], c["group"], bits=4)
         assert a[0] == b[0] == 0
         nan = np.isnan(b[1])
         assert (np.isnan(a[1]) == nan).all()

@@ -450,6 +450,7 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     a.w = lin->w.data;
     a.panels = lin->w.panels;
     a.ksteps = lin->w.ksteps;
+    a.weight_bits = 8u;
     a.wscale = lin->scales;
     a.bias_i32 = lin->bias;
     a.wsum = lin->weight_sums;
@@ -557,8 +558,8 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
         set_error("packed_linear_create: null tensor or zero extent");
         return VXHIP_INVALID_ARGUMENT;
     }
-    if (weight_bits != 8u) {
-        set_error("packed_linear_create: only 8-bit weights run on this backend (got %u)", weight_bits);
+    if (weight_bits != 8u && weight_bits != 4u) {
+        set_error("packed_linear_create: 8- and 4-bit weights run on this backend (got %u)", weight_bits);
         return VXHIP_BACKEND_UNSUPPORTED;
     }
     if (group_size != 32u && group_size != 64u && group_size != 128u && group_size != 256u) {
@@ -568,7 +569,8 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
     if ((uint64_t)k * n > (uint64_t)1 << 40) return VXHIP_INVALID_ARGUMENT;
     int device = 0;
     VXHIP_TRY(hipGetDevice(&device));
-    const uint32_t words = (k + 3u) / 4u;
+    // vx_packed_words (packed_linear_ops.inc:246-248)
+    const uint32_t words = (k / 32u) * weight_bits + ((k % 32u) * weight_bits + 31u) / 32u;
     const uint32_t groups = (k + group_size - 1u) / group_size;
     const uint32_t n_pad = ((n + 31u) / 32u + kPanelPad - 1) / kPanelPad * kPanelPad * 32u;
     std::vector<float> st((size_t)groups * n_pad, 1.0f), hb(n_pad, 0.0f);
@@ -607,7 +609,9 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
     TRY_OR_FAIL(hipMemcpy(pl->scales_t, st.data(), st.size() * sizeof(float), hipMemcpyHostToDevice));
     TRY_OR_FAIL(hipMemcpy(pl->bias, hb.data(), n_pad * sizeof(float), hipMemcpyHostToDevice));
     // offset-binary codes: value = code - 128, i.e. the byte with its top bit flipped
-    VxHipStatus s2 = pack_weight(nullptr, raw, (size_t)words * 4u, n, k, true, &pl->w);
+    VxHipStatus s2 = weight_bits == 4u
+                         ? pack_weight_nibbles(nullptr, (const uint32_t*)raw, words, n, k, &pl->w)
+                         : pack_weight(nullptr, raw, (size_t)words * 4u, n, k, true, &pl->w);
     if (s2 != VXHIP_OK) return fail(s2);
     TRY_OR_FAIL(hipDeviceSynchronize());
 #undef TRY_OR_FAIL
@@ -639,6 +643,7 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
     a.w = pl->w.data;
     a.panels = pl->w.panels;
     a.ksteps = pl->w.ksteps;
+    a.weight_bits = pl->w.bits;
     a.row_scale = row_scales;
     a.scales_t = pl->scales_t;
     a.bias_f32 = pl->bias;
@@ -689,6 +694,10 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
     if (!rows) return 0;
     if (!use_device(ctx->device)) return -1;
     const uint32_t k = pl->w.k, n_pad = pl->w.panels * 32u;
+    if (acc_dev && pl->w.bits != 8u) {
+        set_error("packed_linear_forward_a8: the int32 sums are produced for 8-bit weights only");
+        return -1;
+    }
     if (acc_dev && (uint64_t)k * 127u * 128u > (uint64_t)INT32_MAX) {
         set_error("packed_linear_forward_a8: full-K int32 sums are not provable for K=%u", k);
         return -1;
@@ -740,8 +749,8 @@ int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, c
         rows > 0x7fffffffull)
         return -1;
     const uint32_t bits = groups ? (uint32_t)groups : 4u;
-    if (bits != 8u || normalize != 8) {
-        set_error("packed_linear_f32: this backend runs weight_bits=8 under DYNAMIC_I8 only");
+    if ((bits != 8u && bits != 4u) || normalize != 8) {
+        set_error("packed_linear_f32: this backend runs weight_bits 8 and 4 under DYNAMIC_I8 only");
         return -1;
     }
     VxHipContext* ctx = default_context();

@@ -28,11 +28,21 @@ VxHipStatus hip_status(hipError_t e, const char* what);
 // v_mfma_i32_32x32x32_i8, and half a block pair is one operand of
 // v_mfma_i32_16x16x64_i8.  Panels are padded to a multiple of 8 and steps to
 // a multiple of 4 with zero weights, so tiles never need a weight-side bound.
+//
+// Four-bit weights (bits == 4) keep the same panels and the same 1 KiB blocks,
+// but a block then covers the pair of steps (2t, 2t+1): byte j of lane l's 16
+// holds W[32*panel + l%32][64*t + 16*(l/32) + j] in its low nibble and the
+// weight 32 columns further on in its high nibble, both as 4-bit two's
+// complement.  (w << 4) & 0xf0f0f0f0 and w & 0xf0f0f0f0 therefore turn a
+// block into the two MFMA operands of its steps with every weight scaled by
+// 16, which the exact integer dot undoes with an arithmetic shift.  `ksteps`
+// counts blocks per panel in both forms.
 struct PackedWeight {
     int8_t* data = nullptr;
     uint32_t n = 0, k = 0;
     uint32_t panels = 0;   // padded
-    uint32_t ksteps = 0;   // padded
+    uint32_t ksteps = 0;   // padded; 1 KiB blocks per panel
+    uint32_t bits = 8;
     size_t bytes() const { return (size_t)panels * ksteps * 1024u; }
 };
 
@@ -96,6 +106,9 @@ VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes);
 // flip: XOR 0x80 (U8 or offset-binary source -> signed byte).
 VxHipStatus pack_weight(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
                         uint32_t n, uint32_t k, bool flip, PackedWeight* out);
+// raw_dev: [n] rows of `row_words` I32 words of offset-by-8 nibbles, lowest nibble first.
+VxHipStatus pack_weight_nibbles(hipStream_t stream, const uint32_t* raw_dev, uint32_t row_words,
+                                uint32_t n, uint32_t k, PackedWeight* out);
 VxHipStatus weight_row_stats(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
                              uint32_t n, uint32_t k, bool flip, const int32_t* zero_points_signed,
                              int32_t* sums_dev, int32_t* absmax_dev /* single word */);
@@ -124,6 +137,7 @@ struct LinearArgs {
     uint32_t rows, n, k;
     const int8_t* w;        // packed
     uint32_t panels, ksteps;
+    uint32_t weight_bits;   // 8, or 4 (DequantF32 only): see PackedWeight
     // requant: per-channel arrays are padded to n_pad and 16-byte aligned
     const float* wscale;    // [n_pad] weight scales
     const int32_t* bias_i32;// [n_pad] accumulator-domain bias

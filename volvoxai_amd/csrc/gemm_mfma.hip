@@ -96,12 +96,17 @@ constexpr int KS = 4;  // k-steps of 32 per stage: 128 bytes of k, one cache lin
 // WN x WM wavefronts, each owning TN x TM MFMA tiles of 32x32.  MODE is the
 // Epilogue; GK = k-steps per scale group (DequantF32).  FAST selects the
 // straight-line requantizing epilogue (needs n % 16 == 0, a byte output and no
-// accumulator dump); otherwise the guarded per-quad epilogue runs.
-template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST>
+// accumulator dump); otherwise the guarded per-quad epilogue runs.  W4: four-bit weights
+// (DequantF32 only); a 1 KiB weight block then holds two k-steps, travels through LDS packed
+// and is split into the two MFMA operands in registers.
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4>
 __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams p) {
     constexpr int NWAVES = WN * WM;
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
-    constexpr int WBLK = (BN / 32) * KS, XBLK = BM / 8;  // 1 KiB blocks per stage
+    constexpr int SPB = W4 ? 2 : 1;   // k-steps per weight block
+    constexpr int KB = KS / SPB;      // weight blocks per panel and stage
+    constexpr int WBLK = (BN / 32) * KB, XBLK = BM / 8;  // 1 KiB blocks per stage
+    static_assert(!W4 || MODE == (int)Epilogue::DequantF32, "four-bit weights dequantize only");
     static_assert(WBLK % NWAVES == 0 && XBLK % NWAVES == 0, "blocks must divide over waves");
     constexpr int WLOADS = WBLK / NWAVES, XLOADS = XBLK / NWAVES;
     constexpr int STAGE_BYTES = (WBLK + XBLK) * 1024;
@@ -134,7 +139,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     // ---- per-lane load sources ---------------------------------------------
-    // Weights: block b = wave + t*NWAVES of the stage is (panel b/KS, step b%KS); its address is
+    // Weights: block b = wave + t*NWAVES of the stage is (panel b/KB, block b%KB); its address is
     // a uniform base plus the lane's 16*lane.  Activations: a per-lane row offset plus a chunk
     // offset that is the same for all of a lane's loads of one k-block.
     const uint32_t w_lane = lane * 16u;
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         char* base = lds_raw + stage * STAGE_BYTES;
         if constexpr (t < WLOADS) {
             const uint32_t b = wave + t * NWAVES;
-            const int8_t* src = w_tile + (size_t)(b / KS) * panel_bytes + (size_t)(kb * KS + b % KS) * 1024u;
+            const int8_t* src = w_tile + (size_t)(b / KB) * panel_bytes + (size_t)(kb * KB + b % KB) * 1024u;
             load_to_lds16(src + w_lane, base + b * 1024);
         } else {
             // k-chunks past the row end pair with zero weights: clamp the address
@@ -233,7 +238,8 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                         for (int e = 0; e < 4; e++) {
                             const int r = q * 4 + e;
                             const float gs = __fmul_rn(row_scale[j], sw[e]);
-                            const float term = __fmul_rn((float)acc[i][j][r], gs);
+                            // four-bit operands carry a factor 16; the dot is exact, so is the shift
+                            const float term = __fmul_rn((float)(acc[i][j][r] >> (W4 ? 4 : 0)), gs);
                             fsum[i][j][r] = __float_as_int(
                                 __fadd_rn(__int_as_float(fsum[i][j][r]), term));
                             // groups that end inside a k-block restart from the MFMA's zero C operand
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // ---- fragment addressing ---------------------------------------------------
     // weights: block (panel, step) at 1 KiB granularity, lane slot 16*lane
     // activations: row (wave_m*TM+j)*32 + lane%32 of 128 bytes, chunk 2s + lane/32 at slot chunk ^ (row%8)
-    const uint32_t w_frag = (uint32_t)(wave_n * TN * KS) * 1024u + lane * 16u;
+    const uint32_t w_frag = (uint32_t)(wave_n * TN * KB) * 1024u + lane * 16u;
     const uint32_t x_row = WBLK * 1024u + ((uint32_t)(wave_m * TM * 32) + (lane & 31)) * 128u;
     uint32_t x_slot[KS];
 #pragma unroll
@@ -257,11 +263,19 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
 
     // fragment r of a k-step, in the order the MFMAs want them: w0, x0 .. x(TM-1), w1 .. w(TN-1)
     constexpr int READS = TN + TM, MF = TN * TM;
-    auto read_one = [&](auto r_tag, const char* stage, int s, v4i (&wf)[TN], v4i (&xf)[TM]) {
+    // Four-bit weights: the packed block of steps (s, s+1) is read at even s into wraw and split
+    // by the step that first uses it; odd s has no weight read.
+    v4i wraw[W4 ? TN : 1];
+    auto read_one = [&](auto r_tag, const char* stage, auto s_tag, v4i (&wf)[TN], v4i (&xf)[TM]) {
         constexpr int r = decltype(r_tag)::value;
+        constexpr int s = decltype(s_tag)::value;
         if constexpr (r == 0 || r > TM) {
             constexpr int i = r == 0 ? 0 : r - TM;
-            wf[i] = *reinterpret_cast<const v4i*>(stage + w_frag + (i * KS + s) * 1024);
+            if constexpr (!W4) {
+                wf[i] = *reinterpret_cast<const v4i*>(stage + w_frag + (i * KS + s) * 1024);
+            } else if constexpr ((s & 1) == 0) {
+                wraw[i] = *reinterpret_cast<const v4i*>(stage + w_frag + (i * KB + s / 2) * 1024);
+            }
         } else {
             constexpr int j = r - 1;
             xf[j] = *reinterpret_cast<const v4i*>(stage + x_row + j * 32 * 128 + x_slot[s]);
@@ -309,6 +323,15 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         static_for<MF>([&](auto m_tag) {
             constexpr int m = decltype(m_tag)::value;
             constexpr int i = m / TM, j = m % TM;
+            if constexpr (W4 && (S & 1) == 0 && j == 0) {
+                // low nibbles: this step's operand; high nibbles: the next step's (fragment
+                // buffer 1, whose last readers were issued in the previous step)
+#pragma unroll
+                for (int d = 0; d < 4; d++) {
+                    wf[0][i][d] = (wraw[i][d] << 4) & (int)0xf0f0f0f0u;
+                    wf[1][i][d] = wraw[i][d] & (int)0xf0f0f0f0u;
+                }
+            }
             if constexpr (VXHIP_PROBE_NO_MFMA) {
                 acc[i][j][0] += wf[CB][i][0] ^ xf[CB][j][1];
             } else {
@@ -322,7 +345,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             if constexpr (READ) {
                 static_for<READS>([&](auto r_tag) {
                     constexpr int r = decltype(r_tag)::value;
-                    if constexpr ((r * (MF - 1)) / READS == m) read_one(r_tag, rstage, RS, wf[NB], xf[NB]);
+                    if constexpr ((r * (MF - 1)) / READS == m) read_one(r_tag, rstage, rs_tag, wf[NB], xf[NB]);
                 });
             }
             if constexpr (NL > 0) {
@@ -347,7 +370,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         probe_real = __builtin_amdgcn_s_memrealtime();
     }
     if (nkb > 1) static_for<NLOADS>([&](auto t) { issue_one(t, 1, 1); });
-    static_for<READS>([&](auto r) { read_one(r, lds_raw, 0, wf[0], xf[0]); });
+    static_for<READS>([&](auto r) { read_one(r, lds_raw, IC<0>{}, wf[0], xf[0]); });
     auto k_block = [&](uint32_t kb, auto last_tag) {
         constexpr bool LAST = decltype(last_tag)::value;
         const int cur = kb & 1;
@@ -542,12 +565,12 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     }
 }
 
-template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST>
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
-    constexpr int LDS = 2 * ((BN / 32) * KS + BM / 8) * 1024 + BN * 16;
+    constexpr int LDS = 2 * ((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + BN * 16;
     static bool configured = false;
-    auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST>;
+    auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST, W4>;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) !=
             hipSuccess)
@@ -564,16 +587,16 @@ bool launch_one(hipStream_t s, const LinearArgs& a) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int WN, int WM, int TN, int TM, int MODE, int GK>
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool W4 = false>
 bool launch_cfg(hipStream_t s, const LinearArgs& a) {
     if constexpr (MODE != (int)Epilogue::DequantF32) {
         if ((a.n % 16u) == 0u && a.y && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u)
-            return launch_one<WN, WM, TN, TM, MODE, GK, true>(s, a);
+            return launch_one<WN, WM, TN, TM, MODE, GK, true, false>(s, a);
     }
-    return launch_one<WN, WM, TN, TM, MODE, GK, false>(s, a);
+    return launch_one<WN, WM, TN, TM, MODE, GK, false, W4>(s, a);
 }
 
-template <int MODE, int GK>
+template <int MODE, int GK, bool W4 = false>
 const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     auto forced = [&](const char* tag) { return force && strstr(force, tag) != nullptr; };
     const uint64_t big_tiles = (uint64_t)((a.n + 255) / 256) * ((a.rows + 255) / 256);
@@ -585,8 +608,8 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
             big = (uint64_t)((a.n + 127) / 128) * ((a.rows + 255) / 256) >= (uint64_t)cu_count * 3 / 4;
         // int32 tile accumulators plus f32 running sums: keep the wave tile at 64x64.  With a
         // scale group per k-step the eight-wave tile runs out of registers, so it stays with four.
-        if (big && GK > 1) return launch_cfg<2, 4, 2, 2, MODE, GK>(s, a) ? "t128x256" : nullptr;
-        return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
+        if (big && GK > 1) return launch_cfg<2, 4, 2, 2, MODE, GK, W4>(s, a) ? "t128x256" : nullptr;
+        return launch_cfg<2, 2, 2, 2, MODE, GK, W4>(s, a) ? "t128x128" : nullptr;
     } else {
         // Largest tile (channels x rows) that still gives every compute unit work; names are BNxBM.
         const auto tiles = [&](uint32_t bn, uint32_t bm) {
@@ -612,6 +635,7 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
 const char* launch_gemm_mfma(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (a.ldx < 16u || (a.ldx % 16u) != 0u || ((uintptr_t)a.x % 16u) != 0u) return nullptr;
     if ((uint64_t)a.rows * a.ldx > 0xffffffffull) return nullptr;  // 32-bit activation offsets
+    if (a.weight_bits != 8u && !(a.weight_bits == 4u && a.mode == Epilogue::DequantF32)) return nullptr;
     const char* tile = nullptr;
     static thread_local char name[96];
     const char* family = nullptr;
@@ -625,6 +649,17 @@ const char* launch_gemm_mfma(hipStream_t s, const LinearArgs& a, int cu_count, c
             family = "hip.qlinear.mfma-i8-rowscale";
             break;
         case Epilogue::DequantF32:
+            if (a.weight_bits == 4u) {
+                family = "hip.packed-linear.w4a8-mfma";
+                switch (a.group_size) {
+                    case 32: tile = dispatch_tile<(int)Epilogue::DequantF32, 1, true>(s, a, cu_count, force); break;
+                    case 64: tile = dispatch_tile<(int)Epilogue::DequantF32, 2, true>(s, a, cu_count, force); break;
+                    case 128: tile = dispatch_tile<(int)Epilogue::DequantF32, 4, true>(s, a, cu_count, force); break;
+                    case 256: tile = dispatch_tile<(int)Epilogue::DequantF32, 8, true>(s, a, cu_count, force); break;
+                    default: return nullptr;
+                }
+                break;
+            }
             family = "hip.packed-linear.a8-mfma";
             switch (a.group_size) {
                 case 32: tile = dispatch_tile<(int)Epilogue::DequantF32, 1>(s, a, cu_count, force); break;

@@ -28,6 +28,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <type_traits>
+
 // tuning probe: per-workgroup phase timestamps (100 MHz ticks) through the unused bias_row pointer
 #ifndef VXHIP_GEMV_PROBE
 #define VXHIP_GEMV_PROBE 0
@@ -49,23 +51,32 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 }
 
 // MODE: Epilogue.  GK: k-steps of 32 per scale group (1, 2, 4 or 8).  WAVES:
-// wavefronts of the workgroup, all sharing one panel.
-template <int MODE, int GK, int WAVES>
+// wavefronts of the workgroup, all sharing one panel.  W4: four-bit weights, a 1 KiB block
+// then carries two k-steps and is split into their operands in registers (three VALU
+// operations per dword), so the stream is half as long for the same K.
+template <int MODE, int GK, int WAVES, bool W4>
 __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
+    static_assert(F || !W4, "four-bit weights exist for the dequantizing epilogue only");
+    constexpr int SPB = W4 ? 2 : 1;              // k-steps per 1 KiB block
+    constexpr int UNIT = GK > SPB ? GK : SPB;    // a wave's run is a whole number of these
     uint64_t probe[4] = {0, 0, 0, 0};
     if (VXHIP_GEMV_PROBE) probe[0] = __builtin_amdgcn_s_memrealtime();
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // wave-uniform, and known to the compiler as such: the bounds of the wave's run and every
+    // branch on them are then scalar.  (That is needed, not only cheaper: an MFMA is not
+    // predicated by the EXEC mask, so a guard the compiler took for divergent and turned into
+    // EXEC masking around a lone MFMA would not guard it.)
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t panel = blockIdx.x;
     const uint32_t rows = a.rows;
 
     // this wave's run of k-steps, aligned to whole groups
     const uint32_t steps = (a.k + 31u) / 32u;
-    const uint32_t chunks = (steps + GK - 1) / GK;
+    const uint32_t chunks = (steps + UNIT - 1) / UNIT;
     const uint32_t per = (chunks + WAVES - 1) / WAVES;
-    const uint32_t t0 = min((uint32_t)wave * per * GK, steps);
-    const uint32_t t1 = min((uint32_t)(wave + 1) * per * GK, steps);
+    const uint32_t t0 = min((uint32_t)wave * per * UNIT, steps);
+    const uint32_t t1 = min((uint32_t)(wave + 1) * per * UNIT, steps);
 
     const int8_t* wp = a.w + (size_t)panel * a.ksteps * 1024u + lane * 16u;
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
@@ -77,11 +88,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     int32_t* parts = reinterpret_cast<int32_t*>(gemv_lds);
     const bool row_live = (uint32_t)(lane & 31) < rows;
 
-    v4i wbuf[kDepth], xbuf[kDepth];
+    // slot <- the block that starts at k-step t (t even for four-bit weights) and the
+    // activation chunks of its steps
+    v4i wbuf[kDepth], xbuf[kDepth][SPB];
     auto issue = [&](int slot, uint32_t t) {
-        wbuf[slot] = load_stream(wp + (size_t)t * 1024u);
-        const uint32_t chunk = min(t * 2u + half, last_chunk);
-        xbuf[slot] = *reinterpret_cast<const v4i*>(xp + chunk * 16u);
+        wbuf[slot] = load_stream(wp + (size_t)(t / SPB) * 1024u);
+#pragma unroll
+        for (int h = 0; h < SPB; h++) {
+            const uint32_t chunk = min((t + h) * 2u + half, last_chunk);
+            xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + chunk * 16u);
+        }
     };
 
     v16i acc;
@@ -131,39 +147,69 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
         if (row_live) {
 #pragma unroll
             for (int q = 0; q < 4; q++)
+                // four-bit operands carry a factor 16, which the exact dot sheds here
                 *reinterpret_cast<v4i*>(parts + ((size_t)slab * rows + (lane & 31)) * 32u + q * 8 + half * 4) =
-                    v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+                    v4i{acc[q * 4] >> (W4 ? 4 : 0), acc[q * 4 + 1] >> (W4 ? 4 : 0),
+                        acc[q * 4 + 2] >> (W4 ? 4 : 0), acc[q * 4 + 3] >> (W4 ? 4 : 0)};
         }
     };
 
+    auto stash_scales = [&]() {
+        if constexpr (F) {
 #pragma unroll
-    for (int i = 0; i < kDepth; i++)
-        if (t0 + i < t1) issue(i, t0 + i);
-    if constexpr (F) {
-#pragma unroll
-        for (int u = 0; u < SCALE_SLOTS; u++) {
-            const uint32_t e = sc_base + threadIdx.x + u * WAVES * 64;
-            if (e < a.groups * 32u) lds_scales[e] = sc[u];
-        }
-    }
-
-    for (uint32_t t = t0; t < t1; t += kDepth) {
-#pragma unroll
-        for (int i = 0; i < kDepth; i++) {
-            if (t + i < t1) {
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wbuf[i], xbuf[i], acc, 0, 0, 0);
-                if constexpr (F) {
-                    // a group closes after GK steps (t0 is group aligned) or at the row end
-                    if ((t + i + 1) % GK == 0 || t + i + 1 == t1) {
-                        park((t + i) / GK);
-#pragma unroll
-                        for (int r = 0; r < 16; r++) acc[r] = 0;
-                    }
-                }
-                if (t + i + kDepth < t1) issue(i, t + i + kDepth);
+            for (int u = 0; u < SCALE_SLOTS; u++) {
+                const uint32_t e = sc_base + threadIdx.x + u * WAVES * 64;
+                if (e < a.groups * 32u) lds_scales[e] = sc[u];
             }
         }
+    };
+    // One round: the MFMAs of the kDepth blocks that start at k-step t, each slot refilled with
+    // the block kDepth further on as soon as it has been consumed.  STEADY rounds lie wholly
+    // inside the run and so does the round after them: nothing in them is conditional, which
+    // lets the wait before each MFMA name exactly the loads it needs (a refill under a branch
+    // makes the count of outstanding loads unknown and every wait a full drain of the queue).
+    auto round = [&](uint32_t t, auto steady_tag) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+#pragma unroll
+        for (int i = 0; i < kDepth; i++) {
+#pragma unroll
+            for (int h = 0; h < SPB; h++) {
+                const uint32_t tt = t + i * SPB + h;
+                if (STEADY || tt < t1) {
+                    v4i wop = wbuf[i];
+                    if constexpr (W4) {
+#pragma unroll
+                        for (int d = 0; d < 4; d++)
+                            wop[d] = (h == 0 ? wbuf[i][d] << 4 : wbuf[i][d]) & (int)0xf0f0f0f0u;
+                    }
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, xbuf[i][h], acc, 0, 0, 0);
+                    if constexpr (F) {
+                        // a group closes after GK steps (t0 is group aligned) or at the row end
+                        if ((tt + 1) % GK == 0 || (!STEADY && tt + 1 == t1)) {
+                            park(tt / GK);
+#pragma unroll
+                            for (int r = 0; r < 16; r++) acc[r] = 0;
+                        }
+                    }
+                }
+            }
+            if (STEADY || t + (i + kDepth) * SPB < t1) issue(i, t + (i + kDepth) * SPB);
+        }
+    };
+    constexpr uint32_t ROUND = kDepth * SPB;  // k-steps per round
+    uint32_t t = t0;
+    if (t1 - t0 >= 2 * ROUND) {
+#pragma unroll
+        for (int i = 0; i < kDepth; i++) issue(i, t0 + i * SPB);
+        stash_scales();
+        for (; t + 2 * ROUND <= t1; t += ROUND) round(t, std::true_type{});
+    } else {
+#pragma unroll
+        for (int i = 0; i < kDepth; i++)
+            if (t0 + i * SPB < t1) issue(i, t0 + i * SPB);
+        stash_scales();
     }
+    for (; t < t1; t += ROUND) round(t, std::false_type{});
     if constexpr (!F) park(wave);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (VXHIP_GEMV_PROBE) probe[1] = __builtin_amdgcn_s_memrealtime();
@@ -223,9 +269,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     }
 }
 
-template <int MODE, int GK, int WAVES>
+template <int MODE, int GK, int WAVES, bool W4>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
-    auto kern = gemv_panel_kernel<MODE, GK, WAVES>;
+    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4>;
     if (lds > 64u * 1024u) {
         static bool configured = false;
         if (!configured) {
@@ -239,9 +285,11 @@ bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int MODE, int GK>
+template <int MODE, int GK, bool W4 = false>
 const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
-    const uint32_t steps = (a.k + 31u) / 32u;
+    // blocks of the stream per panel, and the units a wave's run is made of
+    constexpr uint32_t SPB = W4 ? 2 : 1, UNIT = GK > SPB ? GK : SPB;
+    const uint32_t steps = ((a.k + 31u) / 32u + SPB - 1u) / SPB;  // 1 KiB blocks per panel
     // Measured at K=4096, N=14336: 4 blocks in flight per wave and 16 blocks per wave (two
     // workgroups of 8 waves resident per CU) stream fastest; more waves or deeper queues cost
     // occupancy, fewer leave the memory system short of requests.
@@ -249,7 +297,7 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
     // Few panels (small N) leave most of the device idle and every wave latency bound on its
     // own short run: then split K further, down to one scale group per wave, until about 4096
     // waves are in flight.
-    const uint32_t panels = (a.n + 31u) / 32u, chunks = (steps + GK - 1) / GK;
+    const uint32_t panels = (a.n + 31u) / 32u, chunks = ((a.k + 31u) / 32u + UNIT - 1) / UNIT;
     for (int more = waves * 2; more <= 16 && (uint32_t)more <= chunks && panels * (uint32_t)more <= 4096u; more *= 2)
         waves = more;
     if (force && strstr(force, "w16")) waves = 16;
@@ -261,10 +309,10 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
     // the MFMA GEMM takes shapes whose group dots or scales do not fit
     if (lds > 156u * 1024u) return nullptr;
     bool ok = false;
-    if (waves == 16) ok = launch_panel<MODE, GK, 16>(s, a, lds);
-    else if (waves == 8) ok = launch_panel<MODE, GK, 8>(s, a, lds);
-    else if (waves == 4) ok = launch_panel<MODE, GK, 4>(s, a, lds);
-    else ok = launch_panel<MODE, GK, 2>(s, a, lds);
+    if (waves == 16) ok = launch_panel<MODE, GK, 16, W4>(s, a, lds);
+    else if (waves == 8) ok = launch_panel<MODE, GK, 8, W4>(s, a, lds);
+    else if (waves == 4) ok = launch_panel<MODE, GK, 4, W4>(s, a, lds);
+    else ok = launch_panel<MODE, GK, 2, W4>(s, a, lds);
     return !ok ? nullptr : waves == 16 ? "w16" : waves == 8 ? "w8" : waves == 4 ? "w4" : "w2";
 }
 
@@ -275,6 +323,7 @@ const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count,
     if (a.rows == 0u || a.rows > kMaxGemvRows || a.ldx < 16u || (a.ldx % 16u) != 0u ||
         ((uintptr_t)a.x % 16u) != 0u)
         return nullptr;
+    if (a.weight_bits != 8u && !(a.weight_bits == 4u && a.mode == Epilogue::DequantF32)) return nullptr;
     const char* kind = nullptr;
     const char* family = nullptr;
     switch (a.mode) {
@@ -287,6 +336,17 @@ const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count,
             kind = launch_mode<(int)Epilogue::RequantRow, 1>(s, a, force);
             break;
         case Epilogue::DequantF32:
+            if (a.weight_bits == 4u) {
+                family = "hip.packed-linear.w4a8-gemv-mfma";
+                switch (a.group_size) {
+                    case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1, true>(s, a, force); break;
+                    case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2, true>(s, a, force); break;
+                    case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4, true>(s, a, force); break;
+                    case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8, true>(s, a, force); break;
+                    default: return nullptr;
+                }
+                break;
+            }
             family = "hip.packed-linear.a8-gemv-mfma";
             switch (a.group_size) {
                 case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1>(s, a, force); break;

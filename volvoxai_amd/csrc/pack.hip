@@ -35,6 +35,36 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(
     *reinterpret_cast<uint4*>(out + slot * 16u) = v;
 }
 
+// Four-bit form: one thread produces one 16-byte lane slot, i.e. 16 weights of each of the
+// block's two steps.  Source codes are offset by 8 (packed_linear_ops.inc:476-477); code ^ 8
+// is the same value as a 4-bit two's complement number.
+__global__ __launch_bounds__(256) void pack_nibble_kernel(
+        const uint32_t* __restrict__ raw, uint32_t row_words, uint32_t n, uint32_t k,
+        uint32_t panels, uint32_t kblocks, uint8_t* __restrict__ out) {
+    const size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)panels * kblocks * 64u;
+    if (slot >= total) return;
+    const uint32_t lane = (uint32_t)(slot & 63u);
+    const size_t block = slot >> 6;
+    const uint32_t pair = (uint32_t)(block % kblocks);
+    const uint32_t panel = (uint32_t)(block / kblocks);
+    const uint32_t row = panel * 32u + (lane & 31u);
+    const uint32_t k0 = pair * 64u + (lane >> 5) * 16u;
+    uint32_t words[4] = {0u, 0u, 0u, 0u};
+    if (row < n) {
+        const uint32_t* src = raw + (size_t)row * row_words;
+        auto value = [&](uint32_t kk) -> uint32_t {
+            // padding is the value zero
+            return kk < k ? (((src[kk >> 3] >> ((kk & 7u) * 4u)) & 15u) ^ 8u) : 0u;
+        };
+        for (uint32_t j = 0; j < 16u; j++) {
+            const uint32_t b = value(k0 + j) | (value(k0 + 32u + j) << 4);
+            words[j >> 2] |= b << ((j & 3u) * 8u);
+        }
+    }
+    *reinterpret_cast<uint4*>(out + slot * 16u) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
 // One wavefront per output channel: sum of signed bytes and max |w - zp|.
 __global__ __launch_bounds__(256) void weight_row_stats_kernel(
         const uint8_t* __restrict__ raw, size_t row_stride, uint32_t n, uint32_t k, uint32_t flip,
@@ -72,6 +102,22 @@ VxHipStatus pack_weight(hipStream_t stream, const uint8_t* raw_dev, size_t row_s
     const unsigned blocks = (unsigned)((slots + 255u) / 256u);
     hipLaunchKernelGGL(pack_weight_kernel, dim3(blocks), dim3(256), 0, stream, raw_dev, row_stride,
                        n, k, flip ? 1u : 0u, out->panels, out->ksteps, (uint8_t*)out->data);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus pack_weight_nibbles(hipStream_t stream, const uint32_t* raw_dev, uint32_t row_words,
+                                uint32_t n, uint32_t k, PackedWeight* out) {
+    out->n = n;
+    out->k = k;
+    out->bits = 4;
+    out->panels = ((n + kPanelRows - 1) / kPanelRows + kPanelPad - 1) / kPanelPad * kPanelPad;
+    const uint32_t steps = ((k + kStepK - 1) / kStepK + kStepPad - 1) / kStepPad * kStepPad;
+    out->ksteps = steps / 2u;
+    VXHIP_TRY(hipMalloc((void**)&out->data, out->bytes()));
+    const size_t slots = (size_t)out->panels * out->ksteps * 64u;
+    hipLaunchKernelGGL(pack_nibble_kernel, dim3((unsigned)((slots + 255u) / 256u)), dim3(256), 0, stream,
+                       raw_dev, row_words, n, k, out->panels, out->ksteps, (uint8_t*)out->data);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

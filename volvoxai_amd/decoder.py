@@ -56,6 +56,18 @@ def pack_w8_words(w: np.ndarray) -> np.ndarray:
     return codes.view("<u4").reshape(n, words)
 
 
+def pack_w4_words(w: np.ndarray) -> np.ndarray:
+    """int8 [n, k] with values -8..7 -> W4 words [n, vx_packed_words(k, 4)]: code = w + 8,
+    element 8i+j in nibble j of word i, absent elements as the zero code 8
+    (native/src/kernels/packed_linear_ops.inc:246-248, 476-477)."""
+    n, k = w.shape
+    words = (k // 32) * 4 + ((k % 32) * 4 + 31) // 32
+    codes = np.full((n, words * 8), 8, np.uint8)
+    codes[:, :k] = (w.astype(np.int16) + 8).astype(np.uint8) & 15
+    pairs = codes[:, 0::2] | (codes[:, 1::2] << 4)
+    return np.ascontiguousarray(pairs).view("<u4").reshape(n, words)
+
+
 def init_weights(cfg: DecoderConfig, seed: int) -> dict:
     """Random-init weights of the architecture: int8 uniform +-127 with per-channel scales
     ~U(0.002, 0.01) for every linear, f32 embedding and norm gains."""
