@@ -245,6 +245,19 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     pl.close()
 
 
+def test_packed_w4_one_shot_entry(oracle):
+    """The vx_llm_forward_f32-shaped HOST entry with groups=4, and groups=0, which the reference
+    reads as 4 (packed_linear_ops.inc:1547); widths it does not run are declined."""
+    import volvoxai_amd as vx
+    c = cases.packed_case(6, 200, 9, 64, 21, special_rows=True)
+    words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], 9, 64, bits=4)
+    for groups in (4, 0):
+        st, y = vx.packed_linear_f32(c["x"], words, c["scales"], c["bias"], 200, 9, 64, groups=groups)
+        assert st == 0 and same_f32(y, want)
+    assert vx.packed_linear_f32(c["x"], words, c["scales"], c["bias"], 200, 9, 64, groups=3)[0] == -1
+
+
 def test_random_shape_sweep_packed_w4(ctx, oracle):
     """Thirty seeded W4 shapes: ragged K (partial last word, block and group), every group size,
     rows on both sides of the GEMV/GEMM boundary."""

@@ -267,8 +267,14 @@ def test_packed_package_refusals(registered, tmp_path):
     g, w = packed_package(tmp_path / "a", c["x"].shape, words, c["scales"], c["bias"], 32)
     for arithmetic in ("f32", "f16", "f32_fast", "dynamic_i4"):
         assert inspect(registered, g, w, arithmetic)[0] == -7  # only DYNAMIC_I8 is this arithmetic
-    g, w = packed_package(tmp_path / "b", c["x"].shape, words, c["scales"], c["bias"], 32, bits=4)
+    g, w = packed_package(tmp_path / "b", c["x"].shape, words, c["scales"], c["bias"], 32, bits=3)
     assert inspect(registered, g, w, "dynamic_i8")[0] == -7
+    # four-bit weights are offered, with their own word count: W8 words under weight_bits 4 are malformed
+    g, w = packed_package(tmp_path / "b4", c["x"].shape, words, c["scales"], c["bias"], 32, bits=4)
+    assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+    w4 = Oracle().pack_w4_words(cases.four_bit(c["w"]))
+    g, w = packed_package(tmp_path / "b4ok", c["x"].shape, w4, c["scales"], c["bias"], 32, bits=4)
+    assert inspect(registered, g, w, "dynamic_i8")[:4] == (0, 96, 5, 1)
     g, w = packed_package(tmp_path / "c", c["x"].shape, words, c["scales"], c["bias"], 48)
     assert inspect(registered, g, w, "dynamic_i8")[0] == -5
     g, w = packed_package(tmp_path / "d", c["x"].shape, words[:, :-1], c["scales"], c["bias"], 32)
@@ -394,6 +400,19 @@ def test_packed_linear_package_matches_oracle(registered, oracle, tmp_path, rows
     # the same package under another arithmetic is refused before anything is allocated
     r2, _ = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", n, arithmetic="f32")
     assert r2.status == -7 and r2.failed_stage == 3 and r2.writes == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,k,n,group", [(3, 96, 5, 32), (1, 4096, 512, 128), (40, 1000, 264, 64)])
+def test_packed_linear_w4_package_matches_oracle(registered, oracle, tmp_path, rows, k, n, group):
+    c = cases.packed_case(rows, k, n, group, rows + k)
+    words = oracle.pack_w4_words(cases.four_bit(c["w"]))
+    g, w = packed_package(tmp_path / "p4", c["x"].shape, words, c["scales"], c["bias"], group, bits=4)
+    r, y = run(registered, g, w, c["x"], "x", "f32", "logits", "f32", n, arithmetic="dynamic_i8")
+    assert r.status == 0, r.message
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, bits=4)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
+    assert b"hip.packed-linear" in r.execute_route
 
 
 @pytest.mark.gpu

@@ -4,7 +4,7 @@
  * The provider compiles single-node W8A8 packages:
  *   - one QLinear / QGemm / QMatMul node in the volvox-affine-safetensors/v1
  *     representation (docs/w8a8-safetensors.md:13-59, validation list :158-175);
- *   - one PackedLinear node with weight_bits 8 under DYNAMIC_I8 packed
+ *   - one PackedLinear node with weight_bits 8 or 4 under DYNAMIC_I8 packed
  *     arithmetic (node form: native/tests/test_packed_arithmetic.inc:35-37).
  * Anything else is refused with BACKEND_UNSUPPORTED before a compiled instance
  * exists, which is what shape_domain.support = FULL promises
@@ -58,6 +58,7 @@ typedef struct PackagePlan {
     const float* group_scales;
     const float* bias_f32;
     uint32_t group_size;
+    uint32_t weight_bits;
     /* mapped files */
     VxstFile** files;
     size_t file_count;
@@ -346,9 +347,9 @@ static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedAri
         !bits->is_integer || !weight_name || !scale_name)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s' lacks weight, scale or parameters",
                       plan->node_id);
-    if (bits->integer != 8)
-        return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "PackedLinear node '%s': only weight_bits 8 is offered",
-                      plan->node_id);
+    if (bits->integer != 8 && bits->integer != 4)
+        return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
+                      "PackedLinear node '%s': weight_bits 8 and 4 are offered", plan->node_id);
     if (group->integer != 32 && group->integer != 64 && group->integer != 128 && group->integer != 256)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s': group_size must be 32, 64, 128 or 256",
                       plan->node_id);
@@ -356,11 +357,13 @@ static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedAri
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s' needs float32 input and output",
                       plan->node_id);
     plan->group_size = (uint32_t)group->integer;
-    const int64_t words = ((int64_t)plan->d_in + 3) / 4;
+    plan->weight_bits = (uint32_t)bits->integer;
+    /* vx_packed_words (src/kernels/packed_linear_ops.inc:246-248) */
+    const int64_t words = ((int64_t)plan->d_in / 32) * bits->integer + (((int64_t)plan->d_in % 32) * bits->integer + 31) / 32;
     const int64_t groups = ((int64_t)plan->d_in + plan->group_size - 1) / plan->group_size;
     if (find_tensor(plan, weight_name, &weight) != 1 || (strcmp(weight.dtype, "I32") && strcmp(weight.dtype, "U32")) ||
         weight.rank != 2 || weight.shape[0] != (int64_t)plan->d_out || weight.shape[1] != words)
-        return refuse(failure, VX_STATUS_INVALID_GRAPH, "packed weight '%s' is not I32 [d_out, ceil(d_in/4)]",
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "packed weight '%s' is not I32 [d_out, words(d_in, weight_bits)]",
                       weight_name);
     if (find_tensor(plan, scale_name, &scale) != 1 || strcmp(scale.dtype, "F32") || scale.rank != 2 ||
         scale.shape[0] != (int64_t)plan->d_out || scale.shape[1] != groups)
@@ -629,7 +632,7 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.qlinear");
     } else {
         status = (VxStatus)vxhip_packed_linear_create(plan.packed_words, plan.group_scales, plan.bias_f32, plan.d_in,
-                                                      plan.d_out, plan.group_size, 8, &compiled->packed);
+                                                      plan.d_out, plan.group_size, plan.weight_bits, &compiled->packed);
         snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.packed-linear");
     }
     plan_release(&plan);
