@@ -311,8 +311,9 @@ def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
             "decode_linear_variant": step_variant, "prefill_linear_variant": prefill_variant,
             "weight_bytes_read_per_step": weight_bytes,
             "decode_hbm_GBs": weight_bytes / (decode_s / (new_tokens - 1)) / 1e9,
-            "glue": "PyTorch-ROCm f32 ops (RMSNorm, RoPE, GQA attention over a KV cache, SwiGLU); one HIP graph per "
-                    "decode step"}
+            "glue": "HIP kernels of the same library (embedding gather, residual+RMSNorm+prepare, RoPE+KV append, "
+                    "GQA attention, SwiGLU+prepare, argmax+advance); torch SDPA for the prompt's attention only; "
+                    "one HIP graph per decode step"}
 
 
 def main():

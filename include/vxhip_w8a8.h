@@ -125,6 +125,23 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* context, const float* q_dev,
                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
                                 uint32_t max_seq, float* out_dev);
 
+/* Embedding lookup (src/kernels/embedding.inc:5-16): out [count, d_model] row i
+ * = table [vocab, d_model] row tokens_dev[i] (int32 ids as in the reference).
+ * An id outside the table gives a zero row and raises fault bit 2 of
+ * vxhip_context_fault_flags (the reference reads out of bounds there). */
+VxHipStatus vxhip_embedding_gather_f32(VxHipContext* context, const int32_t* tokens_dev,
+                                       const float* table_dev, uint32_t count,
+                                       uint32_t d_model, uint32_t vocab, float* out_dev);
+/* ArgMax over the last axis of input [rows, n] (argmax_axis_typed with inner 1,
+ * src/kernels/reduction_argmax.inc:211-235): strictly-greater scan, so the first
+ * index wins ties, a NaN is never chosen and a NaN in element 0 keeps index 0.
+ * indices_dev int32 [rows].  advance_dev (optional, no counterpart in the
+ * reference) are up to 64 int64 counters incremented by one in the same launch:
+ * a greedy decode loop keeps its position on the device that way. */
+VxHipStatus vxhip_argmax_rows_f32(VxHipContext* context, const float* input_dev,
+                                  uint32_t rows, uint32_t n, int32_t* indices_dev,
+                                  int64_t* advance_dev, uint32_t advance_count);
+
 /* Measurement aid with no counterpart in the reference: runs a register-only
  * v_mfma_i32_32x32x32_i8 loop (16 accumulators per wave, one wave per SIMD,
  * `rounds` x 16 MFMAs per wave) and reports the int8 rate it reached, the

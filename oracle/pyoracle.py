@@ -227,6 +227,21 @@ class Oracle:
         assert st == 0
         return out
 
+    def embedding(self, tokens, table):
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        out = np.zeros((tokens.size, table.shape[1]), dtype=np.float32)
+        self.lib.vxo_embedding_f32.restype = None
+        self.lib.vxo_embedding_f32(tokens.ctypes.data_as(C.c_void_p), _ptr(table, _f32p), _ptr(out, _f32p),
+                                   C.c_uint32(tokens.size), C.c_uint32(table.shape[1]))
+        return out
+
+    def argmax_rows(self, x):
+        out = np.zeros(x.shape[0], dtype=np.int32)
+        self.lib.vxo_argmax_rows_f32.restype = None
+        self.lib.vxo_argmax_rows_f32(_ptr(x, _f32p), C.c_uint32(x.shape[0]), C.c_uint32(x.shape[1]),
+                                     _ptr(out, _i32p))
+        return out
+
     def ptq_pack_bias(self, b, s_in, w_scales):
         out = np.zeros(b.shape, dtype=np.int32)
         st = self.lib.vxo_ptq_pack_bias_i32(_ptr(b, _f32p), b.size, _f(s_in),
@@ -373,6 +388,22 @@ class Reference:
         a.y_elements[0] = y.size
         st = self.lib.vx_llm_forward_f32(C.byref(a))
         return int(st), y
+
+    def embedding(self, tokens, table):
+        """embedding_f32 (src/kernels/embedding.inc:5-16); pointers travel as integers."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        out = np.zeros((tokens.size, table.shape[1]), dtype=np.float32)
+        self.lib.embedding_f32.restype = None
+        self.lib.embedding_f32(C.c_size_t(tokens.ctypes.data), C.c_size_t(table.ctypes.data),
+                               C.c_size_t(out.ctypes.data), C.c_int(tokens.size), C.c_int(table.shape[1]))
+        return out
+
+    def argmax_rows(self, x):
+        """argmax_f32 (src/kernels/reduction_argmax.inc:237-240): indices come back as f32."""
+        out = np.zeros(x.shape[0], dtype=np.float32)
+        self.lib.argmax_f32.restype = None
+        self.lib.argmax_f32(_ptr(x, _f32p), _ptr(out, _f32p), C.c_int(x.shape[0]), C.c_int(x.shape[1]))
+        return out.astype(np.int32)
 
     def ptq_pack_bias(self, b, s_in, w_scales):
         out = np.zeros(b.shape, dtype=np.int32)

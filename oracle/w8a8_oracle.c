@@ -453,3 +453,29 @@ void vxo_pack_w4_words(const int8_t* weight, uint32_t n, uint32_t k,
         }
     }
 }
+
+/* ---- decoder glue either side of the linears --------------------------- */
+
+void vxo_embedding_f32(const int32_t* tokens, const float* table, float* out,
+                       uint32_t count, uint32_t d_model) {
+    for (uint32_t i = 0; i < count; i++)
+        memcpy(out + (uint64_t)i * d_model,
+               table + (uint64_t)tokens[i] * d_model, sizeof(float) * d_model);
+}
+
+void vxo_argmax_rows_f32(const float* input, uint32_t rows, uint32_t n,
+                         int32_t* indices) {
+    for (uint32_t r = 0; r < rows; r++) {
+        const float* x = input + (uint64_t)r * n;
+        double best = x[0];
+        int32_t best_index = 0;
+        for (uint32_t i = 1; i < n; i++) {
+            const double v = x[i];
+            if (v > best) { /* strict: first index on ties, NaN never greater */
+                best = v;
+                best_index = (int32_t)i;
+            }
+        }
+        indices[r] = best_index;
+    }
+}

@@ -142,6 +142,13 @@ void vxo_pack_w8_words(const int8_t* weight, uint32_t n, uint32_t k,
 void vxo_pack_w4_words(const int8_t* weight, uint32_t n, uint32_t k,
                        uint32_t* packed);
 
+/* src/kernels/embedding.inc:5-16 (ids must lie inside the table) */
+void vxo_embedding_f32(const int32_t* tokens, const float* table, float* out,
+                       uint32_t count, uint32_t d_model);
+/* argmax_axis_typed with inner == 1 (src/kernels/reduction_argmax.inc:211-235) */
+void vxo_argmax_rows_f32(const float* input, uint32_t rows, uint32_t n,
+                         int32_t* indices);
+
 #ifdef __cplusplus
 }
 #endif

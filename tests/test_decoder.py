@@ -11,6 +11,14 @@ def small_config():
                          max_seq=32)
 
 
+def test_w4_word_packing_matches_the_oracle(oracle):
+    from volvoxai_amd.decoder import pack_w4_words
+    rng = np.random.default_rng(0)
+    for n, k in [(3, 75), (5, 64), (2, 1), (4, 1000)]:
+        w = rng.integers(-8, 8, (n, k)).astype(np.int8)
+        assert (pack_w4_words(w) == oracle.pack_w4_words(w)).all()
+
+
 def test_word_packing_matches_the_oracle(oracle):
     from volvoxai_amd.decoder import pack_w8_words
     rng = np.random.default_rng(3)
@@ -149,3 +157,37 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
     assert np.abs(first_logits - want_logits[0]).max() <= 2e-4 * scale
     assert (got == want_tokens).all(), (got, want_tokens)
     assert "a8-" in variant
+
+
+@pytest.mark.gpu
+def test_embedding_gather_and_argmax_kernels(ctx, oracle):
+    import torch
+    from volvoxai_amd import w8a8
+    from test_oracle import glue_argmax_rows
+    rng = np.random.default_rng(4)
+    for rows, n in [(12, 37), (32, 32000), (5, 4096), (3, 1023), (2, 1)]:
+        x = glue_argmax_rows() if n == 37 else rng.normal(0, 1, (rows, n)).astype(np.float32)
+        if n == 32000:
+            x[4, 31999] = x[4, 17] = 40.0      # tie across threads and waves -> first
+            x[5, 0] = np.nan
+        counters = torch.tensor([7, 100], dtype=torch.int64, device="cuda")
+        got = w8a8.argmax_rows(ctx, torch.from_numpy(x).cuda(), advance=counters)
+        ctx.synchronize()
+        assert (got.cpu().numpy() == oracle.argmax_rows(x)).all(), (rows, n)
+        assert counters.tolist() == [8, 101]
+    for d in (24, 1024, 7):
+        table = rng.normal(0, 1, (50, d)).astype(np.float32)
+        tokens = np.array([[0, 49], [7, 7], [13, 2]], np.int32)
+        out = w8a8.embedding_gather(ctx, torch.from_numpy(tokens).cuda(), torch.from_numpy(table).cuda())
+        ctx.synchronize()
+        assert (out.cpu().numpy() == oracle.embedding(tokens.reshape(-1), table)).all()
+    assert ctx.fault_flags() == 0
+    # ids outside the table: zero rows and a sticky fault bit (on a context of its own)
+    import volvoxai_amd as vx
+    own = vx.Context(0, torch.cuda.current_stream())
+    bad = w8a8.embedding_gather(own, torch.tensor([3, 50, -1], dtype=torch.int32, device="cuda"),
+                                torch.from_numpy(table).cuda())
+    own.synchronize()
+    bad = bad.cpu().numpy()
+    assert (bad[0] == table[3]).all() and not bad[1:].any() and own.fault_flags() & 2
+    own.close()

@@ -243,6 +243,35 @@ def test_live_reference_packed_and_bias_rule(oracle, reference):
     assert st1 == st2 == 0 and (q1 == q2).all()
 
 
+def glue_argmax_rows():
+    """Rows that separate the scan's rules: ties, a NaN at the front, in the middle, infinities."""
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, (12, 37)).astype(np.float32)
+    x[1, :] = 0.5                              # all equal -> 0
+    x[2, 5] = x[2, 20] = 9.0                   # tie -> first
+    x[3, 0] = np.nan                           # NaN in element 0 keeps 0
+    x[4, 7] = np.nan; x[4, 30] = 8.0           # NaN elsewhere is skipped
+    x[5, :] = -np.inf                          # all -inf -> 0
+    x[6, 3] = np.inf; x[6, 4] = np.inf
+    x[7, :] = np.nan
+    x[8, 0] = -0.0; x[8, 1:] = -1.0; x[8, 9] = 0.0   # +0 does not beat -0
+    x[9, 36] = 50.0                            # last element
+    return x
+
+
+def test_live_reference_embedding_and_argmax(oracle, reference):
+    x = glue_argmax_rows()
+    got = oracle.argmax_rows(x)
+    assert (got == reference.argmax_rows(x)).all()
+    assert got[:10].tolist() == [int(np.argmax(x[0])), 0, 5, 0, 30, 0, 3, 0, 0, 36]
+    big = np.random.default_rng(2).normal(0, 1, (3, 32000)).astype(np.float32)
+    assert (oracle.argmax_rows(big) == np.argmax(big, axis=1)).all()
+    table = np.random.default_rng(3).normal(0, 1, (50, 24)).astype(np.float32)
+    tokens = np.array([0, 49, 7, 7, 13], np.int32)
+    e = oracle.embedding(tokens, table)
+    assert (e == reference.embedding(tokens, table)).all() and (e == table[tokens]).all()
+
+
 # ---- what the mathematics fixes ---------------------------------------------------
 
 def test_accumulator_is_the_integer_gemm(oracle):

@@ -51,6 +51,7 @@ constexpr uint32_t kMaxGemvRows = 32;  // the MFMA operand has 32 row slots
 
 enum FaultBits : uint32_t {
     kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive
+    kFaultBadToken = 2u,        // an embedding lookup was asked for a row outside the table
 };
 
 }  // namespace vxhip

@@ -255,6 +255,78 @@ bool device_ready(VxHipContext* ctx) {
     return ctx && hipSetDevice(ctx->device) == hipSuccess;
 }
 
+// Embedding lookup (embedding.inc:5-16): out[i] = table[tokens[i]], one workgroup per token.
+// The reference reads whatever an id outside the table points at; here such a row is zeros and
+// a fault bit is raised.
+__global__ __launch_bounds__(256) void embedding_gather_kernel(const int32_t* __restrict__ tokens,
+                                                               const float* __restrict__ table,
+                                                               float* __restrict__ out, uint32_t d, uint32_t vocab,
+                                                               uint32_t* fault) {
+    const int32_t id = tokens[blockIdx.x];
+    const bool ok = id >= 0 && (uint32_t)id < vocab;
+    const float* src = table + (size_t)(ok ? id : 0) * d;
+    float* dst = out + (size_t)blockIdx.x * d;
+    if (!ok && threadIdx.x == 0) atomicOr(fault, (uint32_t)kFaultBadToken);
+    if ((d & 3u) == 0u) {
+        for (uint32_t j = threadIdx.x * 4u; j < d; j += blockDim.x * 4u) {
+            const float4 v = ok ? *reinterpret_cast<const float4*>(src + j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4*>(dst + j) = v;
+        }
+    } else {
+        for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) dst[j] = ok ? src[j] : 0.0f;
+    }
+}
+
+// ArgMax over the last axis (reduction_argmax.inc:211-235): a scan in index order that replaces
+// the best only on a strictly greater value, so ties keep the first index, a NaN is never
+// chosen, and a NaN in element 0 wins the row (nothing compares greater than it).  A candidate
+// (v, i) beats (bv, bi) if v > bv, or v == bv and i < bi, which gives the same answer in any
+// evaluation order.  One workgroup per row; `advance` (optional) are counters the first
+// workgroup increments, e.g. the decode position.
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restrict__ x, uint32_t n,
+                                                           int32_t* __restrict__ out, int64_t* advance,
+                                                           uint32_t advance_count) {
+    const float* row = x + (size_t)blockIdx.x * n;
+    float bv = -INFINITY;
+    uint32_t bi = 0xffffffffu;
+    auto offer = [&](float v, uint32_t i) {
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    };
+    if ((n & 3u) == 0u && ((uintptr_t)row & 15u) == 0u) {
+        for (uint32_t j = threadIdx.x * 4u; j < n; j += blockDim.x * 4u) {
+            const float4 v = *reinterpret_cast<const float4*>(row + j);
+            offer(v.x, j);
+            offer(v.y, j + 1u);
+            offer(v.z, j + 2u);
+            offer(v.w, j + 3u);
+        }
+    } else {
+        for (uint32_t j = threadIdx.x; j < n; j += blockDim.x) offer(row[j], j);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_down(bv, off, 64);
+        const uint32_t oi = __shfl_down(bi, off, 64);
+        offer(ov, oi);
+    }
+    __shared__ float wave_v[16];
+    __shared__ uint32_t wave_i[16];
+    const uint32_t wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    if ((threadIdx.x & 63u) == 0u) {
+        wave_v[wave] = bv;
+        wave_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < waves; w++) offer(wave_v[w], wave_i[w]);
+        const float first = row[0];
+        out[blockIdx.x] = (first != first || bi == 0xffffffffu) ? 0 : (int32_t)bi;
+    }
+    if (blockIdx.x == 0 && advance && threadIdx.x < advance_count) advance[threadIdx.x] += 1;
+}
+
 }  // namespace
 }  // namespace vxhip
 
@@ -357,6 +429,35 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
     else if (together == 2u) VXHIP_LAUNCH_ATTENTION(2);
     else VXHIP_LAUNCH_ATTENTION(1);
 #undef VXHIP_LAUNCH_ATTENTION
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_embedding_gather_f32(VxHipContext* ctx, const int32_t* tokens_dev, const float* table_dev,
+                                       uint32_t count, uint32_t d_model, uint32_t vocab, float* out_dev) {
+    if (!ctx || !tokens_dev || !table_dev || !out_dev || !d_model || !vocab) {
+        set_error("embedding_gather_f32: null argument or empty table");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!count) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    hipLaunchKernelGGL(embedding_gather_kernel, dim3(count), dim3(256), 0, ctx->stream, tokens_dev, table_dev,
+                       out_dev, d_model, vocab, ctx->fault_dev);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_argmax_rows_f32(VxHipContext* ctx, const float* input_dev, uint32_t rows, uint32_t n,
+                                  int32_t* indices_dev, int64_t* advance_dev, uint32_t advance_count) {
+    if (!ctx || !input_dev || !indices_dev || !n || (advance_count && !advance_dev) || advance_count > 64u) {
+        set_error("argmax_rows_f32: null argument, empty axis or more than 64 counters");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    const uint32_t block = n >= 4096u ? 1024u : n >= 1024u ? 256u : 64u;
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(block), 0, ctx->stream, input_dev, n, indices_dev,
+                       advance_dev, advance_count);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

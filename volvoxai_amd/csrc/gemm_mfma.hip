@@ -316,7 +316,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // of them a step or two later measured slower, they then land too late.)
     auto step = [&](auto s_tag, auto read_tag, auto rs_tag, const char* rstage, auto nl_tag, uint32_t load_kb,
                     int load_stage, uint32_t kb) {
-        constexpr int S = decltype(s_tag)::value, RS = decltype(rs_tag)::value;
+        constexpr int S = decltype(s_tag)::value;
         constexpr bool READ = decltype(read_tag)::value;
         constexpr int NL = decltype(nl_tag)::value;
         constexpr int CB = S & 1, NB = CB ^ 1;

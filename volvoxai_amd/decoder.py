@@ -136,7 +136,8 @@ class W8A8Decoder:
         self.k_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
         self.v_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
         # state of the decode loop, on the device so a captured step advances by itself
-        self.tokens = torch.zeros(rows, dtype=torch.int64, device=dev)
+        # (int32 ids on the fused path, as the reference's embedding takes them)
+        self.tokens = torch.zeros(rows, dtype=torch.int32 if fused else torch.int64, device=dev)
         self.position = torch.zeros(1, dtype=torch.int64, device=dev)
         self.history = torch.zeros((cfg.max_seq, rows), dtype=torch.int64, device=dev)
         self.slots = torch.arange(cfg.max_seq, device=dev)
@@ -187,11 +188,12 @@ class W8A8Decoder:
         a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
         return self._linear_a8(L["down"], a8, sc)
 
-    def _forward_fused(self, tokens, positions):
-        """tokens int64 [rows, t] -> logits of the last position and their argmax."""
+    def _forward_fused(self, tokens, positions, next_tokens=None, advance=None):
+        """tokens int32 [rows, t] -> logits of the last position and their argmax (int32, written
+        to `next_tokens` when given; `advance` counters are incremented by the same launch)."""
         cfg = self.cfg
         rows, t = tokens.shape
-        x2 = self.embedding[tokens].reshape(rows * t, cfg.hidden)
+        x2 = vx.embedding_gather(self.ctx, tokens.reshape(-1), self.embedding)
         delta = None
         for li in range(cfg.layers):
             delta = self._layer_fused(li, x2, delta, positions, rows, t)
@@ -200,7 +202,7 @@ class W8A8Decoder:
             delta = delta.reshape(rows, t, cfg.hidden)[:, -1, :].contiguous()
         a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, delta, self.gain_f, cfg.eps)
         logits = self._linear_a8(self.lm_head, a8, sc)
-        return logits, logits.argmax(dim=-1)
+        return logits, vx.argmax_rows(self.ctx, logits, out=next_tokens, advance=advance)
 
     def _rmsnorm(self, x, gain):
         xd = x.double()
@@ -253,7 +255,7 @@ class W8A8Decoder:
             slots = self.slots[:t]
             visible = self.slots[None, :] <= slots[:, None]
             if self.fused:
-                self.last_logits, nxt = self._forward_fused(prompt, slots)
+                self.last_logits, nxt = self._forward_fused(prompt.to(torch.int32).contiguous(), slots)
             else:
                 x = self.embedding[prompt]
                 for li in range(cfg.layers):
@@ -269,15 +271,17 @@ class W8A8Decoder:
     def _step(self):
         torch, cfg = self.torch, self.cfg
         pos = self.position
+        if self.fused:
+            # the argmax launch writes the next ids over the current ones and advances the position
+            self.last_logits, nxt = self._forward_fused(self.tokens[:, None], pos, next_tokens=self.tokens,
+                                                        advance=self.position)
+            return nxt
         visible = self.slots[None, :] <= pos[:, None]
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        if self.fused:
-            self.last_logits, nxt = self._forward_fused(self.tokens[:, None], pos)
-        else:
-            x = self.embedding[self.tokens][:, None, :]
-            for li in range(cfg.layers):
-                x = self._layer(li, x, cos, sin, pos, visible)
-            self.last_logits, nxt = self._head(x[:, 0, :])
+        x = self.embedding[self.tokens][:, None, :]
+        for li in range(cfg.layers):
+            x = self._layer(li, x, cos, sin, pos, visible)
+        self.last_logits, nxt = self._head(x[:, 0, :])
         self.tokens.copy_(nxt)
         self.position.add_(1)
         return nxt

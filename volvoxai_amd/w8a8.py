@@ -263,6 +263,31 @@ def gqa_attention(ctx: Context, q, k_cache, v_cache, positions):
     return out
 
 
+def embedding_gather(ctx: Context, tokens_i32, table, out=None):
+    """out[i] = table[tokens_i32[i]]; tokens int32 of any shape, table [vocab, d] f32."""
+    import torch
+    count = tokens_i32.numel()
+    vocab, d = table.shape
+    if out is None:
+        out = torch.empty((count, d), dtype=torch.float32, device=table.device)
+    _check(library().vxhip_embedding_gather_f32(ctx._h, _dp(tokens_i32), _dp(table), count, d, vocab, _dp(out)),
+           "vxhip_embedding_gather_f32")
+    return out
+
+
+def argmax_rows(ctx: Context, x, out=None, advance=None):
+    """First index of the row maximum of x [rows, n] as int32 [rows]; `advance` (int64 tensor of up
+    to 64 counters) is incremented by one in the same launch."""
+    import torch
+    rows, n = x.shape
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=x.device)
+    _check(library().vxhip_argmax_rows_f32(ctx._h, _dp(x), rows, n, _dp(out), _dp(advance),
+                                           0 if advance is None else advance.numel()),
+           "vxhip_argmax_rows_f32")
+    return out
+
+
 def packed_prepare_i8(ctx: Context, x):
     import torch
     rows, k = x.shape
