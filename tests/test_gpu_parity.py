@@ -167,15 +167,16 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
                              c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128", "mfma-i8.t256x256", "mfma-i8.t256x128",
-                      "mfma-i8.t128x64", "mfma-i8.t256x128w4"):
+        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128s2", "mfma-i8.t256x256", "mfma-i8.t256x128",
+                      "mfma-i8.t128x64s2", "mfma-i8.t256x128w4", "mfma-i8.t128x128s4", "mfma-i8.t128x64s4",
+                      "mfma-i8.t64x64"):
             vx.force_variant(force)
             (ok, y), variant = run_resident_qlinear(vx, ctx, c)
             assert ok == 1 and (y == want).all(), variant
             seen.add(variant)
     finally:
         vx.force_variant(None)
-    assert len(seen) == 7, seen
+    assert len(seen) == 10, seen
 
 
 @pytest.mark.parametrize("group", [32, 64, 128, 256])
@@ -189,7 +190,8 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256"):
+        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+                      "a8-mfma.t64x64"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -197,8 +199,8 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    # one scale group per k-step has no eight-wave tile: both GEMM requests run the same one
-    assert len(seen) == (3 if group == 32 else 4), seen
+    # one scale group per k-step has no eight-wave tile: that request runs the four-wave one
+    assert len(seen) == (5 if group == 32 else 6), seen
     pl.close()
 
 
@@ -233,7 +235,8 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256"):
+        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+                      "a8-mfma.t64x64"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -241,7 +244,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert all("w4a8" in v for v in seen) and len(seen) == (3 if group == 32 else 4), seen
+    assert all("w4a8" in v for v in seen) and len(seen) == (5 if group == 32 else 6), seen
     pl.close()
 
 

@@ -98,9 +98,16 @@ constexpr int KS = 4;  // k-steps of 32 per stage: 128 bytes of k, one cache lin
 // straight-line requantizing epilogue (needs n % 16 == 0, a byte output and no
 // accumulator dump); otherwise the guarded per-quad epilogue runs.  W4: four-bit weights
 // (DequantF32 only); a 1 KiB weight block then holds two k-steps, travels through LDS packed
-// and is split into the two MFMA operands in registers.
-template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4>
+// and is split into the two MFMA operands in registers.  NS: LDS stages (a power of two).  Two
+// are all that fits beside a 256x256 tile; a launch of few small tiles is bound by the latency
+// of one k-block's loads per iteration instead, and with four stages three k-blocks are in
+// flight while one is consumed.
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4, int NS>
 __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams p) {
+    static_assert(NS >= 2 && (NS & (NS - 1)) == 0, "stage count must be a power of two");
+    // (the dequantizing epilogue loads group scales inside the loop; the compiler's wait for them
+    // would, with loads completing in order, pull in every k-block requested before them)
+    static_assert(NS == 2 || MODE != (int)Epilogue::DequantF32, "deep staging is for the requantizing modes");
     constexpr int NWAVES = WN * WM;
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
     constexpr int SPB = W4 ? 2 : 1;   // k-steps per weight block
@@ -292,10 +299,12 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // The instruction order inside a k-step is written out and fenced (sched_barrier) rather
     // than left to the scheduler: MFMA m is preceded by the fragment reads and operand loads
     // whose turn it is, so LDS reads, global->LDS loads and MFMAs issue evenly mixed.
-    static_for<NLOADS>([&](auto t) { issue_one(t, 0, 0); });
+    static_for<NS - 1>([&](auto b_tag) {
+        static_for<NLOADS>([&](auto t) { issue_one(t, decltype(b_tag)::value, decltype(b_tag)::value); });
+    });
     // per-channel epilogue constants of this tile (structure of arrays, so a lane's four
     // consecutive channels are one ds_read_b128 each), computed while the first stage is in flight
-    float* lds_f0 = reinterpret_cast<float*>(lds_raw + 2 * STAGE_BYTES);
+    float* lds_f0 = reinterpret_cast<float*>(lds_raw + NS * STAGE_BYTES);
     int32_t* lds_cb = reinterpret_cast<int32_t*>(lds_f0 + BN);
     float* lds_bo = reinterpret_cast<float*>(lds_cb + BN);
     int32_t* lds_zw = reinterpret_cast<int32_t*>(lds_bo + BN);
@@ -363,17 +372,20 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         }
     };
 
-    wait_vmcnt<0>();
+    // k-block 0 has landed; the NS-2 younger ones may still be on their way
+    wait_vmcnt<(NS - 2) * NLOADS>();
     wg_barrier();
     if (VXHIP_PROBE_CLOCK) {
         probe_cycles = __builtin_readcyclecounter();
         probe_real = __builtin_amdgcn_s_memrealtime();
     }
-    if (nkb > 1) static_for<NLOADS>([&](auto t) { issue_one(t, 1, 1); });
+    // (unconditional: a block past the end is clamped to the last one, and the waits below
+    // count on every block having been requested)
+    static_for<NLOADS>([&](auto t) { issue_one(t, NS - 1, NS - 1); });
     static_for<READS>([&](auto r) { read_one(r, lds_raw, IC<0>{}, wf[0], xf[0]); });
     auto k_block = [&](uint32_t kb, auto last_tag) {
         constexpr bool LAST = decltype(last_tag)::value;
-        const int cur = kb & 1;
+        const int cur = kb & (NS - 1);
         const char* stage = lds_raw + cur * STAGE_BYTES;
         static_for<KS - 1>([&](auto s_tag) {
             constexpr int S = decltype(s_tag)::value;
@@ -381,10 +393,11 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         });
         if constexpr (!LAST) {
             wait_lgkm0();     // my reads of this stage have landed in registers
-            if (!VXHIP_PROBE_NO_VMWAIT) wait_vmcnt<0>();  // my loads of the next stage have landed
+            // my loads of the next k-block have landed (the NS-2 blocks after it need not have)
+            if (!VXHIP_PROBE_NO_VMWAIT) wait_vmcnt<(NS - 2) * NLOADS>();
             wg_barrier();
-            step(IC<KS - 1>{}, std::true_type{}, IC<0>{}, lds_raw + (cur ^ 1) * STAGE_BYTES, IC<NLOADS>{},
-                 kb + 2, cur, kb);
+            step(IC<KS - 1>{}, std::true_type{}, IC<0>{}, lds_raw + ((cur + 1) & (NS - 1)) * STAGE_BYTES,
+                 IC<NLOADS>{}, kb + NS, cur, kb);
         } else {
             step(IC<KS - 1>{}, std::false_type{}, IC<0>{}, stage, IC<0>{}, 0u, 0, kb);
         }
@@ -565,12 +578,14 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     }
 }
 
-template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4>
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4, int NS>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
-    constexpr int LDS = 2 * ((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + BN * 16;
+    // the stages and, behind them, the per-channel epilogue constants
+    constexpr int LDS = NS * ((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + BN * 16;
+    static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
     static bool configured = false;
-    auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST, W4>;
+    auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST, W4, NS>;
     if (!configured) {
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) !=
             hipSuccess)
@@ -587,45 +602,62 @@ bool launch_one(hipStream_t s, const LinearArgs& a) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int WN, int WM, int TN, int TM, int MODE, int GK, bool W4 = false>
+template <int WN, int WM, int TN, int TM, int MODE, int GK, bool W4 = false, int NS = 2>
 bool launch_cfg(hipStream_t s, const LinearArgs& a) {
     if constexpr (MODE != (int)Epilogue::DequantF32) {
         if ((a.n % 16u) == 0u && a.y && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u)
-            return launch_one<WN, WM, TN, TM, MODE, GK, true, false>(s, a);
+            return launch_one<WN, WM, TN, TM, MODE, GK, true, false, NS>(s, a);
     }
-    return launch_one<WN, WM, TN, TM, MODE, GK, false, W4>(s, a);
+    return launch_one<WN, WM, TN, TM, MODE, GK, false, W4, NS>(s, a);
 }
 
 template <int MODE, int GK, bool W4 = false>
 const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     auto forced = [&](const char* tag) { return force && strstr(force, tag) != nullptr; };
-    const uint64_t big_tiles = (uint64_t)((a.n + 255) / 256) * ((a.rows + 255) / 256);
-    bool big = big_tiles >= (uint64_t)cu_count * 3 / 4;
-    if (forced("t256x256")) big = true;
-    if (forced("t128x128")) big = false;
     if constexpr (MODE == (int)Epilogue::DequantF32) {
-        if (!forced("t256x256") && !forced("t128x128"))
-            big = (uint64_t)((a.n + 127) / 128) * ((a.rows + 255) / 256) >= (uint64_t)cu_count * 3 / 4;
-        // int32 tile accumulators plus f32 running sums: keep the wave tile at 64x64.  With a
-        // scale group per k-step the eight-wave tile runs out of registers, so it stays with four.
-        if (big && GK > 1) return launch_cfg<2, 4, 2, 2, MODE, GK, W4>(s, a) ? "t128x256" : nullptr;
-        return launch_cfg<2, 2, 2, 2, MODE, GK, W4>(s, a) ? "t128x128" : nullptr;
+        // int32 tile accumulators plus f32 running sums: the wave tile is at most 64x64, and with
+        // a scale group per k-step the eight-wave tile runs out of registers.  A wave folds a
+        // group (four VALU operations per output) strictly after that group's MFMAs, so its time
+        // per k-block grows with its tile: few rows or few channels take narrower tiles, which
+        // also puts more workgroups on the device.
+        const auto tiles = [&](uint32_t bn, uint32_t bm) {
+            return (uint64_t)((a.n + bn - 1) / bn) * ((a.rows + bm - 1) / bm);
+        };
+        const uint64_t enough = (uint64_t)cu_count * 3 / 4;
+        int pick = a.rows <= 64u ? 3 : tiles(128, 256) >= enough && GK > 1 ? 0 : tiles(128, 128) >= enough ? 1
+                   : tiles(64, 128) >= enough ? 2 : 3;
+        if (forced("t256x256")) pick = GK > 1 ? 0 : 1;
+        if (forced("t128x128")) pick = 1;
+        if (forced("t64x128")) pick = 2;
+        if (forced("t64x64")) pick = 3;
+        if (pick == 0) return launch_cfg<2, 4, 2, 2, MODE, GK, W4>(s, a) ? "t128x256" : nullptr;
+        if (pick == 1) return launch_cfg<2, 2, 2, 2, MODE, GK, W4>(s, a) ? "t128x128" : nullptr;
+        if (pick == 2) return launch_cfg<2, 2, 1, 2, MODE, GK, W4>(s, a) ? "t64x128" : nullptr;
+        return launch_cfg<2, 2, 1, 1, MODE, GK, W4>(s, a) ? "t64x64" : nullptr;
     } else {
         // Largest tile (channels x rows) that still gives every compute unit work; names are BNxBM.
         const auto tiles = [&](uint32_t bn, uint32_t bm) {
             return (uint64_t)((a.n + bn - 1) / bn) * ((a.rows + bm - 1) / bm);
         };
         const uint64_t enough = (uint64_t)cu_count * 3 / 4;
-        int pick = tiles(256, 256) >= enough ? 0 : tiles(256, 128) >= enough ? 1 : tiles(128, 128) >= enough ? 2 : 3;
+        int pick = tiles(256, 256) >= enough ? 0 : tiles(256, 128) >= enough ? 1 : tiles(128, 128) >= enough ? 2
+                   : tiles(128, 64) >= enough ? 3 : 4;
         if (forced("t256x256")) pick = 0;
         if (forced("t256x128")) pick = 1;
         if (forced("t128x128")) pick = 2;
         if (forced("t128x64")) pick = 3;
+        if (forced("t64x64")) pick = 4;
         if (pick == 0 && forced("w4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256w4" : nullptr;
         if (pick == 0) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
         if (pick == 1 && forced("w4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128w4" : nullptr;
         if (pick == 1) return launch_cfg<2, 4, 4, 1, MODE, GK>(s, a) ? "t256x128" : nullptr;
+        // one round of tiles or less: the k loop waits on each k-block's loads in turn; four
+        // stages keep three k-blocks in flight (the small tiles leave the LDS for them)
+        const bool deep = forced("s4") || (!forced("s2") && tiles(128, pick == 2 ? 128 : 64) <= (uint64_t)cu_count * 3 / 2);
+        if (pick == 4) return launch_cfg<2, 2, 1, 1, MODE, GK, false, 4>(s, a) ? "t64x64s4" : nullptr;
+        if (pick == 2 && deep) return launch_cfg<2, 2, 2, 2, MODE, GK, false, 4>(s, a) ? "t128x128s4" : nullptr;
         if (pick == 2) return launch_cfg<2, 2, 2, 2, MODE, GK>(s, a) ? "t128x128" : nullptr;
+        if (deep) return launch_cfg<2, 2, 2, 1, MODE, GK, false, 4>(s, a) ? "t128x64s4" : nullptr;
         return launch_cfg<2, 2, 2, 1, MODE, GK>(s, a) ? "t128x64" : nullptr;
     }
 }
