@@ -142,9 +142,11 @@ def packed_package(tmp, x_shape, words, scales, bias, group, bits=8, mutate=None
 
 
 def inspect(host, graph, weights, arithmetic="f32"):
+    """weights: one SafeTensors path, or a list of them (a sharded package)."""
     _, provider, _ = host
-    paths = (C.c_char_p * 1)(str(weights).encode())
-    src = ModelSource(C.sizeof(ModelSource), str(graph).encode(), paths, 1, None, 0)
+    files = list(weights) if isinstance(weights, (list, tuple)) else [weights]
+    paths = (C.c_char_p * len(files))(*[str(f).encode() for f in files])
+    src = ModelSource(C.sizeof(ModelSource), str(graph).encode(), paths, len(files), None, 0)
     d_in, d_out, packed = C.c_uint32(0), C.c_uint32(0), C.c_int32(0)
     msg = C.create_string_buffer(256)
     st = provider.volvoxai_hip_gfx950_inspect_package(C.byref(src), ARITH[arithmetic], C.byref(d_in), C.byref(d_out),
@@ -281,6 +283,23 @@ def test_packed_package_refusals(registered, tmp_path):
     assert inspect(registered, g, w, "dynamic_i8")[0] == -5
     g, w = packed_package(tmp_path / "e", c["x"].shape, words, c["scales"][:, :-1], c["bias"], 32)
     assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+
+
+def test_sharded_weight_files(registered, tmp_path):
+    """The model source may name several SafeTensors files (docs/w8a8-safetensors.md:84-108): a tensor
+    is looked up across all of them and must exist exactly once."""
+    from oracle.pyoracle import Oracle
+    c = cases.packed_case(3, 96, 5, 32, 1)
+    words = Oracle().pack_w8_words(c["w"])
+    g, w = packed_package(tmp_path / "one", c["x"].shape, words, c["scales"], c["bias"], 32)
+    a, b = tmp_path / "one" / "a.safetensors", tmp_path / "one" / "b.safetensors"
+    write_safetensors(a, {"w#as_i32": words.astype(np.uint32)})
+    write_safetensors(b, {"s": c["scales"].astype(np.float32), "b": c["bias"].astype(np.float32)})
+    assert inspect(registered, g, [a, b], "dynamic_i8")[:4] == (0, 96, 5, 1)
+    assert inspect(registered, g, [b, a], "dynamic_i8")[:4] == (0, 96, 5, 1)
+    assert inspect(registered, g, [a], "dynamic_i8")[0] == -5          # scales and bias are missing
+    assert inspect(registered, g, [a, b, w], "dynamic_i8")[0] == -5    # every tensor now exists twice
+    assert inspect(registered, g, [a, tmp_path / "absent.safetensors"], "dynamic_i8")[0] == -4
 
 
 def test_malformed_documents_are_refused(registered, tmp_path):
