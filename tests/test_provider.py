@@ -302,6 +302,24 @@ def test_sharded_weight_files(registered, tmp_path):
     assert inspect(registered, g, [a, tmp_path / "absent.safetensors"], "dynamic_i8")[0] == -4
 
 
+def test_readers_survive_mutated_documents_under_sanitizers(tmp_path):
+    """The JSON and SafeTensors readers, built with AddressSanitizer and UBSan (host code only), fed every
+    truncation and thousands of byte mutations of a valid package: each is parsed or refused, none read
+    out of bounds (the program aborts on the first finding)."""
+    import subprocess
+    from oracle.pyoracle import Oracle
+    here = Path(__file__).parent / "provider_host"
+    built = subprocess.run(["make", "-C", str(here), "parser_mutations"], capture_output=True, text=True)
+    if built.returncode != 0:
+        pytest.skip("sanitizer build unavailable: " + built.stderr[-200:])
+    c = cases.packed_case(3, 96, 5, 32, 1)
+    g, w = packed_package(tmp_path / "p", c["x"].shape, Oracle().pack_w8_words(c["w"]), c["scales"], c["bias"], 32)
+    r = subprocess.run([str(here / "parser_mutations"), str(g), str(w), str(tmp_path / "mutant.bin")],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "parsed" in r.stdout and "refused" in r.stdout
+
+
 def test_malformed_documents_are_refused(registered, tmp_path):
     k = KAT
     g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
