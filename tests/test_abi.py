@@ -22,7 +22,8 @@ def test_kernel_variant_table_shape():
     rows = vx.kernel_variants()
     ids = {r["id"] for r in rows}
     assert {"hip.qlinear.mfma-i8", "hip.qlinear.gemv-mfma", "hip.packed-linear.a8-mfma",
-            "hip.packed-linear.a8-gemv-mfma"} <= ids
+            "hip.packed-linear.a8-gemv-mfma", "hip.packed-linear.w4a8-mfma",
+            "hip.packed-linear.w4a8-gemv-mfma"} <= ids
     for r in rows:
         assert r["backend"] == 0 and r["id"].startswith("hip.") and r["priority"] > 0
         assert r["operator_kind"] in (1002, 1005, 1007, 1036)

@@ -216,6 +216,8 @@ def test_packed_w4_reference_vectors(ctx, oracle, entry):
     ctx.synchronize()
     y = host(y)
     assert st == 0 and "w4a8" in ctx.last_variant
+    family = ctx.last_variant.rsplit(".", 1)[0]  # the id without the tile or wave suffix
+    assert family in {r["id"] for r in vx.kernel_variants()}, ctx.last_variant
     if not np.isnan(y).any():
         assert sha(y) == entry["expected"]["sha256"], f"f32 bits differ from the reference ({ctx.last_variant})"
     _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=4)
