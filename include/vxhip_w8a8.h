@@ -234,12 +234,13 @@ int vxhip_qlinear_i8u8(const void* input, const void* weight,
 
 /* packed_words [n, vx_packed_words(k, bits)] I32 words
  * (src/kernels/packed_linear_ops.inc:246-248): weight_bits 8 = offset-binary
- * bytes (code - 128), four per word; weight_bits 4 = nibbles (code - 8),
- * eight per word, lowest first (:474-480).  scales [n, ceil(k/G)], bias [n] or
+ * bytes (code - 128), four per word; weight_bits 4 / 2 = nibbles (code - 8) /
+ * bit pairs (code - 2), lowest first; weight_bits 3 = a dense bitstream over
+ * the row (code - 4) (:249-254, 472-480).  scales [n, ceil(k/G)], bias [n] or
  * NULL, group_size in {32,64,128,256} (docs/packed-linear-design.md:24-32;
  * physical shapes as checked at src/runtime/engine_runtime_llm.inc:94-99).
  * Other widths return VXHIP_BACKEND_UNSUPPORTED.  HOST pointers, not retained.
- * Four-bit weights stay four-bit in device memory. */
+ * Widths below 8 are held as four-bit weights in device memory. */
 VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words,
                                        const float* scales, const float* bias,
                                        uint32_t k, uint32_t n,
@@ -259,7 +260,7 @@ VxHipStatus vxhip_packed_prepare_i8(VxHipContext* context,
                                     uint32_t k, int8_t* prepared_dev,
                                     float* row_scales_dev);
 
-/* vx_packed_linear_forward with normalize==8, groups==8 or 4
+/* vx_packed_linear_forward with normalize==8, groups in {8, 4, 3, 2}
  * (src/kernels/packed_linear_ops.inc:1545-1621) on resident f32 rows.
  * Returns 0 on success, -1 on a rejected descriptor (reference convention). */
 int vxhip_packed_linear_forward_f32(VxHipContext* context,
@@ -283,8 +284,8 @@ int vxhip_packed_linear_forward_a8(VxHipContext* context,
  * (src/kernels/llm_ops.h:38-53) is not reproduced here; this one-shot HOST
  * entry takes the same values as plain arguments: x=input f32 [rows,k],
  * packed_weight, scale, bias (optional), y=out [rows,n], key_dim=k,
- * value_dim=n, rate=group_size, groups=weight_bits (8 or 4; 0 means 4 as in
- * the reference), normalize=8.
+ * value_dim=n, rate=group_size, groups=weight_bits (8, 4, 3 or 2; 0 means 4
+ * as in the reference), normalize=8.
  * Returns 0 / -1 like vx_llm_forward_f32 (src/kernels/llm_ops.inc:41-56). */
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
                             const float* scale, const float* bias,

@@ -188,6 +188,15 @@ class Oracle:
             _ptr(y, _f32p), _ptr(acc, _i32p), rows, k, n, group, bits)
         return st, y, acc
 
+    def pack_low_bit_words(self, w, bits):
+        n, k = w.shape
+        words = (k // 32) * bits + ((k % 32) * bits + 31) // 32
+        out = np.zeros((n, words), dtype=np.uint32)
+        self.lib.vxo_pack_low_bit_words.restype = None
+        self.lib.vxo_pack_low_bit_words(_ptr(w, _i8p), C.c_uint32(n), C.c_uint32(k), C.c_uint32(bits),
+                                        _ptr(out, _u32p))
+        return out
+
     def pack_w4_words(self, w):
         n, k = w.shape
         words = (k // 32) * 4 + ((k % 32) * 4 + 31) // 32

@@ -226,11 +226,21 @@ static int group_size_ok(uint32_t g) {
     return g == 32u || g == 64u || g == 128u || g == 256u;
 }
 
-/* src/kernels/packed_linear_ops.inc:474-480: W8 codes are offset by 128, W4
- * codes by 8; both little-endian within their I32 word. */
+/* src/kernels/packed_linear_ops.inc:472-480: codes are offset by half their
+ * range (W8 128, W4 8, W2 2), little-endian within their I32 word; W3 is a
+ * dense bitstream over the row (:249-254), offset 4. */
 static int32_t packed_code(const uint32_t* row_words, uint32_t k, uint32_t bits) {
     if (bits == 4u)
         return (int32_t)((row_words[k / 8u] >> ((k % 8u) * 4u)) & 15u) - 8;
+    if (bits == 2u)
+        return (int32_t)((row_words[k / 16u] >> ((k % 16u) * 2u)) & 3u) - 2;
+    if (bits == 3u) {
+        const uint64_t bit = (uint64_t)k * 3u;
+        const uint32_t shift = (uint32_t)(bit % 32u);
+        uint32_t value = row_words[bit / 32u] >> shift;
+        if (shift > 29u) value |= row_words[bit / 32u + 1u] << (32u - shift);
+        return (int32_t)(value & 7u) - 4;
+    }
     return (int32_t)((row_words[k / 4u] >> ((k % 4u) * 8u)) & 255u) - 128;
 }
 
@@ -247,7 +257,7 @@ int vxo_packed_linear_a8_bits(const int8_t* activation, const float* row_scales,
                               uint32_t group_size, uint32_t weight_bits) {
     if (!activation || !row_scales || !packed || !scales || !output || !k ||
         !n || !group_size_ok(group_size) ||
-        (weight_bits != 4u && weight_bits != 8u))
+        (weight_bits != 2u && weight_bits != 3u && weight_bits != 4u && weight_bits != 8u))
         return -1;
     const uint32_t words = packed_words(k, weight_bits);
     const uint32_t groups = (k + group_size - 1u) / group_size;
@@ -477,5 +487,25 @@ void vxo_argmax_rows_f32(const float* input, uint32_t rows, uint32_t n,
             }
         }
         indices[r] = best_index;
+    }
+}
+
+void vxo_pack_low_bit_words(const int8_t* weight, uint32_t n, uint32_t k,
+                            uint32_t bits, uint32_t* packed) {
+    const uint32_t words = packed_words(k, bits);
+    const uint32_t offset = 1u << (bits - 1u), mask = (1u << bits) - 1u;
+    for (uint32_t o = 0; o < n; o++) {
+        uint32_t* row = packed + (uint64_t)o * words;
+        for (uint32_t w = 0; w < words; w++) row[w] = 0;
+        /* every code slot of the row's words, absent elements as the code of zero */
+        const uint32_t slots = (uint32_t)(((uint64_t)words * 32u) / bits);
+        for (uint32_t j = 0; j < slots; j++) {
+            const uint32_t code =
+                (j < k ? (uint32_t)((int32_t)weight[(uint64_t)o * k + j] + (int32_t)offset) : offset) & mask;
+            const uint64_t bit = (uint64_t)j * bits;
+            const uint32_t shift = (uint32_t)(bit % 32u);
+            row[bit / 32u] |= code << shift;
+            if (shift + bits > 32u) row[bit / 32u + 1u] |= code >> (32u - shift);
+        }
     }
 }

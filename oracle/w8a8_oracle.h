@@ -100,10 +100,10 @@ int vxo_packed_linear_a8(const int8_t* activation, const float* row_scales,
                          int32_t* accumulators, uint64_t rows, uint32_t k,
                          uint32_t n, uint32_t group_size);
 
-/* The same two routines for 4-bit weights as well (weight_bits 4 or 8):
+/* The same two routines for every packed width (weight_bits 2, 3, 4 or 8):
  * I32 words [n, vx_packed_words(k, bits)] (src/kernels/packed_linear_ops.inc:
- * 246-248), W4 codes offset by 8, eight per word, lowest nibble first (integer
- * dot :474-477; single-row body :1493-1504). */
+ * 246-248); codes offset by half their range, lowest bits first, W3 a dense
+ * bitstream (:249-254; integer dot :472-480; single-row body :1493-1504). */
 int vxo_packed_linear_forward_bits(const float* input, const uint32_t* packed,
                                    const float* scales, const float* bias,
                                    float* output, uint64_t rows, uint32_t k,
@@ -148,6 +148,11 @@ void vxo_embedding_f32(const int32_t* tokens, const float* table, float* out,
 /* argmax_axis_typed with inner == 1 (src/kernels/reduction_argmax.inc:211-235) */
 void vxo_argmax_rows_f32(const float* input, uint32_t rows, uint32_t n,
                          int32_t* indices);
+
+/* Codes of any packed width below 8 (values in [-2^(bits-1), 2^(bits-1)) stored
+ * + 2^(bits-1)), the layout packed_code() reads; the tail holds the zero code. */
+void vxo_pack_low_bit_words(const int8_t* weight, uint32_t n, uint32_t k,
+                            uint32_t bits, uint32_t* packed);
 
 #ifdef __cplusplus
 }

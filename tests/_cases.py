@@ -157,10 +157,14 @@ def packed_case(rows, k, n, group, seed, with_bias=True, special_rows=False):
     return dict(x=x, w=w, scales=scales, bias=bias, group=group, k=k, n=n)
 
 
+def low_bit(w, bits):
+    """int8 weights reduced to the value range of a `bits`-wide code, -2^(bits-1) .. 2^(bits-1)-1
+    (arithmetic shift, so signs and the rough distribution are kept)."""
+    return (w.astype(np.int8) >> (8 - bits)).astype(np.int8)
+
+
 def four_bit(w):
-    """int8 weights reduced to the W4 value range -8..7 (arithmetic shift, so signs and the
-    rough distribution are kept)."""
-    return (w.astype(np.int8) >> 4).astype(np.int8)
+    return low_bit(w, 4)
 
 
 def decode_case(rows, k, n, group, seed):

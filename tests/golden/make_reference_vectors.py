@@ -89,7 +89,7 @@ def main():
     orc = Oracle()
     out = {"_comment": "Outputs of the reference's C kernels on the seeded inputs of tests/_cases.py; "
                        "written by tests/golden/make_reference_vectors.py.",
-           "qlinear": [], "rowscale": [], "packed": [], "packed_w4": []}
+           "qlinear": [], "rowscale": [], "packed": [], "packed_w4": [], "packed_w3": [], "packed_w2": []}
     for kind, params in QLINEAR_CASES:
         c = build_case(kind, params)
         args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
@@ -124,6 +124,11 @@ def main():
         st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=4)
         assert st == 0
         out["packed_w4"].append({"params": params, "expected": digest(y)})
+        for bits in (3, 2):
+            words = orc.pack_low_bit_words(cases.low_bit(c["w"], bits), bits)
+            st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
+            assert st == 0
+            out[f"packed_w{bits}"].append({"params": params, "expected": digest(y)})
     path = Path(__file__).with_name("reference_vectors.json")
     path.write_text(json.dumps(out, indent=1) + "\n")
     print("wrote", path, path.stat().st_size, "bytes")

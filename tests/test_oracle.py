@@ -163,6 +163,35 @@ def test_packed_w4_matches_reference_vectors(oracle, entry):
     check_digest(y, entry["expected"])
 
 
+@pytest.mark.parametrize("bits", [3, 2])
+def test_packed_low_bit_matches_reference_vectors(oracle, bits):
+    for entry in VECTORS[f"packed_w{bits}"]:
+        c = cases.packed_case(**entry["params"])
+        words = oracle.pack_low_bit_words(cases.low_bit(c["w"], bits), bits)
+        st, y = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
+        assert st == 0
+        check_digest(y, entry["expected"])
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4])
+def test_packed_low_bit_codes_read_back(oracle, bits):
+    """Code j of a row sits at bit j*bits of the row's words (a three-bit code may straddle two
+    words); a one-hot activation reads exactly that weight back."""
+    k, n = 75, 2
+    rng = np.random.default_rng(bits)
+    w = rng.integers(-(1 << (bits - 1)), 1 << (bits - 1), (n, k)).astype(np.int8)
+    words = oracle.pack_low_bit_words(w, bits)
+    assert words.shape == (n, (k // 32) * bits + ((k % 32) * bits + 31) // 32)
+    stream = int.from_bytes(words[1].tobytes(), "little")
+    for j in (0, 9, 10, 20, 21, 31, 32, 74):
+        assert ((stream >> (j * bits)) & ((1 << bits) - 1)) - (1 << (bits - 1)) == int(w[1, j])
+    scales = np.ones((n, 3), np.float32)
+    for j in (0, 10, 21, 42, 74):
+        a8 = np.zeros((1, k), np.int8); a8[0, j] = 1
+        st, y, _ = oracle.packed_linear_a8(a8, np.ones(1, np.float32), words, scales, None, n, 32, bits=bits)
+        assert st == 0 and y[0].tolist() == w[:, j].astype(np.float32).tolist()
+
+
 def test_packed_w4_codes_and_group_dots(oracle):
     """Nibble j of word j//8 holds value+8, lowest nibble first; a one-hot activation reads one
     weight back, and the group dots are the plain integer products."""
@@ -228,13 +257,14 @@ def test_live_reference_packed_and_bias_rule(oracle, reference):
         nan = np.isnan(b[1])
         assert (np.isnan(a[1]) == nan).all()
         assert (a[1].view(np.uint32)[~nan] == b[1].view(np.uint32)[~nan]).all()
-        w4 = oracle.pack_w4_words(cases.four_bit(c["w"]))
-        a = oracle.packed_linear(x, w4, c["scales"], c["bias"], c["n"], c["group"], bits=4)
-        b = reference.packed_linear(x, w4, c["scales"], c["bias"], c["n"], c["group"], bits=4)
-        assert a[0] == b[0] == 0
-        nan = np.isnan(b[1])
-        assert (np.isnan(a[1]) == nan).all()
-        assert (a[1].view(np.uint32)[~nan] == b[1].view(np.uint32)[~nan]).all()
+        for bits in (4, 3, 2):
+            lw = oracle.pack_low_bit_words(cases.low_bit(c["w"], bits), bits)
+            a = oracle.packed_linear(x, lw, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
+            b = reference.packed_linear(x, lw, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
+            assert a[0] == b[0] == 0
+            nan = np.isnan(b[1])
+            assert (np.isnan(a[1]) == nan).all()
+            assert (a[1].view(np.uint32)[~nan] == b[1].view(np.uint32)[~nan]).all()
     rng = np.random.default_rng(9)
     b = rng.normal(0, 0.3, 64).astype(np.float32)
     sw = rng.uniform(0.002, 0.02, 64).astype(np.float32)

@@ -269,7 +269,7 @@ def test_packed_package_refusals(registered, tmp_path):
     g, w = packed_package(tmp_path / "a", c["x"].shape, words, c["scales"], c["bias"], 32)
     for arithmetic in ("f32", "f16", "f32_fast", "dynamic_i4"):
         assert inspect(registered, g, w, arithmetic)[0] == -7  # only DYNAMIC_I8 is this arithmetic
-    g, w = packed_package(tmp_path / "b", c["x"].shape, words, c["scales"], c["bias"], 32, bits=3)
+    g, w = packed_package(tmp_path / "b", c["x"].shape, words, c["scales"], c["bias"], 32, bits=5)
     assert inspect(registered, g, w, "dynamic_i8")[0] == -7
     # four-bit weights are offered, with their own word count: W8 words under weight_bits 4 are malformed
     g, w = packed_package(tmp_path / "b4", c["x"].shape, words, c["scales"], c["bias"], 32, bits=4)

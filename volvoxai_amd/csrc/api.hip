@@ -558,8 +558,8 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
         set_error("packed_linear_create: null tensor or zero extent");
         return VXHIP_INVALID_ARGUMENT;
     }
-    if (weight_bits != 8u && weight_bits != 4u) {
-        set_error("packed_linear_create: 8- and 4-bit weights run on this backend (got %u)", weight_bits);
+    if (weight_bits != 8u && weight_bits != 4u && weight_bits != 3u && weight_bits != 2u) {
+        set_error("packed_linear_create: weight_bits must be 2, 3, 4 or 8 (got %u)", weight_bits);
         return VXHIP_BACKEND_UNSUPPORTED;
     }
     if (group_size != 32u && group_size != 64u && group_size != 128u && group_size != 256u) {
@@ -609,8 +609,8 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
     TRY_OR_FAIL(hipMemcpy(pl->scales_t, st.data(), st.size() * sizeof(float), hipMemcpyHostToDevice));
     TRY_OR_FAIL(hipMemcpy(pl->bias, hb.data(), n_pad * sizeof(float), hipMemcpyHostToDevice));
     // offset-binary codes: value = code - 128, i.e. the byte with its top bit flipped
-    VxHipStatus s2 = weight_bits == 4u
-                         ? pack_weight_nibbles(nullptr, (const uint32_t*)raw, words, n, k, &pl->w)
+    VxHipStatus s2 = weight_bits != 8u
+                         ? pack_weight_nibbles(nullptr, (const uint32_t*)raw, words, n, k, weight_bits, &pl->w)
                          : pack_weight(nullptr, raw, (size_t)words * 4u, n, k, true, &pl->w);
     if (s2 != VXHIP_OK) return fail(s2);
     TRY_OR_FAIL(hipDeviceSynchronize());
@@ -749,8 +749,8 @@ int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, c
         rows > 0x7fffffffull)
         return -1;
     const uint32_t bits = groups ? (uint32_t)groups : 4u;
-    if ((bits != 8u && bits != 4u) || normalize != 8) {
-        set_error("packed_linear_f32: this backend runs weight_bits 8 and 4 under DYNAMIC_I8 only");
+    if ((bits != 8u && bits != 4u && bits != 3u && bits != 2u) || normalize != 8) {
+        set_error("packed_linear_f32: this backend runs weight_bits 2, 3, 4 and 8 under DYNAMIC_I8 only");
         return -1;
     }
     VxHipContext* ctx = default_context();

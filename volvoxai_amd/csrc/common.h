@@ -107,9 +107,10 @@ VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes);
 // flip: XOR 0x80 (U8 or offset-binary source -> signed byte).
 VxHipStatus pack_weight(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
                         uint32_t n, uint32_t k, bool flip, PackedWeight* out);
-// raw_dev: [n] rows of `row_words` I32 words of offset-by-8 nibbles, lowest nibble first.
+// raw_dev: [n] rows of `row_words` I32 words of 2-, 3- or 4-bit codes, offset by half their range,
+// lowest bits first; all are stored as four-bit weights (out->bits == 4).
 VxHipStatus pack_weight_nibbles(hipStream_t stream, const uint32_t* raw_dev, uint32_t row_words,
-                                uint32_t n, uint32_t k, PackedWeight* out);
+                                uint32_t n, uint32_t k, uint32_t bits, PackedWeight* out);
 VxHipStatus weight_row_stats(hipStream_t stream, const uint8_t* raw_dev, size_t row_stride,
                              uint32_t n, uint32_t k, bool flip, const int32_t* zero_points_signed,
                              int32_t* sums_dev, int32_t* absmax_dev /* single word */);

@@ -36,10 +36,12 @@ __global__ __launch_bounds__(256) void pack_weight_kernel(
 }
 
 // Four-bit form: one thread produces one 16-byte lane slot, i.e. 16 weights of each of the
-// block's two steps.  Source codes are offset by 8 (packed_linear_ops.inc:476-477); code ^ 8
-// is the same value as a 4-bit two's complement number.
+// block's two steps.  Source codes of `bits` = 2, 3 or 4 bits are offset by half their range
+// (packed_linear_ops.inc:472-477; three-bit codes are a dense bitstream over the row, :249-254);
+// every such value fits a 4-bit two's complement number, which is what the block stores, so
+// the narrower widths run on the four-bit kernels unchanged.
 __global__ __launch_bounds__(256) void pack_nibble_kernel(
-        const uint32_t* __restrict__ raw, uint32_t row_words, uint32_t n, uint32_t k,
+        const uint32_t* __restrict__ raw, uint32_t row_words, uint32_t n, uint32_t k, uint32_t bits,
         uint32_t panels, uint32_t kblocks, uint8_t* __restrict__ out) {
     const size_t slot = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t total = (size_t)panels * kblocks * 64u;
@@ -54,8 +56,13 @@ __global__ __launch_bounds__(256) void pack_nibble_kernel(
     if (row < n) {
         const uint32_t* src = raw + (size_t)row * row_words;
         auto value = [&](uint32_t kk) -> uint32_t {
-            // padding is the value zero
-            return kk < k ? (((src[kk >> 3] >> ((kk & 7u) * 4u)) & 15u) ^ 8u) : 0u;
+            if (kk >= k) return 0u;  // padding is the value zero
+            const uint64_t bit = (uint64_t)kk * bits;
+            const uint32_t shift = (uint32_t)(bit & 31u);
+            uint32_t code = src[bit >> 5] >> shift;
+            if (shift + bits > 32u) code |= src[(bit >> 5) + 1u] << (32u - shift);
+            code &= (1u << bits) - 1u;
+            return (code - (1u << (bits - 1u))) & 15u;
         };
         for (uint32_t j = 0; j < 16u; j++) {
             const uint32_t b = value(k0 + j) | (value(k0 + 32u + j) << 4);
@@ -107,7 +114,7 @@ VxHipStatus pack_weight(hipStream_t stream, const uint8_t* raw_dev, size_t row_s
 }
 
 VxHipStatus pack_weight_nibbles(hipStream_t stream, const uint32_t* raw_dev, uint32_t row_words,
-                                uint32_t n, uint32_t k, PackedWeight* out) {
+                                uint32_t n, uint32_t k, uint32_t bits, PackedWeight* out) {
     out->n = n;
     out->k = k;
     out->bits = 4;
@@ -117,7 +124,7 @@ VxHipStatus pack_weight_nibbles(hipStream_t stream, const uint32_t* raw_dev, uin
     VXHIP_TRY(hipMalloc((void**)&out->data, out->bytes()));
     const size_t slots = (size_t)out->panels * out->ksteps * 64u;
     hipLaunchKernelGGL(pack_nibble_kernel, dim3((unsigned)((slots + 255u) / 256u)), dim3(256), 0, stream,
-                       raw_dev, row_words, n, k, out->panels, out->ksteps, (uint8_t*)out->data);
+                       raw_dev, row_words, n, k, bits, out->panels, out->ksteps, (uint8_t*)out->data);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

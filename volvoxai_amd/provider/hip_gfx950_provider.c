@@ -4,7 +4,7 @@
  * The provider compiles single-node W8A8 packages:
  *   - one QLinear / QGemm / QMatMul node in the volvox-affine-safetensors/v1
  *     representation (docs/w8a8-safetensors.md:13-59, validation list :158-175);
- *   - one PackedLinear node with weight_bits 8 or 4 under DYNAMIC_I8 packed
+ *   - one PackedLinear node with weight_bits 8, 4, 3 or 2 under DYNAMIC_I8 packed
  *     arithmetic (node form: native/tests/test_packed_arithmetic.inc:35-37).
  * Anything else is refused with BACKEND_UNSUPPORTED before a compiled instance
  * exists, which is what shape_domain.support = FULL promises
@@ -347,9 +347,9 @@ static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedAri
         !bits->is_integer || !weight_name || !scale_name)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s' lacks weight, scale or parameters",
                       plan->node_id);
-    if (bits->integer != 8 && bits->integer != 4)
+    if (bits->integer != 8 && bits->integer != 4 && bits->integer != 3 && bits->integer != 2)
         return refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
-                      "PackedLinear node '%s': weight_bits 8 and 4 are offered", plan->node_id);
+                      "PackedLinear node '%s': weight_bits must be 2, 3, 4 or 8", plan->node_id);
     if (group->integer != 32 && group->integer != 64 && group->integer != 128 && group->integer != 256)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "PackedLinear node '%s': group_size must be 32, 64, 128 or 256",
                       plan->node_id);
