@@ -15,6 +15,8 @@ import pytest
 
 import _cases as cases
 
+I8, U8 = cases.DTYPE_I8, cases.DTYPE_U8
+
 ROOT = Path(__file__).resolve().parent.parent
 PROVIDER = ROOT / "volvoxai_amd" / "lib" / "libvxhip_provider.so"
 MOCK = ROOT / "tests" / "provider_host" / "libvx_mock_host.so"
@@ -139,6 +141,57 @@ def packed_package(tmp, x_shape, words, scales, bias, group, bits=8, mutate=None
     (tmp / "graph.json").write_text(json.dumps(graph, separators=(",", ":")))
     write_safetensors(tmp / "model.safetensors", tensors)
     return tmp / "graph.json", tmp / "model.safetensors"
+
+
+def chain_package(tmp, x_shape, in_name, in_dtype, nodes, tensors, affine):
+    """A graph whose nodes form a chain.  nodes: (id, opType, extra inputs, output tensor, d_out, dtype,
+    params); affine: byte tensor or weight name -> (scale tensor, zero-point tensor[, axis])."""
+    lead = list(x_shape[:-1])
+    graph_nodes, current = [], in_name
+    for node_id, op, extra, out_name, d_out, dtype, params in nodes:
+        graph_nodes.append({"id": node_id, "opType": op, "inputs": dict({"input": current}, **extra),
+                            "outputs": {"out": {"tensor": out_name, "shape": lead + [d_out], "dtype": dtype}},
+                            "params": params})
+        current = out_name
+    table = {}
+    for name, ref in affine.items():
+        table[name] = {"scheme": "per_tensor", "scale_tensor": ref[0], "zero_point_tensor": ref[1]}
+        if len(ref) == 3:
+            table[name].update(scheme="per_axis", axis=ref[2])
+    graph = {"format": "volvox-graph/v1", "dimensions": {},
+             "inputs": {in_name: {"shape": list(x_shape), "dtype": in_dtype}},
+             "nodes": graph_nodes, "outputs": [current],
+             "execution": {"stateless": {}, "entrypoints": [{"name": "evaluate", "effect": 1, "allowed_ranges": [1],
+                                                             "inputs": [in_name], "outputs": [current]}]}}
+    if table:
+        graph["quantization"] = {"format": "volvox-affine-safetensors/v1", "tensors": table}
+    tmp.mkdir(parents=True, exist_ok=True)
+    (tmp / "graph.json").write_text(json.dumps(graph, separators=(",", ":")))
+    write_safetensors(tmp / "model.safetensors", tensors)
+    return tmp / "graph.json", tmp / "model.safetensors"
+
+
+def sandwich(tmp, x_shape, c1, c2=None, mutate=None):
+    """QuantizeLinear -> QLinear [-> QLinear] -> DequantizeLinear over f32 rows; c1/c2 are
+    cases.qlinear_random_case dictionaries (int8 throughout, c2 reads what c1 writes)."""
+    tensors = {"in.s": np.array([c1["s_in"]], np.float32), "in.z": np.array([c1["zp_in"]], np.int8),
+               "w1": c1["w"], "w1.s": c1["scales"], "w1.z": c1["zps"].astype(np.int8), "b1": c1["bias"],
+               "h.s": np.array([c1["s_out"]], np.float32), "h.z": np.array([c1["zp_out"]], np.int8)}
+    affine = {"xq": ("in.s", "in.z"), "w1": ("w1.s", "w1.z", 0), "hq": ("h.s", "h.z")}
+    nodes = [("q", "QuantizeLinear", {"scale": "in.s", "zero_point": "in.z"}, "xq", c1["w"].shape[1], "int8", {}),
+             ("fc1", "QLinear", {"weight": "w1", "bias": "b1"}, "hq", c1["w"].shape[0], "int8", {})]
+    last, last_d, last_affine = "hq", c1["w"].shape[0], ("h.s", "h.z")
+    if c2 is not None:
+        tensors.update({"w2": c2["w"], "w2.s": c2["scales"], "w2.z": c2["zps"].astype(np.int8), "b2": c2["bias"],
+                        "y.s": np.array([c2["s_out"]], np.float32), "y.z": np.array([c2["zp_out"]], np.int8)})
+        affine.update({"w2": ("w2.s", "w2.z", 0), "yq": ("y.s", "y.z")})
+        nodes.append(("fc2", "QGemm", {"weight": "w2", "bias": "b2"}, "yq", c2["w"].shape[0], "int8", {}))
+        last, last_d, last_affine = "yq", c2["w"].shape[0], ("y.s", "y.z")
+    nodes.append(("dq", "DequantizeLinear", {"scale": last_affine[0], "zero_point": last_affine[1]}, "y", last_d,
+                  "float32", {}))
+    if mutate:
+        mutate(nodes, tensors, affine)
+    return chain_package(tmp, x_shape, "x", "float32", nodes, tensors, affine), last_d
 
 
 def inspect(host, graph, weights, arithmetic="f32"):
@@ -283,6 +336,38 @@ def test_packed_package_refusals(registered, tmp_path):
     assert inspect(registered, g, w, "dynamic_i8")[0] == -5
     g, w = packed_package(tmp_path / "e", c["x"].shape, words, c["scales"][:, :-1], c["bias"], 32)
     assert inspect(registered, g, w, "dynamic_i8")[0] == -5
+
+
+def test_reads_node_chains(registered, tmp_path):
+    c1 = cases.qlinear_random_case(4, 48, 24, 5, I8, I8, I8, False)
+    c2 = cases.qlinear_random_case(4, 24, 10, 6, I8, I8, I8, False)
+    c2["s_in"], c2["zp_in"] = c1["s_out"], c1["zp_out"]
+    (g, w), d_out = sandwich(tmp_path / "ok", (4, 48), c1, c2)
+    assert inspect(registered, g, w)[:4] == (0, 48, 10, 0)
+
+    # the second linear reads the first node's output instead of the one before it: not a chain
+    (g, w), _ = sandwich(tmp_path / "dag", (4, 48), c1, c2)
+    doc = json.loads(g.read_text())
+    doc["nodes"][2]["inputs"]["input"] = "xq"
+    g.write_text(json.dumps(doc))
+    st, *_, msg = inspect(registered, g, w)
+    assert st == -7 and "chain" in msg
+
+    def other_parameters(nodes, tensors, affine):  # the node and the table disagree about the input's scale
+        tensors["in.s2"] = np.array([0.5], np.float32)
+        nodes[0] = ("q", "QuantizeLinear", {"scale": "in.s2", "zero_point": "in.z"}, "xq", 48, "int8", {})
+    (g, w), _ = sandwich(tmp_path / "bad", (4, 48), c1, mutate=other_parameters)
+    assert inspect(registered, g, w)[0] == -5
+
+    def widen(nodes, tensors, affine):  # a boundary node may not change the row length
+        nodes[0] = ("q", "QuantizeLinear", {"scale": "in.s", "zero_point": "in.z"}, "xq", 49, "int8", {})
+    (g, w), _ = sandwich(tmp_path / "wide", (4, 48), c1, mutate=widen)
+    assert inspect(registered, g, w)[0] == -5
+
+    def unknown(nodes, tensors, affine):
+        nodes.insert(2, ("act", "QGELU", {}, "gq", 24, "int8", {}))
+    (g, w), _ = sandwich(tmp_path / "op", (4, 48), c1, mutate=unknown)
+    assert inspect(registered, g, w)[0] == -7
 
 
 def test_sharded_weight_files(registered, tmp_path):
@@ -450,6 +535,56 @@ def test_packed_linear_w4_package_matches_oracle(registered, oracle, tmp_path, r
     _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, bits=4)
     assert (y.view(np.uint32) == want.view(np.uint32)).all()
     assert b"hip.packed-linear" in r.execute_route
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,two", [(3, False), (40, True), (1, True)])
+def test_quantize_linear_dequantize_chain_matches_oracle(registered, oracle, tmp_path, rows, two):
+    """QuantizeLinear -> QLinear (-> QGemm) -> DequantizeLinear in one compiled model: every node's
+    bytes are the oracle's, and the intermediate tensors never leave the device."""
+    c1 = cases.qlinear_random_case(rows, 200, 96, 15, I8, I8, I8, False)
+    c2 = cases.qlinear_random_case(rows, 96, 36, 16, I8, I8, I8, False) if two else None
+    x = np.random.default_rng(3).normal(0, 40 * c1["s_in"], (rows, 200)).astype(np.float32)
+    x[0, :4] = [np.nan, np.inf, -np.inf, 0.5 * c1["s_in"]]
+    if two:
+        c2["s_in"], c2["zp_in"] = c1["s_out"], c1["zp_out"]
+    (g, w), d_out = sandwich(tmp_path / "c", x.shape, c1, c2)
+    r, y = run(registered, g, w, x, "x", "f32", "y", "f32", d_out)
+    assert r.status == 0, r.message
+    ok, q = oracle.quantize(x, c1["s_in"], c1["zp_in"], I8)
+    ok1, h = oracle.qlinear(q, c1["w"], c1["bias"], c1["scales"], c1["zps"], c1["s_in"], c1["zp_in"], c1["s_out"],
+                            c1["zp_out"], I8, I8, I8)
+    assert ok == 1 and ok1 == 1
+    last = c1
+    if two:
+        ok2, h = oracle.qlinear(h, c2["w"], c2["bias"], c2["scales"], c2["zps"], c2["s_in"], c2["zp_in"], c2["s_out"],
+                                c2["zp_out"], I8, I8, I8)
+        assert ok2 == 1
+        last = c2
+    _, want = oracle.dequantize(h, last["s_out"], last["zp_out"], I8)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
+    assert (b"nodes=4" if two else b"nodes=3") in r.execute_route
+
+
+@pytest.mark.gpu
+def test_packed_linear_chain_matches_oracle(registered, oracle, tmp_path):
+    """Two PackedLinear nodes (W8 then W4) back to back: the f32 rows of the first are what the second
+    prepares and multiplies."""
+    a = cases.packed_case(9, 256, 130, 64, 41)
+    b = cases.packed_case(9, 130, 40, 32, 42)
+    wa, wb = oracle.pack_w8_words(a["w"]), oracle.pack_w4_words(cases.four_bit(b["w"]))
+    nodes = [("up", "PackedLinear", {"weight": "wa", "scale": "sa", "bias": "ba"}, "h", 130, "float32",
+              {"group_size": 64, "weight_bits": 8}),
+             ("down", "PackedLinear", {"weight": "wb", "scale": "sb", "bias": "bb"}, "y", 40, "float32",
+              {"group_size": 32, "weight_bits": 4})]
+    tensors = {"wa#as_i32": wa, "sa": a["scales"], "ba": a["bias"], "wb#as_i32": wb, "sb": b["scales"], "bb": b["bias"]}
+    g, w = chain_package(tmp_path / "mlp", a["x"].shape, "x", "float32", nodes, tensors, {})
+    r, y = run(registered, g, w, a["x"], "x", "f32", "y", "f32", 40, arithmetic="dynamic_i8")
+    assert r.status == 0, r.message
+    _, h = oracle.packed_linear(a["x"], wa, a["scales"], a["bias"], 130, 64)
+    _, want = oracle.packed_linear(h, wb, b["scales"], b["bias"], 40, 32, bits=4)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
+    assert r.attested_arithmetic == ARITH["dynamic_i8"] and b"nodes=2" in r.execute_route
 
 
 @pytest.mark.gpu

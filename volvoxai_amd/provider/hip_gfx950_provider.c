@@ -1,12 +1,15 @@
 /* Backend provider "hip-gfx950": plugs libvxhip_w8a8 into the unchanged
  * VolvoxAI runtime through its provider SPI (native/include/volvoxai_backend.h:168-259).
  *
- * The provider compiles single-node W8A8 packages:
- *   - one QLinear / QGemm / QMatMul node in the volvox-affine-safetensors/v1
+ * The provider compiles W8A8 packages whose graph is one node or a chain of nodes, each reading
+ * the tensor the one before it wrote (one graph input, one graph output):
+ *   - QLinear / QGemm / QMatMul in the volvox-affine-safetensors/v1
  *     representation (docs/w8a8-safetensors.md:13-59, validation list :158-175);
- *   - one PackedLinear node with weight_bits 8, 4, 3 or 2 under DYNAMIC_I8 packed
- *     arithmetic (node form: native/tests/test_packed_arithmetic.inc:35-37).
- * Anything else is refused with BACKEND_UNSUPPORTED before a compiled instance
+ *   - PackedLinear with weight_bits 8, 4, 3 or 2 under DYNAMIC_I8 packed
+ *     arithmetic (node form: native/tests/test_packed_arithmetic.inc:35-37);
+ *   - QuantizeLinear / DequantizeLinear with per-tensor parameters (node form: inputs
+ *     input, scale, zero_point; python/tests/test_transpose_quantization_dynamic.py:29-37).
+ * Intermediate tensors of a chain stay in device memory.  Anything else is refused with BACKEND_UNSUPPORTED before a compiled instance
  * exists, which is what shape_domain.support = FULL promises
  * (native/include/volvoxai_backend.h:112-118).
  *
@@ -35,9 +38,17 @@ typedef struct HipRuntime {
     char device_name[VX_REPORT_DEVICE_CAPACITY];
 } HipRuntime;
 
-typedef enum PlanKind { PLAN_QLINEAR = 1, PLAN_PACKED_LINEAR = 2 } PlanKind;
+typedef enum PlanKind {
+    PLAN_QLINEAR = 1,
+    PLAN_PACKED_LINEAR = 2,
+    PLAN_QUANTIZE = 3,
+    PLAN_DEQUANTIZE = 4
+} PlanKind;
 
-/* Host-side result of reading a package; tensor pointers borrow the mapped weight files. */
+#define MAX_CHAIN_NODES 64u
+
+/* Host-side result of reading one node; tensor pointers borrow the mapped weight files, which
+ * belong to the ChainPlan. */
 typedef struct PackagePlan {
     PlanKind kind;
     char node_id[NAME_CAPACITY];
@@ -59,14 +70,43 @@ typedef struct PackagePlan {
     const float* bias_f32;
     uint32_t group_size;
     uint32_t weight_bits;
-    /* mapped files */
+    /* QuantizeLinear / DequantizeLinear: parameters of the byte side */
+    float boundary_scale;
+    int32_t boundary_zero_point;
+    /* mapped files (borrowed) */
     VxstFile** files;
     size_t file_count;
 } PackagePlan;
 
+/* The whole graph: its nodes in execution order and the files they read. */
+typedef struct ChainPlan {
+    PackagePlan* nodes;
+    size_t count;
+    VxstFile** files;
+    size_t file_count;
+    char input_name[NAME_CAPACITY];
+    char output_name[NAME_CAPACITY];
+    uint32_t d_in, d_out;
+    VxDataType input_dtype, output_dtype;
+    int any_packed;
+} ChainPlan;
+
+/* One compiled node. */
+typedef struct HipStage {
+    PlanKind kind;
+    uint32_t d_in, d_out;
+    VxDataType input_dtype, output_dtype;
+    VxHipQLinear* qlinear;
+    VxHipPackedLinear* packed;
+    float input_scale, output_scale; /* QLinear; the byte side of a boundary node in input_scale */
+    int32_t input_zero_point, output_zero_point;
+} HipStage;
+
 typedef struct HipCompiled {
     HipRuntime* runtime;
-    PlanKind kind;
+    HipStage* stages;
+    size_t stage_count;
+    uint64_t widest_row_bytes; /* of any tensor of the chain, graph input and output included */
     char input_name[NAME_CAPACITY];
     char output_name[NAME_CAPACITY];
     uint32_t d_in, d_out;
@@ -81,20 +121,15 @@ typedef struct HipCompiled {
     int batch_capable;
     char graph_fingerprint[256];
     char batch_proof_identity[256];
-    VxHipQLinear* qlinear;
-    VxHipPackedLinear* packed;
-    float input_scale, output_scale;
-    int32_t input_zero_point, output_zero_point;
     char route[128];
 } HipCompiled;
 
 typedef struct HipContext {
     HipCompiled* compiled;
     VxHipContext* ctx;
-    void* input_dev;
-    void* output_dev;
+    void* work_dev[2]; /* a node reads one and writes the other */
     void* output_host;
-    size_t input_capacity, output_capacity, host_capacity;
+    size_t work_capacity[2], host_capacity;
     int closed;
 } HipContext;
 
@@ -131,12 +166,12 @@ static VxOperationCode code_for(VxStatus status) {
     }
 }
 
-static void attest(VxReport* report, const char* route) {
+static void attest(VxReport* report, size_t nodes, const char* route) {
     if (!report_writable(report)) return;
     report->route_attested = 1;
     report->operator_fallback_used = 0;
-    snprintf(report->route_evidence, sizeof(report->route_evidence), "provider=%s;nodes=1;route=%s", PROVIDER_NAME,
-             route);
+    snprintf(report->route_evidence, sizeof(report->route_evidence), "provider=%s;nodes=%zu;route=%s", PROVIDER_NAME,
+             nodes, route);
     snprintf(report->fallback_evidence, sizeof(report->fallback_evidence), "%s", "operator=none");
 }
 
@@ -153,11 +188,12 @@ static VxStatus refuse(Failure* failure, VxStatus status, const char* format, co
     return status;
 }
 
-static void plan_release(PackagePlan* plan) {
-    for (size_t i = 0; i < plan->file_count; i++) vxst_close(plan->files[i]);
-    free(plan->files);
-    free(plan->weight_zero_points);
-    memset(plan, 0, sizeof(*plan));
+static void chain_release(ChainPlan* chain) {
+    for (size_t i = 0; i < chain->count; i++) free(chain->nodes[i].weight_zero_points);
+    free(chain->nodes);
+    for (size_t i = 0; i < chain->file_count; i++) vxst_close(chain->files[i]);
+    free(chain->files);
+    memset(chain, 0, sizeof(*chain));
 }
 
 static char* read_text_file(const char* path, size_t* length) {
@@ -274,23 +310,63 @@ static int32_t typed_zero_point(const VxstTensor* t, int64_t index) {
     return !strcmp(t->dtype, "I8") ? (int32_t)((const int8_t*)t->data)[index] : (int32_t)t->data[index];
 }
 
-static VxStatus plan_qlinear(PackagePlan* plan, const VxjValue* root, const VxjValue* node, const VxjValue* out,
-                             Failure* failure) {
+/* The central table of affine descriptors, or NULL (with the refusal filled in). */
+static const VxjValue* quantization_table(const VxjValue* root, Failure* failure) {
     static const char* const table_fields[] = {"format", "tensors"};
-    const VxjValue* node_inputs = vxj_member(node, "inputs");
-    const char* weight_name = vxj_member_string(node_inputs, "weight");
-    const char* bias_name = vxj_member_string(node_inputs, "bias");
     const VxjValue* quantization = vxj_member(root, "quantization");
     const VxjValue* table = vxj_member(quantization, "tensors");
     const char* table_format = vxj_member_string(quantization, "format");
+    if (!quantization || !object_has_only(quantization, table_fields, 2) || !table_format ||
+        strcmp(table_format, "volvox-affine-safetensors/v1") || !table || table->kind != VXJ_OBJECT || !table->count) {
+        refuse(failure, VX_STATUS_INVALID_GRAPH, "graph has no volvox-affine-safetensors/v1 quantization table%s", "");
+        return NULL;
+    }
+    return table;
+}
+
+/* QuantizeLinear (float32 -> int8/uint8) or DequantizeLinear (the reverse) with per-tensor
+ * parameters.  The node names its scale and zero point, and the table's descriptor of the byte
+ * tensor must name the same two tensors. */
+static VxStatus plan_boundary(PackagePlan* plan, const VxjValue* root, const VxjValue* node, int quantize,
+                              Failure* failure) {
+    const VxjValue* node_inputs = vxj_member(node, "inputs");
+    const char* scale_name = vxj_member_string(node_inputs, "scale");
+    const char* zp_name = vxj_member_string(node_inputs, "zero_point");
+    const char* byte_name = quantize ? plan->output_name : plan->input_name;
+    const VxDataType byte_dtype = quantize ? plan->output_dtype : plan->input_dtype;
+    const VxDataType real_dtype = quantize ? plan->input_dtype : plan->output_dtype;
+    const VxjValue* table = quantization_table(root, failure);
+    const VxjValue* descriptor;
+    VxstTensor scale, zero_point;
+    VxStatus status;
+    if (!table) return failure->status;
+    if (!scale_name || !zp_name)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "node '%s' names no scale or zero point", plan->node_id);
+    if (real_dtype != VX_DTYPE_F32 || byte_dtype == VX_DTYPE_F32 || plan->d_in != plan->d_out)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH,
+                      "node '%s' must convert between float32 and int8/uint8 of one shape", plan->node_id);
+    status = resolve_affine(plan, table, byte_name, byte_dtype, 2, 0, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    descriptor = vxj_member(table, byte_name);
+    if (strcmp(vxj_member_string(descriptor, "scale_tensor"), scale_name) ||
+        strcmp(vxj_member_string(descriptor, "zero_point_tensor"), zp_name))
+        return refuse(failure, VX_STATUS_INVALID_GRAPH,
+                      "node '%s' and the quantization table name different parameters", plan->node_id);
+    memcpy(&plan->boundary_scale, scale.data, 4);
+    plan->boundary_zero_point = typed_zero_point(&zero_point, 0);
+    plan->kind = quantize ? PLAN_QUANTIZE : PLAN_DEQUANTIZE;
+    return VX_STATUS_OK;
+}
+
+static VxStatus plan_qlinear(PackagePlan* plan, const VxjValue* root, const VxjValue* node, Failure* failure) {
+    const VxjValue* node_inputs = vxj_member(node, "inputs");
+    const char* weight_name = vxj_member_string(node_inputs, "weight");
+    const char* bias_name = vxj_member_string(node_inputs, "bias");
+    const VxjValue* table = quantization_table(root, failure);
     VxstTensor weight, bias, scale, zero_point;
     VxStatus status;
-    (void)out;
+    if (!table) return failure->status;
     if (!weight_name) return refuse(failure, VX_STATUS_INVALID_GRAPH, "QLinear node '%s' names no weight", plan->node_id);
-    if (!quantization || !object_has_only(quantization, table_fields, 2) || !table_format ||
-        strcmp(table_format, "volvox-affine-safetensors/v1") || !table || table->kind != VXJ_OBJECT || !table->count)
-        return refuse(failure, VX_STATUS_INVALID_GRAPH,
-                      "graph has no volvox-affine-safetensors/v1 quantization table%s", "");
     if (plan->input_dtype == VX_DTYPE_F32 || plan->output_dtype == VX_DTYPE_F32)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "QLinear node '%s' needs int8/uint8 input and output",
                       plan->node_id);
@@ -380,15 +456,28 @@ static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedAri
     return VX_STATUS_OK;
 }
 
-/* Reads graph.json and the weight files named by the model source into a plan. */
-static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic arithmetic, PackagePlan* plan,
+/* A positive extent that fits the kernels' 32-bit row lengths, else 0. */
+static uint32_t fixed_extent(const VxjValue* v) {
+    return v && v->kind == VXJ_NUMBER && v->is_integer && v->integer > 0 && v->integer <= INT32_MAX
+               ? (uint32_t)v->integer : 0u;
+}
+
+/* Two declared extents are the same number or the same symbol. */
+static int same_extent(const VxjValue* a, const VxjValue* b) {
+    if (!a || !b || a->kind != b->kind) return 0;
+    if (a->kind == VXJ_NUMBER) return a->is_integer && b->is_integer && a->integer == b->integer;
+    return a->kind == VXJ_STRING && !strcmp(a->string, b->string);
+}
+
+/* Reads graph.json and the weight files named by the model source into a chain of node plans. */
+static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic arithmetic, ChainPlan* chain,
                              Failure* failure) {
     size_t length = 0;
     const char* json_error = NULL;
     char* text;
     VxjValue* root;
     VxStatus status = VX_STATUS_OK;
-    memset(plan, 0, sizeof(*plan));
+    memset(chain, 0, sizeof(*chain));
     text = read_text_file(source->graph_path, &length);
     if (!text) return refuse(failure, VX_STATUS_IO_ERROR, "cannot read graph document '%s'", source->graph_path);
     root = vxj_parse(text, length, &json_error);
@@ -400,80 +489,116 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
         const VxjValue* inputs = vxj_member(root, "inputs");
         const VxjValue* nodes = vxj_member(root, "nodes");
         const VxjValue* outputs = vxj_member(root, "outputs");
-        const VxjValue* node = vxj_item(nodes, 0);
-        const char* op = vxj_member_string(node, "opType");
-        const VxjValue* out = vxj_member(vxj_member(node, "outputs"), "out");
-        const VxjValue* out_shape = vxj_member(out, "shape");
         const VxjValue* graph_input = inputs && inputs->kind == VXJ_OBJECT ? inputs->first : NULL;
         const VxjValue* in_shape = vxj_member(graph_input, "shape");
-        const VxjValue* last;
+        const VxjValue* declared_output = vxj_item(outputs, 0);
+        /* the tensor the next node must read */
+        char current[NAME_CAPACITY];
+        VxDataType current_dtype;
+        uint32_t current_d;
         if (!format || strcmp(format, "volvox-graph/v1")) {
             status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph format is not volvox-graph/v1%s", "");
             break;
         }
-        if (!nodes || nodes->kind != VXJ_ARRAY || nodes->count != 1 || !inputs || inputs->count != 1 || !outputs ||
-            outputs->kind != VXJ_ARRAY || outputs->count != 1) {
+        if (!nodes || nodes->kind != VXJ_ARRAY || !nodes->count || nodes->count > MAX_CHAIN_NODES || !inputs ||
+            inputs->count != 1 || !outputs || outputs->kind != VXJ_ARRAY || outputs->count != 1) {
             status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
-                            "this provider compiles graphs of one node, one input and one output%s", "");
+                            "this provider compiles chains of up to 64 nodes with one input and one output%s", "");
             break;
         }
-        if (!op || !out || !copy_name(plan->node_id, vxj_member_string(node, "id")) ||
-            !copy_name(plan->input_name, graph_input->key) ||
-            !copy_name(plan->output_name, vxj_member_string(out, "tensor")) ||
-            !graph_dtype(vxj_member_string(graph_input, "dtype"), &plan->input_dtype) ||
-            !graph_dtype(vxj_member_string(out, "dtype"), &plan->output_dtype) || !in_shape ||
-            in_shape->kind != VXJ_ARRAY || !in_shape->count || !out_shape || out_shape->kind != VXJ_ARRAY ||
-            out_shape->count != in_shape->count) {
-            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "node or tensor declaration is incomplete%s", "");
+        if (!copy_name(chain->input_name, graph_input->key) ||
+            !graph_dtype(vxj_member_string(graph_input, "dtype"), &chain->input_dtype) || !in_shape ||
+            in_shape->kind != VXJ_ARRAY || !in_shape->count || declared_output->kind != VXJ_STRING ||
+            !copy_name(chain->output_name, declared_output->string)) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph input or output declaration is incomplete%s", "");
             break;
         }
-        {
-            const char* fed = vxj_member_string(vxj_member(node, "inputs"), "input");
-            const VxjValue* declared = vxj_item(outputs, 0);
-            if (!fed || strcmp(fed, plan->input_name) || declared->kind != VXJ_STRING ||
-                strcmp(declared->string, plan->output_name)) {
-                status = refuse(failure, VX_STATUS_INVALID_GRAPH,
-                                "the node must read the graph input and feed the graph output%s", "");
-                break;
-            }
-        }
-        /* dense on the last axis: that extent is a number in both declarations */
-        last = vxj_item(in_shape, in_shape->count - 1);
-        if (last->kind != VXJ_NUMBER || !last->is_integer || last->integer <= 0 || last->integer > INT32_MAX) {
+        /* dense on the last axis: that extent is a number in every declaration */
+        chain->d_in = fixed_extent(vxj_item(in_shape, in_shape->count - 1));
+        if (!chain->d_in) {
             status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the input's last extent must be a fixed d_in%s", "");
             break;
         }
-        plan->d_in = (uint32_t)last->integer;
-        last = vxj_item(out_shape, out_shape->count - 1);
-        if (last->kind != VXJ_NUMBER || !last->is_integer || last->integer <= 0 || last->integer > INT32_MAX) {
-            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the output's last extent must be a fixed d_out%s", "");
-            break;
-        }
-        plan->d_out = (uint32_t)last->integer;
-
-        plan->files = (VxstFile**)calloc(source->weight_path_count ? source->weight_path_count : 1, sizeof(VxstFile*));
-        if (!plan->files) {
+        chain->files = (VxstFile**)calloc(source->weight_path_count ? source->weight_path_count : 1, sizeof(VxstFile*));
+        chain->nodes = (PackagePlan*)calloc(nodes->count, sizeof(PackagePlan));
+        if (!chain->files || !chain->nodes) {
             status = refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
             break;
         }
         for (size_t i = 0; i < source->weight_path_count && status == VX_STATUS_OK; i++) {
             char error[VX_REPORT_MESSAGE_CAPACITY];
-            if (vxst_open(source->weight_paths[i], &plan->files[plan->file_count], error, sizeof(error)) != 0)
+            if (vxst_open(source->weight_paths[i], &chain->files[chain->file_count], error, sizeof(error)) != 0)
                 status = refuse(failure, VX_STATUS_IO_ERROR, "%s", error);
             else
-                plan->file_count++;
+                chain->file_count++;
         }
         if (status != VX_STATUS_OK) break;
 
-        if (!strcmp(op, "QLinear") || !strcmp(op, "QGemm") || !strcmp(op, "QMatMul"))
-            status = plan_qlinear(plan, root, node, out, failure);
-        else if (!strcmp(op, "PackedLinear"))
-            status = plan_packed(plan, node, arithmetic, failure);
-        else
-            status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "operator '%s' is not offered by this provider", op);
+        memcpy(current, chain->input_name, sizeof(current));
+        current_dtype = chain->input_dtype;
+        current_d = chain->d_in;
+        for (const VxjValue* node = nodes->first; node && status == VX_STATUS_OK; node = node->next) {
+            PackagePlan* plan = &chain->nodes[chain->count];
+            const char* op = vxj_member_string(node, "opType");
+            const VxjValue* out = vxj_member(vxj_member(node, "outputs"), "out");
+            const VxjValue* out_shape = vxj_member(out, "shape");
+            const char* fed = vxj_member_string(vxj_member(node, "inputs"), "input");
+            chain->count++;
+            plan->files = chain->files;
+            plan->file_count = chain->file_count;
+            if (!op || !out || !copy_name(plan->node_id, vxj_member_string(node, "id")) ||
+                !copy_name(plan->output_name, vxj_member_string(out, "tensor")) ||
+                !graph_dtype(vxj_member_string(out, "dtype"), &plan->output_dtype) || !out_shape ||
+                out_shape->kind != VXJ_ARRAY || out_shape->count != in_shape->count) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH, "node or tensor declaration is incomplete%s", "");
+                break;
+            }
+            if (!fed || strcmp(fed, current)) {
+                status = refuse(failure, nodes->count == 1 ? VX_STATUS_INVALID_GRAPH : VX_STATUS_BACKEND_UNSUPPORTED,
+                                "node '%s' does not read the tensor before it: only chains are compiled",
+                                plan->node_id);
+                break;
+            }
+            /* rows pass through unchanged: the leading extents are the graph input's */
+            for (size_t axis = 0; axis + 1 < in_shape->count; axis++)
+                if (!same_extent(vxj_item(in_shape, axis), vxj_item(out_shape, axis)))
+                    status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                    "node '%s' changes a leading extent", plan->node_id);
+            if (status != VX_STATUS_OK) break;
+            memcpy(plan->input_name, current, sizeof(current));
+            plan->input_dtype = current_dtype;
+            plan->d_in = current_d;
+            plan->d_out = fixed_extent(vxj_item(out_shape, out_shape->count - 1));
+            if (!plan->d_out) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the last extent of '%s' must be fixed",
+                                plan->output_name);
+                break;
+            }
+            if (!strcmp(op, "QLinear") || !strcmp(op, "QGemm") || !strcmp(op, "QMatMul"))
+                status = plan_qlinear(plan, root, node, failure);
+            else if (!strcmp(op, "PackedLinear"))
+                status = plan_packed(plan, node, arithmetic, failure);
+            else if (!strcmp(op, "QuantizeLinear") || !strcmp(op, "DequantizeLinear"))
+                status = plan_boundary(plan, root, node, op[0] == 'Q', failure);
+            else
+                status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "operator '%s' is not offered by this provider",
+                                op);
+            if (plan->kind == PLAN_PACKED_LINEAR) chain->any_packed = 1;
+            memcpy(current, plan->output_name, sizeof(current));
+            current_dtype = plan->output_dtype;
+            current_d = plan->d_out;
+        }
+        if (status != VX_STATUS_OK) break;
+        if (strcmp(current, chain->output_name)) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the last node must write the graph output '%s'",
+                            chain->output_name);
+            break;
+        }
+        chain->output_dtype = current_dtype;
+        chain->d_out = current_d;
     } while (0);
     vxj_free(root);
-    if (status != VX_STATUS_OK) plan_release(plan);
+    if (status != VX_STATUS_OK) chain_release(chain);
     return status;
 }
 
@@ -516,13 +641,16 @@ static int policy_names(const VxBackendPolicy* policy, const char* name) {
 static void hip_compiled_destroy(void* compiled_instance) {
     HipCompiled* compiled = (HipCompiled*)compiled_instance;
     if (!compiled) return;
-    if (compiled->qlinear) vxhip_qlinear_destroy(compiled->qlinear);
-    if (compiled->packed) vxhip_packed_linear_destroy(compiled->packed);
+    for (size_t i = 0; i < compiled->stage_count; i++) {
+        if (compiled->stages[i].qlinear) vxhip_qlinear_destroy(compiled->stages[i].qlinear);
+        if (compiled->stages[i].packed) vxhip_packed_linear_destroy(compiled->stages[i].packed);
+    }
+    free(compiled->stages);
     free(compiled);
 }
 
 /* The logical specifications the core hands over must describe the same tensors as the graph. */
-static int specs_match(const VxBackendCompileInput* input, const PackagePlan* plan, HipCompiled* compiled) {
+static int specs_match(const VxBackendCompileInput* input, const ChainPlan* plan, HipCompiled* compiled) {
     const VxTensorSpec* in = &input->inputs[0];
     const VxTensorSpec* out = &input->outputs[0];
     if (in->struct_size != sizeof(*in) || out->struct_size != sizeof(*out) || !in->name || !out->name ||
@@ -565,11 +693,12 @@ static int specs_match(const VxBackendCompileInput* input, const PackagePlan* pl
 static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput* input, const VxBackendPolicy* policy,
                             void** out_compiled, VxBackendShapeDomainAttestation* attestation, VxReport* report) {
     HipRuntime* runtime = (HipRuntime*)runtime_instance;
-    PackagePlan plan;
+    ChainPlan plan;
     Failure failure = {VX_STATUS_OK, {0}};
     HipCompiled* compiled;
     VxStatus status;
-    uint64_t rows_max = 1, resident, tensor_bytes;
+    uint64_t rows_max = 1, resident = 0;
+    size_t route_used = 0;
     if (!runtime || !input || input->struct_size != sizeof(*input) || !input->source ||
         input->source->struct_size != sizeof(*input->source) || !input->graph_fingerprint ||
         !input->shape_domain_proof_identity || !out_compiled || !attestation ||
@@ -585,7 +714,7 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
     }
     if (input->input_count != 1 || input->output_count != 1 || !input->inputs || !input->outputs) {
         fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
-                    "this provider compiles graphs of one node, one input and one output");
+                    "this provider compiles graphs with one input and one output");
         return VX_STATUS_BACKEND_UNSUPPORTED;
     }
     status = plan_package(input->source, input->packed_arithmetic, &plan, &failure);
@@ -594,19 +723,20 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         return status;
     }
     compiled = (HipCompiled*)calloc(1, sizeof(*compiled));
-    if (!compiled) {
-        plan_release(&plan);
+    if (compiled) compiled->stages = (HipStage*)calloc(plan.count, sizeof(HipStage));
+    if (!compiled || !compiled->stages) {
+        chain_release(&plan);
+        free(compiled);
         return VX_STATUS_OUT_OF_MEMORY;
     }
     if (!specs_match(input, &plan, compiled)) {
-        plan_release(&plan);
-        free(compiled);
+        chain_release(&plan);
+        hip_compiled_destroy(compiled);
         fill_report(report, runtime, VX_STATUS_INVALID_ARGUMENT, VX_STAGE_COMPILE, VX_CODE_INVALID_ARGUMENT,
                     "logical tensor specifications do not describe the graph's input and output");
         return VX_STATUS_INVALID_ARGUMENT;
     }
     compiled->runtime = runtime;
-    compiled->kind = plan.kind;
     memcpy(compiled->input_name, plan.input_name, sizeof(compiled->input_name));
     memcpy(compiled->output_name, plan.output_name, sizeof(compiled->output_name));
     compiled->d_in = plan.d_in;
@@ -615,27 +745,55 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
     compiled->output_dtype = plan.output_dtype;
     compiled->input_element_bytes = plan.input_dtype == VX_DTYPE_F32 ? 4u : 1u;
     compiled->output_element_bytes = plan.output_dtype == VX_DTYPE_F32 ? 4u : 1u;
-    compiled->input_scale = plan.input_scale;
-    compiled->output_scale = plan.output_scale;
-    compiled->input_zero_point = plan.input_zero_point;
-    compiled->output_zero_point = plan.output_zero_point;
+    compiled->widest_row_bytes = (uint64_t)plan.d_in * compiled->input_element_bytes;
 
-    if (plan.kind == PLAN_QLINEAR) {
-        status = (VxStatus)vxhip_qlinear_create(plan.weight, plan.weight_scales, plan.weight_zero_points, plan.bias_i32,
-                                                plan.d_in, plan.d_out, plan.weight_dtype, &compiled->qlinear);
-        /* a fused integer operator is published only with its multiplier and accumulator-range
-         * contract satisfied (docs/w8a8-safetensors.md:158-175, item 8) */
-        if (status == VX_STATUS_OK &&
-            !vxhip_qlinear_admits(compiled->qlinear, plan.input_scale, plan.input_zero_point, plan.output_scale,
-                                  plan.output_zero_point, (uint32_t)plan.input_dtype, (uint32_t)plan.output_dtype))
-            status = VX_STATUS_INVALID_GRAPH;
-        snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.qlinear");
-    } else {
-        status = (VxStatus)vxhip_packed_linear_create(plan.packed_words, plan.group_scales, plan.bias_f32, plan.d_in,
-                                                      plan.d_out, plan.group_size, plan.weight_bits, &compiled->packed);
-        snprintf(compiled->route, sizeof(compiled->route), "%s", "hip.packed-linear");
+    for (size_t i = 0; i < plan.count && status == VX_STATUS_OK; i++) {
+        const PackagePlan* node = &plan.nodes[i];
+        HipStage* stage = &compiled->stages[compiled->stage_count++];
+        const char* family = "";
+        const uint64_t row_bytes = (uint64_t)node->d_out * (node->output_dtype == VX_DTYPE_F32 ? 4u : 1u);
+        stage->kind = node->kind;
+        stage->d_in = node->d_in;
+        stage->d_out = node->d_out;
+        stage->input_dtype = node->input_dtype;
+        stage->output_dtype = node->output_dtype;
+        if (row_bytes > compiled->widest_row_bytes) compiled->widest_row_bytes = row_bytes;
+        if (node->kind == PLAN_QLINEAR) {
+            stage->input_scale = node->input_scale;
+            stage->output_scale = node->output_scale;
+            stage->input_zero_point = node->input_zero_point;
+            stage->output_zero_point = node->output_zero_point;
+            status = (VxStatus)vxhip_qlinear_create(node->weight, node->weight_scales, node->weight_zero_points,
+                                                    node->bias_i32, node->d_in, node->d_out, node->weight_dtype,
+                                                    &stage->qlinear);
+            /* a fused integer operator is published only with its multiplier and accumulator-range
+             * contract satisfied (docs/w8a8-safetensors.md:158-175, item 8) */
+            if (status == VX_STATUS_OK &&
+                !vxhip_qlinear_admits(stage->qlinear, node->input_scale, node->input_zero_point, node->output_scale,
+                                      node->output_zero_point, (uint32_t)node->input_dtype,
+                                      (uint32_t)node->output_dtype))
+                status = VX_STATUS_INVALID_GRAPH;
+            if (status == VX_STATUS_OK) resident += vxhip_qlinear_resident_bytes(stage->qlinear);
+            family = "hip.qlinear";
+        } else if (node->kind == PLAN_PACKED_LINEAR) {
+            status = (VxStatus)vxhip_packed_linear_create(node->packed_words, node->group_scales, node->bias_f32,
+                                                          node->d_in, node->d_out, node->group_size, node->weight_bits,
+                                                          &stage->packed);
+            if (status == VX_STATUS_OK) resident += vxhip_packed_linear_resident_bytes(stage->packed);
+            family = "hip.packed-linear";
+        } else {
+            stage->input_scale = node->boundary_scale;
+            stage->input_zero_point = node->boundary_zero_point;
+            family = node->kind == PLAN_QUANTIZE ? "hip.quantize-linear" : "hip.dequantize-linear";
+        }
+        if (route_used + 1 < sizeof(compiled->route))
+            route_used += (size_t)snprintf(compiled->route + route_used, sizeof(compiled->route) - route_used, "%s%s",
+                                           i ? ">" : "", family);
+        if (route_used >= sizeof(compiled->route)) route_used = sizeof(compiled->route) - 1u;
     }
-    plan_release(&plan);
+    const int any_packed = plan.any_packed;
+    const size_t node_count = plan.count;
+    chain_release(&plan);
     if (status != VX_STATUS_OK) {
         fill_report(report, runtime, status, VX_STAGE_COMPILE, code_for(status), vxhip_last_error());
         hip_compiled_destroy(compiled);
@@ -651,33 +809,27 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         }
         rows_max *= (uint64_t)compiled->lead_max[axis];
     }
-    resident = compiled->qlinear ? vxhip_qlinear_resident_bytes(compiled->qlinear)
-                                 : vxhip_packed_linear_resident_bytes(compiled->packed);
-    tensor_bytes = rows_max * compiled->d_in * compiled->input_element_bytes;
-    if (rows_max * compiled->d_out * compiled->output_element_bytes > tensor_bytes)
-        tensor_bytes = rows_max * compiled->d_out * compiled->output_element_bytes;
     attestation->graph_fingerprint = input->graph_fingerprint;
     attestation->shape_domain_proof_identity = input->shape_domain_proof_identity;
-    attestation->maximum_tensor_bytes = tensor_bytes;
-    /* weights plus, per context, staged input, output and the int8 staging of a PackedLinear call */
-    attestation->maximum_resident_bytes =
-        resident + rows_max * ((uint64_t)compiled->d_in * (compiled->input_element_bytes + 1u) +
-                               (uint64_t)compiled->d_out * compiled->output_element_bytes + 8u);
+    attestation->maximum_tensor_bytes = rows_max * compiled->widest_row_bytes;
+    /* weights plus, per context, the two work buffers, the int8 staging of a PackedLinear call
+     * (at most one byte per float of its input) and row scales */
+    attestation->maximum_resident_bytes = resident + rows_max * (3u * compiled->widest_row_bytes + 8u);
     attestation->resource_limit_bytes = 0;
     attestation->has_resource_limit = 0;
-    attestation->packed_arithmetic =
-        compiled->packed ? VX_PACKED_ARITHMETIC_DYNAMIC_I8 : input->packed_arithmetic;
+    attestation->packed_arithmetic = any_packed ? VX_PACKED_ARITHMETIC_DYNAMIC_I8 : input->packed_arithmetic;
     *out_compiled = compiled;
-    fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE, "single-node W8A8 package compiled");
-    attest(report, compiled->route);
+    fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE,
+                node_count == 1 ? "single-node W8A8 package compiled" : "W8A8 node chain compiled");
+    attest(report, compiled->stage_count, compiled->route);
     return VX_STATUS_OK;
 }
 
 static void hip_context_destroy(void* context_instance) {
     HipContext* context = (HipContext*)context_instance;
     if (!context) return;
-    if (context->input_dev) vxhip_device_free(context->input_dev);
-    if (context->output_dev) vxhip_device_free(context->output_dev);
+    if (context->work_dev[0]) vxhip_device_free(context->work_dev[0]);
+    if (context->work_dev[1]) vxhip_device_free(context->work_dev[1]);
     free(context->output_host);
     if (context->ctx) vxhip_context_destroy(context->ctx);
     free(context);
@@ -740,15 +892,16 @@ static int binding_admitted(const HipCompiled* compiled, const VxTensorBinding* 
     return binding->byte_size == (size_t)*rows * compiled->d_in * compiled->input_element_bytes;
 }
 
-/* Upload, one linear over all rows, download into the context's host buffer. */
+/* Upload, every node over all rows (each reads one work buffer and writes the other), download
+ * into the context's host buffer. */
 static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, VxReport* report) {
     const HipCompiled* compiled = context->compiled;
     const size_t input_bytes = (size_t)rows * compiled->d_in * compiled->input_element_bytes;
     const size_t output_bytes = (size_t)rows * compiled->d_out * compiled->output_element_bytes;
+    const size_t work_bytes = (size_t)rows * (size_t)compiled->widest_row_bytes;
     VxStatus status;
-    int handled;
-    status = grow_device(&context->input_dev, &context->input_capacity, input_bytes);
-    if (status == VX_STATUS_OK) status = grow_device(&context->output_dev, &context->output_capacity, output_bytes);
+    status = grow_device(&context->work_dev[0], &context->work_capacity[0], work_bytes);
+    if (status == VX_STATUS_OK) status = grow_device(&context->work_dev[1], &context->work_capacity[1], work_bytes);
     if (status == VX_STATUS_OK && output_bytes > context->host_capacity) {
         void* fresh = realloc(context->output_host, output_bytes);
         if (!fresh) status = VX_STATUS_OUT_OF_MEMORY;
@@ -758,20 +911,41 @@ static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, 
         }
     }
     if (status == VX_STATUS_OK)
-        status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->input_dev, input, input_bytes);
-    if (status == VX_STATUS_OK) {
-        if (compiled->qlinear)
-            handled = vxhip_qlinear_forward(context->ctx, compiled->qlinear, context->input_dev, context->output_dev, NULL,
-                                            (uint32_t)rows, compiled->input_scale, compiled->input_zero_point,
-                                            compiled->output_scale, compiled->output_zero_point,
-                                            (uint32_t)compiled->input_dtype, (uint32_t)compiled->output_dtype);
-        else
-            handled = vxhip_packed_linear_forward_f32(context->ctx, compiled->packed, (const float*)context->input_dev,
-                                                      (float*)context->output_dev, (uint32_t)rows) == 0;
+        status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->work_dev[0], input, input_bytes);
+    for (size_t i = 0; i < compiled->stage_count && status == VX_STATUS_OK; i++) {
+        const HipStage* stage = &compiled->stages[i];
+        const void* from = context->work_dev[i & 1u];
+        void* to = context->work_dev[(i + 1u) & 1u];
+        const uint64_t elements = rows * stage->d_in;
+        int handled = 0;
+        switch (stage->kind) {
+            case PLAN_QLINEAR:
+                handled = vxhip_qlinear_forward(context->ctx, stage->qlinear, from, to, NULL, (uint32_t)rows,
+                                                stage->input_scale, stage->input_zero_point, stage->output_scale,
+                                                stage->output_zero_point, (uint32_t)stage->input_dtype,
+                                                (uint32_t)stage->output_dtype);
+                break;
+            case PLAN_PACKED_LINEAR:
+                handled = vxhip_packed_linear_forward_f32(context->ctx, stage->packed, (const float*)from, (float*)to,
+                                                          (uint32_t)rows) == 0;
+                break;
+            case PLAN_QUANTIZE:
+                handled = elements <= UINT32_MAX &&
+                          vxhip_quantize_forward(context->ctx, (const float*)from, (uint32_t)elements, to,
+                                                 stage->input_scale, stage->input_zero_point,
+                                                 (uint32_t)stage->output_dtype);
+                break;
+            case PLAN_DEQUANTIZE:
+                handled = elements <= UINT32_MAX &&
+                          vxhip_dequantize_forward(context->ctx, from, (uint32_t)elements, stage->input_scale,
+                                                   stage->input_zero_point, (uint32_t)stage->input_dtype, (float*)to);
+                break;
+        }
         if (!handled) status = VX_STATUS_EXECUTION_FAILED;
     }
     if (status == VX_STATUS_OK)
-        status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host, context->output_dev, output_bytes);
+        status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host,
+                                                context->work_dev[compiled->stage_count & 1u], output_bytes);
     if (status != VX_STATUS_OK)
         fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
     return status;
@@ -796,7 +970,7 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
                          context->output_host, (size_t)rows * compiled->d_out * compiled->output_element_bytes);
     if (status != VX_STATUS_OK) return status;
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear executed");
-    attest(report, vxhip_context_last_variant(context->ctx));
+    attest(report, compiled->stage_count, vxhip_context_last_variant(context->ctx));
     return VX_STATUS_OK;
 }
 
@@ -860,7 +1034,7 @@ static VxStatus hip_context_execute_batch(void* context_instance, const VxBacken
         if (status != VX_STATUS_OK) return status;
     }
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear batch executed");
-    attest(report, vxhip_context_last_variant(context->ctx));
+    attest(report, compiled->stage_count, vxhip_context_last_variant(context->ctx));
     return VX_STATUS_OK;
 }
 
@@ -904,7 +1078,7 @@ VxStatus volvoxai_hip_gfx950_backend_register(VxReport* report) {
 VxStatus volvoxai_hip_gfx950_inspect_package(const VxModelSource* source, VxPackedArithmetic arithmetic,
                                              uint32_t* d_in, uint32_t* d_out, int32_t* is_packed_linear,
                                              char* message, size_t message_capacity) {
-    PackagePlan plan;
+    ChainPlan plan;
     Failure failure = {VX_STATUS_OK, {0}};
     VxStatus status;
     if (!source || source->struct_size != sizeof(*source)) return VX_STATUS_INVALID_ARGUMENT;
@@ -913,8 +1087,8 @@ VxStatus volvoxai_hip_gfx950_inspect_package(const VxModelSource* source, VxPack
     if (status == VX_STATUS_OK) {
         if (d_in) *d_in = plan.d_in;
         if (d_out) *d_out = plan.d_out;
-        if (is_packed_linear) *is_packed_linear = plan.kind == PLAN_PACKED_LINEAR;
-        plan_release(&plan);
+        if (is_packed_linear) *is_packed_linear = plan.any_packed;
+        chain_release(&plan);
     }
     return status;
 }
