@@ -54,10 +54,21 @@ __global__ __launch_bounds__(1024) void prepare_i8_kernel(
     const float* src = x + (size_t)row * k;
     float maximum = 0.0f;
     uint32_t bad = 0u;
-    for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) {
+    // a thread's first elements stay in registers for the second pass (rows of up to 4096 at
+    // 1024 threads are then read once)
+    constexpr int kKept = 4;
+    float kept[kKept];
+#pragma unroll
+    for (int i = 0; i < kKept; i++) {
+        const uint32_t j = threadIdx.x + i * blockDim.x;
+        kept[i] = j < k ? src[j] : 0.0f;
+        bad |= finite_f32(kept[i]) ? 0u : 1u;
+        maximum = fmaxf(maximum, fabsf(kept[i]));  // fmaxf ignores a NaN operand; `bad` records it
+    }
+    for (uint32_t j = threadIdx.x + kKept * blockDim.x; j < k; j += blockDim.x) {
         const float v = src[j];
         bad |= finite_f32(v) ? 0u : 1u;
-        maximum = fmaxf(maximum, fabsf(v));  // fmaxf ignores a NaN operand; `bad` records it
+        maximum = fmaxf(maximum, fabsf(v));
     }
     for (int off = 32; off > 0; off >>= 1) {
         maximum = fmaxf(maximum, __shfl_down(maximum, off, 64));
@@ -77,7 +88,12 @@ __global__ __launch_bounds__(1024) void prepare_i8_kernel(
     float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
     int8_t* dst = prepared + (size_t)row * ld;
-    for (uint32_t j = threadIdx.x; j < ld; j += blockDim.x) {
+#pragma unroll
+    for (int i = 0; i < kKept; i++) {
+        const uint32_t j = threadIdx.x + i * blockDim.x;
+        if (j < ld) dst[j] = (int8_t)(!bad && j < k ? packed_round_i8(__fdiv_rn(kept[i], scale)) : 0);
+    }
+    for (uint32_t j = threadIdx.x + kKept * blockDim.x; j < ld; j += blockDim.x) {
         int32_t q = 0;
         if (!bad && j < k) q = packed_round_i8(__fdiv_rn(src[j], scale));
         dst[j] = (int8_t)q;

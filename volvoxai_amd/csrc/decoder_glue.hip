@@ -47,15 +47,16 @@ __device__ __forceinline__ float block_sum(float v, float* slots) {
 // clamped to +-127 with a true f32 divide; a non-finite row gets zero codes and a NaN scale.
 __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_t* codes, float* scale_out,
                                             float* slots) {
-    float maximum = 0.0f, bad = 0.0f;
+    // one reduction for both questions: a non-finite element counts as +inf, which no finite
+    // maximum can be
+    float maximum = 0.0f;
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) {
         const float v = vals[j];
-        if (!finite_f32(v)) bad = 1.0f;
-        maximum = fmaxf(maximum, fabsf(v));
+        maximum = fmaxf(maximum, finite_f32(v) ? fabsf(v) : __builtin_inff());
     }
     maximum = block_max(maximum, slots);
-    bad = block_max(bad, slots);
-    float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+    const float bad = maximum == __builtin_inff() ? 1.0f : 0.0f;
+    float scale = maximum == 0.0f || bad != 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x)
         codes[j] = bad != 0.0f ? (int8_t)0 : (int8_t)packed_round_i8(__fdiv_rn(vals[j], scale));
@@ -75,6 +76,8 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
     const uint32_t row = blockIdx.x;
     float* src = x + (size_t)row * d;
     double sum = 0.0;
+    // the first pass's gain is requested with the row, not after the reduction
+    const float gain_first = threadIdx.x < d ? gain[threadIdx.x] : 0.0f;
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) {
         float v = src[j];
         if (delta) {
@@ -92,7 +95,8 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
     const double var = total / (double)d;
     const double inv_std = 1.0 / sqrt(var + eps);
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) {
-        const float y = (float)((double)vals[j] * inv_std * (double)gain[j]);
+        const float gj = j == threadIdx.x ? gain_first : gain[j];
+        const float y = (float)((double)vals[j] * inv_std * (double)gj);
         vals[j] = y;
         if (normalized) normalized[(size_t)row * d + j] = y;
     }
