@@ -191,7 +191,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     seen = set()
     try:
         for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
-                      "a8-mfma.t64x64"):
+                      "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -200,7 +200,8 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     finally:
         vx.force_variant(None)
     # one scale group per k-step has no eight-wave tile: that request runs the four-wave one
-    assert len(seen) == (5 if group == 32 else 6), seen
+    # (the pipelined 128x128 tile exists for one group per k-block only, i.e. G = 128)
+    assert len(seen) == (5 if group == 32 else 7 if group == 128 else 6), seen
     pl.close()
 
 
@@ -258,7 +259,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     seen = set()
     try:
         for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
-                      "a8-mfma.t64x64"):
+                      "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -266,7 +267,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert all("w4a8" in v for v in seen) and len(seen) == (5 if group == 32 else 6), seen
+    assert all("w4a8" in v for v in seen) and len(seen) == (5 if group == 32 else 7 if group == 128 else 6), seen
     pl.close()
 
 

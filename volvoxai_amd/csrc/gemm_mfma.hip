@@ -74,6 +74,11 @@ __device__ __forceinline__ void load_to_lds16(const void* gptr, void* lptr) {
                                      (__attribute__((address_space(3))) void*)lptr, 16, 0, 0);
 }
 
+__device__ __forceinline__ void load_to_lds4(const void* gptr, void* lptr) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
+                                     (__attribute__((address_space(3))) void*)lptr, 4, 0, 0);
+}
+
 struct GemmParams {
     LinearArgs a;
     uint32_t tiles_n, tiles_m;
@@ -116,8 +121,19 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     static_assert(!W4 || MODE == (int)Epilogue::DequantF32, "four-bit weights dequantize only");
     static_assert(WBLK % NWAVES == 0 && XBLK % NWAVES == 0, "blocks must divide over waves");
     constexpr int WLOADS = WBLK / NWAVES, XLOADS = XBLK / NWAVES;
-    constexpr int STAGE_BYTES = (WBLK + XBLK) * 1024;
     constexpr bool F32OUT = MODE == (int)Epilogue::DequantF32;
+    // PIPE (dequantizing epilogue, one scale group per k-block, wave tiles of at most two MFMA
+    // tiles): two sets of tile accumulators by k-block parity.  While the MFMAs of k-block kb fill
+    // one set, the fold of group kb-1 (four VALU operations per output) drains the other in the
+    // MFMAs' shadow, four outputs after each MFMA, instead of following them.  The group's BN
+    // weight scales travel with the operands, as the tail of the stage of the k-block that folds
+    // them: a vector load in the loop would be waited for by the compiler, together with every
+    // operand load requested before it.  (Larger wave tiles do not fit two accumulator sets in
+    // the 256 VGPRs of a two-waves-per-SIMD kernel, and with AGPRs in play the compiler copies
+    // accumulators back and forth wholesale, which measured slower than not overlapping.)
+    constexpr bool PIPE = F32OUT && GK == KS && TN * TM <= 2;
+    constexpr int SCALE_OFF = (WBLK + XBLK) * 1024;
+    constexpr int STAGE_BYTES = SCALE_OFF + (PIPE ? BN * 4 : 0);
     const LinearArgs& a = p.a;
 
     const int lane = threadIdx.x & 63;
@@ -171,6 +187,15 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     auto issue_one = [&](auto t_tag, uint32_t kb, int stage) {
         constexpr int t = decltype(t_tag)::value;
         if (VXHIP_PROBE_NO_LOADS && kb > 0) return;
+        if constexpr (PIPE && t == 0) {
+            // stage of k-block kb: the scales of group kb-1, which that k-block folds (kb = 0
+            // folds zeros; any finite scales do).  64 channels per wavefront, 4 bytes per lane.
+            if (wave < BN / 64) {
+                const uint32_t g = min(max(kb, 1u) - 1u, a.groups - 1u);
+                load_to_lds4(a.scales_t + (size_t)g * a.n_pad + n0 + wave * 64 + lane,
+                             lds_raw + stage * STAGE_BYTES + SCALE_OFF + wave * 256);
+            }
+        }
         kb = min(kb, nkb - 1u);
         if (VXHIP_PROBE_SAME_KB) kb = kb & 1u;  // same two k-blocks over and over: cache hits only
         char* base = lds_raw + stage * STAGE_BYTES;
@@ -187,13 +212,17 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     };
     // ---- accumulators --------------------------------------------------------
     v16i acc[TN][TM];
+    v16i acc_odd[PIPE ? TN : 1][PIPE ? TM : 1];  // PIPE: accumulators of the odd k-blocks
     v16i fsum[F32OUT ? TN : 1][F32OUT ? TM : 1];
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int j = 0; j < TM; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+            for (int r = 0; r < 16; r++) {
+                acc[i][j][r] = 0;
+                if constexpr (PIPE) acc_odd[i][j][r] = 0;
+            }
     if constexpr (F32OUT) {
 #pragma unroll
         for (int i = 0; i < TN; i++)
@@ -231,7 +260,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                     sw_next[i][q] = *reinterpret_cast<const v4f*>(srow + nbase + i * 32 + q * 8);
         }
     };
-    load_scales(0);
+    if constexpr (!PIPE) load_scales(0);
     auto fold_group = [&](uint32_t g) {
         if constexpr (F32OUT) {
 #pragma unroll
@@ -256,6 +285,39 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                 }
             }
             load_scales(g + 1u);
+        }
+    };
+
+    // PIPE: the fold of the accumulator set of parity P, four outputs (one quad of one tile) per
+    // slot.  Slots are ordered (tile column i, quad q, tile row j), so a unit u = (i, q) of four
+    // channel scales serves TM consecutive slots; it is read from the stage one unit ahead, the
+    // first unit of the next k-block from that block's stage (the last unit lies in the step after
+    // the barrier, when that stage has landed).
+    constexpr int UNITS = TN * 4;
+    v4f sw_ring[PIPE ? 2 : 1];
+    const uint32_t sw_lane = (uint32_t)(wave_n * TN * 32 + (lane >> 5) * 4) * 4u + SCALE_OFF;
+    auto read_scale_unit = [&](auto unit_tag, const char* stage) {
+        constexpr int u = decltype(unit_tag)::value;
+        sw_ring[u & 1] = *reinterpret_cast<const v4f*>(stage + sw_lane + ((u / 4) * 32 + (u % 4) * 8) * 4);
+    };
+    auto fold_slot = [&](auto parity_tag, auto idx_tag, const char* stage, const char* next_stage, auto more_tag) {
+        constexpr int P = decltype(parity_tag)::value, IDX = decltype(idx_tag)::value;
+        constexpr int u = IDX / TM, j = IDX % TM, i = u / 4, q = u % 4;
+        if constexpr (j == 0) {
+            if constexpr (u + 1 < UNITS) read_scale_unit(IC<u + 1>{}, stage);
+            else if constexpr (decltype(more_tag)::value) read_scale_unit(IC<0>{}, next_stage);
+        }
+        const v4f sw = sw_ring[u & 1];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int r = q * 4 + e;
+            const int32_t dot = (P == 0 ? acc[i][j][r] : acc_odd[i][j][r]) >> (W4 ? 4 : 0);
+            const float gs = __fmul_rn(row_scale[j], sw[e]);
+            float sum = __fadd_rn(__int_as_float(fsum[i][j][r]), __fmul_rn((float)dot, gs));
+            // the sum is needed only after the loop, and left to itself the optimizer collects all
+            // folds of a k-block behind its MFMAs; this pins each where it is written
+            asm volatile("" : "+v"(sum));
+            fsum[i][j][r] = __float_as_int(sum);
         }
     };
 
@@ -324,8 +386,9 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // load_stage.  (All of a stage's loads go out in the step after the barrier: issuing part
     // of them a step or two later measured slower, they then land too late.)
     auto step = [&](auto s_tag, auto read_tag, auto rs_tag, const char* rstage, auto nl_tag, uint32_t load_kb,
-                    int load_stage, uint32_t kb) {
+                    int load_stage, uint32_t kb, auto parity_tag, const char* cstage) {
         constexpr int S = decltype(s_tag)::value;
+        constexpr int P = decltype(parity_tag)::value;  // k-block parity (PIPE)
         constexpr bool READ = decltype(read_tag)::value;
         constexpr int NL = decltype(nl_tag)::value;
         constexpr int CB = S & 1, NB = CB ^ 1;
@@ -347,8 +410,14 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                 // first k-step of a scale group: accumulate onto zero instead of clearing registers
                 constexpr bool FRESH = F32OUT && GK <= KS && (S % GK) == 0;
                 const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], FRESH ? zero : acc[i][j], 0, 0, 0);
+                if constexpr (PIPE && P == 1)
+                    acc_odd[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j],
+                                                                          FRESH ? zero : acc_odd[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], FRESH ? zero : acc[i][j], 0, 0, 0);
             }
+            // PIPE: one slot (four outputs) of the other set's fold rides behind every MFMA
+            if constexpr (PIPE) fold_slot(IC<P ^ 1>{}, IC<S * MF + m>{}, cstage, rstage, read_tag);
             // after MFMA m: the reads and loads whose slot it is.  Reads keep clear of the
             // step's last MFMAs, which cover the latency of the final read.
             if constexpr (READ) {
@@ -363,9 +432,9 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                     if constexpr ((l * MF) / NL == m) issue_one(l_tag, load_kb, load_stage);
                 });
             }
-            if constexpr (!F32OUT) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (!F32OUT || PIPE) __builtin_amdgcn_sched_barrier(0);
         });
-        if constexpr (F32OUT) {
+        if constexpr (F32OUT && !PIPE) {
             if constexpr (GK <= KS) {
                 if ((S + 1) % GK == 0) fold_group((kb * KS + S) / GK);
             }
@@ -383,13 +452,14 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // count on every block having been requested)
     static_for<NLOADS>([&](auto t) { issue_one(t, NS - 1, NS - 1); });
     static_for<READS>([&](auto r) { read_one(r, lds_raw, IC<0>{}, wf[0], xf[0]); });
-    auto k_block = [&](uint32_t kb, auto last_tag) {
+    if constexpr (PIPE) read_scale_unit(IC<0>{}, lds_raw);
+    auto k_block = [&](uint32_t kb, auto last_tag, auto parity_tag) {
         constexpr bool LAST = decltype(last_tag)::value;
         const int cur = kb & (NS - 1);
         const char* stage = lds_raw + cur * STAGE_BYTES;
         static_for<KS - 1>([&](auto s_tag) {
             constexpr int S = decltype(s_tag)::value;
-            step(s_tag, std::true_type{}, IC<S + 1>{}, stage, IC<0>{}, 0u, 0, kb);
+            step(s_tag, std::true_type{}, IC<S + 1>{}, stage, IC<0>{}, 0u, 0, kb, parity_tag, stage);
         });
         if constexpr (!LAST) {
             wait_lgkm0();     // my reads of this stage have landed in registers
@@ -397,16 +467,41 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             if (!VXHIP_PROBE_NO_VMWAIT) wait_vmcnt<(NS - 2) * NLOADS>();
             wg_barrier();
             step(IC<KS - 1>{}, std::true_type{}, IC<0>{}, lds_raw + ((cur + 1) & (NS - 1)) * STAGE_BYTES,
-                 IC<NLOADS>{}, kb + NS, cur, kb);
+                 IC<NLOADS>{}, kb + NS, cur, kb, parity_tag, stage);
         } else {
-            step(IC<KS - 1>{}, std::false_type{}, IC<0>{}, stage, IC<0>{}, 0u, 0, kb);
+            step(IC<KS - 1>{}, std::false_type{}, IC<0>{}, stage, IC<0>{}, 0u, 0, kb, parity_tag, stage);
         }
         if constexpr (F32OUT && (GK > KS)) {
             if (((kb + 1) * KS) % GK == 0 || kb + 1 == nkb) fold_group((kb * KS) / GK);
         }
     };
-    for (uint32_t kb = 0; kb + 1 < nkb; kb++) k_block(kb, std::false_type{});
-    k_block(nkb - 1u, std::true_type{});
+    if constexpr (PIPE) {
+        // pairs of k-blocks, so that the parity of a block is a compile-time fact; then the one or
+        // two blocks that are left, and the fold of the last group, which has no MFMAs to hide in
+        uint32_t kb = 0;
+        for (; kb + 2 < nkb; kb += 2) {
+            k_block(kb, std::false_type{}, IC<0>{});
+            k_block(kb + 1, std::false_type{}, IC<1>{});
+        }
+        if (kb + 2 == nkb) {
+            k_block(kb, std::false_type{}, IC<0>{});
+            k_block(kb + 1, std::true_type{}, IC<1>{});
+        } else {
+            k_block(kb, std::true_type{}, IC<0>{});
+        }
+        // the last group's scales are the tail of the stage requested as k-block nkb
+        wait_vmcnt<0>();
+        wg_barrier();
+        const char* last_stage = lds_raw + (nkb & (NS - 1)) * STAGE_BYTES;
+        read_scale_unit(IC<0>{}, last_stage);
+        if (nkb & 1u)
+            static_for<TN * TM * 4>([&](auto idx) { fold_slot(IC<0>{}, idx, last_stage, last_stage, std::false_type{}); });
+        else
+            static_for<TN * TM * 4>([&](auto idx) { fold_slot(IC<1>{}, idx, last_stage, last_stage, std::false_type{}); });
+    } else {
+        for (uint32_t kb = 0; kb + 1 < nkb; kb++) k_block(kb, std::false_type{}, IC<0>{});
+        k_block(nkb - 1u, std::true_type{}, IC<0>{});
+    }
     wait_vmcnt<0>();  // nothing of this workgroup may still be writing LDS when the epilogue reuses it
     uint64_t probe_loop_end = 0;
     if (VXHIP_PROBE_CLOCK) {
@@ -582,7 +677,8 @@ template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4, 
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 32, BM = WM * TM * 32;
     // the stages and, behind them, the per-channel epilogue constants
-    constexpr int LDS = NS * ((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + BN * 16;
+    constexpr bool PIPE = MODE == (int)Epilogue::DequantF32 && GK == KS && TN * TM <= 2;  // as in the kernel
+    constexpr int LDS = NS * (((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + (PIPE ? BN * 4 : 0)) + BN * 16;
     static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
     static bool configured = false;
     auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST, W4, NS>;
@@ -630,6 +726,13 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (forced("t128x128")) pick = 1;
         if (forced("t64x128")) pick = 2;
         if (forced("t64x64")) pick = 3;
+        if constexpr (GK == KS) {
+            // one group per k-block: eight waves of 64x32 fold in the shadow of their MFMAs.  Measured
+            // against the plain 128x128 tile: 30 against 42 us at 4096x3072 -> 1024, 36 against 50 us
+            // at 256x4096 -> 14336; the 128x256 tile stays ahead where there is work for it.
+            if ((pick == 1 && !forced("t128x128")) || forced("t128x128p"))
+                return launch_cfg<2, 4, 2, 1, MODE, GK, W4>(s, a) ? "t128x128p" : nullptr;
+        }
         if (pick == 0) return launch_cfg<2, 4, 2, 2, MODE, GK, W4>(s, a) ? "t128x256" : nullptr;
         if (pick == 1) return launch_cfg<2, 2, 2, 2, MODE, GK, W4>(s, a) ? "t128x128" : nullptr;
         if (pick == 2) return launch_cfg<2, 2, 1, 2, MODE, GK, W4>(s, a) ? "t64x128" : nullptr;
