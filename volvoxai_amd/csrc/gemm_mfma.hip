@@ -290,24 +290,26 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
 
     // PIPE: the fold of the accumulator set of parity P, four outputs (one quad of one tile) per
     // slot.  Slots are ordered (tile column i, quad q, tile row j), so a unit u = (i, q) of four
-    // channel scales serves TM consecutive slots; it is read from the stage one unit ahead, the
-    // first unit of the next k-block from that block's stage (the last unit lies in the step after
-    // the barrier, when that stage has landed).
+    // channel scales serves TM consecutive slots; it is read from the stage AHEAD units ahead, the
+    // first units of the next k-block from that block's stage (which has landed in the step after
+    // the barrier; AHEAD is chosen so that no earlier step reaches for it).  Two ahead lets the
+    // wait before a fold name the one read it needs instead of draining the LDS queue.
     constexpr int UNITS = TN * 4;
-    v4f sw_ring[PIPE ? 2 : 1];
+    constexpr int AHEAD = UNITS / KS >= 2 ? 2 : 1;
+    v4f sw_ring[PIPE ? 4 : 1];
     const uint32_t sw_lane = (uint32_t)(wave_n * TN * 32 + (lane >> 5) * 4) * 4u + SCALE_OFF;
     auto read_scale_unit = [&](auto unit_tag, const char* stage) {
         constexpr int u = decltype(unit_tag)::value;
-        sw_ring[u & 1] = *reinterpret_cast<const v4f*>(stage + sw_lane + ((u / 4) * 32 + (u % 4) * 8) * 4);
+        sw_ring[u & 3] = *reinterpret_cast<const v4f*>(stage + sw_lane + ((u / 4) * 32 + (u % 4) * 8) * 4);
     };
     auto fold_slot = [&](auto parity_tag, auto idx_tag, const char* stage, const char* next_stage, auto more_tag) {
         constexpr int P = decltype(parity_tag)::value, IDX = decltype(idx_tag)::value;
         constexpr int u = IDX / TM, j = IDX % TM, i = u / 4, q = u % 4;
         if constexpr (j == 0) {
-            if constexpr (u + 1 < UNITS) read_scale_unit(IC<u + 1>{}, stage);
-            else if constexpr (decltype(more_tag)::value) read_scale_unit(IC<0>{}, next_stage);
+            if constexpr (u + AHEAD < UNITS) read_scale_unit(IC<u + AHEAD>{}, stage);
+            else if constexpr (decltype(more_tag)::value) read_scale_unit(IC<u + AHEAD - UNITS>{}, next_stage);
         }
-        const v4f sw = sw_ring[u & 1];
+        const v4f sw = sw_ring[u & 3];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const int r = q * 4 + e;
@@ -452,7 +454,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // count on every block having been requested)
     static_for<NLOADS>([&](auto t) { issue_one(t, NS - 1, NS - 1); });
     static_for<READS>([&](auto r) { read_one(r, lds_raw, IC<0>{}, wf[0], xf[0]); });
-    if constexpr (PIPE) read_scale_unit(IC<0>{}, lds_raw);
+    if constexpr (PIPE) static_for<AHEAD>([&](auto u_tag) { read_scale_unit(u_tag, lds_raw); });
     auto k_block = [&](uint32_t kb, auto last_tag, auto parity_tag) {
         constexpr bool LAST = decltype(last_tag)::value;
         const int cur = kb & (NS - 1);
@@ -493,7 +495,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         wait_vmcnt<0>();
         wg_barrier();
         const char* last_stage = lds_raw + (nkb & (NS - 1)) * STAGE_BYTES;
-        read_scale_unit(IC<0>{}, last_stage);
+        static_for<AHEAD>([&](auto u_tag) { read_scale_unit(u_tag, last_stage); });
         if (nkb & 1u)
             static_for<TN * TM * 4>([&](auto idx) { fold_slot(IC<0>{}, idx, last_stage, last_stage, std::false_type{}); });
         else
