@@ -580,3 +580,52 @@ def test_random_shape_sweep_packed(ctx, oracle):
                 vx.force_variant(None)
             assert st == 0 and same_f32(host(y), want), (trial, rows, k, n, group, ctx.last_variant)
         pl.close()
+
+
+def test_every_tile_and_stage_variant_on_ragged_shapes(ctx, oracle):
+    """Seeded ragged shapes through every forced GEMM tile, stage count and the pipelined tile, for
+    both epilogue families and every packed width: each must give the oracle's bits."""
+    import volvoxai_amd as vx
+    rng = np.random.default_rng(31)
+    packed_variants = ("a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128", "a8-mfma.t64x64",
+                       "a8-mfma.t128x128p")
+    for trial in range(24):
+        rows = int(rng.choice([3, 33, 65, 128, 200, 257]))
+        k = int(rng.choice([31, 64, 129, 384, 640, 1153]))
+        n = int(rng.choice([5, 33, 64, 129, 256, 300]))
+        group = int(rng.choice([32, 64, 128, 128, 256]))
+        bits = int(rng.choice([8, 4, 3, 2]))
+        c = cases.packed_case(rows, k, n, group, 4000 + trial, with_bias=bool(trial % 2), special_rows=(trial % 5 == 0))
+        w = c["w"] if bits == 8 else cases.low_bit(c["w"], bits)
+        words = oracle.pack_w8_words(w) if bits == 8 else oracle.pack_low_bit_words(w, bits)
+        _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, bits=bits)
+        pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=bits)
+        xd = dev(c["x"])
+        try:
+            for force in packed_variants:
+                vx.force_variant(force)
+                st, y = pl.forward_f32(ctx, xd)
+                ctx.synchronize()
+                assert st == 0 and same_f32(host(y), want), (trial, rows, k, n, group, bits, ctx.last_variant)
+        finally:
+            vx.force_variant(None)
+        pl.close()
+    q_variants = ("mfma-i8.t128x128s2", "mfma-i8.t128x128s4", "mfma-i8.t128x64s2", "mfma-i8.t128x64s4",
+                  "mfma-i8.t64x64", "mfma-i8.t256x128", "mfma-i8.t256x256")
+    for trial in range(24):
+        rows = int(rng.choice([2, 33, 64, 129, 300]))
+        k = int(rng.choice([15, 64, 127, 385, 777, 1024]))
+        n = int(rng.choice([7, 16, 48, 100, 144, 272]))
+        in_dt, w_dt, out_dt = (int(rng.choice([I8, U8])) for _ in range(3))
+        c = cases.qlinear_random_case(rows, k, n, 5000 + trial, in_dt, w_dt, out_dt, bool(trial % 3 == 0))
+        ok_w, want = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
+                                    c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
+        assert ok_w == 1
+        try:
+            for force in q_variants:
+                vx.force_variant(force)
+                (ok, y), variant = run_resident_qlinear(vx, ctx, c)
+                assert ok == 1 and (y == want).all(), (trial, rows, k, n, in_dt, w_dt, out_dt, variant)
+        finally:
+            vx.force_variant(None)
+    assert ctx.fault_flags() == 0
