@@ -125,6 +125,20 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* context, const float* q_dev,
                                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
                                 uint32_t max_seq, float* out_dev);
 
+/* One decode step (one new token per row) of the two entry points above in a
+ * single launch: rotates the q heads and the new k of qkv [rows, (q_heads +
+ * 2*kv_heads) * head_dim] at cache slot position_dev[0], appends the rotated k
+ * and the v to the caches at that slot, and attends over slots 0..position.
+ * out [rows, q_heads * head_dim] holds the same bits as vxhip_rope_append_kv
+ * followed by vxhip_gqa_attention with t = 1. */
+VxHipStatus vxhip_rope_gqa_attention_decode(VxHipContext* context, const float* qkv_dev,
+                                            const float* cos_dev, const float* sin_dev,
+                                            const int64_t* position_dev, uint32_t rows,
+                                            uint32_t q_heads, uint32_t kv_heads,
+                                            uint32_t head_dim, uint32_t max_seq,
+                                            float* k_cache_dev, float* v_cache_dev,
+                                            float* out_dev);
+
 /* Embedding lookup (src/kernels/embedding.inc:5-16): out [count, d_model] row i
  * = table [vocab, d_model] row tokens_dev[i] (int32 ids as in the reference).
  * An id outside the table gives a zero row and raises fault bit 2 of

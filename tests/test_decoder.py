@@ -160,6 +160,33 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,start,q_heads,kv_heads,head_dim", [(3, 0, 4, 2, 64), (2, 7, 16, 8, 128), (5, 255, 4, 4, 32),
+                                                                   (2, 300, 8, 1, 64)])
+def test_fused_decode_attention_equals_the_two_kernels(ctx, rows, start, q_heads, kv_heads, head_dim):
+    """One launch (rotary + cache append + attention) against rope_append_kv followed by gqa_attention
+    on the same inputs: the same output bits and the same caches, at the first slot, in the middle,
+    past 256 slots (a thread then owns two slots) and for a group of eight query heads."""
+    import torch
+    from volvoxai_amd import w8a8
+    rng = np.random.default_rng(rows + start)
+    max_seq = 384
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = torch.from_numpy(rng.normal(0, 1, (rows, 1, width)).astype(np.float32)).cuda()
+    angle = rng.uniform(0, 6.28, (max_seq, head_dim)).astype(np.float32)
+    cos, sin = torch.from_numpy(np.cos(angle)).cuda(), torch.from_numpy(np.sin(angle)).cuda()
+    cache = rng.normal(0, 1, (2, rows, kv_heads, max_seq, head_dim)).astype(np.float32)
+    k1, v1 = torch.from_numpy(cache[0]).cuda(), torch.from_numpy(cache[1]).cuda()
+    k2, v2 = k1.clone(), v1.clone()
+    pos = torch.tensor([start], dtype=torch.int64, device="cuda")
+    q = w8a8.rope_append_kv(ctx, qkv, cos, sin, pos, q_heads, kv_heads, head_dim, k1, v1)
+    want = w8a8.gqa_attention(ctx, q, k1, v1, pos).reshape(rows, -1)
+    got = w8a8.rope_gqa_attention_decode(ctx, qkv.reshape(rows, -1), cos, sin, pos, q_heads, kv_heads, head_dim, k2, v2)
+    ctx.synchronize()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@pytest.mark.gpu
 def test_embedding_gather_and_argmax_kernels(ctx, oracle):
     import torch
     from volvoxai_amd import w8a8

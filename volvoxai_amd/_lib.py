@@ -67,6 +67,7 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_swiglu_prepare_i8": (i32, [vp, vp, u32, u32, vp, vp, vp]),
         "vxhip_rope_append_kv": (i32, [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
         "vxhip_gqa_attention": (i32, [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]),
+        "vxhip_rope_gqa_attention_decode": (i32, [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, vp, vp, vp]),
         "vxhip_embedding_gather_f32": (i32, [vp, vp, vp, u32, u32, u32, vp]),
         "vxhip_argmax_rows_f32": (i32, [vp, vp, u32, u32, vp, vp, u32]),
         "vxhip_probe_mfma_rate": (i32, [vp, u32, u32, C.POINTER(C.c_double), C.POINTER(C.c_double),

@@ -155,32 +155,91 @@ __global__ void rope_append_kernel(const float* __restrict__ qkv, const float* _
 // scores[max_seq] + partial[8][head_dim] floats.  Scores: one thread per visible slot (its whole
 // dot products, 16-byte loads, all independent); P.V: the slots split over eight groups of
 // 32 threads, a thread four channels.
-template <int REP>
+//
+// FUSED (decode, t = 1): q is the qkv row as the linear wrote it.  The workgroup rotates its own
+// query heads and the new key of its KV head itself (the arithmetic of rope_append_kernel), uses
+// that key and the new value from LDS for the slot being appended, and the first workgroup of
+// each KV group also stores them in the caches for later steps; slots before the new one come
+// from the caches, so workgroups do not depend on each other.  Every slot is still handled by
+// the thread, and in the order, that the unfused kernel gives it: the results are the same bits.
+template <int REP, bool FUSED>
 __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restrict__ q,
-                                                            const float* __restrict__ k_cache,
-                                                            const float* __restrict__ v_cache,
+                                                            float* __restrict__ k_cache,
+                                                            float* __restrict__ v_cache,
                                                             const int64_t* __restrict__ positions, uint32_t t,
                                                             uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
-                                                            uint32_t max_seq, float scale, float* __restrict__ out) {
+                                                            uint32_t max_seq, float scale, float* __restrict__ out,
+                                                            const float* __restrict__ cos_table,
+                                                            const float* __restrict__ sin_table) {
     const uint32_t per_head = 9u * head_dim + max_seq;
     float* lds = reinterpret_cast<float*>(glue_lds);
+    float* k_new = lds + REP * per_head;  // FUSED: the appended key and value, head_dim floats each
+    float* v_new = k_new + head_dim;
     __shared__ float slots[4];
     const uint32_t token = blockIdx.x;
     const uint32_t head0 = blockIdx.y * REP;
     const uint32_t row = token / t, i = token % t;
     const uint32_t kvh = head0 / (q_heads / kv_heads);
-    const uint32_t visible = (uint32_t)positions[i] + 1u;  // slots 0 .. position
-    const float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
-    const float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    const uint32_t position = (uint32_t)positions[i];
+    const uint32_t visible = position + 1u;  // slots 0 .. position
+    // slots read from the caches: all visible ones, or all before the one being appended
+    const uint32_t cached = FUSED ? position : visible;
+    float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    if constexpr (FUSED) {
+        const uint32_t width = (q_heads + 2u * kv_heads) * head_dim, half = head_dim / 2u;
+        const float* src = q + (size_t)token * width;
+        const bool writer = head0 % (q_heads / kv_heads) == 0u;
+        auto rotated = [&](const float* head, uint32_t dd) {
+            const float partner = dd < half ? -head[dd + half] : head[dd - half];
+            const float c = cos_table[(size_t)position * head_dim + dd], sn = sin_table[(size_t)position * head_dim + dd];
+            return __fadd_rn(__fmul_rn(head[dd], c), __fmul_rn(partner, sn));
+        };
+        for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u) {
 #pragma unroll
-    for (int h = 0; h < REP; h++)
-        for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
-            lds[h * per_head + dd] = q[((size_t)token * q_heads + head0 + h) * head_dim + dd];
+            for (int h = 0; h < REP; h++) lds[h * per_head + dd] = rotated(src + (size_t)(head0 + h) * head_dim, dd);
+            const float kn = rotated(src + (size_t)(q_heads + kvh) * head_dim, dd);
+            const float vn = src[(size_t)(q_heads + kv_heads + kvh) * head_dim + dd];
+            k_new[dd] = kn;
+            v_new[dd] = vn;
+            if (writer) {
+                kbase[(size_t)position * head_dim + dd] = kn;
+                vbase[(size_t)position * head_dim + dd] = vn;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int h = 0; h < REP; h++)
+            for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
+                lds[h * per_head + dd] = q[((size_t)token * q_heads + head0 + h) * head_dim + dd];
+    }
     __syncthreads();
     float m[REP];
 #pragma unroll
     for (int h = 0; h < REP; h++) m[h] = -INFINITY;
-    for (uint32_t s = threadIdx.x; s < visible; s += 256u) {
+    if constexpr (FUSED) {
+        // the appended slot, from LDS; it is the last slot of the thread that owns it
+        if (threadIdx.x == position % 256u) {
+            float dot[REP];
+#pragma unroll
+            for (int h = 0; h < REP; h++) dot[h] = 0.0f;
+            for (uint32_t c = 0; c < head_dim / 4u; c++) {
+#pragma unroll
+                for (int h = 0; h < REP; h++) {
+                    const float* qs = lds + h * per_head;
+                    dot[h] += qs[4 * c] * k_new[4 * c] + qs[4 * c + 1] * k_new[4 * c + 1] +
+                              qs[4 * c + 2] * k_new[4 * c + 2] + qs[4 * c + 3] * k_new[4 * c + 3];
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < REP; h++) {
+                dot[h] = __fmul_rn(dot[h], scale);
+                lds[h * per_head + head_dim + position] = dot[h];
+                m[h] = fmaxf(m[h], dot[h]);
+            }
+        }
+    }
+    for (uint32_t s = threadIdx.x; s < cached; s += 256u) {
         const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)s * head_dim);
         float dot[REP];
 #pragma unroll
@@ -221,7 +280,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
 #pragma unroll
         for (int h = 0; h < REP; h++) acc[h] = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 8
-        for (uint32_t s = group; s < visible; s += 8u) {
+        for (uint32_t s = group; s < cached; s += 8u) {
             const float4 vv = *reinterpret_cast<const float4*>(vbase + (size_t)s * head_dim + c4);
 #pragma unroll
             for (int h = 0; h < REP; h++) {
@@ -230,6 +289,19 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
                 acc[h].y += p * vv.y;
                 acc[h].z += p * vv.z;
                 acc[h].w += p * vv.w;
+            }
+        }
+        if constexpr (FUSED) {
+            if (group == position % 8u) {  // the appended slot closes its group's sum
+                const float4 vv = *reinterpret_cast<const float4*>(v_new + c4);
+#pragma unroll
+                for (int h = 0; h < REP; h++) {
+                    const float p = lds[h * per_head + head_dim + position];
+                    acc[h].x += p * vv.x;
+                    acc[h].y += p * vv.y;
+                    acc[h].z += p * vv.z;
+                    acc[h].w += p * vv.w;
+                }
             }
         }
 #pragma unroll
@@ -426,13 +498,47 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
         return VXHIP_INVALID_ARGUMENT;
     }
     const dim3 grid(rows * t, q_heads / together);
-#define VXHIP_LAUNCH_ATTENTION(R)                                                                            \
-    hipLaunchKernelGGL(gqa_attention_kernel<R>, grid, dim3(256), lds, ctx->stream, q_dev, k_cache_dev,     \
-                       v_cache_dev, positions_dev, t, q_heads, kv_heads, head_dim, max_seq, scale, out_dev)
+#define VXHIP_LAUNCH_ATTENTION(R)                                                                               \
+    hipLaunchKernelGGL((gqa_attention_kernel<R, false>), grid, dim3(256), lds, ctx->stream, q_dev,              \
+                       const_cast<float*>(k_cache_dev), const_cast<float*>(v_cache_dev), positions_dev, t,     \
+                       q_heads, kv_heads, head_dim, max_seq, scale, out_dev, nullptr, nullptr)
     if (together == 4u) VXHIP_LAUNCH_ATTENTION(4);
     else if (together == 2u) VXHIP_LAUNCH_ATTENTION(2);
     else VXHIP_LAUNCH_ATTENTION(1);
 #undef VXHIP_LAUNCH_ATTENTION
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_rope_gqa_attention_decode(VxHipContext* ctx, const float* qkv_dev, const float* cos_dev,
+                                            const float* sin_dev, const int64_t* position_dev, uint32_t rows,
+                                            uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                            uint32_t max_seq, float* k_cache_dev, float* v_cache_dev,
+                                            float* out_dev) {
+    if (!ctx || !qkv_dev || !cos_dev || !sin_dev || !position_dev || !k_cache_dev || !v_cache_dev || !out_dev ||
+        !q_heads || !kv_heads || q_heads % kv_heads || !head_dim || head_dim % 4u || head_dim > 1024u || !max_seq) {
+        set_error("rope_gqa_attention_decode: null argument or unsupported geometry");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!rows) return VXHIP_OK;
+    if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
+    const float scale = (float)(1.0 / sqrt((double)head_dim));
+    const uint32_t rep = q_heads / kv_heads;
+    const uint32_t together = rep >= 8u && rep % 4u == 0u ? 4u : 1u;  // as in vxhip_gqa_attention
+    const size_t lds = ((size_t)together * (9u * head_dim + max_seq) + 2u * head_dim) * sizeof(float);
+    if (lds > 60u * 1024u) {
+        set_error("rope_gqa_attention_decode: head_dim/max_seq too large for the score buffer");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    const dim3 grid(rows, q_heads / together);
+    if (together == 4u)
+        hipLaunchKernelGGL((gqa_attention_kernel<4, true>), grid, dim3(256), lds, ctx->stream, qkv_dev, k_cache_dev,
+                           v_cache_dev, position_dev, 1u, q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev,
+                           sin_dev);
+    else
+        hipLaunchKernelGGL((gqa_attention_kernel<1, true>), grid, dim3(256), lds, ctx->stream, qkv_dev, k_cache_dev,
+                           v_cache_dev, position_dev, 1u, q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev,
+                           sin_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

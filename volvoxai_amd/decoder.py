@@ -171,6 +171,16 @@ class W8A8Decoder:
         else:
             a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, delta, L["gain1"], cfg.eps)
         qkv = self._linear_a8(L["qkv"], a8, sc).reshape(rows, t, -1)
+        if t == 1:
+            # a decode step: rotary, cache append and attention in one launch
+            attn = vx.rope_gqa_attention_decode(self.ctx, qkv.reshape(rows, -1), self.cos, self.sin, positions,
+                                                cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.k_cache[li],
+                                                self.v_cache[li])
+            o = self._linear(L["o"], attn)
+            a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, o, L["gain2"], cfg.eps)
+            gu = self._linear_a8(L["gate_up"], a8, sc)
+            a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
+            return self._linear_a8(L["down"], a8, sc)
         q = vx.rope_append_kv(self.ctx, qkv, self.cos, self.sin, positions, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
                               self.k_cache[li], self.v_cache[li])
         if t > 1:

@@ -263,6 +263,19 @@ def gqa_attention(ctx: Context, q, k_cache, v_cache, positions):
     return out
 
 
+def rope_gqa_attention_decode(ctx: Context, qkv, cos, sin, position, q_heads, kv_heads, head_dim, k_cache, v_cache):
+    """One decode step: qkv [rows, (q+2kv)*d]; rotary, cache append at slot position[0] and attention
+    in one launch; returns [rows, q_heads*d]."""
+    import torch
+    rows = qkv.shape[0]
+    out = torch.empty((rows, q_heads * head_dim), dtype=torch.float32, device=qkv.device)
+    _check(library().vxhip_rope_gqa_attention_decode(ctx._h, _dp(qkv), _dp(cos), _dp(sin), _dp(position), rows, q_heads,
+                                                     kv_heads, head_dim, k_cache.shape[2], _dp(k_cache), _dp(v_cache),
+                                                     _dp(out)),
+           "vxhip_rope_gqa_attention_decode")
+    return out
+
+
 def embedding_gather(ctx: Context, tokens_i32, table, out=None):
     """out[i] = table[tokens_i32[i]]; tokens int32 of any shape, table [vocab, d] f32."""
     import torch
