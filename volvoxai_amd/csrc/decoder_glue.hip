@@ -162,7 +162,14 @@ __global__ void rope_append_kernel(const float* __restrict__ qkv, const float* _
 // each KV group also stores them in the caches for later steps; slots before the new one come
 // from the caches, so workgroups do not depend on each other.  Every slot is still handled by
 // the thread, and in the order, that the unfused kernel gives it: the results are the same bits.
-template <int REP, bool FUSED>
+//
+// Scores, NC = head_dim / 32 in {1, 2, 4, 8}: eight lanes share a key row, each loading the 16-byte
+// chunks c = lane%8 + 8*i, so one load instruction of a wavefront covers eight rows with whole
+// 128-byte lines (a thread per row touches 64 lines with every load and refetches each of them
+// eight times once the rows outgrow the L1); the eight partial dots meet in three xor-shuffles.
+// Rows of four passes (128 slots) are requested before the first is used.  NC = 0 keeps the
+// thread-per-row loop for other head sizes.
+template <int REP, bool FUSED, int NC>
 __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restrict__ q,
                                                             float* __restrict__ k_cache,
                                                             float* __restrict__ v_cache,
@@ -217,49 +224,116 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     float m[REP];
 #pragma unroll
     for (int h = 0; h < REP; h++) m[h] = -INFINITY;
-    if constexpr (FUSED) {
-        // the appended slot, from LDS; it is the last slot of the thread that owns it
-        if (threadIdx.x == position % 256u) {
-            float dot[REP];
-#pragma unroll
-            for (int h = 0; h < REP; h++) dot[h] = 0.0f;
-            for (uint32_t c = 0; c < head_dim / 4u; c++) {
-#pragma unroll
-                for (int h = 0; h < REP; h++) {
-                    const float* qs = lds + h * per_head;
-                    dot[h] += qs[4 * c] * k_new[4 * c] + qs[4 * c + 1] * k_new[4 * c + 1] +
-                              qs[4 * c + 2] * k_new[4 * c + 2] + qs[4 * c + 3] * k_new[4 * c + 3];
-                }
-            }
+    if constexpr (NC > 0) {
+        const uint32_t lane8 = threadIdx.x & 7u, rowg = threadIdx.x >> 3;
+        // this lane's share of a row's dot with each query head, then the sum over the eight lanes
+        auto finish = [&](float (&dot)[REP], uint32_t slot) {
 #pragma unroll
             for (int h = 0; h < REP; h++) {
-                dot[h] = __fmul_rn(dot[h], scale);
-                lds[h * per_head + head_dim + position] = dot[h];
-                m[h] = fmaxf(m[h], dot[h]);
+                float d = dot[h];
+                d += __shfl_xor(d, 1, 64);
+                d += __shfl_xor(d, 2, 64);
+                d += __shfl_xor(d, 4, 64);
+                d = __fmul_rn(d, scale);
+                if (lane8 == 0u) lds[h * per_head + head_dim + slot] = d;
+                m[h] = fmaxf(m[h], d);
             }
-        }
-    }
-    for (uint32_t s = threadIdx.x; s < cached; s += 256u) {
-        const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)s * head_dim);
-        float dot[REP];
-#pragma unroll
-        for (int h = 0; h < REP; h++) dot[h] = 0.0f;
-#pragma unroll 8
-        for (uint32_t c = 0; c < head_dim / 4u; c++) {
-            const float4 kv = kr[c];
+        };
+        auto accumulate = [&](float (&dot)[REP], const float4& kv, uint32_t c) {
 #pragma unroll
             for (int h = 0; h < REP; h++) {
                 const float* qs = lds + h * per_head;
                 dot[h] += qs[4 * c] * kv.x + qs[4 * c + 1] * kv.y + qs[4 * c + 2] * kv.z + qs[4 * c + 3] * kv.w;
             }
-        }
+        };
+        constexpr int PASSES = 4;
+        for (uint32_t s0 = 0; s0 < cached; s0 += 32u * PASSES) {
+            float4 kv[PASSES][NC];
 #pragma unroll
-        for (int h = 0; h < REP; h++) {
-            dot[h] = __fmul_rn(dot[h], scale);
-            lds[h * per_head + head_dim + s] = dot[h];
-            m[h] = fmaxf(m[h], dot[h]);
+            for (int u = 0; u < PASSES; u++) {
+                const uint32_t srow = min(s0 + u * 32u + rowg, cached - 1u);  // rows past the end: a valid address
+                const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)srow * head_dim);
+#pragma unroll
+                for (int c = 0; c < NC; c++) kv[u][c] = kr[lane8 + 8u * c];
+            }
+#pragma unroll
+            for (int u = 0; u < PASSES; u++) {
+                const uint32_t srow = s0 + u * 32u + rowg;
+                float dot[REP];
+#pragma unroll
+                for (int h = 0; h < REP; h++) dot[h] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < NC; c++) accumulate(dot, kv[u][c], lane8 + 8u * c);
+                // (all 64 lanes take part in the shuffles; rows past the end are dropped here)
+                float keep[REP];
+#pragma unroll
+                for (int h = 0; h < REP; h++) keep[h] = m[h];
+                finish(dot, min(srow, cached - 1u));
+                if (srow >= cached) {
+#pragma unroll
+                    for (int h = 0; h < REP; h++) m[h] = keep[h];
+                }
+            }
+        }
+        if constexpr (FUSED) {
+            // the appended slot, from LDS, by the eight lanes that own it in the unfused kernel and in
+            // the same order of operations
+            if (rowg == position % 32u) {
+                float dot[REP];
+#pragma unroll
+                for (int h = 0; h < REP; h++) dot[h] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < NC; c++)
+                    accumulate(dot, *reinterpret_cast<const float4*>(k_new + 4u * (lane8 + 8u * c)), lane8 + 8u * c);
+                finish(dot, position);
+            }
+        }
+    } else {
+        if constexpr (FUSED) {
+            // the appended slot, from LDS; it is the last slot of the thread that owns it
+            if (threadIdx.x == position % 256u) {
+                float dot[REP];
+#pragma unroll
+                for (int h = 0; h < REP; h++) dot[h] = 0.0f;
+                for (uint32_t c = 0; c < head_dim / 4u; c++) {
+#pragma unroll
+                    for (int h = 0; h < REP; h++) {
+                        const float* qs = lds + h * per_head;
+                        dot[h] += qs[4 * c] * k_new[4 * c] + qs[4 * c + 1] * k_new[4 * c + 1] +
+                                  qs[4 * c + 2] * k_new[4 * c + 2] + qs[4 * c + 3] * k_new[4 * c + 3];
+                    }
+                }
+#pragma unroll
+                for (int h = 0; h < REP; h++) {
+                    dot[h] = __fmul_rn(dot[h], scale);
+                    lds[h * per_head + head_dim + position] = dot[h];
+                    m[h] = fmaxf(m[h], dot[h]);
+                }
+            }
+        }
+        for (uint32_t s = threadIdx.x; s < cached; s += 256u) {
+            const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)s * head_dim);
+            float dot[REP];
+#pragma unroll
+            for (int h = 0; h < REP; h++) dot[h] = 0.0f;
+#pragma unroll 8
+            for (uint32_t c = 0; c < head_dim / 4u; c++) {
+                const float4 kv = kr[c];
+#pragma unroll
+                for (int h = 0; h < REP; h++) {
+                    const float* qs = lds + h * per_head;
+                    dot[h] += qs[4 * c] * kv.x + qs[4 * c + 1] * kv.y + qs[4 * c + 2] * kv.z + qs[4 * c + 3] * kv.w;
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < REP; h++) {
+                dot[h] = __fmul_rn(dot[h], scale);
+                lds[h * per_head + head_dim + s] = dot[h];
+                m[h] = fmaxf(m[h], dot[h]);
+            }
         }
     }
+    __syncthreads();  // scores of a slot are read below by other threads than wrote them
 #pragma unroll
     for (int h = 0; h < REP; h++) {
         float* scores = lds + h * per_head + head_dim;
@@ -329,6 +403,31 @@ uint32_t row_block(uint32_t rows, uint32_t d) {
 
 bool device_ready(VxHipContext* ctx) {
     return ctx && hipSetDevice(ctx->device) == hipSuccess;
+}
+
+// Picks the instance for the query heads per workgroup (4 or 1) and the head size.
+template <bool FUSED>
+void launch_attention(hipStream_t stream, uint32_t together, dim3 grid, size_t lds, const float* q, float* k_cache,
+                      float* v_cache, const int64_t* positions, uint32_t t, uint32_t q_heads, uint32_t kv_heads,
+                      uint32_t head_dim, uint32_t max_seq, float scale, float* out, const float* cos_table,
+                      const float* sin_table) {
+#define VXHIP_ATTENTION(R, NC)                                                                                  \
+    hipLaunchKernelGGL((gqa_attention_kernel<R, FUSED, NC>), grid, dim3(256), lds, stream, q, k_cache, v_cache, \
+                       positions, t, q_heads, kv_heads, head_dim, max_seq, scale, out, cos_table, sin_table)
+#define VXHIP_ATTENTION_HEADS(NC)     \
+    do {                              \
+        if (together == 4u) VXHIP_ATTENTION(4, NC); \
+        else VXHIP_ATTENTION(1, NC);  \
+    } while (0)
+    switch (head_dim) {
+        case 32: VXHIP_ATTENTION_HEADS(1); break;
+        case 64: VXHIP_ATTENTION_HEADS(2); break;
+        case 128: VXHIP_ATTENTION_HEADS(4); break;
+        case 256: VXHIP_ATTENTION_HEADS(8); break;
+        default: VXHIP_ATTENTION_HEADS(0); break;
+    }
+#undef VXHIP_ATTENTION_HEADS
+#undef VXHIP_ATTENTION
 }
 
 // Embedding lookup (embedding.inc:5-16): out[i] = table[tokens[i]], one workgroup per token.
@@ -498,14 +597,9 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
         return VXHIP_INVALID_ARGUMENT;
     }
     const dim3 grid(rows * t, q_heads / together);
-#define VXHIP_LAUNCH_ATTENTION(R)                                                                               \
-    hipLaunchKernelGGL((gqa_attention_kernel<R, false>), grid, dim3(256), lds, ctx->stream, q_dev,              \
-                       const_cast<float*>(k_cache_dev), const_cast<float*>(v_cache_dev), positions_dev, t,     \
-                       q_heads, kv_heads, head_dim, max_seq, scale, out_dev, nullptr, nullptr)
-    if (together == 4u) VXHIP_LAUNCH_ATTENTION(4);
-    else if (together == 2u) VXHIP_LAUNCH_ATTENTION(2);
-    else VXHIP_LAUNCH_ATTENTION(1);
-#undef VXHIP_LAUNCH_ATTENTION
+    launch_attention<false>(ctx->stream, together, grid, lds, q_dev, const_cast<float*>(k_cache_dev),
+                            const_cast<float*>(v_cache_dev), positions_dev, t, q_heads, kv_heads, head_dim, max_seq,
+                            scale, out_dev, nullptr, nullptr);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -531,14 +625,8 @@ VxHipStatus vxhip_rope_gqa_attention_decode(VxHipContext* ctx, const float* qkv_
         return VXHIP_INVALID_ARGUMENT;
     }
     const dim3 grid(rows, q_heads / together);
-    if (together == 4u)
-        hipLaunchKernelGGL((gqa_attention_kernel<4, true>), grid, dim3(256), lds, ctx->stream, qkv_dev, k_cache_dev,
-                           v_cache_dev, position_dev, 1u, q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev,
-                           sin_dev);
-    else
-        hipLaunchKernelGGL((gqa_attention_kernel<1, true>), grid, dim3(256), lds, ctx->stream, qkv_dev, k_cache_dev,
-                           v_cache_dev, position_dev, 1u, q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev,
-                           sin_dev);
+    launch_attention<true>(ctx->stream, together, grid, lds, qkv_dev, k_cache_dev, v_cache_dev, position_dev, 1u,
+                           q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev, sin_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
