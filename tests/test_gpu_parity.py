@@ -167,7 +167,7 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
                              c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w8", "mfma-i8.t128x128s2", "mfma-i8.t256x256", "mfma-i8.t256x128",
+        for force in ("gemv.w2", "gemv.w8c32", "gemv.w8c8", "gemv.w16c16", "mfma-i8.t128x128s2", "mfma-i8.t256x256", "mfma-i8.t256x128",
                       "mfma-i8.t128x64s2", "mfma-i8.t256x128w4", "mfma-i8.t128x128s4", "mfma-i8.t128x64s4",
                       "mfma-i8.t64x64"):
             vx.force_variant(force)
@@ -176,7 +176,7 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
             seen.add(variant)
     finally:
         vx.force_variant(None)
-    assert len(seen) == 10, seen
+    assert len(seen) == 12, seen
 
 
 @pytest.mark.parametrize("group", [32, 64, 128, 256])
@@ -190,7 +190,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+        for force in ("gemv.w2", "gemv.w16c32", "gemv.w16c8", "gemv.w8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
                       "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
@@ -201,7 +201,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
         vx.force_variant(None)
     # one scale group per k-step has no eight-wave tile: that request runs the four-wave one
     # (the pipelined 128x128 tile exists for one group per k-block only, i.e. G = 128)
-    assert len(seen) == (5 if group == 32 else 7 if group == 128 else 6), seen
+    assert len(seen) == (7 if group == 32 else 9 if group == 128 else 8), seen
     pl.close()
 
 
@@ -258,7 +258,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+        for force in ("gemv.w2", "gemv.w16c32", "gemv.w16c8", "gemv.w8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
                       "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
@@ -267,7 +267,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert all("w4a8" in v for v in seen) and len(seen) == (5 if group == 32 else 7 if group == 128 else 6), seen
+    assert all("w4a8" in v for v in seen) and len(seen) == (7 if group == 32 else 9 if group == 128 else 8), seen
     pl.close()
 
 

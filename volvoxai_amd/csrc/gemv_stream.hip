@@ -54,9 +54,19 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 // wavefronts of the workgroup, all sharing one panel.  W4: four-bit weights, a 1 KiB block
 // then carries two k-steps and is split into their operands in registers (three VALU
 // operations per dword), so the stream is half as long for the same K.
-template <int MODE, int GK, int WAVES, bool W4>
+//
+// SPLIT (1, 2 or 4): workgroups per panel.  A matrix of few panels (N = 1024 is 32 of them) leaves
+// most compute units without a workgroup; then SPLIT workgroups share a panel, each taking
+// CH = 32 / SPLIT of its channels.  A workgroup reads only the bytes of a block that hold its
+// channels (whole 128-byte lines: eight channels are lanes 8q..8q+7 and 32+8q..32+8q+7): the other
+// lanes are pointed at the same lines, so nothing in the stream becomes conditional, the MFMA runs
+// on a full operand whose other rows repeat the workgroup's own, and only the accumulator quads of
+// the workgroup's channels are parked, folded and stored.
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT>
 __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
+    constexpr int CH = 32 / SPLIT;     // channels of this workgroup
+    constexpr int QUADS = 4 / SPLIT;   // accumulator quads (8 channels each) of this workgroup
     static_assert(F || !W4, "four-bit weights exist for the dequantizing epilogue only");
     constexpr int SPB = W4 ? 2 : 1;              // k-steps per 1 KiB block
     constexpr int UNIT = GK > SPB ? GK : SPB;    // a wave's run is a whole number of these
@@ -68,8 +78,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     // predicated by the EXEC mask, so a guard the compiler took for divergent and turned into
     // EXEC masking around a lone MFMA would not guard it.)
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const uint32_t panel = blockIdx.x;
+    const uint32_t panel = blockIdx.x / SPLIT, sub = blockIdx.x % SPLIT;
     const uint32_t rows = a.rows;
+    const uint32_t ch0 = panel * 32u + sub * CH;  // first channel of this workgroup
+    // the lane whose 16 bytes of a block this lane loads: itself when its channel is the
+    // workgroup's, else the lane that holds the workgroup's channel at the same offset
+    const uint32_t src_lane = SPLIT == 1 ? (uint32_t)lane : ((lane & 32) | (sub * CH + (lane & (CH - 1))));
 
     // this wave's run of k-steps, aligned to whole groups
     const uint32_t steps = (a.k + 31u) / 32u;
@@ -78,13 +92,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     const uint32_t t0 = min((uint32_t)wave * per * UNIT, steps);
     const uint32_t t1 = min((uint32_t)(wave + 1) * per * UNIT, steps);
 
-    const int8_t* wp = a.w + (size_t)panel * a.ksteps * 1024u + lane * 16u;
+    const int8_t* wp = a.w + (size_t)panel * a.ksteps * 1024u + src_lane * 16u;
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
     const int8_t* xp = a.x + (size_t)m * a.ldx;
     const uint32_t half = lane >> 5;
     const uint32_t last_chunk = (a.k - 1u) / 16u;
 
-    // LDS: F: dots[group][row][32] exact int32 group dots   R: parts[wave][row][32]
+    // LDS: F: dots[group][row][CH] exact int32 group dots   R: parts[wave][row][CH]
     int32_t* parts = reinterpret_cast<int32_t*>(gemv_lds);
     const bool row_live = (uint32_t)(lane & 31) < rows;
 
@@ -106,27 +120,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 
     // The tail's per-output operands (activation scale, bias) are requested now, so that their
     // latency hides behind the stream instead of following it.
-    constexpr int TAIL_ITERS = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);
+    constexpr int TAIL_ITERS = ((int)kMaxGemvRows * CH + WAVES * 64 - 1) / (WAVES * 64);
     float tail_rs[F ? TAIL_ITERS : 1], tail_bias[F ? TAIL_ITERS : 1];
     if constexpr (F) {
 #pragma unroll
         for (int it = 0; it < TAIL_ITERS; it++) {
             const uint32_t o = threadIdx.x + it * WAVES * 64;
-            tail_rs[it] = a.row_scale[min(o >> 5, rows - 1u)];
-            tail_bias[it] = a.bias_f32[panel * 32u + (o & 31u)];  // padded to whole panels
+            tail_rs[it] = a.row_scale[min(o / CH, rows - 1u)];
+            tail_bias[it] = a.bias_f32[ch0 + o % CH];  // padded to whole panels
         }
     }
 
     // F: the panel's group scales [group][32] are fetched first (they are L2 hits and return
     // ahead of the HBM stream) and kept in LDS for the tail.
     constexpr int SCALE_SLOTS = 4;  // per thread; covers groups * 32 <= SCALE_SLOTS * threads
-    float* lds_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)a.groups * rows * 32u;
+    float* lds_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)a.groups * rows * CH;
     float sc[F ? SCALE_SLOTS : 1];
     uint32_t sc_base = 0;
     if constexpr (F) {
-        const uint32_t total = a.groups * 32u;
+        const uint32_t total = a.groups * CH;
         auto fetch = [&](uint32_t e) {
-            return e < total ? a.scales_t[(size_t)(e >> 5) * a.n_pad + panel * 32u + (e & 31u)] : 0.0f;
+            return e < total ? a.scales_t[(size_t)(e / CH) * a.n_pad + ch0 + e % CH] : 0.0f;
         };
         // many groups on few waves: copy all but the last pass before the stream starts
         while (total - sc_base > (uint32_t)(SCALE_SLOTS * WAVES * 64)) {
@@ -146,11 +160,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     auto park = [&](uint32_t slab) {
         if (row_live) {
 #pragma unroll
-            for (int q = 0; q < 4; q++)
+            for (int q = 0; q < 4; q++) {
+                // quad q holds channels 8q..8q+7 of the panel; the test is scalar
+                if (SPLIT > 1 && (uint32_t)(q / QUADS) != sub) continue;
                 // four-bit operands carry a factor 16, which the exact dot sheds here
-                *reinterpret_cast<v4i*>(parts + ((size_t)slab * rows + (lane & 31)) * 32u + q * 8 + half * 4) =
+                *reinterpret_cast<v4i*>(parts + ((size_t)slab * rows + (lane & 31)) * CH + (q % QUADS) * 8 +
+                                        half * 4) =
                     v4i{acc[q * 4] >> (W4 ? 4 : 0), acc[q * 4 + 1] >> (W4 ? 4 : 0),
                         acc[q * 4 + 2] >> (W4 ? 4 : 0), acc[q * 4 + 3] >> (W4 ? 4 : 0)};
+            }
         }
     };
 
@@ -159,7 +177,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
             for (int u = 0; u < SCALE_SLOTS; u++) {
                 const uint32_t e = sc_base + threadIdx.x + u * WAVES * 64;
-                if (e < a.groups * 32u) lds_scales[e] = sc[u];
+                if (e < a.groups * CH) lds_scales[e] = sc[u];
             }
         }
     };
@@ -216,21 +234,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     __syncthreads();
     if (VXHIP_GEMV_PROBE) probe[2] = __builtin_amdgcn_s_memrealtime();
 
-    // Tail: one thread per output, index o = row * 32 + channel.  F: sum += f32(dot_g) *
+    // Tail: one thread per output, index o = row * CH + channel.  F: sum += f32(dot_g) *
     // (s_a * s_w[n][g]) in ascending group order with separate roundings
     // (packed_linear_ops.inc:1498-1504); eight groups' operands are requested before the
     // first add needs one.
-    const size_t slab = (size_t)rows * 32u;
+    const size_t slab = (size_t)rows * CH;
     if constexpr (F) {
 #pragma unroll
         for (int it = 0; it < TAIL_ITERS; it++) {
             const uint32_t o = threadIdx.x + it * WAVES * 64;
-            if (o >= rows * 32u) break;
-            const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
+            if (o >= rows * CH) break;
+            const uint32_t om = o / CH, on = ch0 + o % CH;
             const float rs = tail_rs[it];
             float sum = 0.0f;
             const int32_t* dp = parts + o;
-            const float* sp = lds_scales + (o & 31u);
+            const float* sp = lds_scales + o % CH;
             uint32_t g = 0;
             for (; g + 8u <= a.groups; g += 8u) {
                 int32_t d[8];
@@ -238,19 +256,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
                 for (int u = 0; u < 8; u++) {
                     d[u] = dp[(size_t)(g + u) * slab];
-                    sw[u] = sp[(g + u) * 32u];
+                    sw[u] = sp[(g + u) * CH];
                 }
 #pragma unroll
                 for (int u = 0; u < 8; u++)
                     sum = __fadd_rn(sum, __fmul_rn((float)d[u], __fmul_rn(rs, sw[u])));
             }
             for (; g < a.groups; g++)
-                sum = __fadd_rn(sum, __fmul_rn((float)dp[(size_t)g * slab], __fmul_rn(rs, sp[g * 32u])));
+                sum = __fadd_rn(sum, __fmul_rn((float)dp[(size_t)g * slab], __fmul_rn(rs, sp[g * CH])));
             if (on < a.n) ((float*)a.y)[(size_t)om * a.n + on] = __fadd_rn(sum, tail_bias[it]);
         }
     } else {
-        for (uint32_t o = threadIdx.x; o < rows * 32u; o += WAVES * 64) {
-            const uint32_t om = o >> 5, on = panel * 32u + (o & 31u);
+        for (uint32_t o = threadIdx.x; o < rows * CH; o += WAVES * 64) {
+            const uint32_t om = o / CH, on = ch0 + o % CH;
             float rs = 0.0f;
             if constexpr (MODE == (int)Epilogue::RequantRow) rs = a.row_scale[om];
             int32_t dot = 0;
@@ -269,9 +287,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     }
 }
 
-template <int MODE, int GK, int WAVES, bool W4>
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
-    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4>;
+    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT>;
     if (lds > 64u * 1024u) {
         static bool configured = false;
         if (!configured) {
@@ -281,12 +299,19 @@ bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
             configured = true;
         }
     }
-    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u * SPLIT), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError() == hipSuccess;
 }
 
+template <int MODE, int GK, int WAVES, bool W4>
+bool launch_split(hipStream_t s, const LinearArgs& a, size_t lds, int split) {
+    if (split == 4) return launch_panel<MODE, GK, WAVES, W4, 4>(s, a, lds);
+    if (split == 2) return launch_panel<MODE, GK, WAVES, W4, 2>(s, a, lds);
+    return launch_panel<MODE, GK, WAVES, W4, 1>(s, a, lds);
+}
+
 template <int MODE, int GK, bool W4 = false>
-const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
+const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     // blocks of the stream per panel, and the units a wave's run is made of
     constexpr uint32_t SPB = W4 ? 2 : 1, UNIT = GK > SPB ? GK : SPB;
     const uint32_t steps = ((a.k + 31u) / 32u + SPB - 1u) / SPB;  // 1 KiB blocks per panel
@@ -304,22 +329,37 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, const char* force) {
     else if (force && strstr(force, "w8")) waves = 8;
     else if (force && strstr(force, "w4")) waves = 4;
     else if (force && strstr(force, "w2")) waves = 2;
-    const size_t lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * (a.rows + 1u) * 128u
-                                                          : (size_t)waves * a.rows * 128u;
+    // Fewer panels than half the compute units: two or four workgroups share each panel's
+    // channels (only the 8- and 16-wave kernels are built that way; such shapes have them
+    // unless K is tiny).
+    int split = 1;
+    if (waves >= 8) {
+        split = panels * 4u <= (uint32_t)cu_count ? 4 : panels * 2u <= (uint32_t)cu_count ? 2 : 1;
+        if (force && strstr(force, "c8")) split = 4;
+        else if (force && strstr(force, "c16")) split = 2;
+        else if (force && strstr(force, "c32")) split = 1;
+    }
+    const size_t ch_bytes = 128u / (size_t)split;  // one row of the workgroup's channels, int32 or f32
+    const size_t lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * (a.rows + 1u) * ch_bytes
+                                                          : (size_t)waves * a.rows * ch_bytes;
     // the MFMA GEMM takes shapes whose group dots or scales do not fit
     if (lds > 156u * 1024u) return nullptr;
     bool ok = false;
-    if (waves == 16) ok = launch_panel<MODE, GK, 16, W4>(s, a, lds);
-    else if (waves == 8) ok = launch_panel<MODE, GK, 8, W4>(s, a, lds);
+    if (waves == 16) ok = launch_split<MODE, GK, 16, W4>(s, a, lds, split);
+    else if (waves == 8) ok = launch_split<MODE, GK, 8, W4>(s, a, lds, split);
     else if (waves == 4) ok = launch_panel<MODE, GK, 4, W4>(s, a, lds);
     else ok = launch_panel<MODE, GK, 2, W4>(s, a, lds);
-    return !ok ? nullptr : waves == 16 ? "w16" : waves == 8 ? "w8" : waves == 4 ? "w4" : "w2";
+    if (!ok) return nullptr;
+    static const char* const names[3][4] = {{"w2", "w4", "w8", "w16"},
+                                            {"w2", "w4", "w8c16", "w16c16"},
+                                            {"w2", "w4", "w8c8", "w16c8"}};
+    return names[split == 4 ? 2 : split == 2 ? 1 : 0][waves == 16 ? 3 : waves == 8 ? 2 : waves == 4 ? 1 : 0];
 }
 
 }  // namespace
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
-    (void)cu_count;
+    if (cu_count <= 0) cu_count = 256;
     if (a.rows == 0u || a.rows > kMaxGemvRows || a.ldx < 16u || (a.ldx % 16u) != 0u ||
         ((uintptr_t)a.x % 16u) != 0u)
         return nullptr;
@@ -329,30 +369,30 @@ const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count,
     switch (a.mode) {
         case Epilogue::RequantTensor:
             family = "hip.qlinear.gemv-mfma";
-            kind = launch_mode<(int)Epilogue::RequantTensor, 1>(s, a, force);
+            kind = launch_mode<(int)Epilogue::RequantTensor, 1>(s, a, cu_count, force);
             break;
         case Epilogue::RequantRow:
             family = "hip.qlinear.gemv-mfma-rowscale";
-            kind = launch_mode<(int)Epilogue::RequantRow, 1>(s, a, force);
+            kind = launch_mode<(int)Epilogue::RequantRow, 1>(s, a, cu_count, force);
             break;
         case Epilogue::DequantF32:
             if (a.weight_bits == 4u) {
                 family = "hip.packed-linear.w4a8-gemv-mfma";
                 switch (a.group_size) {
-                    case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1, true>(s, a, force); break;
-                    case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2, true>(s, a, force); break;
-                    case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4, true>(s, a, force); break;
-                    case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8, true>(s, a, force); break;
+                    case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1, true>(s, a, cu_count, force); break;
+                    case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2, true>(s, a, cu_count, force); break;
+                    case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4, true>(s, a, cu_count, force); break;
+                    case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8, true>(s, a, cu_count, force); break;
                     default: return nullptr;
                 }
                 break;
             }
             family = "hip.packed-linear.a8-gemv-mfma";
             switch (a.group_size) {
-                case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1>(s, a, force); break;
-                case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2>(s, a, force); break;
-                case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4>(s, a, force); break;
-                case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8>(s, a, force); break;
+                case 32: kind = launch_mode<(int)Epilogue::DequantF32, 1>(s, a, cu_count, force); break;
+                case 64: kind = launch_mode<(int)Epilogue::DequantF32, 2>(s, a, cu_count, force); break;
+                case 128: kind = launch_mode<(int)Epilogue::DequantF32, 4>(s, a, cu_count, force); break;
+                case 256: kind = launch_mode<(int)Epilogue::DequantF32, 8>(s, a, cu_count, force); break;
                 default: return nullptr;
             }
             break;
