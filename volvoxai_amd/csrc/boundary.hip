@@ -4,6 +4,7 @@
 // elementwise or per-row work.
 #include "common.h"
 #include "device_math.h"
+#include "wave_ops.h"
 
 namespace vxhip {
 
@@ -48,8 +49,8 @@ VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows
 __global__ __launch_bounds__(1024) void prepare_i8_kernel(
         const float* __restrict__ x, uint32_t k, int8_t* __restrict__ prepared, uint32_t ld,
         float* __restrict__ scales) {
-    __shared__ float wave_max[16];
-    __shared__ uint32_t wave_bad[16];
+    __shared__ float slot_max[16];
+    __shared__ uint32_t slot_bad[16];
     const uint32_t row = blockIdx.x;
     const float* src = x + (size_t)row * k;
     float maximum = 0.0f;
@@ -70,20 +71,18 @@ __global__ __launch_bounds__(1024) void prepare_i8_kernel(
         bad |= finite_f32(v) ? 0u : 1u;
         maximum = fmaxf(maximum, fabsf(v));
     }
-    for (int off = 32; off > 0; off >>= 1) {
-        maximum = fmaxf(maximum, __shfl_down(maximum, off, 64));
-        bad |= __shfl_down(bad, off, 64);
-    }
+    maximum = wave_max(maximum);
+    bad = __builtin_amdgcn_ballot_w64(bad != 0u) != 0ull ? 1u : 0u;
     if ((threadIdx.x & 63u) == 0u) {
-        wave_max[threadIdx.x >> 6] = maximum;
-        wave_bad[threadIdx.x >> 6] = bad;
+        slot_max[threadIdx.x >> 6] = maximum;
+        slot_bad[threadIdx.x >> 6] = bad;
     }
     __syncthreads();
-    maximum = wave_max[0];
-    bad = wave_bad[0];
+    maximum = slot_max[0];
+    bad = slot_bad[0];
     for (uint32_t w = 1; w < blockDim.x / 64u; w++) {
-        maximum = fmaxf(maximum, wave_max[w]);
-        bad |= wave_bad[w];
+        maximum = fmaxf(maximum, slot_max[w]);
+        bad |= slot_bad[w];
     }
     float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;

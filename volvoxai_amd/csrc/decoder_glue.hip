@@ -14,6 +14,7 @@
 // All are row-sized, latency-bound kernels; none of them is on the int8 roofline.
 #include "common.h"
 #include "device_math.h"
+#include "wave_ops.h"
 
 #include <math.h>
 
@@ -23,7 +24,7 @@ namespace {
 extern __shared__ __attribute__((aligned(16))) char glue_lds[];
 
 __device__ __forceinline__ float block_max(float v, float* slots) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off, 64));
+    v = wave_max(v);
     if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
     __syncthreads();
     float m = slots[0];
@@ -33,7 +34,7 @@ __device__ __forceinline__ float block_max(float v, float* slots) {
 }
 
 __device__ __forceinline__ float block_sum(float v, float* slots) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    v = wave_sum_to_lane0(v);
     if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
     __syncthreads();
     float s = slots[0];
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
         vals[j] = v;
         sum += (double)v * (double)v;
     }
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+    sum = wave_sum_to_lane0(sum);
     if ((threadIdx.x & 63u) == 0u) dslots[threadIdx.x >> 6] = sum;
     __syncthreads();
     double total = 0.0;
@@ -193,7 +194,69 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     const uint32_t cached = FUSED ? position : visible;
     float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
     float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
-    if constexpr (FUSED) {
+    // Cached rows arrive in blocks that are requested two blocks ahead of their use, the first
+    // two before the query is ready: every workgroup of the launch is resident at once and in the
+    // same phase, each dependent request costs all of them a round trip to a loaded memory
+    // (2-3 us), and up to 256 slots this way cost one for the keys and one for the values.  A
+    // request never depends on a branch: rows past the end are clamped to the last cached one
+    // (row 0 of the cache when there is none), so they cost no memory traffic and the waits
+    // stay exact.
+    // rows of PASSES passes of 32 are in a block (fewer at head size 256, whose rows are twice as
+    // long: the two blocks must leave room for three wavefronts per SIMD where they can)
+    constexpr int PASSES = NC > 4 ? 2 : 4, KC = NC > 0 ? NC : 1;
+    const uint32_t last_cached = max(cached, 1u) - 1u;
+    const uint32_t lane8 = threadIdx.x & 7u, rowg = threadIdx.x >> 3;
+    float4 kv_a[PASSES][KC], kv_b[PASSES][KC];
+    auto request_keys = [&](float4 (&buf)[PASSES][KC], uint32_t s0) {
+#pragma unroll
+        for (int u = 0; u < PASSES; u++) {
+            const uint32_t srow = min(s0 + u * 32u + rowg, last_cached);
+            const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)srow * head_dim);
+#pragma unroll
+            for (int c = 0; c < KC; c++) buf[u][c] = kr[lane8 + 8u * c];
+        }
+    };
+    if constexpr (FUSED && NC > 0) {
+        // (head sizes up to 256: a thread rotates at most one channel)  The operands of the rotation
+        // are requested before the keys: loads return in order, so requested after them they
+        // would hold the query back until every key of both blocks had arrived.
+        const uint32_t width = (q_heads + 2u * kv_heads) * head_dim, half = head_dim / 2u;
+        const float* src = q + (size_t)token * width;
+        const bool writer = head0 % (q_heads / kv_heads) == 0u;
+        const uint32_t dd = threadIdx.x, mate = dd < half ? dd + half : dd - half;
+        const bool rotates = dd < head_dim;
+        float in_q[REP], in_q_mate[REP], in_k = 0.0f, in_k_mate = 0.0f, in_v = 0.0f, in_cos = 0.0f, in_sin = 0.0f;
+#pragma unroll
+        for (int h = 0; h < REP; h++) in_q[h] = in_q_mate[h] = 0.0f;
+        if (rotates) {
+#pragma unroll
+            for (int h = 0; h < REP; h++) {
+                in_q[h] = src[(size_t)(head0 + h) * head_dim + dd];
+                in_q_mate[h] = src[(size_t)(head0 + h) * head_dim + mate];
+            }
+            in_k = src[(size_t)(q_heads + kvh) * head_dim + dd];
+            in_k_mate = src[(size_t)(q_heads + kvh) * head_dim + mate];
+            in_v = src[(size_t)(q_heads + kv_heads + kvh) * head_dim + dd];
+            in_cos = cos_table[(size_t)position * head_dim + dd];
+            in_sin = sin_table[(size_t)position * head_dim + dd];
+        }
+        request_keys(kv_a, 0u);
+        request_keys(kv_b, 32u * PASSES);
+        if (rotates) {
+            auto rotated = [&](float own, float other) {  // the arithmetic of rope_append_kernel
+                return __fadd_rn(__fmul_rn(own, in_cos), __fmul_rn(dd < half ? -other : other, in_sin));
+            };
+#pragma unroll
+            for (int h = 0; h < REP; h++) lds[h * per_head + dd] = rotated(in_q[h], in_q_mate[h]);
+            const float kn = rotated(in_k, in_k_mate);
+            k_new[dd] = kn;
+            v_new[dd] = in_v;
+            if (writer) {
+                kbase[(size_t)position * head_dim + dd] = kn;
+                vbase[(size_t)position * head_dim + dd] = in_v;
+            }
+        }
+    } else if constexpr (FUSED) {
         const uint32_t width = (q_heads + 2u * kv_heads) * head_dim, half = head_dim / 2u;
         const float* src = q + (size_t)token * width;
         const bool writer = head0 % (q_heads / kv_heads) == 0u;
@@ -215,47 +278,85 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
             }
         }
     } else {
+        float in_q[REP];
 #pragma unroll
         for (int h = 0; h < REP; h++)
-            for (uint32_t dd = threadIdx.x; dd < head_dim; dd += 256u)
+            in_q[h] = threadIdx.x < head_dim ? q[((size_t)token * q_heads + head0 + h) * head_dim + threadIdx.x] : 0.0f;
+        if constexpr (NC > 0) {
+            request_keys(kv_a, 0u);
+            request_keys(kv_b, 32u * PASSES);
+        }
+#pragma unroll
+        for (int h = 0; h < REP; h++) {
+            if (threadIdx.x < head_dim) lds[h * per_head + threadIdx.x] = in_q[h];
+            for (uint32_t dd = threadIdx.x + 256u; dd < head_dim; dd += 256u)
                 lds[h * per_head + dd] = q[((size_t)token * q_heads + head0 + h) * head_dim + dd];
+        }
     }
     __syncthreads();
+    // P.V: group g of 32 threads takes slots g, g + 8, ..., a thread four channels of each; the
+    // values come in batches of eight rows, requested two batches ahead like the keys, the first
+    // two before the softmax.  (Requesting them while key blocks are still alive takes more than
+    // 256 registers, which halves the workgroups a compute unit holds and was slower.)
+    const uint32_t group = threadIdx.x >> 5, chunk = threadIdx.x & 31u;
+    constexpr int VROWS = 8;
+    float4 vv_a[VROWS], vv_b[VROWS];
+    auto request_values = [&](float4 (&buf)[VROWS], uint32_t s0, uint32_t c4) {
+#pragma unroll
+        for (int u = 0; u < VROWS; u++) {
+            const uint32_t s = min(s0 + group + 8u * u, last_cached);
+            buf[u] = *reinterpret_cast<const float4*>(vbase + (size_t)s * head_dim + min(c4, head_dim - 4u));
+        }
+    };
+    constexpr uint32_t BATCH = 8u * VROWS;  // slots per batch over the eight groups
     float m[REP];
 #pragma unroll
     for (int h = 0; h < REP; h++) m[h] = -INFINITY;
     if constexpr (NC > 0) {
-        const uint32_t lane8 = threadIdx.x & 7u, rowg = threadIdx.x >> 3;
         // this lane's share of a row's dot with each query head, then the sum over the eight lanes
         auto finish = [&](float (&dot)[REP], uint32_t slot) {
 #pragma unroll
             for (int h = 0; h < REP; h++) {
                 float d = dot[h];
-                d += __shfl_xor(d, 1, 64);
-                d += __shfl_xor(d, 2, 64);
-                d += __shfl_xor(d, 4, 64);
+                // the eight lanes' sum as a butterfly of lane exchanges inside the register file
+                // (an exchange through the LDS crossbar costs a round trip, and the three of a
+                // row depend on each other): partners lane^1, lane^2, then the mirrored lane of
+                // the other quad, whose four lanes all hold that quad's sum by then
+                d += lane_exchange<kDppXor1>(d);
+                d += lane_exchange<kDppXor2>(d);
+                d += lane_exchange<kDppHalfMirror>(d);
                 d = __fmul_rn(d, scale);
                 if (lane8 == 0u) lds[h * per_head + head_dim + slot] = d;
                 m[h] = fmaxf(m[h], d);
             }
         };
-        auto accumulate = [&](float (&dot)[REP], const float4& kv, uint32_t c) {
+        // this lane's chunks of the query heads: registers when they are few (a read from LDS
+        // cannot be hoisted over the score writes by the compiler and would repeat per row)
+        constexpr bool Q_HELD = REP * KC <= 8;
+        float4 q_held[Q_HELD ? REP : 1][Q_HELD ? KC : 1];
+        if constexpr (Q_HELD) {
+#pragma unroll
+            for (int h = 0; h < REP; h++)
+#pragma unroll
+                for (int c = 0; c < KC; c++)
+                    q_held[h][c] = *reinterpret_cast<const float4*>(lds + h * per_head + 4u * (lane8 + 8u * c));
+        }
+        auto accumulate = [&](float (&dot)[REP], const float4& kv, int c) {
 #pragma unroll
             for (int h = 0; h < REP; h++) {
-                const float* qs = lds + h * per_head;
-                dot[h] += qs[4 * c] * kv.x + qs[4 * c + 1] * kv.y + qs[4 * c + 2] * kv.z + qs[4 * c + 3] * kv.w;
+                float4 qv;
+                if constexpr (Q_HELD) qv = q_held[h][c];
+                else qv = *reinterpret_cast<const float4*>(lds + h * per_head + 4u * (lane8 + 8u * c));
+                // fused multiply-adds: the score phase is bound by vector instruction issue (two
+                // wavefronts per SIMD, each a few hundred instructions), and this halves it
+                dot[h] = __builtin_fmaf(qv.x, kv.x, dot[h]);
+                dot[h] = __builtin_fmaf(qv.y, kv.y, dot[h]);
+                dot[h] = __builtin_fmaf(qv.z, kv.z, dot[h]);
+                dot[h] = __builtin_fmaf(qv.w, kv.w, dot[h]);
             }
         };
-        constexpr int PASSES = 4;
-        for (uint32_t s0 = 0; s0 < cached; s0 += 32u * PASSES) {
-            float4 kv[PASSES][NC];
-#pragma unroll
-            for (int u = 0; u < PASSES; u++) {
-                const uint32_t srow = min(s0 + u * 32u + rowg, cached - 1u);  // rows past the end: a valid address
-                const float4* kr = reinterpret_cast<const float4*>(kbase + (size_t)srow * head_dim);
-#pragma unroll
-                for (int c = 0; c < NC; c++) kv[u][c] = kr[lane8 + 8u * c];
-            }
+        constexpr uint32_t BLOCK = 32u * PASSES;  // slots per block
+        auto score_block = [&](float4 (&buf)[PASSES][KC], uint32_t s0) {
 #pragma unroll
             for (int u = 0; u < PASSES; u++) {
                 const uint32_t srow = s0 + u * 32u + rowg;
@@ -263,17 +364,25 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
 #pragma unroll
                 for (int h = 0; h < REP; h++) dot[h] = 0.0f;
 #pragma unroll
-                for (int c = 0; c < NC; c++) accumulate(dot, kv[u][c], lane8 + 8u * c);
-                // (all 64 lanes take part in the shuffles; rows past the end are dropped here)
+                for (int c = 0; c < NC; c++) accumulate(dot, buf[u][c], c);
+                // (all 64 lanes take part in the shuffles; a row past the end repeats the last
+                // cached one, rewrites its score with the same value and is dropped from the
+                // maximum here)
                 float keep[REP];
 #pragma unroll
                 for (int h = 0; h < REP; h++) keep[h] = m[h];
-                finish(dot, min(srow, cached - 1u));
+                finish(dot, min(srow, last_cached));
                 if (srow >= cached) {
 #pragma unroll
                     for (int h = 0; h < REP; h++) m[h] = keep[h];
                 }
             }
+        };
+        for (uint32_t s0 = 0; s0 < cached; s0 += 2u * BLOCK) {
+            score_block(kv_a, s0);
+            request_keys(kv_a, s0 + 2u * BLOCK);
+            if (s0 + BLOCK < cached) score_block(kv_b, s0 + BLOCK);  // (a scalar branch)
+            request_keys(kv_b, s0 + 3u * BLOCK);
         }
         if constexpr (FUSED) {
             // the appended slot, from LDS, by the eight lanes that own it in the unfused kernel and in
@@ -284,7 +393,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
                 for (int h = 0; h < REP; h++) dot[h] = 0.0f;
 #pragma unroll
                 for (int c = 0; c < NC; c++)
-                    accumulate(dot, *reinterpret_cast<const float4*>(k_new + 4u * (lane8 + 8u * c)), lane8 + 8u * c);
+                    accumulate(dot, *reinterpret_cast<const float4*>(k_new + 4u * (lane8 + 8u * c)), c);
                 finish(dot, position);
             }
         }
@@ -333,6 +442,10 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
             }
         }
     }
+    if constexpr (NC > 0) {
+        request_values(vv_a, 0u, chunk * 4u);
+        request_values(vv_b, BATCH, chunk * 4u);
+    }
     __syncthreads();  // scores of a slot are read below by other threads than wrote them
 #pragma unroll
     for (int h = 0; h < REP; h++) {
@@ -348,22 +461,42 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
         for (uint32_t s = threadIdx.x; s < visible; s += 256u) scores[s] = __fdiv_rn(scores[s], sum);
     }
     __syncthreads();
-    const uint32_t group = threadIdx.x >> 5, chunk = threadIdx.x & 31u;
     for (uint32_t c4 = chunk * 4u; c4 < head_dim; c4 += 128u) {
         float4 acc[REP];
 #pragma unroll
         for (int h = 0; h < REP; h++) acc[h] = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 8
-        for (uint32_t s = group; s < cached; s += 8u) {
-            const float4 vv = *reinterpret_cast<const float4*>(vbase + (size_t)s * head_dim + c4);
+        auto weigh = [&](const float4& vv, uint32_t s) {
 #pragma unroll
             for (int h = 0; h < REP; h++) {
                 const float p = lds[h * per_head + head_dim + s];
-                acc[h].x += p * vv.x;
-                acc[h].y += p * vv.y;
-                acc[h].z += p * vv.z;
-                acc[h].w += p * vv.w;
+                acc[h].x = __builtin_fmaf(p, vv.x, acc[h].x);
+                acc[h].y = __builtin_fmaf(p, vv.y, acc[h].y);
+                acc[h].z = __builtin_fmaf(p, vv.z, acc[h].z);
+                acc[h].w = __builtin_fmaf(p, vv.w, acc[h].w);
             }
+        };
+        if constexpr (NC > 0) {
+            auto weigh_batch = [&](float4 (&buf)[VROWS], uint32_t s0) {
+#pragma unroll
+                for (int u = 0; u < VROWS; u++) {
+                    const uint32_t s = s0 + group + 8u * u;
+                    if (s < cached) weigh(buf[u], s);
+                }
+            };
+            if (c4 != chunk * 4u) {  // head sizes above 128: a later pass
+                request_values(vv_a, 0u, c4);
+                request_values(vv_b, BATCH, c4);
+            }
+            for (uint32_t s0 = 0; s0 < cached; s0 += 2u * BATCH) {
+                weigh_batch(vv_a, s0);
+                request_values(vv_a, s0 + 2u * BATCH, c4);
+                if (s0 + BATCH < cached) weigh_batch(vv_b, s0 + BATCH);
+                request_values(vv_b, s0 + 3u * BATCH, c4);
+            }
+        } else {
+#pragma unroll 8
+            for (uint32_t s = group; s < cached; s += 8u)
+                weigh(*reinterpret_cast<const float4*>(vbase + (size_t)s * head_dim + c4), s);
         }
         if constexpr (FUSED) {
             if (group == position % 8u) {  // the appended slot closes its group's sum
@@ -371,10 +504,10 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
 #pragma unroll
                 for (int h = 0; h < REP; h++) {
                     const float p = lds[h * per_head + head_dim + position];
-                    acc[h].x += p * vv.x;
-                    acc[h].y += p * vv.y;
-                    acc[h].z += p * vv.z;
-                    acc[h].w += p * vv.w;
+                    acc[h].x = __builtin_fmaf(p, vv.x, acc[h].x);
+                    acc[h].y = __builtin_fmaf(p, vv.y, acc[h].y);
+                    acc[h].z = __builtin_fmaf(p, vv.z, acc[h].z);
+                    acc[h].w = __builtin_fmaf(p, vv.w, acc[h].w);
                 }
             }
         }
