@@ -23,13 +23,15 @@ namespace {
 
 extern __shared__ __attribute__((aligned(16))) char glue_lds[];
 
+// LAST: nothing writes `slots` again before the kernel ends, so no second barrier is needed.
+template <bool LAST = false>
 __device__ __forceinline__ float block_max(float v, float* slots) {
     v = wave_max(v);
     if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
     __syncthreads();
     float m = slots[0];
     for (uint32_t w = 1; w < blockDim.x / 64u; w++) m = fmaxf(m, slots[w]);
-    __syncthreads();
+    if constexpr (!LAST) __syncthreads();
     return m;
 }
 
@@ -43,7 +45,8 @@ __device__ __forceinline__ float block_sum(float v, float* slots) {
     return s;
 }
 
-// Shared tail of the two *_prepare kernels: the row's f32 values are in `vals` (LDS).
+// Shared tail of the two *_prepare kernels: the row's f32 values are in `vals` (LDS), element j
+// written by thread j % blockDim.x, which is also the thread that reads it here.
 // scale = max|v| / 127 (1.0 for an all-zero row, floored at 2^-126), code = ties-to-even(v / scale)
 // clamped to +-127 with a true f32 divide; a non-finite row gets zero codes and a NaN scale.
 __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_t* codes, float* scale_out,
@@ -55,7 +58,7 @@ __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_
         const float v = vals[j];
         maximum = fmaxf(maximum, finite_f32(v) ? fabsf(v) : __builtin_inff());
     }
-    maximum = block_max(maximum, slots);
+    maximum = block_max<true>(maximum, slots);
     const float bad = maximum == __builtin_inff() ? 1.0f : 0.0f;
     float scale = maximum == 0.0f || bad != 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
@@ -101,7 +104,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
         vals[j] = y;
         if (normalized) normalized[(size_t)row * d + j] = y;
     }
-    __syncthreads();
+    // (no barrier: prepare_row walks the row with the same stride, a thread reads its own writes)
     prepare_row(vals, d, prepared + (size_t)row * d, row_scales + row, slots);
 }
 
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(1024) void swiglu_prepare_kernel(const float* __res
         vals[j] = y;
         if (activated) activated[(size_t)row * inter + j] = y;
     }
-    __syncthreads();
+    // (no barrier: prepare_row walks the row with the same stride, a thread reads its own writes)
     prepare_row(vals, inter, prepared + (size_t)row * inter, row_scales + row, slots);
 }
 
