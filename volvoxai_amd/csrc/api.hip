@@ -76,18 +76,28 @@ struct Carver {
     }
 };
 
-static VxHipContext* default_context() {
-    static thread_local VxHipContext* ctx = nullptr;
-    if (!ctx && vxhip_context_create(0, nullptr, VXHIP_CONTEXT_OWN_STREAM, &ctx) != VXHIP_OK) ctx = nullptr;
-    return ctx;
-}
-
 static bool use_device(int device) {
     if (hipSetDevice(device) != hipSuccess) {
         set_error("hipSetDevice(%d) failed", device);
         return false;
     }
     return true;
+}
+
+// The context of the host-pointer entry points: device 0, one per thread.  Its device is made
+// current on every use, because the handles those entry points create live on the current device.
+static VxHipContext* default_context() {
+    static thread_local VxHipContext* ctx = nullptr;
+    if (!ctx && vxhip_context_create(0, nullptr, VXHIP_CONTEXT_OWN_STREAM, &ctx) != VXHIP_OK) ctx = nullptr;
+    if (ctx && !use_device(ctx->device)) return nullptr;
+    return ctx;
+}
+
+// A compiled weight is used on the device it was created on.
+static bool same_device(const VxHipContext* ctx, int handle_device, const char* who) {
+    if (ctx->device == handle_device) return true;
+    set_error("%s: the handle lives on device %d, the context on device %d", who, handle_device, ctx->device);
+    return false;
 }
 
 // Picks the kernel family for the shape and launches it.
@@ -421,7 +431,7 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
         !qlinear_admission(lin, per_row, input_scale, input_zp, output_scale, output_zp, input_dtype, output_dtype))
         return 0;
     const uint32_t k = lin->w.k, n = lin->w.n;
-    if (!use_device(ctx->device)) return 0;
+    if (!same_device(ctx, lin->device, "qlinear_forward") || !use_device(ctx->device)) return 0;
 
     const bool flip = input_dtype == VXHIP_DTYPE_U8;
     const bool stage = flip || (k % 16u) != 0u || ((uintptr_t)input_dev % 16u) != 0u;
@@ -692,7 +702,7 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
         return -1;
     }
     if (!rows) return 0;
-    if (!use_device(ctx->device)) return -1;
+    if (!same_device(ctx, pl->device, "packed_linear_forward_a8") || !use_device(ctx->device)) return -1;
     const uint32_t k = pl->w.k, n_pad = pl->w.panels * 32u;
     if (acc_dev && pl->w.bits != 8u) {
         set_error("packed_linear_forward_a8: the int32 sums are produced for 8-bit weights only");
@@ -727,7 +737,7 @@ int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* 
         return -1;
     }
     if (!rows) return 0;
-    if (!use_device(ctx->device)) return -1;
+    if (!same_device(ctx, pl->device, "packed_linear_forward_f32") || !use_device(ctx->device)) return -1;
     const uint32_t k = pl->w.k;
     const uint32_t ld = (k + 15u) / 16u * 16u;
     Carver sizes{nullptr};

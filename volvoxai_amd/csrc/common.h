@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/vxhip_w8a8.h"
 
 namespace vxhip {
@@ -171,6 +173,18 @@ struct LinearArgs {
 // gemm_mfma.hip / gemv_stream.hip: return the variant id that ran, or null if
 // the shape is outside the kernel's domain (nothing launched).
 const char* launch_gemm_mfma(hipStream_t s, const LinearArgs& a, int cu_count, const char* force);
+// A kernel's dynamic-LDS limit is an attribute per device: raised once per device and kernel
+// (`done` holds one bit per device ordinal; a racing second call only repeats the request).
+inline bool raise_lds_limit(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return false;
+    const uint64_t bit = 1ull << device;
+    if (done.load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+    done.fetch_or(bit, std::memory_order_release);
+    return true;
+}
+
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force);
 
 const char* forced_variant();

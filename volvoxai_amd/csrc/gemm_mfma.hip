@@ -682,14 +682,9 @@ bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr bool PIPE = MODE == (int)Epilogue::DequantF32 && GK == KS && TN * TM <= 2;  // as in the kernel
     constexpr int LDS = NS * (((BN / 32) * KS / (W4 ? 2 : 1) + BM / 8) * 1024 + (PIPE ? BN * 4 : 0)) + BN * 16;
     static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
-    static bool configured = false;
+    static std::atomic<uint64_t> configured{0};
     auto kern = gemm_mfma_kernel<WN, WM, TN, TM, MODE, GK, FAST, W4, NS>;
-    if (!configured) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS) !=
-            hipSuccess)
-            return false;
-        configured = true;
-    }
+    if (!raise_lds_limit((const void*)kern, LDS, configured)) return false;
     GemmParams p;
     p.a = a;
     p.tiles_n = (a.n + BN - 1) / BN;

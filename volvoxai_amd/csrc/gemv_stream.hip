@@ -291,13 +291,8 @@ template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT>;
     if (lds > 64u * 1024u) {
-        static bool configured = false;
-        if (!configured) {
-            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=
-                hipSuccess)
-                return false;
-            configured = true;
-        }
+        static std::atomic<uint64_t> configured{0};
+        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured)) return false;
     }
     hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u * SPLIT), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError() == hipSuccess;
