@@ -314,7 +314,7 @@ def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
             "weight_bytes_read_per_step": weight_bytes,
             "decode_hbm_GBs": weight_bytes / (decode_s / (new_tokens - 1)) / 1e9,
             "glue": "HIP kernels of the same library (embedding gather, residual+RMSNorm+prepare, RoPE+KV append, "
-                    "GQA attention, SwiGLU+prepare, argmax+advance); torch SDPA for the prompt's attention only; "
+                    "prompt and decode GQA attention, SwiGLU+prepare, argmax+advance); "
                     "one HIP graph per decode step"}
 
 

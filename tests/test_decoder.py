@@ -131,6 +131,37 @@ def test_rope_append_and_attention_kernels(ctx, rows, t, start):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,t,start,q_heads,kv_heads,head_dim,max_seq", [
+    (2, 128, 0, 16, 8, 128, 256),   # the benchmark's prompt
+    (1, 40, 13, 8, 1, 64, 70),      # eight query heads per KV head, a prompt continued at slot 13
+    (2, 9, 100, 4, 4, 256, 131),    # one head per KV head, the largest head size, an odd cache length
+    (1, 200, 0, 2, 1, 32, 1000),    # a long cache: fewer tokens share a workgroup
+    (3, 5, 2, 4, 2, 64, 32),        # too few tokens for the prompt kernel: the per-token one
+])
+def test_prompt_attention(ctx, rows, t, start, q_heads, kv_heads, head_dim, max_seq):
+    """Causal grouped-query attention of t prompt tokens per row over the caches, against a float64
+    statement of its definition (every token sees the slots up to its own)."""
+    import volvoxai_amd.w8a8 as vx
+    rng = np.random.default_rng(t * 7 + head_dim)
+    q = rng.normal(0, 1, (rows, t, q_heads, head_dim)).astype(np.float32)
+    k_cache = rng.normal(0, 1, (rows, kv_heads, max_seq, head_dim)).astype(np.float32)
+    v_cache = rng.normal(0, 1, (rows, kv_heads, max_seq, head_dim)).astype(np.float32)
+    positions = np.arange(start, start + t, dtype=np.int64)
+    out = vx.gqa_attention(ctx, _dev(q), _dev(k_cache), _dev(v_cache), _dev(positions))
+    ctx.synchronize()
+    got = out.cpu().numpy().reshape(rows, t, q_heads, head_dim)
+    rep = q_heads // kv_heads
+    for h in range(q_heads):
+        kk, vv = k_cache[:, h // rep].astype(np.float64), v_cache[:, h // rep].astype(np.float64)
+        sc = np.einsum("btd,bsd->bts", q[:, :, h].astype(np.float64), kk) / np.sqrt(head_dim)
+        sc[:, np.arange(max_seq)[None, :] > positions[:, None]] = -np.inf
+        p = np.exp(sc - sc.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        want = np.einsum("bts,bsd->btd", p, vv)
+        assert np.allclose(got[:, :, h], want, rtol=2e-5, atol=2e-6), h
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):

@@ -531,6 +531,177 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     }
 }
 
+// Prompt attention (t > 1 tokens per row).  The kernel above gives every (token, head) its own
+// workgroup, so a prompt of t tokens reads each key and value row t times.  Here a workgroup takes
+// `tq` consecutive tokens of one row and the `rep` query heads of one KV head, qw = tq * rep <= 32
+// queries, and walks that KV head's rows once for all of them, 64 slots at a time through LDS:
+//   scores   thread (slot = tid % 64, wavefront) holds eight queries' dots with one staged key row;
+//            the eight queries are the same for the whole wavefront, so they are read through the
+//            scalar cache straight from global memory and cost no LDS bandwidth (as LDS broadcast
+//            reads they took nine tenths of it and bounded the kernel)
+//   softmax  a wavefront per query, over the slots that query may see (slot <= its position)
+//   P.V      thread (four channels, tid / 32) holds four queries' sums over the staged value rows
+// The arithmetic is that of the kernel above (f32, scores scaled after the dot, exp(x - max),
+// a true division by the sum) with fused multiply-adds and its own summation order.
+// grid (rows * ceil(t / tq), kv_heads), block 256.
+// LDS: scores [qw][score_pitch], staged rows [64][head_dim + 4].
+constexpr uint32_t kPrefillQueries = 32u, kPrefillSlots = 64u;
+
+__global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restrict__ q,
+                                                          const float* __restrict__ k_cache,
+                                                          const float* __restrict__ v_cache,
+                                                          const int64_t* __restrict__ positions, uint32_t t,
+                                                          uint32_t tq, uint32_t q_heads, uint32_t kv_heads,
+                                                          uint32_t head_dim, uint32_t max_seq, float scale,
+                                                          float* __restrict__ out) {
+    __shared__ uint32_t visible[kPrefillQueries];  // slots query i may see; 0: no such query
+    const uint32_t rep = q_heads / kv_heads, qw = tq * rep;
+    const uint32_t blocks = (t + tq - 1u) / tq;
+    const uint32_t row = blockIdx.x / blocks, i0 = (blockIdx.x % blocks) * tq, kvh = blockIdx.y;
+    const uint32_t hd4 = head_dim / 4u, pitch = head_dim + 4u, score_pitch = (max_seq + 3u) & ~3u;
+    float* sc = reinterpret_cast<float*>(glue_lds);
+    float* stage = sc + (size_t)qw * score_pitch;
+    const float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    const float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
+    auto token_of = [&](uint32_t qi) { return i0 + qi / rep; };
+    auto head_of = [&](uint32_t qi) { return kvh * rep + qi % rep; };
+
+    if (threadIdx.x < kPrefillQueries) {
+        const uint32_t qi = threadIdx.x;
+        uint32_t v = 0u;
+        if (qi < qw && token_of(qi) < t) v = min((uint32_t)positions[token_of(qi)] + 1u, max_seq);
+        visible[qi] = v;
+    }
+    __syncthreads();
+    uint32_t span = 0u;  // slots any query of the workgroup sees
+    for (uint32_t qi = 0; qi < qw; qi++) span = max(span, visible[qi]);
+
+    // rows s0 .. s0+63 of a cache (zeros past the span) into the stage
+    // (four loads are requested before the first is stored: one round trip, not four)
+    auto stage_rows = [&](const float* base, uint32_t s0) {
+        const uint32_t total = kPrefillSlots * hd4;
+        for (uint32_t e0 = threadIdx.x; e0 < total; e0 += 4u * 256u) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t e = e0 + u * 256u, srow = s0 + e / hd4;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (e < total && srow < span)
+                    v[u] = *reinterpret_cast<const float4*>(base + (size_t)srow * head_dim + 4u * (e % hd4));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t e = e0 + u * 256u;
+                if (e < total) *reinterpret_cast<float4*>(stage + (size_t)(e / hd4) * pitch + 4u * (e % hd4)) = v[u];
+            }
+        }
+    };
+
+    {   // scores
+        const uint32_t slot = threadIdx.x & 63u;
+        const uint32_t first = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) * 8u);  // wave-uniform
+        // (queries past qw, or of tokens past t, repeat a valid one; their dots are dropped below)
+        const float* qrow[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t qi = min(first + j, qw - 1u);
+            qrow[j] = q + ((size_t)(row * t + min(token_of(qi), t - 1u)) * q_heads + head_of(qi)) * head_dim;
+        }
+        for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {
+            stage_rows(kbase, s0);
+            __syncthreads();
+            float dot[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) dot[j] = 0.0f;
+            const float* krow = stage + (size_t)slot * pitch;
+            for (uint32_t c = 0; c < hd4; c++) {
+                const float4 kv = *reinterpret_cast<const float4*>(krow + 4u * c);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float4 qv = *reinterpret_cast<const float4*>(qrow[j] + 4u * c);
+                    dot[j] = __builtin_fmaf(qv.x, kv.x, dot[j]);
+                    dot[j] = __builtin_fmaf(qv.y, kv.y, dot[j]);
+                    dot[j] = __builtin_fmaf(qv.z, kv.z, dot[j]);
+                    dot[j] = __builtin_fmaf(qv.w, kv.w, dot[j]);
+                }
+            }
+            const uint32_t s = s0 + slot;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t qi = first + j;
+                if (qi < qw && s < visible[qi]) sc[(size_t)qi * score_pitch + s] = __fmul_rn(dot[j], scale);
+            }
+            __syncthreads();
+        }
+    }
+    {   // softmax: probabilities over the visible slots, zeros from there to the span
+        const uint32_t lane = threadIdx.x & 63u;
+        for (uint32_t qi = threadIdx.x >> 6; qi < qw; qi += 4u) {  // (uniform per wavefront)
+            float* mine = sc + (size_t)qi * score_pitch;
+            const uint32_t seen = visible[qi];
+            if (seen != 0u) {
+                float m = -INFINITY;
+                for (uint32_t s = lane; s < seen; s += 64u) m = fmaxf(m, mine[s]);
+                m = wave_max(m);
+                float sum = 0.0f;
+                for (uint32_t s = lane; s < seen; s += 64u) {
+                    const float e = expf(mine[s] - m);
+                    mine[s] = e;
+                    sum += e;
+                }
+                sum = wave_sum(sum);
+                for (uint32_t s = lane; s < seen; s += 64u) mine[s] = __fdiv_rn(mine[s], sum);
+            }
+            for (uint32_t s = seen + lane; s < span; s += 64u) mine[s] = 0.0f;
+        }
+    }
+    __syncthreads();
+    {   // P.V
+        const uint32_t c4 = (threadIdx.x & 31u) * 4u, first = (threadIdx.x >> 5) * 4u;
+        float4 acc[2][4];  // channel passes c4 and c4 + 128 (head sizes up to 256) x four queries
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[pass][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {
+            stage_rows(vbase, s0);
+            __syncthreads();
+            const uint32_t rows_here = min(kPrefillSlots, span - s0);
+            for (uint32_t r = 0; r < rows_here; r++) {
+                float p[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) p[j] = sc[(size_t)min(first + j, qw - 1u) * score_pitch + s0 + r];
+#pragma unroll
+                for (int pass = 0; pass < 2; pass++) {
+                    const uint32_t cc = c4 + pass * 128u;
+                    if (cc < head_dim) {
+                        const float4 vv = *reinterpret_cast<const float4*>(stage + (size_t)r * pitch + cc);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            acc[pass][j].x = __builtin_fmaf(p[j], vv.x, acc[pass][j].x);
+                            acc[pass][j].y = __builtin_fmaf(p[j], vv.y, acc[pass][j].y);
+                            acc[pass][j].z = __builtin_fmaf(p[j], vv.z, acc[pass][j].z);
+                            acc[pass][j].w = __builtin_fmaf(p[j], vv.w, acc[pass][j].w);
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t qi = first + j;
+            if (qi >= qw || token_of(qi) >= t) continue;
+            float* dst = out + ((size_t)(row * t + token_of(qi)) * q_heads + head_of(qi)) * head_dim;
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const uint32_t cc = c4 + pass * 128u;
+                if (cc < head_dim) *reinterpret_cast<float4*>(dst + cc) = acc[pass][j];
+            }
+        }
+    }
+}
+
 // Few rows leave most of the device idle and the kernel latency bound: then a row gets a full
 // 1024-thread workgroup; with many rows 256 threads per row keep more rows resident.
 uint32_t row_block(uint32_t rows, uint32_t d) {
@@ -723,6 +894,34 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     const float scale = (float)(1.0 / sqrt((double)head_dim));
     const uint32_t rep = q_heads / kv_heads;
+    if (t >= 8u && rep <= kPrefillQueries && head_dim <= 256u) {
+        // a prompt: tokens share the walk over the cache, as many per workgroup as the LDS holds
+        uint32_t tq = kPrefillQueries / rep;
+        auto lds_for = [&](uint32_t tokens) {
+            const size_t qw = (size_t)tokens * rep;
+            return (qw * ((max_seq + 3u) & ~3u) + (size_t)kPrefillSlots * (head_dim + 4u)) * sizeof(float);
+        };
+        while (tq > 1u && lds_for(tq) > 150u * 1024u) tq /= 2u;
+        // two workgroups per compute unit hide each other's staging, if four tokens or more still
+        // share a walk then
+        if (lds_for(tq) > 78u * 1024u) {
+            uint32_t fewer = tq;
+            while (fewer > 4u && lds_for(fewer) > 78u * 1024u) fewer /= 2u;
+            if (lds_for(fewer) <= 78u * 1024u) tq = fewer;
+        }
+        if (lds_for(tq) <= 150u * 1024u) {
+            static std::atomic<uint64_t> configured{0};
+            if (!raise_lds_limit((const void*)gqa_prefill_kernel, 152 * 1024, configured)) {  // (plus its static 128 bytes)
+                set_error("gqa_attention: the prompt kernel's LDS limit could not be raised");
+                return VXHIP_EXECUTION_FAILED;
+            }
+            const dim3 grid(rows * ((t + tq - 1u) / tq), kv_heads);
+            hipLaunchKernelGGL(gqa_prefill_kernel, grid, dim3(256), lds_for(tq), ctx->stream, q_dev, k_cache_dev,
+                               v_cache_dev, positions_dev, t, tq, q_heads, kv_heads, head_dim, max_seq, scale, out_dev);
+            VXHIP_TRY(hipGetLastError());
+            return VXHIP_OK;
+        }
+    }
     // Query heads per workgroup.  Sharing a KV head's rows between its query heads halves the
     // reads but also the workgroups; at decode sizes the kernel is latency bound and one head per
     // workgroup measured faster (18 us against 26 us for 32 rows x 16 heads x 256 slots).

@@ -48,6 +48,16 @@ __device__ __forceinline__ float wave_max(float v) {
     return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
+// The sum over the 64 lanes, in every lane, as a butterfly (pairs, quads, eights, rows, then the
+// four rows): for callers that need no particular order.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += lane_exchange<kDppXor1>(v);
+    v += lane_exchange<kDppXor2>(v);
+    v += lane_exchange<kDppHalfMirror>(v);
+    v += lane_exchange<kDppMirror>(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+
 // The sum over the 64 lanes in the order of a shuffle-down tree with offsets 32, 16, 8, 4, 2, 1
 // (bit for bit what that tree gives), valid in lane 0 only.  The two steps that cross rows are
 // shuffles; the four inside the row are DPP moves.

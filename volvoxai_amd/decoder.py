@@ -183,15 +183,8 @@ class W8A8Decoder:
             return self._linear_a8(L["down"], a8, sc)
         q = vx.rope_append_kv(self.ctx, qkv, self.cos, self.sin, positions, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
                               self.k_cache[li], self.v_cache[li])
-        if t > 1:
-            # prompt (positions 0..t-1): every query attends causally to the t new slots; the
-            # library's kernel is shaped for single-token steps, so this goes to PyTorch's
-            # fused attention
-            attn = self.torch.nn.functional.scaled_dot_product_attention(
-                q.permute(0, 2, 1, 3), self.k_cache[li][:, :, :t], self.v_cache[li][:, :, :t], is_causal=True,
-                enable_gqa=True).permute(0, 2, 1, 3)
-        else:
-            attn = vx.gqa_attention(self.ctx, q, self.k_cache[li], self.v_cache[li], positions)
+        # the prompt: every token attends to the cache slots up to its own
+        attn = vx.gqa_attention(self.ctx, q, self.k_cache[li], self.v_cache[li], positions)
         o = self._linear(L["o"], attn.reshape(rows * t, cfg.q_dim))
         a8, sc = vx.add_rmsnorm_prepare_i8(self.ctx, x2, o, L["gain2"], cfg.eps)
         gu = self._linear_a8(L["gate_up"], a8, sc)
