@@ -448,6 +448,14 @@ def main():
                                 "traffic": MEASURED_TRAFFIC_BYTES["gemv_1x4096x14336"],
                                 "kernel": ctx.last_variant, "bytes_per_launch": gb, "avg_kernel_ms": gmean,
                                 "median_kernel_ms": gmed, "min_kernel_ms": gmin}
+        # What the memory system gives a kernel of this size that only reads (same bytes, buffers
+        # rotated the same way): the practical ceiling next to the 8 TB/s on the data sheet.
+        plain = [torch.randint(0, 255, (Kg * Ng,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
+        torch.cuda.synchronize()
+        probe = ctx.probe_stream_read(plain, launches=60)
+        probe["gemv_rate_over_plain_read"] = out["roofline_gemv"]["achieved"] / probe["GBs"]
+        out["hbm_ceiling_probe"] = probe
+        del plain
         if args.only == "gemv":
             out.update(value=out["gemv"]["value"], unit="GB/s", ms_per_step=gwall_ms,
                        config={"workload": out["gemv"]["workload"]}, roofline=out["roofline_gemv"])

@@ -166,6 +166,17 @@ VxHipStatus vxhip_argmax_rows_f32(VxHipContext* context, const float* input_dev,
 VxHipStatus vxhip_probe_mfma_rate(VxHipContext* context, uint32_t rounds,
                                   uint32_t random_operands, double* tops,
                                   double* shader_mhz, double* microseconds);
+/* Its HBM counterpart, also without a counterpart in the reference: `launches`
+ * launches of a kernel that only reads, each one whole buffer of bytes_each
+ * bytes (16-byte aligned device pointers, taken in rotation so that a buffer
+ * smaller than the 256 MB Infinity Cache is not served from it), timed
+ * back to back; reports the rate per launch and the time of one.  This is the
+ * ceiling of a bandwidth-bound kernel of that size on this device, launch ramp
+ * and drain included.  Synchronises the context's stream. */
+VxHipStatus vxhip_probe_stream_read(VxHipContext* context, const void* const* buffers_dev,
+                                    uint32_t buffer_count, size_t bytes_each,
+                                    uint32_t launches, double* gigabytes_per_second,
+                                    double* microseconds);
 
 /* Device memory for hosts without HIP headers. */
 VxHipStatus vxhip_device_malloc(size_t bytes, void** out_device_pointer);

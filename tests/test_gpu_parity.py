@@ -629,3 +629,22 @@ def test_every_tile_and_stage_variant_on_ragged_shapes(ctx, oracle):
         finally:
             vx.force_variant(None)
     assert ctx.fault_flags() == 0
+
+
+def test_ceiling_probes_report_rates(ctx):
+    """The two measurement aids: a register-only MFMA loop and a read-only kernel.  Rates are
+    machine facts, so only their sanity is checked, and that bad arguments are refused."""
+    import torch
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import VxHipError
+    m = ctx.probe_mfma_rate(32, True)
+    assert 100.0 < m["tops"] < 6000.0 and 300.0 < m["shader_mhz"] < 3500.0
+    bufs = [torch.zeros((1 << 20) + 48, dtype=torch.uint8, device="cuda") for _ in range(3)]
+    r = ctx.probe_stream_read(bufs, launches=9)
+    assert r["bytes"] == (1 << 20) + 48 and r["GBs"] > 1.0 and r["microseconds"] > 0.0
+    with pytest.raises(VxHipError):
+        ctx.probe_stream_read([bufs[0][1:17]], launches=1)  # not 16-byte aligned
+    with pytest.raises(VxHipError):
+        ctx.probe_stream_read([bufs[0][:8]], launches=1)    # less than one 16-byte word
+    assert vx is not None
+

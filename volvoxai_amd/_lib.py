@@ -72,6 +72,8 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_argmax_rows_f32": (i32, [vp, vp, u32, u32, vp, vp, u32]),
         "vxhip_probe_mfma_rate": (i32, [vp, u32, u32, C.POINTER(C.c_double), C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)]),
+        "vxhip_probe_stream_read": (i32, [vp, C.POINTER(C.c_void_p), u32, sz, u32, C.POINTER(C.c_double),
+                                          C.POINTER(C.c_double)]),
         "vxhip_device_malloc": (i32, [sz, pp]),
         "vxhip_device_free": (None, [vp]),
         "vxhip_memcpy_to_device": (i32, [vp, vp, vp, sz]),

@@ -47,10 +47,80 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i* __restrict__ 
     if (fold == 0x12345) sink[0] = fold;  // keeps the accumulators alive
 }
 
+// The HBM counterpart: the same bytes a GEMV streams, read and folded into a word that is never
+// stored -- no MFMA, no LDS, no tail.  What this reaches is what the memory system gives a
+// kernel of that size, launch ramp and drain included.
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ data, size_t count,
+                                                          uint32_t* sink) {
+    const size_t stride = (size_t)gridDim.x * 256u;
+    size_t i = (size_t)blockIdx.x * 256u + threadIdx.x;
+    uint32_t fold = 0u;
+    for (; i + 3u * stride < count; i += 4u * stride) {  // four loads in flight per thread
+        const uint4 a = data[i], b = data[i + stride], c = data[i + 2u * stride], d = data[i + 3u * stride];
+        fold ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < count; i += stride) {
+        const uint4 a = data[i];
+        fold ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+    if (fold == 0x9e3779b9u) sink[0] = fold;  // keeps the loads alive; practically never true
+}
+
 }  // namespace
 }  // namespace vxhip
 
 using namespace vxhip;
+
+extern "C" VxHipStatus vxhip_probe_stream_read(VxHipContext* ctx, const void* const* buffers_dev,
+                                               uint32_t buffer_count, size_t bytes_each, uint32_t launches,
+                                               double* gigabytes_per_second, double* microseconds) {
+    if (!ctx || !buffers_dev || !buffer_count || bytes_each < 16u || !launches || !gigabytes_per_second) {
+        set_error("probe_stream_read: null argument, no buffer or no launch");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    for (uint32_t i = 0; i < buffer_count; i++) {
+        if (!buffers_dev[i] || ((uintptr_t)buffers_dev[i] % 16u) != 0u) {
+            set_error("probe_stream_read: buffer %u is null or not 16-byte aligned", i);
+            return VXHIP_INVALID_ARGUMENT;
+        }
+    }
+    VXHIP_TRY(hipSetDevice(ctx->device));
+    uint32_t* sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    VxHipStatus st = VXHIP_OK;
+    auto check = [&](hipError_t e, const char* what) {
+        if (st == VXHIP_OK && e != hipSuccess) st = hip_status(e, what);
+    };
+    check(hipMalloc((void**)&sink, 64), "hipMalloc");
+    check(hipEventCreate(&e0), "hipEventCreate");
+    check(hipEventCreate(&e1), "hipEventCreate");
+    const size_t count = bytes_each / 16u;
+    const int groups = 16 * (ctx->cu_count > 0 ? ctx->cu_count : 256);  // measured best among 4, 8, 16 per CU
+    float ms = 0.0f;
+    if (st == VXHIP_OK) {
+        for (uint32_t i = 0; i < buffer_count; i++)  // warm-up, one pass over every buffer
+            hipLaunchKernelGGL(stream_read_kernel, dim3(groups), dim3(256), 0, ctx->stream,
+                               (const uint4*)buffers_dev[i], count, sink);
+        check(hipStreamSynchronize(ctx->stream), "warm-up launches");
+        check(hipEventRecord(e0, ctx->stream), "record");
+        for (uint32_t i = 0; i < launches; i++)
+            hipLaunchKernelGGL(stream_read_kernel, dim3(groups), dim3(256), 0, ctx->stream,
+                               (const uint4*)buffers_dev[i % buffer_count], count, sink);
+        check(hipGetLastError(), "launch");
+        check(hipEventRecord(e1, ctx->stream), "record");
+        check(hipEventSynchronize(e1), "sync");
+        check(hipEventElapsedTime(&ms, e0, e1), "elapsed");
+    }
+    if (st == VXHIP_OK) {
+        const double us = (double)ms * 1e3 / launches;
+        *gigabytes_per_second = (double)(count * 16u) / us / 1e3;
+        if (microseconds) *microseconds = us;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    return st;
+}
 
 extern "C" VxHipStatus vxhip_probe_mfma_rate(VxHipContext* ctx, uint32_t rounds, uint32_t random_operands,
                                              double* tops, double* shader_mhz, double* microseconds) {

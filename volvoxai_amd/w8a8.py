@@ -96,6 +96,18 @@ class Context:
                                                C.byref(mhz), C.byref(us)), "vxhip_probe_mfma_rate")
         return {"tops": tops.value, "shader_mhz": mhz.value, "microseconds": us.value}
 
+    def probe_stream_read(self, buffers, launches=60) -> dict:
+        """A kernel that only reads, one whole buffer (device tensors of equal size, rotated) per
+        launch: the rate and time per launch the memory system gives a kernel of that size."""
+        nbytes = buffers[0].numel() * buffers[0].element_size()
+        if any(b.numel() * b.element_size() != nbytes for b in buffers):
+            raise ValueError("probe_stream_read: buffers differ in size")
+        pointers = (C.c_void_p * len(buffers))(*[b.data_ptr() for b in buffers])
+        gbs, us = C.c_double(0), C.c_double(0)
+        _check(library().vxhip_probe_stream_read(self._h, pointers, len(buffers), nbytes, int(launches), C.byref(gbs),
+                                                 C.byref(us)), "vxhip_probe_stream_read")
+        return {"GBs": gbs.value, "microseconds": us.value, "bytes": nbytes // 16 * 16, "buffers_rotated": len(buffers)}
+
 
 class QLinear:
     """Compiled scope of one QLinear/QMatMul/QGemm node: prepacked weights."""
