@@ -544,7 +544,7 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
 // The arithmetic is that of the kernel above (f32, scores scaled after the dot, exp(x - max),
 // a true division by the sum) with fused multiply-adds and its own summation order.
 // grid (rows * ceil(t / tq), kv_heads), block 256.
-// LDS: scores [qw][score_pitch], staged rows [64][head_dim + 4].
+// LDS: scores [qw][max_seq rounded up to 64], staged rows [64][head_dim + 4].
 constexpr uint32_t kPrefillQueries = 32u, kPrefillSlots = 64u;
 
 __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restrict__ q,
@@ -558,7 +558,8 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
     const uint32_t rep = q_heads / kv_heads, qw = tq * rep;
     const uint32_t blocks = (t + tq - 1u) / tq;
     const uint32_t row = blockIdx.x / blocks, i0 = (blockIdx.x % blocks) * tq, kvh = blockIdx.y;
-    const uint32_t hd4 = head_dim / 4u, pitch = head_dim + 4u, score_pitch = (max_seq + 3u) & ~3u;
+    // (a score row is a whole number of 64-slot blocks, so that P.V never has to guard a slot)
+    const uint32_t hd4 = head_dim / 4u, pitch = head_dim + 4u, score_pitch = (max_seq + 63u) & ~63u;
     float* sc = reinterpret_cast<float*>(glue_lds);
     float* stage = sc + (size_t)qw * score_pitch;
     const float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * head_dim;
@@ -576,26 +577,29 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
     uint32_t span = 0u;  // slots any query of the workgroup sees
     for (uint32_t qi = 0; qi < qw; qi++) span = max(span, visible[qi]);
 
-    // rows s0 .. s0+63 of a cache (zeros past the span) into the stage
-    // (four loads are requested before the first is stored: one round trip, not four)
-    auto stage_rows = [&](const float* base, uint32_t s0) {
-        const uint32_t total = kPrefillSlots * hd4;
-        for (uint32_t e0 = threadIdx.x; e0 < total; e0 += 4u * 256u) {
-            float4 v[4];
+    // Rows s0 .. s0+63 of a cache (zeros past the span) go to the stage in two steps: requested
+    // into registers, stored to LDS a block later -- the request of the next block is in flight
+    // while this one is being used.
+    constexpr int kStageRegs = 16;  // 64 rows x 256 floats over 256 threads, as 16-byte words
+    const uint32_t stage_words = kPrefillSlots * hd4;
+    auto fetch_rows = [&](const float* base, uint32_t s0, float4 (&v)[kStageRegs]) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint32_t e = e0 + u * 256u, srow = s0 + e / hd4;
-                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (e < total && srow < span)
-                    v[u] = *reinterpret_cast<const float4*>(base + (size_t)srow * head_dim + 4u * (e % hd4));
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const uint32_t e = e0 + u * 256u;
-                if (e < total) *reinterpret_cast<float4*>(stage + (size_t)(e / hd4) * pitch + 4u * (e % hd4)) = v[u];
-            }
+        for (int u = 0; u < kStageRegs; u++) {
+            const uint32_t e = threadIdx.x + u * 256u, srow = s0 + e / hd4;
+            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e < stage_words && srow < span)
+                v[u] = *reinterpret_cast<const float4*>(base + (size_t)srow * head_dim + 4u * (e % hd4));
         }
     };
+    auto commit_rows = [&](const float4 (&v)[kStageRegs]) {
+#pragma unroll
+        for (int u = 0; u < kStageRegs; u++) {
+            const uint32_t e = threadIdx.x + u * 256u;
+            if (e < stage_words) *reinterpret_cast<float4*>(stage + (size_t)(e / hd4) * pitch + 4u * (e % hd4)) = v[u];
+        }
+    };
+    float4 ahead[kStageRegs];
+    fetch_rows(kbase, 0u, ahead);
 
     {   // scores
         const uint32_t slot = threadIdx.x & 63u;
@@ -608,13 +612,17 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
             qrow[j] = q + ((size_t)(row * t + min(token_of(qi), t - 1u)) * q_heads + head_of(qi)) * head_dim;
         }
         for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {
-            stage_rows(kbase, s0);
+            commit_rows(ahead);
             __syncthreads();
+            // the next block of keys, or after the last one the first block of values
+            if (s0 + kPrefillSlots < span) fetch_rows(kbase, s0 + kPrefillSlots, ahead);
+            else fetch_rows(vbase, 0u, ahead);
             float dot[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) dot[j] = 0.0f;
             const float* krow = stage + (size_t)slot * pitch;
-            for (uint32_t c = 0; c < hd4; c++) {
+#pragma unroll 4
+            for (uint32_t c = 0; c < hd4; c++) {  // (unrolled: the loads of four steps go out together)
                 const float4 kv = *reinterpret_cast<const float4*>(krow + 4u * c);
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -652,7 +660,8 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
                 sum = wave_sum(sum);
                 for (uint32_t s = lane; s < seen; s += 64u) mine[s] = __fdiv_rn(mine[s], sum);
             }
-            for (uint32_t s = seen + lane; s < span; s += 64u) mine[s] = 0.0f;
+            const uint32_t span_blocks = (span + kPrefillSlots - 1u) / kPrefillSlots * kPrefillSlots;
+            for (uint32_t s = seen + lane; s < span_blocks; s += 64u) mine[s] = 0.0f;
         }
     }
     __syncthreads();
@@ -664,10 +673,13 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[pass][j] = make_float4(0.f, 0.f, 0.f, 0.f);
         for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {
-            stage_rows(vbase, s0);
+            commit_rows(ahead);
             __syncthreads();
-            const uint32_t rows_here = min(kPrefillSlots, span - s0);
-            for (uint32_t r = 0; r < rows_here; r++) {
+            if (s0 + kPrefillSlots < span) fetch_rows(vbase, s0 + kPrefillSlots, ahead);
+            // (every row of the block: the staged rows past the span are zeros and so are their
+            // probabilities, and a fixed count lets the reads of eight rows go out together)
+#pragma unroll 8
+            for (uint32_t r = 0; r < kPrefillSlots; r++) {
                 float p[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) p[j] = sc[(size_t)min(first + j, qw - 1u) * score_pitch + s0 + r];
@@ -899,7 +911,7 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
         uint32_t tq = kPrefillQueries / rep;
         auto lds_for = [&](uint32_t tokens) {
             const size_t qw = (size_t)tokens * rep;
-            return (qw * ((max_seq + 3u) & ~3u) + (size_t)kPrefillSlots * (head_dim + 4u)) * sizeof(float);
+            return (qw * ((max_seq + 63u) & ~63u) + (size_t)kPrefillSlots * (head_dim + 4u)) * sizeof(float);
         };
         while (tq > 1u && lds_for(tq) > 150u * 1024u) tq /= 2u;
         // two workgroups per compute unit hide each other's staging, if four tokens or more still
