@@ -194,20 +194,31 @@ def bench_other_configs(torch, vx, cases, ctx):
     """configs[1] at M=4,16, configs[2] at M=512,2048 and configs[4] (M=2048, K=14336, N=4096,
     dynamic per-token scales, f32 dequant+bias): time per call with inputs resident."""
     from volvoxai_amd.decoder import pack_w8_words
+    from volvoxai_amd.w8a8 import operand_order_codes
     res = {}
     # decode GEMV, M = 4 and 16 (rotating weight copies as for M = 1)
     Kg, Ng, G, copies = 4096, 14336, 128, 6
     d = cases.decode_case(16, Kg, Ng, G, 14336)
     words = pack_w8_words(d["w"])
     pls = [vx.PackedLinear(words, d["scales"], d["bias"], Kg, Ng, G) for _ in range(copies)]
+    # With more than one row the int8 codes are handed over the way the library's preparation
+    # kernels write them for a decode context: the rows' 16-byte chunks interleaved (operand
+    # order), which the GEMV loads as whole cache lines.  The row-major figure stays beside it.
+    octx = vx.Context(0, torch.cuda.current_stream())
+    octx.set_activation_layout(True)
     for m in (4, 16):
         a8 = torch.from_numpy(d["a8"][:m]).cuda()
+        o8 = torch.from_numpy(operand_order_codes(d["a8"][:m])).cuda()
         ars = torch.from_numpy(d["row_scales"][:m]).cuda()
         y = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
-        ms = region_ms(lambda i: pls[i % copies].forward_a8(ctx, a8, ars, out=y), 100, torch)
+        y_rows = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
+        ms = region_ms(lambda i: pls[i % copies].forward_a8(octx, o8, ars, out=y), 100, torch)
+        ms_rows = region_ms(lambda i: pls[i % copies].forward_a8(ctx, a8, ars, out=y_rows), 100, torch)
         gb = gemv_algorithmic_bytes(m, Kg, Ng)
         res[f"gemv_M{m}_K4096_N14336"] = {"ms": ms, "GBs": gb / (ms * 1e-3) / 1e9, "frac_hbm": gb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                           "variant": ctx.last_variant}
+                                           "variant": octx.last_variant, "activations": "operand order",
+                                           "ms_with_row_major_activations": ms_rows,
+                                           "same_bits_either_way": bool(torch.equal(y.view(torch.int32), y_rows.view(torch.int32)))}
     for p in pls:
         p.close()
     # the same decode shape with four-bit weights: half the weight bytes, same scales and output
@@ -217,14 +228,15 @@ def bench_other_configs(torch, vx, cases, ctx):
     w4copies = 2 * copies
     pls = [vx.PackedLinear(w4words, d["scales"], d["bias"], Kg, Ng, G, weight_bits=4) for _ in range(w4copies)]
     for m in (1, 16):
-        a8 = torch.from_numpy(d["a8"][:m]).cuda()
+        o8 = torch.from_numpy(operand_order_codes(d["a8"][:m])).cuda()
         ars = torch.from_numpy(d["row_scales"][:m]).cuda()
         y = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
-        ms = region_ms(lambda i: pls[i % w4copies].forward_a8(ctx, a8, ars, out=y), 100, torch)
+        ms = region_ms(lambda i: pls[i % w4copies].forward_a8(octx, o8, ars, out=y), 100, torch)
         gb = gemv_algorithmic_bytes(m, Kg, Ng) - Kg * Ng // 2
         res[f"w4a8_gemv_M{m}_K4096_N14336"] = {"ms": ms, "GBs": gb / (ms * 1e-3) / 1e9,
                                                 "frac_hbm": gb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                                "variant": ctx.last_variant}
+                                                "variant": octx.last_variant, "activations": "operand order"}
+    octx.close()
     a8 = torch.from_numpy(np.tile(d["a8"], (128, 1))).cuda()
     ars = torch.from_numpy(np.tile(d["row_scales"], 128)).cuda()
     y = torch.empty((2048, Ng), dtype=torch.float32, device="cuda")

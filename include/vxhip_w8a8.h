@@ -79,6 +79,25 @@ const char* vxhip_context_last_variant(const VxHipContext* context);
 /* Device-side fault word accumulated by kernels (non-finite multiplier seen,
  * ...); reading it synchronises the stream.  0 = clean. */
 VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
+/* Layout of prepared activations (int8 codes) handed between entry points on
+ * this context; no counterpart in the reference, whose prepared rows
+ * (src/kernels/llm_ops.h:30-32) are row major.
+ *   VXHIP_ACTIVATIONS_ROW_MAJOR (default): [rows, k] bytes.
+ *   VXHIP_ACTIVATIONS_OPERAND32: calls with rows <= 32 exchange the codes in
+ *     the order the streaming GEMV loads them: the 16-byte chunks of the rows
+ *     interleaved, code j of row r at ((j / 16) * 32 + r) * 16 + j % 16.  Such a
+ *     buffer ALWAYS holds 32 * ceil(k / 16) * 16 bytes, whatever `rows` is, and
+ *     must be 16-byte aligned.  Calls with rows > 32 stay row major.
+ * It applies to what vxhip_packed_prepare_i8, vxhip_rmsnorm_prepare_i8,
+ * vxhip_add_rmsnorm_prepare_i8 and vxhip_swiglu_prepare_i8 write and to what
+ * vxhip_packed_linear_forward_a8 reads.  With 32 rows the GEMVs of a decoder
+ * layer run 0.5-2 us shorter each (a row-major load of one k-step touches 32
+ * cache lines for its 1 KiB). */
+#define VXHIP_ACTIVATIONS_ROW_MAJOR 0u
+#define VXHIP_ACTIVATIONS_OPERAND32 1u
+VxHipStatus vxhip_context_set_activation_layout(VxHipContext* context, uint32_t layout);
+/* Bytes a prepared-activation buffer needs on this context for `rows` x k. */
+size_t vxhip_context_prepared_bytes(const VxHipContext* context, uint32_t rows, uint32_t k);
 
 /* ---- decoder glue around the PackedLinear calls ------------------------- */
 /* The steps either side of the linears of a decoder layer (the components the

@@ -648,3 +648,44 @@ def test_ceiling_probes_report_rates(ctx):
         ctx.probe_stream_read([bufs[0][:8]], launches=1)    # less than one 16-byte word
     assert vx is not None
 
+
+
+@pytest.mark.parametrize("rows,k,n,group", [(1, 4096, 96, 128), (5, 1000, 36, 32), (16, 1537, 130, 64),
+                                            (32, 1024, 1056, 128), (27, 24, 40, 256), (32, 5000, 300, 32)])
+def test_operand_order_activations(oracle, rows, k, n, group):
+    """A context set to exchange prepared activations in the GEMV's operand order: the prepared
+    bytes are the row-major codes re-ordered, the linear gives the oracle's bits from them (also
+    where no GEMV takes the shape and the rows are copied back out for the GEMM, the last case),
+    and calls with more than 32 rows stay row major."""
+    import torch
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    c = cases.packed_case(rows, k, n, group, 900 + rows, True, special_rows=(rows >= 5))
+    words = oracle.pack_w8_words(c["w"])
+    _, want = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], n, group)
+    plain, blocked = vx.Context(0, None), vx.Context(0, None)
+    blocked.set_activation_layout(True)
+    xd = dev(c["x"])
+    codes, scales = packed_prepare_i8(plain, xd)
+    bcodes, bscales = packed_prepare_i8(blocked, xd)
+    plain.synchronize(), blocked.synchronize()
+    chunks = (k + 15) // 16
+    assert bcodes.numel() == 32 * chunks * 16
+    padded = np.zeros((rows, chunks * 16), np.int8)
+    padded[:, :k] = host(codes)
+    got = host(bcodes).reshape(chunks, 32, 16)[:, :rows].transpose(1, 0, 2).reshape(rows, chunks * 16)
+    assert (got == padded).all() and same_f32(host(bscales), host(scales))
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+    st, y = pl.forward_a8(blocked, bcodes, bscales)
+    blocked.synchronize()
+    assert st == 0 and same_f32(host(y), want), blocked.last_variant
+    assert ("gemv" in blocked.last_variant) == (k != 5000)
+    if k == 1000:  # more than 32 rows on the same context: row major, through the GEMM
+        big = cases.packed_case(40, k, n, group, 77, True)
+        _, want_big = oracle.packed_linear(big["x"], words, c["scales"], c["bias"], n, group)
+        a8, sc = packed_prepare_i8(blocked, dev(big["x"]))
+        assert tuple(a8.shape) == (40, k)
+        st, y = pl.forward_a8(blocked, a8, sc)
+        blocked.synchronize()
+        assert st == 0 and same_f32(host(y), want_big)
+    pl.close(), plain.close(), blocked.close()

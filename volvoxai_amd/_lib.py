@@ -74,6 +74,8 @@ def _declare(L: C.CDLL) -> None:
                                         C.POINTER(C.c_double)]),
         "vxhip_probe_stream_read": (i32, [vp, C.POINTER(C.c_void_p), u32, sz, u32, C.POINTER(C.c_double),
                                           C.POINTER(C.c_double)]),
+        "vxhip_context_set_activation_layout": (i32, [vp, u32]),
+        "vxhip_context_prepared_bytes": (sz, [vp, u32, u32]),
         "vxhip_device_malloc": (i32, [sz, pp]),
         "vxhip_device_free": (None, [vp]),
         "vxhip_memcpy_to_device": (i32, [vp, vp, vp, sz]),

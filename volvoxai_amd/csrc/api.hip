@@ -220,6 +220,18 @@ VxHipStatus vxhip_context_fault_flags(VxHipContext* ctx, uint32_t* flags) {
     return VXHIP_OK;
 }
 
+VxHipStatus vxhip_context_set_activation_layout(VxHipContext* ctx, uint32_t layout) {
+    if (!ctx || layout > VXHIP_ACTIVATIONS_OPERAND32) return VXHIP_INVALID_ARGUMENT;
+    ctx->activation_layout = layout;
+    return VXHIP_OK;
+}
+
+size_t vxhip_context_prepared_bytes(const VxHipContext* ctx, uint32_t rows, uint32_t k) {
+    if (ctx && ctx->activation_layout == VXHIP_ACTIVATIONS_OPERAND32 && rows <= kOperandOrderRows)
+        return (size_t)kOperandOrderRows * ((k + 15u) / 16u * 16u);
+    return (size_t)rows * k;
+}
+
 VxHipStatus vxhip_device_malloc(size_t bytes, void** out) {
     if (!out) return VXHIP_INVALID_ARGUMENT;
     *out = nullptr;
@@ -637,16 +649,22 @@ VxHipStatus vxhip_packed_prepare_i8(VxHipContext* ctx, const float* input_dev, u
     if (!rows) return VXHIP_OK;
     if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
     ctx->last_variant = "hip.packed-linear.prepare-i8";
-    return launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared_dev, k, row_scales_dev);
+    const bool operand_order = ctx->activation_layout == VXHIP_ACTIVATIONS_OPERAND32 && rows <= kOperandOrderRows;
+    return launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared_dev,
+                             operand_order ? ActivationLayout{(k + 15u) / 16u * 16u, 1u} : ActivationLayout{k, 0u},
+                             row_scales_dev);
 }
 
+// operand_order: a8 is in operand order (rows <= 32), which only the GEMV reads; -2 then says that
+// no GEMV takes the shape and the caller has to come back with row-major activations.
 static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const int8_t* a8, uint32_t lda,
-                         const float* row_scales, float* y, int32_t* acc, const int32_t* zeros,
-                         uint32_t rows) {
+                         bool operand_order, const float* row_scales, float* y, int32_t* acc,
+                         const int32_t* zeros, uint32_t rows) {
     LinearArgs a{};
     a.mode = Epilogue::DequantF32;
     a.x = a8;
     a.ldx = lda;
+    a.x_operand_order = operand_order ? 1u : 0u;
     a.rows = rows;
     a.n = pl->w.n;
     a.k = pl->w.k;
@@ -665,7 +683,7 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
     const char* id = nullptr;
     if (y) {
         id = run_linear(ctx, a);
-        if (!id) return -1;
+        if (!id) return operand_order ? -2 : -1;
     }
     if (acc) {
         // exact full-K int32 sums: the same kernels in requantizing mode with the byte output
@@ -687,7 +705,7 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
         b.out_lo = -128;
         b.out_hi = 127;
         const char* id2 = run_linear(ctx, b);
-        if (!id2) return -1;
+        if (!id2) return operand_order && !y ? -2 : -1;
         if (!id) id = id2;
     }
     ctx->last_variant = id;
@@ -712,7 +730,14 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
         set_error("packed_linear_forward_a8: full-K int32 sums are not provable for K=%u", k);
         return -1;
     }
-    const bool stage = (k % 16u) != 0u || ((uintptr_t)activation_dev % 16u) != 0u;
+    const bool operand_order = ctx->activation_layout == VXHIP_ACTIVATIONS_OPERAND32 && rows <= kOperandOrderRows;
+    if (operand_order && ((uintptr_t)activation_dev % 16u) != 0u) {
+        set_error("packed_linear_forward_a8: operand-order activations must be 16-byte aligned");
+        return -1;
+    }
+    // row-major rows are used in place when they are aligned whole chunks; operand order is
+    // used in place by the GEMV and copied out to rows only if the call ends up on the GEMM
+    const bool stage = operand_order || (k % 16u) != 0u || ((uintptr_t)activation_dev % 16u) != 0u;
     const uint32_t ld = stage ? (k + 15u) / 16u * 16u : k;
     Carver sizes{nullptr};
     sizes.take<int32_t>(acc_dev ? n_pad : 0);
@@ -723,10 +748,16 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
     int8_t* staged = c.take<int8_t>(stage ? (size_t)rows * ld : 0);
     // a fill kernel rather than a memset node, so the call stays graph-capturable
     if (acc_dev && launch_fill_u32(ctx->stream, (uint32_t*)zeros, n_pad, 0u) != VXHIP_OK) return -1;
+    if (operand_order) {
+        const int st = packed_run_a8(ctx, pl, activation_dev, ld, true, row_scales_dev, output_dev, acc_dev, zeros, rows);
+        if (st != -2) return st;
+        if (launch_unblock_activations(ctx->stream, activation_dev, rows, k, staged, ld) != VXHIP_OK) return -1;
+        return packed_run_a8(ctx, pl, staged, ld, false, row_scales_dev, output_dev, acc_dev, zeros, rows);
+    }
     if (stage && launch_stage_activations(ctx->stream, activation_dev, rows, k, false, staged, ld, nullptr) !=
                      VXHIP_OK)
         return -1;
-    return packed_run_a8(ctx, pl, stage ? staged : activation_dev, ld, row_scales_dev, output_dev, acc_dev,
+    return packed_run_a8(ctx, pl, stage ? staged : activation_dev, ld, false, row_scales_dev, output_dev, acc_dev,
                          zeros, rows);
 }
 
@@ -740,15 +771,25 @@ int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* 
     if (!same_device(ctx, pl->device, "packed_linear_forward_f32") || !use_device(ctx->device)) return -1;
     const uint32_t k = pl->w.k;
     const uint32_t ld = (k + 15u) / 16u * 16u;
+    // the prepared rows never leave this call: up to 32 rows go to the GEMV in its operand order
+    const bool operand_order = rows <= kOperandOrderRows;
+    const size_t prepared_rows = operand_order ? kOperandOrderRows : rows;
     Carver sizes{nullptr};
     sizes.take<float>(rows);
-    sizes.take<int8_t>((size_t)rows * ld);
+    sizes.take<int8_t>(prepared_rows * ld);
     if (ensure_scratch(ctx, sizes.off + 256u) != VXHIP_OK) return -1;
     Carver c{(char*)ctx->scratch};
     float* row_scales = c.take<float>(rows);
-    int8_t* prepared = c.take<int8_t>((size_t)rows * ld);
-    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ld, row_scales) != VXHIP_OK) return -1;
-    return packed_run_a8(ctx, pl, prepared, ld, row_scales, output_dev, nullptr, nullptr, rows);
+    int8_t* prepared = c.take<int8_t>(prepared_rows * ld);
+    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, operand_order ? 1u : 0u},
+                          row_scales) != VXHIP_OK)
+        return -1;
+    const int st = packed_run_a8(ctx, pl, prepared, ld, operand_order, row_scales, output_dev, nullptr, nullptr, rows);
+    if (st != -2) return st;
+    // no GEMV takes the shape (or a GEMM tile is forced): once more, as rows, for the GEMM
+    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, 0u}, row_scales) != VXHIP_OK)
+        return -1;
+    return packed_run_a8(ctx, pl, prepared, ld, false, row_scales, output_dev, nullptr, nullptr, rows);
 }
 
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, const float* scale,

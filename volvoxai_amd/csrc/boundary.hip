@@ -47,8 +47,9 @@ VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows
 // A row holding NaN or Inf gets zero codes and a NaN scale, which makes every
 // output of that row NaN downstream as the reference requires (:1495).
 __global__ __launch_bounds__(1024) void prepare_i8_kernel(
-        const float* __restrict__ x, uint32_t k, int8_t* __restrict__ prepared, uint32_t ld,
+        const float* __restrict__ x, uint32_t k, int8_t* __restrict__ prepared, const ActivationLayout layout,
         float* __restrict__ scales) {
+    const uint32_t ld = layout.ld;
     __shared__ float slot_max[16];
     __shared__ uint32_t slot_bad[16];
     const uint32_t row = blockIdx.x;
@@ -86,25 +87,53 @@ __global__ __launch_bounds__(1024) void prepare_i8_kernel(
     }
     float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
-    int8_t* dst = prepared + (size_t)row * ld;
 #pragma unroll
     for (int i = 0; i < kKept; i++) {
         const uint32_t j = threadIdx.x + i * blockDim.x;
-        if (j < ld) dst[j] = (int8_t)(!bad && j < k ? packed_round_i8(__fdiv_rn(kept[i], scale)) : 0);
+        if (j < ld)
+            prepared[activation_offset(layout, row, j)] =
+                (int8_t)(!bad && j < k ? packed_round_i8(__fdiv_rn(kept[i], scale)) : 0);
     }
     for (uint32_t j = threadIdx.x + kKept * blockDim.x; j < ld; j += blockDim.x) {
         int32_t q = 0;
         if (!bad && j < k) q = packed_round_i8(__fdiv_rn(src[j], scale));
-        dst[j] = (int8_t)q;
+        prepared[activation_offset(layout, row, j)] = (int8_t)q;
     }
     if (threadIdx.x == 0) scales[row] = bad ? __builtin_nanf("") : scale;
 }
 
 VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
-                              int8_t* prepared, uint32_t ld, float* scales) {
+                              int8_t* prepared, ActivationLayout layout, float* scales) {
+    // (operand order has room for 32 rows, and its rows are whole 16-byte chunks)
+    if (layout.operand_order && (rows > kOperandOrderRows || layout.ld != (k + 15u) / 16u * 16u))
+        return VXHIP_INVALID_ARGUMENT;
     // few long rows: latency bound, give each row a full workgroup
     const uint32_t block = rows <= 256u && k >= 1024u ? 1024u : 256u;
-    hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(block), 0, s, x, k, prepared, ld, scales);
+    hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(block), 0, s, x, k, prepared, layout, scales);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
+// one thread per 16-byte chunk of a row
+__global__ __launch_bounds__(256) void unblock_activations_kernel(const int8_t* __restrict__ blocked,
+                                                                  uint32_t rows, uint32_t chunks,
+                                                                  int8_t* __restrict__ row_major, uint32_t ld) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= rows * chunks) return;
+    const uint32_t row = i / chunks, chunk = i % chunks;
+    *reinterpret_cast<uint4*>(row_major + (size_t)row * ld + chunk * 16u) =
+        *reinterpret_cast<const uint4*>(blocked + ((size_t)chunk * kOperandOrderRows + row) * 16u);
+}
+
+VxHipStatus launch_unblock_activations(hipStream_t s, const int8_t* blocked, uint32_t rows, uint32_t k,
+                                       int8_t* row_major, uint32_t ld) {
+    const uint32_t chunks = (k + 15u) / 16u;
+    if (rows > kOperandOrderRows || ld < chunks * 16u || (ld % 16u) != 0u || ((uintptr_t)blocked % 16u) != 0u ||
+        ((uintptr_t)row_major % 16u) != 0u)
+        return VXHIP_INVALID_ARGUMENT;
+    if (!rows) return VXHIP_OK;
+    hipLaunchKernelGGL(unblock_activations_kernel, dim3((rows * chunks + 255u) / 256u), dim3(256), 0, s, blocked,
+                       rows, chunks, row_major, ld);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

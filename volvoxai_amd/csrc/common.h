@@ -74,6 +74,7 @@ struct VxHipContext {
     int div_used = 0, div_next = 0;
     const char* last_variant = "";
     int cu_count = 0;
+    uint32_t activation_layout = 0;  // VXHIP_ACTIVATIONS_*: what the prepare entry points write for rows <= 32
 };
 
 struct VxHipQLinear {
@@ -120,8 +121,25 @@ VxHipStatus weight_row_stats(hipStream_t stream, const uint8_t* raw_dev, size_t 
 // boundary.hip ---------------------------------------------------------------
 VxHipStatus launch_stage_activations(hipStream_t s, const void* x, uint32_t rows, uint32_t k,
                                      bool flip, int8_t* staged, uint32_t ld, int32_t* rowsum);
+// Where code j of activation row `row` lives.  Row major: row * ld + j.  Operand order (at most
+// 32 rows): the row's 16-byte chunks interleaved with those of the other rows,
+// ((j / 16) * 32 + row) * 16 + j % 16, which is how a wavefront of the streaming GEMV wants them:
+// the 64 lanes' loads of one k-step are then 1 KiB in a row (8 cache lines) instead of 32 bytes
+// from each of 32 lines.  Such a buffer always holds 32 rows of ceil(k / 16) chunks.
+struct ActivationLayout {
+    uint32_t ld;
+    uint32_t operand_order;
+};
+__host__ __device__ inline size_t activation_offset(ActivationLayout layout, uint32_t row, uint32_t j) {
+    return layout.operand_order ? ((size_t)(j >> 4) * 32u + row) * 16u + (j & 15u) : (size_t)row * layout.ld + j;
+}
+constexpr uint32_t kOperandOrderRows = 32;
+
 VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
-                              int8_t* prepared, uint32_t ld, float* scales);
+                              int8_t* prepared, ActivationLayout layout, float* scales);
+// operand-order activations (rows <= 32, k codes each) back to row-major rows of ld bytes
+VxHipStatus launch_unblock_activations(hipStream_t s, const int8_t* blocked, uint32_t rows, uint32_t k,
+                                       int8_t* row_major, uint32_t ld);
 VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t value);
 // Counts, over every f32 mantissa of the dividend, where the one- and the two-correction
 // division by `divisor` differ from IEEE division: counters[0] and counters[1].
@@ -136,8 +154,9 @@ enum class Epilogue : int { RequantTensor = 0, RequantRow = 1, DequantF32 = 2 };
 
 struct LinearArgs {
     Epilogue mode;
-    const int8_t* x;        // signed activations [rows][ldx]
+    const int8_t* x;        // signed activations [rows][ldx], or in operand order (GEMV only)
     uint32_t ldx;
+    uint32_t x_operand_order;  // see ActivationLayout; rows <= 32
     uint32_t rows, n, k;
     const int8_t* w;        // packed
     uint32_t panels, ksteps;

@@ -49,8 +49,10 @@ __device__ __forceinline__ float block_sum(float v, float* slots) {
 // written by thread j % blockDim.x, which is also the thread that reads it here.
 // scale = max|v| / 127 (1.0 for an all-zero row, floored at 2^-126), code = ties-to-even(v / scale)
 // clamped to +-127 with a true f32 divide; a non-finite row gets zero codes and a NaN scale.
-__device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_t* codes, float* scale_out,
-                                            float* slots) {
+// The codes of row `row` go where `layout` puts them (row-major rows of d bytes, or operand order,
+// whose last 16-byte chunk is filled up with zeros).
+__device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_t* codes, ActivationLayout layout,
+                                            uint32_t row, float* scale_out, float* slots) {
     // one reduction for both questions: a non-finite element counts as +inf, which no finite
     // maximum can be
     float maximum = 0.0f;
@@ -63,7 +65,10 @@ __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_
     float scale = maximum == 0.0f || bad != 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
     if (scale < 0x1p-126f) scale = 0x1p-126f;
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x)
-        codes[j] = bad != 0.0f ? (int8_t)0 : (int8_t)packed_round_i8(__fdiv_rn(vals[j], scale));
+        codes[activation_offset(layout, row, j)] =
+            bad != 0.0f ? (int8_t)0 : (int8_t)packed_round_i8(__fdiv_rn(vals[j], scale));
+    if (layout.operand_order)
+        for (uint32_t j = d + threadIdx.x; j < layout.ld; j += blockDim.x) codes[activation_offset(layout, row, j)] = 0;
     if (threadIdx.x == 0) *scale_out = bad != 0.0f ? __builtin_nanf("") : scale;
 }
 
@@ -72,6 +77,7 @@ __device__ __forceinline__ void prepare_row(const float* vals, uint32_t d, int8_
 __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict__ x, const float* __restrict__ delta,
                                                               const float* __restrict__ gain, uint32_t d, double eps,
                                                               int8_t* __restrict__ prepared,
+                                                              const ActivationLayout layout,
                                                               float* __restrict__ row_scales,
                                                               float* __restrict__ normalized) {
     float* vals = reinterpret_cast<float*>(glue_lds);
@@ -105,11 +111,12 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
         if (normalized) normalized[(size_t)row * d + j] = y;
     }
     // (no barrier: prepare_row walks the row with the same stride, a thread reads its own writes)
-    prepare_row(vals, d, prepared + (size_t)row * d, row_scales + row, slots);
+    prepare_row(vals, d, prepared, layout, row, row_scales + row, slots);
 }
 
 __global__ __launch_bounds__(1024) void swiglu_prepare_kernel(const float* __restrict__ gate_up, uint32_t inter,
                                                              int8_t* __restrict__ prepared,
+                                                             const ActivationLayout layout,
                                                              float* __restrict__ row_scales,
                                                              float* __restrict__ activated) {
     float* vals = reinterpret_cast<float*>(glue_lds);
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(1024) void swiglu_prepare_kernel(const float* __res
         if (activated) activated[(size_t)row * inter + j] = y;
     }
     // (no barrier: prepare_row walks the row with the same stride, a thread reads its own writes)
-    prepare_row(vals, inter, prepared + (size_t)row * inter, row_scales + row, slots);
+    prepare_row(vals, inter, prepared, layout, row, row_scales + row, slots);
 }
 
 // grid (rows * t, q_heads + 2 * kv_heads), block head_dim.  Token (row, i) sits at cache slot
@@ -724,6 +731,14 @@ bool device_ready(VxHipContext* ctx) {
     return ctx && hipSetDevice(ctx->device) == hipSuccess;
 }
 
+// What a prepare entry point writes: row-major rows of d codes, or, on a context set to
+// VXHIP_ACTIVATIONS_OPERAND32 and for at most 32 rows, operand order.
+ActivationLayout prepared_layout(const VxHipContext* ctx, uint32_t rows, uint32_t d) {
+    if (ctx->activation_layout == VXHIP_ACTIVATIONS_OPERAND32 && rows <= kOperandOrderRows)
+        return ActivationLayout{(d + 15u) / 16u * 16u, 1u};
+    return ActivationLayout{d, 0u};
+}
+
 // Picks the instance for the query heads per workgroup (4 or 1) and the head size.
 template <bool FUSED>
 void launch_attention(hipStream_t stream, uint32_t together, dim3 grid, size_t lds, const float* q, float* k_cache,
@@ -839,7 +854,7 @@ VxHipStatus vxhip_rmsnorm_prepare_i8(VxHipContext* ctx, const float* input_dev, 
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(row_block(rows, d)), d * sizeof(float), ctx->stream,
                        const_cast<float*>(input_dev), (const float*)nullptr, gain_dev, d, eps, prepared_dev,
-                       row_scales_dev, normalized_dev);
+                       prepared_layout(ctx, rows, d), row_scales_dev, normalized_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -854,8 +869,8 @@ VxHipStatus vxhip_add_rmsnorm_prepare_i8(VxHipContext* ctx, float* residual_dev,
     if (!rows) return VXHIP_OK;
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     hipLaunchKernelGGL(rmsnorm_prepare_kernel, dim3(rows), dim3(row_block(rows, d)), d * sizeof(float), ctx->stream,
-                       residual_dev,
-                       delta_dev, gain_dev, d, eps, prepared_dev, row_scales_dev, (float*)nullptr);
+                       residual_dev, delta_dev, gain_dev, d, eps, prepared_dev, prepared_layout(ctx, rows, d),
+                       row_scales_dev, (float*)nullptr);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -869,8 +884,8 @@ VxHipStatus vxhip_swiglu_prepare_i8(VxHipContext* ctx, const float* gate_up_dev,
     if (!rows) return VXHIP_OK;
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     hipLaunchKernelGGL(swiglu_prepare_kernel, dim3(rows), dim3(row_block(rows, inter)), inter * sizeof(float),
-                       ctx->stream,
-                       gate_up_dev, inter, prepared_dev, row_scales_dev, activated_dev);
+                       ctx->stream, gate_up_dev, inter, prepared_dev, prepared_layout(ctx, rows, inter), row_scales_dev,
+                       activated_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }

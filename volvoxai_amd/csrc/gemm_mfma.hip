@@ -765,6 +765,7 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
 }  // namespace
 
 const char* launch_gemm_mfma(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
+    if (a.x_operand_order) return nullptr;  // the tiles are staged from row-major activations
     if (a.ldx < 16u || (a.ldx % 16u) != 0u || ((uintptr_t)a.x % 16u) != 0u) return nullptr;
     if ((uint64_t)a.rows * a.ldx > 0xffffffffull) return nullptr;  // 32-bit activation offsets
     if (a.weight_bits != 8u && !(a.weight_bits == 4u && a.mode == Epilogue::DequantF32)) return nullptr;

@@ -94,7 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 
     const int8_t* wp = a.w + (size_t)panel * a.ksteps * 1024u + src_lane * 16u;
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
-    const int8_t* xp = a.x + (size_t)m * a.ldx;
+    // row-major rows, or operand order: the row's 16-byte chunks 512 bytes apart (see
+    // ActivationLayout), which makes the 64 lanes' loads of a k-step one contiguous KiB
+    const int8_t* xp = a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
+    const uint32_t x_chunk_pitch = a.x_operand_order ? 16u * kOperandOrderRows : 16u;
     const uint32_t half = lane >> 5;
     const uint32_t last_chunk = (a.k - 1u) / 16u;
 
@@ -110,7 +113,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
         for (int h = 0; h < SPB; h++) {
             const uint32_t chunk = min((t + h) * 2u + half, last_chunk);
-            xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + chunk * 16u);
+            xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
         }
     };
 
@@ -355,9 +358,9 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (cu_count <= 0) cu_count = 256;
-    if (a.rows == 0u || a.rows > kMaxGemvRows || a.ldx < 16u || (a.ldx % 16u) != 0u ||
-        ((uintptr_t)a.x % 16u) != 0u)
-        return nullptr;
+    if (a.rows == 0u || a.rows > kMaxGemvRows || ((uintptr_t)a.x % 16u) != 0u) return nullptr;
+    if (!a.x_operand_order && (a.ldx < 16u || (a.ldx % 16u) != 0u)) return nullptr;
+    static_assert(kMaxGemvRows <= kOperandOrderRows, "an operand-order buffer holds every row of a GEMV");
     if (a.weight_bits != 8u && !(a.weight_bits == 4u && a.mode == Epilogue::DequantF32)) return nullptr;
     const char* kind = nullptr;
     const char* family = nullptr;

@@ -112,6 +112,9 @@ class W8A8Decoder:
         self.torch, self.cfg, self.rows, self.fused = torch, cfg, rows, fused
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
+        # prepared activations of up to 32 rows travel between the glue kernels and the GEMVs in
+        # the GEMV's operand order (the fused path only: the other prepares inside each linear)
+        self.ctx.set_activation_layout(fused)
         dev = "cuda"
 
         def make(lin):
@@ -155,7 +158,7 @@ class W8A8Decoder:
 
     def _linear_a8(self, pl, a8, scales):
         torch = self.torch
-        out = torch.empty((a8.shape[0], pl.n), dtype=torch.float32, device=a8.device)
+        out = torch.empty((scales.shape[0], pl.n), dtype=torch.float32, device=a8.device)
         st, _ = pl.forward_a8(self.ctx, a8, scales, out=out)
         if st != 0:
             raise RuntimeError(_library().vxhip_last_error().decode())

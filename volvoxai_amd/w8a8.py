@@ -84,6 +84,21 @@ class Context:
     def last_variant(self) -> str:
         return library().vxhip_context_last_variant(self._h).decode()
 
+    def set_activation_layout(self, operand_order: bool):
+        """Prepared activations of calls with up to 32 rows in the GEMV's operand order (True) or
+        row major (False, the default); see vxhip_context_set_activation_layout."""
+        _check(library().vxhip_context_set_activation_layout(self._h, 1 if operand_order else 0),
+               "vxhip_context_set_activation_layout")
+
+    def prepared_buffer(self, rows: int, k: int, device):
+        """An int8 buffer for the prepared codes of rows x k in this context's layout: [rows, k] row
+        major, or flat (32 * ceil(k/16) * 16 bytes) in operand order."""
+        import torch
+        nbytes = library().vxhip_context_prepared_bytes(self._h, rows, k)
+        if nbytes == rows * k:
+            return torch.empty((rows, k), dtype=torch.int8, device=device)
+        return torch.empty((nbytes,), dtype=torch.int8, device=device)
+
     def fault_flags(self) -> int:
         v = C.c_uint32(0)
         _check(library().vxhip_context_fault_flags(self._h, C.byref(v)), "vxhip_context_fault_flags")
@@ -207,7 +222,7 @@ class PackedLinear:
     def forward_a8(self, ctx: Context, a8, row_scales, out=None, want_accumulators=False,
                    accumulators=None):
         import torch
-        rows = a8.shape[0]
+        rows = row_scales.shape[0]  # (a8 is flat when the context exchanges operand-order activations)
         if out is None:
             out = torch.empty((rows, self.n), dtype=torch.float32, device=a8.device)
         if want_accumulators and accumulators is None:
@@ -221,7 +236,7 @@ def rmsnorm_prepare_i8(ctx: Context, x, gain, eps, want_normalized=False):
     """RMSNorm then activation preparation of x [rows, d]; returns (codes int8, row scales[, normalized f32])."""
     import torch
     rows, d = x.shape
-    a8 = torch.empty((rows, d), dtype=torch.int8, device=x.device)
+    a8 = ctx.prepared_buffer(rows, d, x.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
     normalized = torch.empty((rows, d), dtype=torch.float32, device=x.device) if want_normalized else None
     _check(library().vxhip_rmsnorm_prepare_i8(ctx._h, _dp(x), _dp(gain), rows, d, float(eps), _dp(a8), _dp(scales),
@@ -233,7 +248,7 @@ def add_rmsnorm_prepare_i8(ctx: Context, residual, delta, gain, eps):
     """residual += delta in place, then RMSNorm and preparation of the updated rows."""
     import torch
     rows, d = residual.shape
-    a8 = torch.empty((rows, d), dtype=torch.int8, device=residual.device)
+    a8 = ctx.prepared_buffer(rows, d, residual.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=residual.device)
     _check(library().vxhip_add_rmsnorm_prepare_i8(ctx._h, _dp(residual), _dp(delta), _dp(gain), rows, d, float(eps),
                                                   _dp(a8), _dp(scales)), "vxhip_add_rmsnorm_prepare_i8")
@@ -245,7 +260,7 @@ def swiglu_prepare_i8(ctx: Context, gate_up, want_activated=False):
     import torch
     rows, two = gate_up.shape
     inter = two // 2
-    a8 = torch.empty((rows, inter), dtype=torch.int8, device=gate_up.device)
+    a8 = ctx.prepared_buffer(rows, inter, gate_up.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=gate_up.device)
     act = torch.empty((rows, inter), dtype=torch.float32, device=gate_up.device) if want_activated else None
     _check(library().vxhip_swiglu_prepare_i8(ctx._h, _dp(gate_up), rows, inter, _dp(a8), _dp(scales), _dp(act)),
@@ -313,10 +328,26 @@ def argmax_rows(ctx: Context, x, out=None, advance=None):
     return out
 
 
+def operand_order_codes(a8):
+    """Row-major int8 codes [rows <= 32, k] (numpy) re-ordered the way a context with
+    set_activation_layout(True) exchanges them: flat, 32 * ceil(k/16) * 16 bytes, code j of row r
+    at ((j // 16) * 32 + r) * 16 + j % 16, zeros elsewhere."""
+    a8 = np.ascontiguousarray(a8, dtype=np.int8)
+    rows, k = a8.shape
+    if rows > 32:
+        raise ValueError("operand order holds at most 32 rows")
+    chunks = (k + 15) // 16
+    padded = np.zeros((rows, chunks * 16), np.int8)
+    padded[:, :k] = a8
+    out = np.zeros((chunks, 32, 16), np.int8)
+    out[:, :rows] = padded.reshape(rows, chunks, 16).transpose(1, 0, 2)
+    return out.reshape(-1)
+
+
 def packed_prepare_i8(ctx: Context, x):
     import torch
     rows, k = x.shape
-    a8 = torch.empty((rows, k), dtype=torch.int8, device=x.device)
+    a8 = ctx.prepared_buffer(rows, k, x.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
     _check(library().vxhip_packed_prepare_i8(ctx._h, _dp(x), rows, k, _dp(a8), _dp(scales)),
            "vxhip_packed_prepare_i8")
