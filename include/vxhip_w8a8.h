@@ -76,8 +76,11 @@ VxHipStatus vxhip_context_synchronize(VxHipContext* context);
  * "hip.qlinear.mfma-i8.t256x256" -- the string a provider reports as
  * route_evidence (runtime/public_api_model_lifecycle.inc:748-751). */
 const char* vxhip_context_last_variant(const VxHipContext* context);
-/* Device-side fault word accumulated by kernels (non-finite multiplier seen,
- * ...); reading it synchronises the stream.  0 = clean. */
+/* Device-side fault word accumulated by kernels; reading it synchronises the
+ * stream.  0 = clean.  Bit 1: a requantization multiplier was not finite and
+ * positive.  Bit 2: an embedding id outside the table (its row is zeros).
+ * Bit 4: a cache position at or past max_seq was given to the rotary/attention
+ * entry points (that token's caches and output are left untouched). */
 VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
 /* Layout of prepared activations (int8 codes) handed between entry points on
  * this context; no counterpart in the reference, whose prepared rows

@@ -218,6 +218,39 @@ def test_fused_decode_attention_equals_the_two_kernels(ctx, rows, start, q_heads
 
 
 @pytest.mark.gpu
+def test_a_position_outside_the_cache_is_refused_on_the_device():
+    """A cache slot at or past max_seq reaches the kernels only as a value in device memory: they
+    leave the caches and that token's output alone and raise fault bit 4."""
+    import torch
+    import volvoxai_amd as vx
+    from volvoxai_amd import w8a8
+    own = vx.Context(0, None)  # fault bits are sticky: not the shared context
+    rng = np.random.default_rng(5)
+    rows, q_heads, kv_heads, head_dim, max_seq = 2, 4, 2, 64, 48
+    width = (q_heads + 2 * kv_heads) * head_dim
+    angle = rng.uniform(0, 6.28, (max_seq, head_dim)).astype(np.float32)
+    cos, sin = torch.from_numpy(np.cos(angle)).cuda(), torch.from_numpy(np.sin(angle)).cuda()
+    cache = rng.normal(0, 1, (2, rows, kv_heads, max_seq, head_dim)).astype(np.float32)
+    k, v = torch.from_numpy(cache[0]).cuda(), torch.from_numpy(cache[1]).cuda()
+    k0, v0 = k.clone(), v.clone()
+    qkv = torch.from_numpy(rng.normal(0, 1, (rows, width)).astype(np.float32)).cuda()
+    bad = torch.tensor([max_seq], dtype=torch.int64, device="cuda")
+    w8a8.rope_gqa_attention_decode(own, qkv, cos, sin, bad, q_heads, kv_heads, head_dim, k, v)
+    assert own.fault_flags() == 4 and torch.equal(k, k0) and torch.equal(v, v0)
+    w8a8.rope_append_kv(own, qkv.reshape(rows, 1, width), cos, sin, bad, q_heads, kv_heads, head_dim, k, v)
+    # a prompt whose last tokens run past the cache: the tokens inside are attended as usual
+    t = 12
+    positions = torch.arange(max_seq - 8, max_seq - 8 + t, dtype=torch.int64, device="cuda")
+    q = torch.from_numpy(rng.normal(0, 1, (rows, t, q_heads, head_dim)).astype(np.float32)).cuda()
+    out = w8a8.gqa_attention(own, q, k, v, positions)
+    inside = w8a8.gqa_attention(own, q[:, :8].contiguous(), k, v, positions[:8])
+    own.synchronize()
+    assert own.fault_flags() == 4 and torch.equal(k, k0) and torch.equal(v, v0)
+    assert torch.allclose(out[:, :8], inside, rtol=2e-5, atol=2e-6)
+    own.close()
+
+
+@pytest.mark.gpu
 def test_embedding_gather_and_argmax_kernels(ctx, oracle):
     import torch
     from volvoxai_amd import w8a8

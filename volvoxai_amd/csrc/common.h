@@ -54,6 +54,7 @@ constexpr uint32_t kMaxGemvRows = 32;  // the MFMA operand has 32 row slots
 enum FaultBits : uint32_t {
     kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive
     kFaultBadToken = 2u,        // an embedding lookup was asked for a row outside the table
+    kFaultBadPosition = 4u,     // a cache slot at or past max_seq was named: nothing read or written there
 };
 
 }  // namespace vxhip

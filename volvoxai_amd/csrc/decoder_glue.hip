@@ -141,12 +141,17 @@ __global__ void rope_append_kernel(const float* __restrict__ qkv, const float* _
                                    const float* __restrict__ sin_table, const int64_t* __restrict__ positions,
                                    uint32_t t, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
                                    uint32_t max_seq, float* __restrict__ q_out, float* __restrict__ k_cache,
-                                   float* __restrict__ v_cache) {
+                                   float* __restrict__ v_cache, uint32_t* __restrict__ fault) {
     const uint32_t token = blockIdx.x, head = blockIdx.y, dd = threadIdx.x;
     const uint32_t row = token / t, i = token % t;
     const uint32_t width = (q_heads + 2u * kv_heads) * head_dim;
     const float* src = qkv + (size_t)token * width + (size_t)head * head_dim;
-    const uint32_t slot = (uint32_t)positions[i];
+    const uint64_t named = (uint64_t)positions[i];
+    if (named >= max_seq) {  // outside the caches and the tables: touch nothing, say so
+        if (dd == 0) atomicOr(fault, (uint32_t)kFaultBadPosition);
+        return;
+    }
+    const uint32_t slot = (uint32_t)named;
     const uint32_t half = head_dim / 2u;
     const float v = src[dd];
     if (head >= q_heads + kv_heads) {  // value head: plain append
@@ -188,7 +193,8 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
                                                             uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
                                                             uint32_t max_seq, float scale, float* __restrict__ out,
                                                             const float* __restrict__ cos_table,
-                                                            const float* __restrict__ sin_table) {
+                                                            const float* __restrict__ sin_table,
+                                                            uint32_t* __restrict__ fault) {
     const uint32_t per_head = 9u * head_dim + max_seq;
     float* lds = reinterpret_cast<float*>(glue_lds);
     float* k_new = lds + REP * per_head;  // FUSED: the appended key and value, head_dim floats each
@@ -198,7 +204,12 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     const uint32_t head0 = blockIdx.y * REP;
     const uint32_t row = token / t, i = token % t;
     const uint32_t kvh = head0 / (q_heads / kv_heads);
-    const uint32_t position = (uint32_t)positions[i];
+    const uint64_t named = (uint64_t)positions[i];
+    if (named >= max_seq) {  // (the whole workgroup) outside the caches: touch nothing, say so
+        if (threadIdx.x == 0) atomicOr(fault, (uint32_t)kFaultBadPosition);
+        return;
+    }
+    const uint32_t position = (uint32_t)named;
     const uint32_t visible = position + 1u;  // slots 0 .. position
     // slots read from the caches: all visible ones, or all before the one being appended
     const uint32_t cached = FUSED ? position : visible;
@@ -560,7 +571,7 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
                                                           const int64_t* __restrict__ positions, uint32_t t,
                                                           uint32_t tq, uint32_t q_heads, uint32_t kv_heads,
                                                           uint32_t head_dim, uint32_t max_seq, float scale,
-                                                          float* __restrict__ out) {
+                                                          float* __restrict__ out, uint32_t* __restrict__ fault) {
     __shared__ uint32_t visible[kPrefillQueries];  // slots query i may see; 0: no such query
     const uint32_t rep = q_heads / kv_heads, qw = tq * rep;
     const uint32_t blocks = (t + tq - 1u) / tq;
@@ -577,7 +588,11 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
     if (threadIdx.x < kPrefillQueries) {
         const uint32_t qi = threadIdx.x;
         uint32_t v = 0u;
-        if (qi < qw && token_of(qi) < t) v = min((uint32_t)positions[token_of(qi)] + 1u, max_seq);
+        if (qi < qw && token_of(qi) < t) {
+            const uint64_t named = (uint64_t)positions[token_of(qi)];
+            if (named >= max_seq) atomicOr(fault, (uint32_t)kFaultBadPosition);  // (its output row is left as it is)
+            else v = (uint32_t)named + 1u;
+        }
         visible[qi] = v;
     }
     __syncthreads();
@@ -710,7 +725,7 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const uint32_t qi = first + j;
-            if (qi >= qw || token_of(qi) >= t) continue;
+            if (qi >= qw || token_of(qi) >= t || visible[qi] == 0u) continue;
             float* dst = out + ((size_t)(row * t + token_of(qi)) * q_heads + head_of(qi)) * head_dim;
 #pragma unroll
             for (int pass = 0; pass < 2; pass++) {
@@ -744,10 +759,10 @@ template <bool FUSED>
 void launch_attention(hipStream_t stream, uint32_t together, dim3 grid, size_t lds, const float* q, float* k_cache,
                       float* v_cache, const int64_t* positions, uint32_t t, uint32_t q_heads, uint32_t kv_heads,
                       uint32_t head_dim, uint32_t max_seq, float scale, float* out, const float* cos_table,
-                      const float* sin_table) {
+                      const float* sin_table, uint32_t* fault) {
 #define VXHIP_ATTENTION(R, NC)                                                                                  \
     hipLaunchKernelGGL((gqa_attention_kernel<R, FUSED, NC>), grid, dim3(256), lds, stream, q, k_cache, v_cache, \
-                       positions, t, q_heads, kv_heads, head_dim, max_seq, scale, out, cos_table, sin_table)
+                       positions, t, q_heads, kv_heads, head_dim, max_seq, scale, out, cos_table, sin_table, fault)
 #define VXHIP_ATTENTION_HEADS(NC)     \
     do {                              \
         if (together == 4u) VXHIP_ATTENTION(4, NC); \
@@ -903,7 +918,7 @@ VxHipStatus vxhip_rope_append_kv(VxHipContext* ctx, const float* qkv_dev, const 
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     hipLaunchKernelGGL(rope_append_kernel, dim3(rows * t, q_heads + 2u * kv_heads), dim3(head_dim), 0, ctx->stream,
                        qkv_dev, cos_dev, sin_dev, positions_dev, t, q_heads, kv_heads, head_dim, max_seq, q_out_dev,
-                       k_cache_dev, v_cache_dev);
+                       k_cache_dev, v_cache_dev, ctx->fault_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -944,7 +959,8 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
             }
             const dim3 grid(rows * ((t + tq - 1u) / tq), kv_heads);
             hipLaunchKernelGGL(gqa_prefill_kernel, grid, dim3(256), lds_for(tq), ctx->stream, q_dev, k_cache_dev,
-                               v_cache_dev, positions_dev, t, tq, q_heads, kv_heads, head_dim, max_seq, scale, out_dev);
+                               v_cache_dev, positions_dev, t, tq, q_heads, kv_heads, head_dim, max_seq, scale, out_dev,
+                               ctx->fault_dev);
             VXHIP_TRY(hipGetLastError());
             return VXHIP_OK;
         }
@@ -961,7 +977,7 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
     const dim3 grid(rows * t, q_heads / together);
     launch_attention<false>(ctx->stream, together, grid, lds, q_dev, const_cast<float*>(k_cache_dev),
                             const_cast<float*>(v_cache_dev), positions_dev, t, q_heads, kv_heads, head_dim, max_seq,
-                            scale, out_dev, nullptr, nullptr);
+                            scale, out_dev, nullptr, nullptr, ctx->fault_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
@@ -988,7 +1004,7 @@ VxHipStatus vxhip_rope_gqa_attention_decode(VxHipContext* ctx, const float* qkv_
     }
     const dim3 grid(rows, q_heads / together);
     launch_attention<true>(ctx->stream, together, grid, lds, qkv_dev, k_cache_dev, v_cache_dev, position_dev, 1u,
-                           q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev, sin_dev);
+                           q_heads, kv_heads, head_dim, max_seq, scale, out_dev, cos_dev, sin_dev, ctx->fault_dev);
     VXHIP_TRY(hipGetLastError());
     return VXHIP_OK;
 }
