@@ -68,6 +68,9 @@ def write_safetensors(path, tensors):
              np.dtype(np.uint32): "U32", np.dtype(np.float32): "F32"}
     header, blobs, offset = {}, [], 0
     for name, arr in tensors.items():
+        if name == "__metadata__":  # free-form strings beside the tensors
+            header[name] = dict(arr)
+            continue
         arr = np.ascontiguousarray(arr)
         dtype = names[arr.dtype]
         if name.endswith("#as_i32"):  # packed words are stored as I32
@@ -305,6 +308,13 @@ def _drop(path):
     ("weight shape", lambda g, t: t.__setitem__("projection.weight", np.zeros((4, 5), np.int8)), -5),
     ("bias dtype", lambda g, t: t.__setitem__("projection.bias", np.zeros(4, np.float32)), -5),
     ("dangling weight", lambda g, t: t.pop("projection.weight"), -5),
+    # representations the v1 format retired (docs/w8a8-safetensors.md:176-188, :100-102)
+    ("retired graph field", lambda g, t: g.__setitem__("weights_quantization", {"projection.weight": "int8"}), -5),
+    ("retired storage field", lambda g, t: g.__setitem__("weights_quantization_storage", "safetensors"), -5),
+    ("inline input quantization", lambda g, t: g["inputs"]["hidden_q"].__setitem__("quantization", {"scale": 0.5}), -5),
+    ("node outputs_quantization", lambda g, t: g["nodes"][0].__setitem__("outputs_quantization", {"out": {}}), -5),
+    ("retired safetensors metadata", lambda g, t: t.__setitem__("__metadata__", {"weights_quantization": "int8"}), -5),
+    ("unrelated safetensors metadata", lambda g, t: t.__setitem__("__metadata__", {"exported_by": "a test"}), 0),
 ])
 def test_qlinear_package_refusals(registered, tmp_path, name, mutate, status):
     k = KAT

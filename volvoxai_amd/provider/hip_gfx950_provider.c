@@ -500,6 +500,15 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
             status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph format is not volvox-graph/v1%s", "");
             break;
         }
+        /* representations v1 retired: an artifact that carries one is not a v1 package
+         * (docs/w8a8-safetensors.md:176-188) */
+        if (vxj_member(root, "weights_quantization") || vxj_member(root, "weights_quantization_storage") ||
+            (graph_input && graph_input->kind == VXJ_OBJECT && vxj_member(graph_input, "quantization"))) {
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                            "the graph carries a retired quantization field (weights_quantization, "
+                            "weights_quantization_storage or an inline input quantization)%s", "");
+            break;
+        }
         if (!nodes || nodes->kind != VXJ_ARRAY || !nodes->count || nodes->count > MAX_CHAIN_NODES || !inputs ||
             inputs->count != 1 || !outputs || outputs->kind != VXJ_ARRAY || outputs->count != 1) {
             status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
@@ -527,10 +536,17 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
         }
         for (size_t i = 0; i < source->weight_path_count && status == VX_STATUS_OK; i++) {
             char error[VX_REPORT_MESSAGE_CAPACITY];
-            if (vxst_open(source->weight_paths[i], &chain->files[chain->file_count], error, sizeof(error)) != 0)
+            if (vxst_open(source->weight_paths[i], &chain->files[chain->file_count], error, sizeof(error)) != 0) {
                 status = refuse(failure, VX_STATUS_IO_ERROR, "%s", error);
-            else
-                chain->file_count++;
+            } else {
+                const VxstFile* opened = chain->files[chain->file_count++];
+                /* SafeTensors metadata is no quantization authority, and the retired keys make the
+                 * file invalid (docs/w8a8-safetensors.md:100-102) */
+                if (vxst_metadata_has(opened, "weights_quantization") ||
+                    vxst_metadata_has(opened, "weights_quantization_storage"))
+                    status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                    "weight file '%s' carries retired quantization metadata", source->weight_paths[i]);
+            }
         }
         if (status != VX_STATUS_OK) break;
 
@@ -544,6 +560,11 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
             const VxjValue* out_shape = vxj_member(out, "shape");
             const char* fed = vxj_member_string(vxj_member(node, "inputs"), "input");
             chain->count++;
+            if (node->kind == VXJ_OBJECT && vxj_member(node, "outputs_quantization")) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                "a node carries the retired outputs_quantization field%s", "");
+                break;
+            }
             plan->files = chain->files;
             plan->file_count = chain->file_count;
             if (!op || !out || !copy_name(plan->node_id, vxj_member_string(node, "id")) ||

@@ -112,3 +112,9 @@ int vxst_find(const VxstFile* f, const char* name, VxstTensor* out) {
     out->data = f->payload + b->integer;
     return 1;
 }
+
+int vxst_metadata_has(const VxstFile* f, const char* key) {
+    if (!f || !key) return 0;
+    const VxjValue* metadata = vxj_member(f->header, "__metadata__");
+    return metadata && metadata->kind == VXJ_OBJECT && vxj_member(metadata, key) != NULL;
+}

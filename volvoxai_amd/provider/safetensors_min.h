@@ -25,5 +25,7 @@ int vxst_open(const char* path, VxstFile** out, char* error, size_t error_capaci
 void vxst_close(VxstFile* file);
 /* 1 and *out filled if the file holds a tensor of that name, else 0. */
 int vxst_find(const VxstFile* file, const char* name, VxstTensor* out);
+/* 1 when the file's __metadata__ object has the key. */
+int vxst_metadata_has(const VxstFile* file, const char* key);
 
 #endif
