@@ -132,7 +132,10 @@ def test_rope_append_and_attention_kernels(ctx, rows, t, start):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("rows,t,start,q_heads,kv_heads,head_dim,max_seq", [
-    (2, 128, 0, 16, 8, 128, 256),   # the benchmark's prompt
+    (2, 128, 0, 16, 8, 128, 256),   # the benchmark's prompt (head size 128: the matrix-pipe kernel)
+    (1, 70, 5, 8, 2, 128, 200),     # the same kernel with ragged blocks, four query heads per KV head
+    (3, 9, 0, 3, 1, 128, 64),       # and with query rows left empty (27 of 32 used)
+    (1, 16, 0, 2, 2, 128, 9000),    # head size 128 with a cache too long for its 32 score rows
     (1, 40, 13, 8, 1, 64, 70),      # eight query heads per KV head, a prompt continued at slot 13
     (2, 9, 100, 4, 4, 256, 131),    # one head per KV head, the largest head size, an odd cache length
     (1, 200, 0, 2, 1, 32, 1000),    # a long cache: fewer tokens share a workgroup

@@ -736,6 +736,173 @@ __global__ __launch_bounds__(256) void gqa_prefill_kernel(const float* __restric
     }
 }
 
+// The same prompt attention for head size 128 on the f32 matrix pipes (v_mfma_f32_32x32x2f32: full
+// f32 products and sums, not a reduced-precision format).  The queries of a workgroup are the 32
+// rows of the A operand and stay in registers for the whole kernel: lane l holds query l % 32 and,
+// for the scores, 32 of its 128 channels.  Per 64-slot block:
+//   scores  wavefront w takes slots 32 * (w & 1) .. +31 and channels 64 * (w >> 1) .. +63: 32 MFMAs,
+//           each adding the channel pair (c, c + 32) of the lane halves; the two channel halves of
+//           a slot tile are added through the score rows in LDS (one stores, one adds and scales)
+//   P.V     wavefront w takes output channels 32 * w .. +31: 32 MFMAs, each adding the slot pair
+//           (s, s + 32); the sums stay in 16 accumulator registers across the blocks
+// Softmax and staging are those of the kernel above.  A workgroup's score rows are always 32.
+// (The kernel above reads its queries through the scalar cache, which two workgroups per compute
+// unit overflow: 189 us per launch of a 32-row, 128-token prompt against 102 us here.)
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void gqa_prefill_mfma_kernel(const float* __restrict__ q,
+                                                               const float* __restrict__ k_cache,
+                                                               const float* __restrict__ v_cache,
+                                                               const int64_t* __restrict__ positions, uint32_t t,
+                                                               uint32_t tq, uint32_t q_heads, uint32_t kv_heads,
+                                                               uint32_t max_seq, float scale, float* __restrict__ out,
+                                                               uint32_t* __restrict__ fault) {
+    constexpr uint32_t HD = 128u, HD4 = HD / 4u, PITCH = HD + 4u;
+    __shared__ uint32_t visible[kPrefillQueries];
+    const uint32_t rep = q_heads / kv_heads, qw = tq * rep;
+    const uint32_t blocks = (t + tq - 1u) / tq;
+    const uint32_t row = blockIdx.x / blocks, i0 = (blockIdx.x % blocks) * tq, kvh = blockIdx.y;
+    const uint32_t score_pitch = (max_seq + 63u) & ~63u;
+    float* sc = reinterpret_cast<float*>(glue_lds);             // [32][score_pitch]
+    float* stage = sc + (size_t)kPrefillQueries * score_pitch;  // [64][PITCH]
+    const float* kbase = k_cache + ((size_t)row * kv_heads + kvh) * max_seq * HD;
+    const float* vbase = v_cache + ((size_t)row * kv_heads + kvh) * max_seq * HD;
+    const uint32_t lane = threadIdx.x & 63u, r = lane & 31u, h = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    auto token_of = [&](uint32_t qi) { return i0 + qi / rep; };
+    auto head_of = [&](uint32_t qi) { return kvh * rep + qi % rep; };
+
+    if (threadIdx.x < kPrefillQueries) {
+        const uint32_t qi = threadIdx.x;
+        uint32_t v = 0u;
+        if (qi < qw && token_of(qi) < t) {
+            const uint64_t named = (uint64_t)positions[token_of(qi)];
+            if (named >= max_seq) atomicOr(fault, (uint32_t)kFaultBadPosition);  // (its output row is left as it is)
+            else v = (uint32_t)named + 1u;
+        }
+        visible[qi] = v;
+    }
+    // this lane's 32 channels of query r for the scores (zeros for a query that does not exist)
+    const uint32_t score_channel = 64u * (wave >> 1) + 32u * h;
+    float qreg[32];
+    {
+        const bool exists = r < qw && token_of(r) < t;
+        const float* src = q + ((size_t)(row * t + (exists ? token_of(r) : 0u)) * q_heads + head_of(exists ? r : 0u)) * HD +
+                           score_channel;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float4 v = exists ? *reinterpret_cast<const float4*>(src + 4 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            qreg[4 * j] = v.x, qreg[4 * j + 1] = v.y, qreg[4 * j + 2] = v.z, qreg[4 * j + 3] = v.w;
+        }
+    }
+    __syncthreads();
+    uint32_t span = 0u;
+    for (uint32_t qi = 0; qi < qw; qi++) span = max(span, visible[qi]);
+    const uint32_t span_blocks = (span + kPrefillSlots - 1u) / kPrefillSlots * kPrefillSlots;
+
+    constexpr int kStageRegs = 8;  // 64 rows x 128 floats over 256 threads, as 16-byte words
+    auto fetch_rows = [&](const float* base, uint32_t s0, float4 (&v)[kStageRegs]) {
+#pragma unroll
+        for (int u = 0; u < kStageRegs; u++) {
+            const uint32_t e = threadIdx.x + u * 256u, srow = s0 + e / HD4;
+            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (srow < span) v[u] = *reinterpret_cast<const float4*>(base + (size_t)srow * HD + 4u * (e % HD4));
+        }
+    };
+    auto commit_rows = [&](const float4 (&v)[kStageRegs]) {
+#pragma unroll
+        for (int u = 0; u < kStageRegs; u++) {
+            const uint32_t e = threadIdx.x + u * 256u;
+            *reinterpret_cast<float4*>(stage + (size_t)(e / HD4) * PITCH + 4u * (e % HD4)) = v[u];
+        }
+    };
+    float4 ahead[kStageRegs];
+    fetch_rows(kbase, 0u, ahead);
+
+    // The 16 accumulator registers of a lane are rows 8 * (v / 4) + 4 * h + v % 4 of column r.
+    auto tile_row = [&](int v) { return 8u * (uint32_t)(v / 4) + 4u * h + (uint32_t)(v % 4); };
+
+    for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {  // scores
+        commit_rows(ahead);
+        __syncthreads();
+        if (s0 + kPrefillSlots < span) fetch_rows(kbase, s0 + kPrefillSlots, ahead);
+        else fetch_rows(vbase, 0u, ahead);
+        const uint32_t slot_tile = 32u * (wave & 1u);
+        const float* krow = stage + (size_t)(slot_tile + r) * PITCH + score_channel;
+        v16f acc;
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float4 kv = *reinterpret_cast<const float4*>(krow + 4 * j);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[4 * j], kv.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[4 * j + 1], kv.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[4 * j + 2], kv.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[4 * j + 3], kv.w, acc, 0, 0, 0);
+        }
+        float* tile = sc + s0 + slot_tile + r;  // + query * score_pitch
+        if ((wave >> 1) == 0u) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) tile[(size_t)tile_row(v) * score_pitch] = acc[v];
+        }
+        __syncthreads();
+        if ((wave >> 1) == 1u) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float* at = tile + (size_t)tile_row(v) * score_pitch;
+                *at = __fmul_rn(__fadd_rn(*at, acc[v]), scale);
+            }
+        }
+        __syncthreads();
+    }
+    {   // softmax: probabilities over the visible slots, zeros from there to the end of the last block
+        for (uint32_t qi = wave; qi < kPrefillQueries; qi += 4u) {
+            float* mine = sc + (size_t)qi * score_pitch;
+            const uint32_t seen = qi < qw ? visible[qi] : 0u;
+            if (seen != 0u) {
+                float m = -INFINITY;
+                for (uint32_t s = lane; s < seen; s += 64u) m = fmaxf(m, mine[s]);
+                m = wave_max(m);
+                float sum = 0.0f;
+                for (uint32_t s = lane; s < seen; s += 64u) {
+                    const float e = expf(mine[s] - m);
+                    mine[s] = e;
+                    sum += e;
+                }
+                sum = wave_sum(sum);
+                for (uint32_t s = lane; s < seen; s += 64u) mine[s] = __fdiv_rn(mine[s], sum);
+            }
+            for (uint32_t s = seen + lane; s < span_blocks; s += 64u) mine[s] = 0.0f;
+        }
+    }
+    __syncthreads();
+    v16f o;
+#pragma unroll
+    for (int v = 0; v < 16; v++) o[v] = 0.0f;
+    for (uint32_t s0 = 0; s0 < span; s0 += kPrefillSlots) {  // P.V
+        commit_rows(ahead);
+        __syncthreads();
+        if (s0 + kPrefillSlots < span) fetch_rows(vbase, s0 + kPrefillSlots, ahead);
+        const float* prow = sc + (size_t)r * score_pitch + s0 + 32u * h;      // probabilities of query r
+        const float* vcol = stage + (size_t)(32u * h) * PITCH + 32u * wave + r;  // channel 32 * wave + r
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float4 pv = *reinterpret_cast<const float4*>(prow + 4 * j);
+            o = __builtin_amdgcn_mfma_f32_32x32x2f32(pv.x, vcol[(size_t)(4 * j) * PITCH], o, 0, 0, 0);
+            o = __builtin_amdgcn_mfma_f32_32x32x2f32(pv.y, vcol[(size_t)(4 * j + 1) * PITCH], o, 0, 0, 0);
+            o = __builtin_amdgcn_mfma_f32_32x32x2f32(pv.z, vcol[(size_t)(4 * j + 2) * PITCH], o, 0, 0, 0);
+            o = __builtin_amdgcn_mfma_f32_32x32x2f32(pv.w, vcol[(size_t)(4 * j + 3) * PITCH], o, 0, 0, 0);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const uint32_t qi = tile_row(v);
+        if (qi >= qw || token_of(qi) >= t || visible[qi] == 0u) continue;
+        out[((size_t)(row * t + token_of(qi)) * q_heads + head_of(qi)) * HD + 32u * wave + r] = o[v];
+    }
+}
+
 // Few rows leave most of the device idle and the kernel latency bound: then a row gets a full
 // 1024-thread workgroup; with many rows 256 threads per row keep more rows resident.
 uint32_t row_block(uint32_t rows, uint32_t d) {
@@ -936,6 +1103,25 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     const float scale = (float)(1.0 / sqrt((double)head_dim));
     const uint32_t rep = q_heads / kv_heads;
+    if (t >= 8u && rep <= kPrefillQueries && head_dim == 128u) {
+        // a prompt at head size 128: the matrix-pipe kernel, if its 32 score rows fit
+        const size_t lds = ((size_t)kPrefillQueries * ((max_seq + 63u) & ~63u) + (size_t)kPrefillSlots * (128u + 4u)) *
+                           sizeof(float);
+        if (lds <= 150u * 1024u) {
+            static std::atomic<uint64_t> configured{0};
+            if (!raise_lds_limit((const void*)gqa_prefill_mfma_kernel, 152 * 1024, configured)) {
+                set_error("gqa_attention: the prompt kernel's LDS limit could not be raised");
+                return VXHIP_EXECUTION_FAILED;
+            }
+            const uint32_t tq = kPrefillQueries / rep;
+            const dim3 grid(rows * ((t + tq - 1u) / tq), kv_heads);
+            hipLaunchKernelGGL(gqa_prefill_mfma_kernel, grid, dim3(256), lds, ctx->stream, q_dev, k_cache_dev,
+                               v_cache_dev, positions_dev, t, tq, q_heads, kv_heads, max_seq, scale, out_dev,
+                               ctx->fault_dev);
+            VXHIP_TRY(hipGetLastError());
+            return VXHIP_OK;
+        }
+    }
     if (t >= 8u && rep <= kPrefillQueries && head_dim <= 256u) {
         // a prompt: tokens share the walk over the cache, as many per workgroup as the LDS holds
         uint32_t tq = kPrefillQueries / rep;
