@@ -35,16 +35,6 @@ __device__ __forceinline__ float block_max(float v, float* slots) {
     return m;
 }
 
-__device__ __forceinline__ float block_sum(float v, float* slots) {
-    v = wave_sum_to_lane0(v);
-    if ((threadIdx.x & 63u) == 0u) slots[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = slots[0];
-    for (uint32_t w = 1; w < blockDim.x / 64u; w++) s += slots[w];
-    __syncthreads();
-    return s;
-}
-
 // Shared tail of the two *_prepare kernels: the row's f32 values are in `vals` (LDS), element j
 // written by thread j % blockDim.x, which is also the thread that reads it here.
 // scale = max|v| / 127 (1.0 for an all-zero row, floored at 2^-126), code = ties-to-even(v / scale)
@@ -199,7 +189,6 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
     float* lds = reinterpret_cast<float*>(glue_lds);
     float* k_new = lds + REP * per_head;  // FUSED: the appended key and value, head_dim floats each
     float* v_new = k_new + head_dim;
-    __shared__ float slots[4];
     const uint32_t token = blockIdx.x;
     const uint32_t head0 = blockIdx.y * REP;
     const uint32_t row = token / t, i = token % t;
@@ -467,19 +456,36 @@ __global__ __launch_bounds__(256) void gqa_attention_kernel(const float* __restr
         request_values(vv_a, 0u, chunk * 4u);
         request_values(vv_b, BATCH, chunk * 4u);
     }
-    __syncthreads();  // scores of a slot are read below by other threads than wrote them
+    // Softmax.  The heads' maxima cross the workgroup in one exchange (every thread scored slots
+    // of every head); after that the 4 / REP wavefronts of a group own one head each, so the heads'
+    // exponentials, sums and divisions run side by side instead of one head after the other.
+    {
+        constexpr uint32_t GROUP = 256u / REP, GROUP_WAVES = 4u / REP;
+        __shared__ float wave_maxima[4 * REP], wave_sums[4];
+        const uint32_t wave = threadIdx.x >> 6, own = threadIdx.x / GROUP, at = threadIdx.x % GROUP;
 #pragma unroll
-    for (int h = 0; h < REP; h++) {
-        float* scores = lds + h * per_head + head_dim;
-        const float mh = block_max(m[h], slots);
+        for (int h = 0; h < REP; h++) {
+            const float mw = wave_max(m[h]);
+            if ((threadIdx.x & 63u) == 0u) wave_maxima[wave * REP + h] = mw;
+        }
+        __syncthreads();  // (also: the scores of a slot are read below by other threads than wrote them)
+        float mh = wave_maxima[own];
+#pragma unroll
+        for (uint32_t w = 1; w < 4u; w++) mh = fmaxf(mh, wave_maxima[w * REP + own]);
+        float* scores = lds + own * per_head + head_dim;
         float sum = 0.0f;
-        for (uint32_t s = threadIdx.x; s < visible; s += 256u) {
+        for (uint32_t s = at; s < visible; s += GROUP) {
             const float e = expf(scores[s] - mh);
             scores[s] = e;
             sum += e;
         }
-        sum = block_sum(sum, slots);
-        for (uint32_t s = threadIdx.x; s < visible; s += 256u) scores[s] = __fdiv_rn(scores[s], sum);
+        sum = wave_sum_to_lane0(sum);
+        if ((threadIdx.x & 63u) == 0u) wave_sums[wave] = sum;
+        __syncthreads();
+        float total = wave_sums[own * GROUP_WAVES];
+#pragma unroll
+        for (uint32_t w = 1; w < GROUP_WAVES; w++) total += wave_sums[own * GROUP_WAVES + w];
+        for (uint32_t s = at; s < visible; s += GROUP) scores[s] = __fdiv_rn(scores[s], total);
     }
     __syncthreads();
     for (uint32_t c4 = chunk * 4u; c4 < head_dim; c4 += 128u) {
