@@ -156,6 +156,10 @@ int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
                 !vxo_multiplier(row_scales[r], weight_scales[n], output_scale, &m))
                 return 0;
         }
+    /* the real-valued bias is part of the descriptor: a value that is not finite declines the call */
+    if (bias_f32)
+        for (uint32_t n = 0; n < d_out; n++)
+            if (!finite_f32(bias_f32[n])) return 0;
     for (uint32_t r = 0; r < rows; r++) {
         for (uint32_t n = 0; n < d_out; n++) {
             /* the reference loop with rows = 1 and input_scale = row_scales[r] */

@@ -10,11 +10,15 @@
  * Parity status: every function below is pinned by the reference's own
  * known-answer vectors (tests/golden/reference_kats.json) and, where the
  * reference tree is available, by a byte comparison against the reference C
- * compiled from its own sources (oracle/_ref).  The one exception is the
- * optional f32 bias of vxo_qlinear_rowscale_i8u8: the reference has no
- * real-valued bias in its requantizing linear, so that term is an extension
- * ("parity unpinned" for that term only; with it absent the function is the
- * reference's per-row call and is pinned like the rest).
+ * compiled from its own sources (oracle/_ref).  The optional f32 bias of
+ * vxo_qlinear_rowscale_i8u8 has no reference counterpart (the reference's
+ * requantizing linear has an accumulator-domain bias only), so no reference
+ * vector can cover it; it is pinned instead by what its definition fixes:
+ * hand-derived cases in which another order of the additions, a single
+ * rounding or a reciprocal product give a different byte, and a seeded sweep
+ * against the rule evaluated in exact rationals with explicit roundings
+ * (tests/test_oracle.py).  With the bias absent the function is the
+ * reference's per-row call and is pinned like the rest.
  */
 #ifndef VXO_W8A8_ORACLE_H
 #define VXO_W8A8_ORACLE_H
@@ -61,7 +65,8 @@ int vxo_qlinear_i8u8(const void* input, const void* weight,
  * (may be NULL) is an EXTENSION with no reference counterpart: after the
  * reference transform t = f32(f32(acc)*mult) + f32(zp), the term
  * f32(bias_f32[n] / output_scale) is added with one more f32 rounding before
- * the saturating round.  With bias_f32 == NULL the bytes are the reference's. */
+ * the saturating round.  With bias_f32 == NULL the bytes are the reference's.
+ * A bias that is not finite declines the call, like an invalid scale. */
 int vxo_qlinear_rowscale_i8u8(const int8_t* input, const void* weight,
                               const int32_t* bias_i32, const float* bias_f32,
                               const float* weight_scales,

@@ -356,3 +356,106 @@ def test_ptq_rules(oracle):
     assert q.tolist() == [0, -127, 54]
     st, b = oracle.ptq_pack_bias(np.array([0.25, -0.75], np.float32), 0.5, np.array([0.5, 0.25], np.float32))
     assert st == 0 and b.tolist() == [1, -6]
+
+
+# ---- the real-valued bias of the per-token requantizing form (no reference counterpart) ------
+
+def _rn32(q):
+    """Round an exact rational to the nearest binary32 value, ties to even, by integer arithmetic
+    alone (normal range only): the definition of one IEEE rounding, independent of the host FPU."""
+    from fractions import Fraction
+    q = Fraction(q)
+    if q == 0:
+        return Fraction(0)
+    sign, mag = (-1 if q < 0 else 1), abs(q)
+    e = 0
+    while mag >= 2:
+        mag /= 2; e += 1
+    while mag < 1:
+        mag *= 2; e -= 1
+    assert -126 <= e <= 127
+    scaled = mag * (1 << 23)              # in [2^23, 2^24)
+    lo = scaled.numerator // scaled.denominator
+    rem = scaled - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (lo & 1)):
+        lo += 1
+    return sign * Fraction(lo, 1 << 23) * Fraction(2) ** e
+
+
+def _round_half_even(q):
+    from fractions import Fraction
+    lo = q.numerator // q.denominator
+    rem = q - lo
+    return lo + 1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (lo & 1)) else lo
+
+
+def _bias_rule(acc, s_row, s_w, s_y, zp, bias, lo=-128, hi=127):
+    """The extension's definition, in exact rationals with one explicit rounding per step:
+    y = sat_rne( rn( rn( rn(rn(acc) * rn(rn(s_row*s_w)/s_y)) + zp ) + rn(bias/s_y) ) )."""
+    from fractions import Fraction as Fr
+    mult = _rn32(_rn32(Fr(s_row) * Fr(s_w)) / Fr(s_y))
+    t1 = _rn32(_rn32(Fr(acc)) * mult)
+    t2 = _rn32(t1 + zp)
+    t = _rn32(t2 + _rn32(Fr(bias) / Fr(s_y)))
+    return max(lo, min(hi, _round_half_even(t)))
+
+
+def _one(oracle, x, w, s_row, s_w, s_y, zp, bias, out_dtype=I8):
+    ok, y, acc = oracle.qlinear_rowscale(
+        np.array([[x]], np.int8), np.array([[w]], np.int8), np.array([s_w], np.float32), np.zeros(1, np.int32),
+        np.array([s_row], np.float32), s_y, zp, out_dtype=out_dtype, bias_f32=np.array([bias], np.float32))
+    return ok, int(y[0, 0]), int(acc[0, 0])
+
+
+def test_rowscale_f32_bias_order_and_roundings(oracle):
+    """t = f32(f32(f32(acc)*mult) + zp), then t + f32(bias/s_y) as one more rounding, then the
+    saturating ties-even round.  Inputs where a plausible other form gives another byte."""
+    # (a) zero point first, then bias.  acc = 1, mult = 0.5 + 2^-24 (one ulp above a half), zp = 1,
+    # bias = -1: 1.5 + 2^-24 is a tie between 1.5 and 1.5 + 2^-23 and goes to the even 1.5; minus 1
+    # is the tie 0.5 -> 0.  Bias first (exact -0.5 + 2^-24, then + 1 = 0.5 + 2^-24 -> 1) and a single
+    # rounding of the exact sum (0.5 + 2^-24 -> 1) both give 1.
+    m = float.fromhex("0x1.000002p-1")
+    assert _one(oracle, 1, 1, m, 1.0, 1.0, 1, -1.0) == (1, 0, 1)
+    assert _bias_rule(1, m, 1.0, 1.0, 1, -1.0) == 0
+    # (b) bias / s_y is a true division, rounded once.  s_y = 0.05f, bias = 0x1.a00002p+0: the
+    # quotient lies within half an ulp (2^-19) of 32.5, so the term is the tie 32.5 -> 32; a product
+    # with the rounded reciprocal of 0.05f lands one ulp above and would give 33.
+    from fractions import Fraction as Fr
+    s_y, bias = float(np.float32(0.05)), float.fromhex("0x1.a00002p+0")
+    assert abs(Fr(bias) / Fr(s_y) - Fr(65, 2)) < Fr(1, 1 << 19)
+    assert float(np.float32(np.float32(bias) * np.float32(np.float32(1.0) / np.float32(0.05)))) > 32.5
+    assert _one(oracle, 0, 1, 1.0, 1.0, s_y, 0, bias) == (1, 32, 0)
+    # (c) the bias is in real units, not in output units and not in accumulator units
+    assert _one(oracle, 3, 1, 0.5, 0.5, 0.25, 0, 1.0) == (1, 7, 3)      # 3 * (0.25/0.25) + 1/0.25
+    # (d) ties to even after the bias, both directions, and a negative tie
+    assert _one(oracle, 2, 1, 1.0, 1.0, 1.0, 0, 0.5)[1] == 2            # 2.5 -> 2
+    assert _one(oracle, 3, 1, 1.0, 1.0, 1.0, 0, 0.5)[1] == 4            # 3.5 -> 4
+    assert _one(oracle, -2, 1, 1.0, 1.0, 1.0, 0, -0.5)[1] == -2         # -2.5 -> -2
+    # (e) saturation is applied after the bias, in both byte domains
+    assert _one(oracle, 120, 1, 1.0, 1.0, 1.0, 0, 10.0)[1] == 127
+    assert _one(oracle, -120, 1, 1.0, 1.0, 1.0, 0, -300.0)[1] == -128
+    assert _one(oracle, 100, 1, 1.0, 1.0, 1.0, 7, 200.0, out_dtype=U8)[1] == 255
+    assert _one(oracle, -100, 1, 1.0, 1.0, 1.0, 7, 0.25, out_dtype=U8)[1] == 0
+    # (f) a bias that is not finite is a bad descriptor: the whole call is declined
+    for bad in (np.nan, np.inf, -np.inf):
+        assert _one(oracle, 1, 1, 1.0, 1.0, 1.0, 0, bad)[0] == 0
+
+
+def test_rowscale_f32_bias_against_exact_rationals(oracle):
+    """Seeded small cases: every output byte equals the rule evaluated in exact rationals with
+    explicit roundings (no host floating point on the checking side)."""
+    rng = np.random.default_rng(314)
+    rows, k, n = 5, 9, 6
+    x = rng.integers(-127, 128, (rows, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    s_w = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    s_row = rng.uniform(0.01, 0.05, rows).astype(np.float32)
+    bias = rng.normal(0, 0.4, n).astype(np.float32)
+    for s_y, zp in ((np.float32(0.05), 0), (np.float32(0.0123), -3)):
+        ok, y, acc = oracle.qlinear_rowscale(x, w, s_w, np.zeros(n, np.int32), s_row, s_y, zp, bias_f32=bias)
+        assert ok == 1 and (acc == x.astype(np.int64) @ w.astype(np.int64).T).all()
+        for r in range(rows):
+            for c in range(n):
+                assert int(y[r, c]) == _bias_rule(int(acc[r, c]), float(s_row[r]), float(s_w[c]), float(s_y), zp,
+                                                  float(bias[c])), (r, c)
+        assert len(np.unique(y)) > 8  # not all saturated
