@@ -80,8 +80,29 @@ const char* vxhip_context_last_variant(const VxHipContext* context);
  * stream.  0 = clean.  Bit 1: a requantization multiplier was not finite and
  * positive.  Bit 2: an embedding id outside the table (its row is zeros).
  * Bit 4: a cache position at or past max_seq was given to the rotary/attention
- * entry points (that token's caches and output are left untouched). */
+ * entry points (that token's caches and output are left untouched).  Bit 8: a
+ * real-valued bias given to vxhip_qlinear_forward_rowscale was not finite.
+ *
+ * What the host can check it checks before anything is launched, and declines.
+ * Values that live in device memory (the row scales and the real-valued bias of
+ * vxhip_qlinear_forward_rowscale, token ids, cache positions) can only be checked
+ * by the kernels: where the reference's CPU rule would decline the whole call
+ * (src/kernels/w8a8_affine.h:169-181) the kernel raises the bit and still writes
+ * output bytes, which are then meaningless.  The return value of such a call is
+ * therefore provisional until this word has been read as 0.  The word is sticky:
+ * it keeps every bit raised since the context was created or since the last
+ * vxhip_context_clear_fault_flags. */
 VxHipStatus vxhip_context_fault_flags(VxHipContext* context, uint32_t* flags);
+/* Clears the fault word, ordered on the context's stream after the work already
+ * enqueued (asynchronous; no counterpart in the reference). */
+VxHipStatus vxhip_context_clear_fault_flags(VxHipContext* context);
+/* Grows the context's scratch (activation staging, prepared rows) to at least
+ * `bytes` now instead of inside a later call.  Entry points size the scratch by
+ * themselves; a block that is outgrown is kept until vxhip_context_destroy, so a
+ * HIP graph captured on this context stays valid when a later, larger call
+ * grows it.  Reserving up front only avoids holding the outgrown blocks.  No
+ * counterpart in the reference. */
+VxHipStatus vxhip_context_reserve_scratch(VxHipContext* context, size_t bytes);
 /* Layout of prepared activations (int8 codes) handed between entry points on
  * this context; no counterpart in the reference, whose prepared rows
  * (src/kernels/llm_ops.h:30-32) are row major.

@@ -258,6 +258,40 @@ class Oracle:
         return st, out
 
 
+def packed_linear_a8_blocked(a8, row_scales, w, scales, bias, group):
+    """PackedLinear / DYNAMIC_I8 from prepared activations, vectorised for shapes the scalar C
+    restatement would take minutes on (TEST INFRASTRUCTURE like the rest of this module).
+
+    The same rule as vxo_packed_linear_a8 (src/kernels/packed_linear_ops.inc:1498-1504, :1533):
+    per storage group g in ascending order  sum = f32(sum + f32(f32(dot_g) * f32(s_a * s_w[n][g]))),
+    then  y = f32(sum + bias[n]).  The group dots are exact: int8 products summed in float64
+    through BLAS stay below 2^53 by a wide margin (|dot_g| <= 256 * 127 * 128).  numpy's float32
+    arithmetic is one IEEE rounding per operation and never fused.
+
+    a8 int8 [rows, k], row_scales f32 [rows], w int8 [n, k] (the signed weights, not the packed
+    words), scales f32 [n, ceil(k/group)], bias f32 [n] or None.  Returns (y f32 [rows, n],
+    acc int64 [rows, n] = the full-K sums).  Rows with a NaN scale give NaN rows."""
+    rows, k = a8.shape
+    n = w.shape[0]
+    groups = (k + group - 1) // group
+    assert scales.shape == (n, groups)
+    total = np.zeros((rows, n), dtype=np.float32)
+    acc = np.zeros((rows, n), dtype=np.int64)
+    rs = row_scales.astype(np.float32)[:, None]
+    with np.errstate(invalid="ignore"):
+        for g in range(groups):
+            lo, hi = g * group, min(k, (g + 1) * group)
+            dot = a8[:, lo:hi].astype(np.float64) @ w[:, lo:hi].astype(np.float64).T
+            acc += dot.astype(np.int64)
+            gs = (rs * scales[None, :, g].astype(np.float32)).astype(np.float32)
+            term = (dot.astype(np.float32) * gs).astype(np.float32)
+            total = (total + term).astype(np.float32)
+        if bias is not None:
+            total = (total + bias.astype(np.float32)[None, :]).astype(np.float32)
+    total[np.isnan(row_scales)] = np.nan
+    return total, acc
+
+
 class _LLMOpArgs(C.Structure):
     """Field order of VxLLMOpArgs (src/kernels/llm_ops.h:38-53)."""
     _fields_ = [(n, C.c_int32) for n in (

@@ -7,12 +7,19 @@ import numpy as np
 
 
 class DecoderRef:
-    def __init__(self, cfg, weights, oracle, rope_tables):
-        self.cfg, self.w, self.orc = cfg, weights, oracle
+    def __init__(self, cfg, weights, oracle, rope_tables, blocked=False):
+        """blocked=True runs the linears through the oracle's vectorised PackedLinear (same bits as
+        the scalar one, pinned in tests/test_oracle.py): the benchmark's dimensions in seconds."""
+        self.cfg, self.w, self.orc, self.blocked = cfg, weights, oracle, blocked
         self.cos, self.sin = rope_tables(cfg)
         self.packed = {}
 
     def linear(self, key, lin, x2d):
+        if self.blocked:
+            from oracle.pyoracle import packed_linear_a8_blocked
+            a8, s, fin = self.orc.packed_prepare(np.ascontiguousarray(x2d, np.float32))
+            s = np.where(fin == 1, s, np.nan).astype(np.float32)
+            return packed_linear_a8_blocked(a8, s, lin["w"], lin["scales"], None, self.cfg.group)[0]
         if key not in self.packed:
             self.packed[key] = self.orc.pack_w8_words(lin["w"])
         _, y = self.orc.packed_linear(np.ascontiguousarray(x2d, np.float32), self.packed[key], lin["scales"], None,
@@ -47,13 +54,21 @@ class DecoderRef:
             v_cache[li] = np.concatenate([v_cache[li], v.transpose(0, 2, 1, 3)], axis=2)
             seq = k_cache[li].shape[2]
             qg = q.transpose(0, 2, 1, 3).reshape(rows, cfg.kv_heads, rep, t, cfg.head_dim)
-            scores = np.einsum("bgrtd,bgsd->bgrts", qg, k_cache[li]).astype(np.float32) * np.float32(1.0 / np.sqrt(cfg.head_dim))
+            if self.blocked:  # the same f32 products through BLAS: the benchmark's prompt in seconds
+                scores = np.matmul(qg.reshape(rows, cfg.kv_heads, rep * t, cfg.head_dim),
+                                   k_cache[li].transpose(0, 1, 3, 2)).reshape(rows, cfg.kv_heads, rep, t, seq)
+            else:
+                scores = np.einsum("bgrtd,bgsd->bgrts", qg, k_cache[li]).astype(np.float32)
+            scores = scores * np.float32(1.0 / np.sqrt(cfg.head_dim))
             visible = np.arange(seq)[None, :] <= (start + np.arange(t))[:, None]
             scores = np.where(visible[None, None, None], scores, -np.inf)
             scores = scores - scores.max(-1, keepdims=True)
             p = np.exp(scores).astype(np.float32)
             p = p / p.sum(-1, keepdims=True)
-            ctxv = np.einsum("bgrts,bgsd->bgrtd", p, v_cache[li]).astype(np.float32)
+            if self.blocked:
+                ctxv = np.matmul(p.reshape(rows, cfg.kv_heads, rep * t, seq), v_cache[li])
+            else:
+                ctxv = np.einsum("bgrts,bgsd->bgrtd", p, v_cache[li]).astype(np.float32)
             attn = ctxv.reshape(rows, cfg.q_heads, t, cfg.head_dim).transpose(0, 2, 1, 3).reshape(rows * t, cfg.q_dim)
             x = x + self.linear((li, "o"), L["o"], attn).reshape(rows, t, -1)
             h = self.rmsnorm(x, L["norm2"])

@@ -176,7 +176,8 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
     prompt = np.random.default_rng(2).integers(0, cfg.vocab, (rows, prompt_len))
     want_tokens, want_logits = DecoderRef(cfg, weights, oracle, rope_tables).generate(prompt, new)
 
-    dec = W8A8Decoder(cfg, weights, rows, fused=fused)
+    from _decoder_torch import TorchGlueDecoder
+    dec = (W8A8Decoder if fused else TorchGlueDecoder)(cfg, weights, rows)
     pd = torch.from_numpy(prompt).cuda()
     torch.cuda.synchronize()
     dec.prefill(pd)
@@ -191,6 +192,72 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
     assert np.abs(first_logits - want_logits[0]).max() <= 2e-4 * scale
     assert (got == want_tokens).all(), (got, want_tokens)
     assert "a8-" in variant
+
+
+@pytest.mark.gpu
+def test_decoder_at_benchmark_dimensions(oracle):
+    """Two layers of the benchmark decoder at its own dimensions (hidden 1024, 16 query / 8 KV heads
+    of 128, SwiGLU 3072, vocabulary 32000), 32 rows, 128-token prompts: prefill and decode steps,
+    eager and replayed from the HIP graph, token for token against the CPU restatement.  A row
+    whose two best reference logits are closer than the glue's rounding noise is compared up to
+    that step only (the f32 glue sums in another order than numpy)."""
+    import torch
+    from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights, rope_tables
+    cfg = DecoderConfig(layers=2)
+    assert (cfg.hidden, cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.inter, cfg.vocab) == (1024, 16, 8, 128, 3072, 32000)
+    weights = init_weights(cfg, 5)
+    rows, prompt_len, new = 32, 128, 4
+    prompt = np.random.default_rng(1).integers(0, cfg.vocab, (rows, prompt_len))
+    want_tokens, want_logits = DecoderRef(cfg, weights, oracle, rope_tables, blocked=True).generate(prompt, new)
+    dec = W8A8Decoder(cfg, weights, rows)
+    pd = torch.from_numpy(prompt).cuda()
+    dec.prefill(pd)
+    first_logits = dec.last_logits.cpu().numpy()
+    eager = dec.decode(new - 1).cpu().numpy()
+    dec.prefill(pd)
+    dec.capture()
+    replayed = dec.decode(new - 1).cpu().numpy()
+    variant = dec.ctx.last_variant
+    dec.close()
+    scale = np.abs(want_logits[0]).max()
+    assert np.abs(first_logits - want_logits[0]).max() <= 2e-4 * scale
+    assert (eager == replayed).all()
+    # rows stay comparable while every step so far had a clear winner in the reference
+    clear = np.ones(rows, bool)
+    compared = 0
+    for step in range(new):
+        top2 = np.sort(want_logits[step], axis=1)[:, -2:]
+        clear &= (top2[:, 1] - top2[:, 0]) > 4e-4 * scale
+        assert (eager[step][clear] == want_tokens[step][clear]).all(), step
+        compared += int(clear.sum())
+    assert compared >= new * rows * 3 // 4, "too few rows with a clear winner to call this a comparison"
+    assert "a8-" in variant
+
+
+@pytest.mark.gpu
+def test_longer_prompt_after_capture_keeps_the_graph_valid(oracle):
+    """A HIP graph of a decode step holds the addresses of the context's scratch.  A later prefill
+    with a longer prompt outgrows that scratch; the library keeps the old block alive, so replaying
+    the graph afterwards gives exactly the tokens of an eager run."""
+    import torch
+    from volvoxai_amd.decoder import W8A8Decoder, init_weights
+    from volvoxai_amd.decoder import DecoderConfig
+    cfg = DecoderConfig(layers=2, hidden=256, q_heads=4, kv_heads=2, head_dim=64, inter=512, vocab=1000, group=128,
+                        max_seq=2100)
+    weights = init_weights(cfg, 3)
+    rows = 3
+    rng = np.random.default_rng(9)
+    short, long = rng.integers(0, cfg.vocab, (rows, 2)), rng.integers(0, cfg.vocab, (rows, 2048))
+    dec = W8A8Decoder(cfg, weights, rows)
+    dec.prefill(torch.from_numpy(short).cuda())
+    dec.capture()                                   # scratch sized for 3 x 2 tokens (1 MiB) is baked into the graph
+    dec.prefill(torch.from_numpy(long).cuda())      # 3 x 2048 prepared rows of 256 bytes: the scratch grows
+    replayed = dec.decode(5).cpu().numpy()
+    dec.graph = None
+    dec.prefill(torch.from_numpy(long).cuda())
+    eager = dec.decode(5).cpu().numpy()
+    dec.close()
+    assert (replayed == eager).all()
 
 
 @pytest.mark.gpu

@@ -167,8 +167,8 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
                              c["zp_out"], c["in_dtype"], c["w_dtype"], c["out_dtype"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w8c32", "gemv.w8c8", "gemv.w16c16", "mfma-i8.t128x128s2", "mfma-i8.t256x256", "mfma-i8.t256x128",
-                      "mfma-i8.t128x64s2", "mfma-i8.t256x128w4", "mfma-i8.t128x128s4", "mfma-i8.t128x64s4",
+        for force in ("gemv.wv2", "gemv.wv8c32", "gemv.wv8c8", "gemv.wv16c16", "mfma-i8.t128x128s2", "mfma-i8.t256x256", "mfma-i8.t256x128",
+                      "mfma-i8.t128x64s2", "mfma-i8.t256x128wv4", "mfma-i8.t128x128s4", "mfma-i8.t128x64s4",
                       "mfma-i8.t64x64"):
             vx.force_variant(force)
             (ok, y), variant = run_resident_qlinear(vx, ctx, c)
@@ -190,7 +190,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16c32", "gemv.w16c8", "gemv.w8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+        for force in ("gemv.wv2", "gemv.wv16c32", "gemv.wv16c8", "gemv.wv8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
                       "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
@@ -258,7 +258,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     xd = dev(c["x"])
     seen = set()
     try:
-        for force in ("gemv.w2", "gemv.w16c32", "gemv.w16c8", "gemv.w8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
+        for force in ("gemv.wv2", "gemv.wv16c32", "gemv.wv16c8", "gemv.wv8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
                       "a8-mfma.t64x64", "a8-mfma.t128x128p"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
@@ -377,9 +377,9 @@ def test_config1_cpu_route_shape(ctx, oracle):
     assert ok3 == 1 and same_f32(deq, want_deq)
 
 
-@pytest.mark.parametrize("rows", [512, 4096])
+@pytest.mark.parametrize("rows", [512, 2048, 4096])
 def test_prefill_shape_config3_subblocks(ctx, oracle, rows):
-    """M in {512,4096}, K=N=4096, per-token x per-channel scale, requant to int8
+    """M in {512,2048,4096}, K=N=4096, per-token x per-channel scale, requant to int8
     at output scale 0.05.  An output sub-block depends only on its own rows of A
     and B, so the oracle checks random sub-blocks at full problem size; the
     int32 accumulators of the whole output are checked against an f64 GEMM."""
@@ -466,6 +466,104 @@ def test_outlier_large_k_config5_reduced_rows(ctx, oracle):
                                    np.ascontiguousarray(bias[cs]), len(cs), g)
     assert same_f32(host(y)[:, cs], want)
     pl.close()
+
+
+def test_outlier_large_k_config5_full_size(ctx, oracle):
+    """The whole shape, M=2048, K=14336, N=4096, f32 rows with 1% outlier channels: the prepared
+    codes and scales against the oracle on sampled rows, the full-K int32 sums of the whole output
+    against an f64 GEMM, and the f32 outputs against the oracle on random sub-blocks (an output
+    depends only on its own row of activations and its own weight row)."""
+    import torch
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    rows, k, n, g = 2048, 14336, 4096, 128
+    rng = np.random.default_rng(55)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[:, rng.choice(k, k // 100, replace=False)] *= 20.0
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    chan = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    scales = np.repeat(chan[:, None], k // g, axis=1).copy()
+    bias = rng.normal(0, 0.1, n).astype(np.float32)
+    words = oracle.pack_w8_words(w)
+    pl = vx.PackedLinear(words, scales, bias, k, n, g)
+    xd = dev(x)
+    st, y = pl.forward_f32(ctx, xd)
+    ctx.synchronize()
+    variant = ctx.last_variant
+    assert st == 0 and "a8-mfma" in variant
+    a8, sc = packed_prepare_i8(ctx, xd)
+    st, y2, acc = pl.forward_a8(ctx, a8, sc, want_accumulators=True)
+    ctx.synchronize()
+    assert st == 0 and torch.equal(y.view(torch.int32), y2.view(torch.int32))
+    exact = a8.double() @ dev(w).double().T  # |sum| <= 14336 * 127 * 127 < 2^53: exact in f64
+    assert torch.equal(acc.double(), exact)
+    del exact
+    y, a8, sc = host(y), host(a8), host(sc)
+    rs = np.sort(rng.choice(rows, 48, replace=False))
+    want_a, want_s, fin = oracle.packed_prepare(x[rs])
+    assert fin.all() and (a8[rs] == want_a).all() and (sc[rs].view(np.uint32) == want_s.view(np.uint32)).all()
+    for _ in range(3):
+        rs = np.sort(rng.choice(rows, 24, replace=False))
+        cs = np.sort(rng.choice(n, 40, replace=False))
+        _, want = oracle.packed_linear(np.ascontiguousarray(x[rs]), np.ascontiguousarray(words[cs]),
+                                       np.ascontiguousarray(scales[cs]), np.ascontiguousarray(bias[cs]), len(cs), g)
+        assert same_f32(y[np.ix_(rs, cs)], want), variant
+    pl.close()
+
+
+# ---- values only the device can check -------------------------------------------------------
+
+def test_device_side_faults_are_raised_and_cleared(oracle):
+    """Row scales and the real-valued bias of the per-token form live in device memory, so the host
+    admission cannot see them.  Where the CPU rule declines the call, the kernels raise a sticky
+    fault bit (1: a multiplier is not finite and positive; 8: a bias is not finite), in both kernel
+    families; clearing the word is ordered on the stream."""
+    import torch
+    import volvoxai_amd as vx
+    own = vx.Context(0, torch.cuda.current_stream())  # fault bits are sticky: not the shared context
+    for rows, bad_row in ((8, 3), (160, 77)):         # the streaming GEMV and the MFMA GEMM
+        c = cases.rowscale_case(rows, 256, 64, 5)
+        lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, I8)
+        xd, bd = dev(c["x"]), dev(c["bias_f32"])
+        ok, _ = lin.forward_rowscale(own, xd, dev(c["row_scales"]), c["s_out"], 0, bias_f32=bd)
+        assert ok == 1 and own.fault_flags() == 0
+        for value in (0.0, -1.0, np.nan, np.inf):
+            rs = c["row_scales"].copy()
+            rs[bad_row] = value
+            assert oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], rs, c["s_out"], 0)[0] == 0
+            ok, _ = lin.forward_rowscale(own, xd, dev(rs), c["s_out"], 0, bias_f32=bd)
+            assert ok == 1 and own.fault_flags() == 1, (rows, value, own.last_variant)  # provisional 1, then the bit
+            own.clear_fault_flags()
+            assert own.fault_flags() == 0
+        for value in (np.nan, -np.inf):
+            b = c["bias_f32"].copy()
+            b[9] = value
+            assert oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], c["row_scales"], c["s_out"], 0,
+                                           bias_f32=b)[0] == 0
+            ok, _ = lin.forward_rowscale(own, xd, dev(c["row_scales"]), c["s_out"], 0, bias_f32=dev(b))
+            assert ok == 1 and own.fault_flags() == 8, (rows, value, own.last_variant)
+            own.clear_fault_flags()
+        # the word is clean again and a good call stays clean
+        ok, y = lin.forward_rowscale(own, xd, dev(c["row_scales"]), c["s_out"], 0, bias_f32=bd)
+        _, want, _ = oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], c["row_scales"], c["s_out"], 0,
+                                             bias_f32=c["bias_f32"])
+        assert ok == 1 and own.fault_flags() == 0 and (host(y) == want).all()
+        lin.close()
+    own.close()
+
+
+def test_two_contexts_keep_their_own_variant_ids(ctx):
+    """The id of the kernel that ran is held per context, not per thread."""
+    import torch
+    import volvoxai_amd as vx
+    other = vx.Context(0, torch.cuda.current_stream())
+    small = cases.qlinear_random_case(4, 256, 64, 2)
+    big = cases.qlinear_random_case(64, 256, 128, 2)
+    (ok1, _), v1 = run_resident_qlinear(vx, ctx, big)
+    (ok2, _), v2 = run_resident_qlinear(vx, other, small)
+    assert ok1 == ok2 == 1 and "gemv" in v2 and "mfma-i8" in v1
+    assert ctx.last_variant == v1 and other.last_variant == v2  # the second launch did not overwrite the first
+    other.close()
 
 
 # ---- boundaries and edge cases ------------------------------------------------------------

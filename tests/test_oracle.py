@@ -459,3 +459,30 @@ def test_rowscale_f32_bias_against_exact_rationals(oracle):
                 assert int(y[r, c]) == _bias_rule(int(acc[r, c]), float(s_row[r]), float(s_w[c]), float(s_y), zp,
                                                   float(bias[c])), (r, c)
         assert len(np.unique(y)) > 8  # not all saturated
+
+
+def test_blocked_packed_linear_equals_the_scalar_restatement(oracle):
+    """The vectorised form used for full-size shapes gives the scalar restatement's bits (which the
+    reference digests pin), ragged K and partial groups included, and a NaN scale marks its row."""
+    from oracle.pyoracle import packed_linear_a8_blocked
+    for entry in VECTORS["packed"][:6]:
+        c = cases.packed_case(**entry["params"])
+        a8, s, fin = oracle.packed_prepare(c["x"])
+        s = np.where(fin == 1, s, np.nan).astype(np.float32)
+        got, acc = packed_linear_a8_blocked(a8, s, c["w"], c["scales"], c["bias"], c["group"])
+        _, want = oracle.packed_linear(c["x"], oracle.pack_w8_words(c["w"]), c["scales"], c["bias"], c["n"], c["group"])
+        nan = np.isnan(want)
+        assert (np.isnan(got) == nan).all() and (got.view(np.uint32)[~nan] == want.view(np.uint32)[~nan]).all()
+        if not nan.any():
+            check_digest(got, entry["expected"])
+            assert (acc == a8.astype(np.int64) @ c["w"].astype(np.int64).T).all()
+    rng = np.random.default_rng(6)
+    for rows, k, n, g in [(3, 300, 17, 64), (2, 4096, 9, 128), (5, 95, 4, 32)]:
+        a8 = rng.integers(-127, 128, (rows, k)).astype(np.int8)
+        w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+        rs = rng.uniform(0.01, 0.05, rows).astype(np.float32)
+        sc = rng.uniform(0.002, 0.01, (n, (k + g - 1) // g)).astype(np.float32)
+        b = rng.normal(0, 0.1, n).astype(np.float32)
+        got, _ = packed_linear_a8_blocked(a8, rs, w, sc, b, g)
+        _, want, _ = oracle.packed_linear_a8(a8, rs, oracle.pack_w8_words(w), sc, b, n, g)
+        assert (got.view(np.uint32) == want.view(np.uint32)).all()

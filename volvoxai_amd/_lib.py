@@ -62,6 +62,8 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_context_synchronize": (i32, [vp]),
         "vxhip_context_last_variant": (C.c_char_p, [vp]),
         "vxhip_context_fault_flags": (i32, [vp, C.POINTER(u32)]),
+        "vxhip_context_clear_fault_flags": (i32, [vp]),
+        "vxhip_context_reserve_scratch": (i32, [vp, sz]),
         "vxhip_rmsnorm_prepare_i8": (i32, [vp, vp, vp, u32, u32, C.c_double, vp, vp, vp]),
         "vxhip_add_rmsnorm_prepare_i8": (i32, [vp, vp, vp, vp, u32, u32, C.c_double, vp, vp]),
         "vxhip_swiglu_prepare_i8": (i32, [vp, vp, u32, u32, vp, vp, vp]),

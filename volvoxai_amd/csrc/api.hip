@@ -53,15 +53,25 @@ static bool multiplier_ok(float s_in, float s_w, float s_out) {
 
 VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes) {
     if (bytes <= ctx->scratch_bytes) return VXHIP_OK;
-    // earlier launches may still read the old block
-    VXHIP_TRY(hipStreamSynchronize(ctx->stream));
-    if (ctx->scratch) VXHIP_TRY(hipFree(ctx->scratch));
-    ctx->scratch = nullptr;
-    ctx->scratch_bytes = 0;
-    const size_t want = (bytes + (1u << 20)) & ~((size_t)(1u << 20) - 1u);
-    VXHIP_TRY(hipMalloc(&ctx->scratch, want));
+    // The outgrown block is retired, not freed: launches in flight may still read it, and a HIP
+    // graph captured on this context keeps its address and may be replayed after this call.
+    // Growing at least doubles the block, so the retired ones add up to less than the live one.
+    if (ctx->scratch && ctx->retired_count == VxHipContext::kRetiredSlots) {
+        set_error("context scratch grew more often than %d times", VxHipContext::kRetiredSlots);
+        return VXHIP_INTERNAL;
+    }
+    size_t want = (bytes + (1u << 20)) & ~((size_t)(1u << 20) - 1u);
+    if (want < 2 * ctx->scratch_bytes) want = 2 * ctx->scratch_bytes;
+    void* fresh = nullptr;
+    VXHIP_TRY(hipMalloc(&fresh, want));
+    if (ctx->scratch) ctx->retired[ctx->retired_count++] = ctx->scratch;
+    ctx->scratch = fresh;
     ctx->scratch_bytes = want;
     return VXHIP_OK;
+}
+
+void set_last_variant(VxHipContext* ctx, const char* id) {
+    snprintf(ctx->last_variant, sizeof ctx->last_variant, "%s", id ? id : "");
 }
 
 struct Carver {
@@ -199,6 +209,7 @@ void vxhip_context_destroy(VxHipContext* ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
+    for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
     if (ctx->fault_dev) (void)hipFree(ctx->fault_dev);
     if (ctx->div_proof_dev) (void)hipFree(ctx->div_proof_dev);
     if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -218,6 +229,19 @@ VxHipStatus vxhip_context_fault_flags(VxHipContext* ctx, uint32_t* flags) {
     VXHIP_TRY(hipMemcpyAsync(flags, ctx->fault_dev, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     VXHIP_TRY(hipStreamSynchronize(ctx->stream));
     return VXHIP_OK;
+}
+
+VxHipStatus vxhip_context_clear_fault_flags(VxHipContext* ctx) {
+    if (!ctx) return VXHIP_INVALID_ARGUMENT;
+    if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
+    // a fill kernel on the context's stream: ordered after the launches that may still raise bits
+    return launch_fill_u32(ctx->stream, ctx->fault_dev, 1u, 0u);
+}
+
+VxHipStatus vxhip_context_reserve_scratch(VxHipContext* ctx, size_t bytes) {
+    if (!ctx) return VXHIP_INVALID_ARGUMENT;
+    if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
+    return ensure_scratch(ctx, bytes);
 }
 
 VxHipStatus vxhip_context_set_activation_layout(VxHipContext* ctx, uint32_t layout) {
@@ -502,7 +526,7 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
         set_error("qlinear_forward: no kernel variant accepts rows=%u k=%u n=%u", rows, k, n);
         return 0;
     }
-    ctx->last_variant = id;
+    set_last_variant(ctx, id);
     return 1;
 }
 
@@ -648,7 +672,7 @@ VxHipStatus vxhip_packed_prepare_i8(VxHipContext* ctx, const float* input_dev, u
     if (!ctx || !input_dev || !prepared_dev || !row_scales_dev || !k) return VXHIP_INVALID_ARGUMENT;
     if (!rows) return VXHIP_OK;
     if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
-    ctx->last_variant = "hip.packed-linear.prepare-i8";
+    set_last_variant(ctx, "hip.packed-linear.prepare-i8");
     const bool operand_order = ctx->activation_layout == VXHIP_ACTIVATIONS_OPERAND32 && rows <= kOperandOrderRows;
     return launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared_dev,
                              operand_order ? ActivationLayout{(k + 15u) / 16u * 16u, 1u} : ActivationLayout{k, 0u},
@@ -708,7 +732,7 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
         if (!id2) return operand_order && !y ? -2 : -1;
         if (!id) id = id2;
     }
-    ctx->last_variant = id;
+    set_last_variant(ctx, id);
     return 0;
 }
 
@@ -833,7 +857,7 @@ int vxhip_quantize_forward(VxHipContext* ctx, const float* input_dev, uint32_t e
         !zero_point_ok(zp, dtype))
         return 0;
     if (!use_device(ctx->device)) return 0;
-    ctx->last_variant = "hip.quantize-linear.elementwise";
+    set_last_variant(ctx, "hip.quantize-linear.elementwise");
     return launch_quantize(ctx->stream, input_dev, elements, output_dev, scale, zp,
                            dtype == VXHIP_DTYPE_I8) == VXHIP_OK;
 }
@@ -842,7 +866,7 @@ int vxhip_dequantize_forward(VxHipContext* ctx, const void* input_dev, uint32_t 
                              int32_t zp, uint32_t dtype, float* output_dev) {
     if (!ctx || !input_dev || !output_dev || !byte_dtype(dtype)) return 0;
     if (!use_device(ctx->device)) return 0;
-    ctx->last_variant = "hip.dequantize-linear.elementwise";
+    set_last_variant(ctx, "hip.dequantize-linear.elementwise");
     return launch_dequantize(ctx->stream, input_dev, elements, scale, zp, dtype == VXHIP_DTYPE_I8,
                              output_dev) == VXHIP_OK;
 }

@@ -55,6 +55,7 @@ enum FaultBits : uint32_t {
     kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive
     kFaultBadToken = 2u,        // an embedding lookup was asked for a row outside the table
     kFaultBadPosition = 4u,     // a cache slot at or past max_seq was named: nothing read or written there
+    kFaultBadBias = 8u,         // a real-valued bias of the per-token requantizing form was not finite
 };
 
 }  // namespace vxhip
@@ -63,9 +64,14 @@ struct VxHipContext {
     int device = 0;
     hipStream_t stream = nullptr;
     bool own_stream = false;
-    // grow-only scratch (activation staging, per-channel parameters, prepared rows)
+    // grow-only scratch (activation staging, per-channel parameters, prepared rows).  A block that
+    // has been outgrown is kept until the context is destroyed: a HIP graph captured on this
+    // context has the block's address baked into its kernel nodes and may be replayed later.
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    static constexpr int kRetiredSlots = 48;  // sizes at least double, so this is never reached
+    void* retired[kRetiredSlots] = {};
+    int retired_count = 0;
     uint32_t* fault_dev = nullptr;
     // Exhaustive exactness proofs of the short division sequences, one pair of mismatch
     // counters per divisor seen (the output scales of the calls made on this context).
@@ -73,7 +79,7 @@ struct VxHipContext {
     uint32_t* div_proof_dev = nullptr;          // [kDivisorSlots][2]
     uint32_t div_bits[kDivisorSlots] = {};      // bit pattern of the divisor proved in each slot
     int div_used = 0, div_next = 0;
-    const char* last_variant = "";
+    char last_variant[96] = "";  // a copy: the launchers' name buffers are per thread, not per context
     int cu_count = 0;
     uint32_t activation_layout = 0;  // VXHIP_ACTIVATIONS_*: what the prepare entry points write for rows <= 32
 };
@@ -105,6 +111,7 @@ struct VxHipPackedLinear {
 namespace vxhip {
 
 VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes);
+void set_last_variant(VxHipContext* ctx, const char* id);
 
 // pack.hip ------------------------------------------------------------------
 // raw_dev: [n] rows of `row_stride` bytes holding k weight bytes each.

@@ -44,7 +44,12 @@ __device__ __forceinline__ ChannelConsts channel_consts(const LinearArgs& a, uin
     } else {
         c.f0 = sw;
         c.cb = a.bias_i32[n];
-        if (a.bias_row && n < a.n) c.bo = __fdiv_rn(a.bias_row[n], a.output_scale);
+        if (a.bias_row && n < a.n) {
+            const float b = a.bias_row[n];
+            // a bias that is not finite is a bad descriptor (the CPU rule declines the call)
+            if (!(fabsf(b) <= 3.402823466e38f)) atomicOr(a.fault, (uint32_t)kFaultBadBias);
+            c.bo = __fdiv_rn(b, a.output_scale);
+        }
     }
     return c;
 }

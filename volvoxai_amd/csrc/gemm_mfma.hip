@@ -32,26 +32,6 @@
 #include <type_traits>
 #include <utility>
 
-// Compile-time probes used only when tuning (all off in the shipped build):
-// leave out one ingredient of the main loop to see what bounds it.
-#ifndef VXHIP_PROBE_NO_LOADS
-#define VXHIP_PROBE_NO_LOADS 0
-#endif
-#ifndef VXHIP_PROBE_NO_MFMA
-#define VXHIP_PROBE_NO_MFMA 0
-#endif
-#ifndef VXHIP_PROBE_SAME_KB
-#define VXHIP_PROBE_SAME_KB 0
-#endif
-#ifndef VXHIP_PROBE_CLOCK
-#define VXHIP_PROBE_CLOCK 0
-#endif
-#ifndef VXHIP_PROBE_NO_VMWAIT
-#define VXHIP_PROBE_NO_VMWAIT 0
-#endif
-#ifndef VXHIP_PROBE_NO_EPILOGUE
-#define VXHIP_PROBE_NO_EPILOGUE 0
-#endif
 namespace vxhip {
 
 namespace {
@@ -146,8 +126,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // its own L2).  Give XCD x the x-th contiguous run of tiles, and order
     // tiles so a run is a compact block of the output: that block's operand
     // slices are then shared through one L2 instead of being fetched by all.
-    uint64_t probe_cycles = 0, probe_real = 0, probe_start = 0;
-    if (VXHIP_PROBE_CLOCK) probe_start = __builtin_amdgcn_s_memrealtime();
     const uint32_t total = p.tiles_n * p.tiles_m;
     const uint32_t per_xcd = (total + 7u) / 8u;
     const uint32_t lin = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
@@ -186,7 +164,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     constexpr int NLOADS = WLOADS + XLOADS;
     auto issue_one = [&](auto t_tag, uint32_t kb, int stage) {
         constexpr int t = decltype(t_tag)::value;
-        if (VXHIP_PROBE_NO_LOADS && kb > 0) return;
         if constexpr (PIPE && t == 0) {
             // stage of k-block kb: the scales of group kb-1, which that k-block folds (kb = 0
             // folds zeros; any finite scales do).  64 channels per wavefront, 4 bytes per lane.
@@ -197,7 +174,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             }
         }
         kb = min(kb, nkb - 1u);
-        if (VXHIP_PROBE_SAME_KB) kb = kb & 1u;  // same two k-blocks over and over: cache hits only
         char* base = lds_raw + stage * STAGE_BYTES;
         if constexpr (t < WLOADS) {
             const uint32_t b = wave + t * NWAVES;
@@ -406,18 +382,14 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
                     wf[1][i][d] = wraw[i][d] & (int)0xf0f0f0f0u;
                 }
             }
-            if constexpr (VXHIP_PROBE_NO_MFMA) {
-                acc[i][j][0] += wf[CB][i][0] ^ xf[CB][j][1];
-            } else {
-                // first k-step of a scale group: accumulate onto zero instead of clearing registers
-                constexpr bool FRESH = F32OUT && GK <= KS && (S % GK) == 0;
-                const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                if constexpr (PIPE && P == 1)
-                    acc_odd[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j],
-                                                                          FRESH ? zero : acc_odd[i][j], 0, 0, 0);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], FRESH ? zero : acc[i][j], 0, 0, 0);
-            }
+            // first k-step of a scale group: accumulate onto zero instead of clearing registers
+            constexpr bool FRESH = F32OUT && GK <= KS && (S % GK) == 0;
+            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            if constexpr (PIPE && P == 1)
+                acc_odd[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j],
+                                                                      FRESH ? zero : acc_odd[i][j], 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[CB][i], xf[CB][j], FRESH ? zero : acc[i][j], 0, 0, 0);
             // PIPE: one slot (four outputs) of the other set's fold rides behind every MFMA
             if constexpr (PIPE) fold_slot(IC<P ^ 1>{}, IC<S * MF + m>{}, cstage, rstage, read_tag);
             // after MFMA m: the reads and loads whose slot it is.  Reads keep clear of the
@@ -446,10 +418,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     // k-block 0 has landed; the NS-2 younger ones may still be on their way
     wait_vmcnt<(NS - 2) * NLOADS>();
     wg_barrier();
-    if (VXHIP_PROBE_CLOCK) {
-        probe_cycles = __builtin_readcyclecounter();
-        probe_real = __builtin_amdgcn_s_memrealtime();
-    }
     // (unconditional: a block past the end is clamped to the last one, and the waits below
     // count on every block having been requested)
     static_for<NLOADS>([&](auto t) { issue_one(t, NS - 1, NS - 1); });
@@ -466,7 +434,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         if constexpr (!LAST) {
             wait_lgkm0();     // my reads of this stage have landed in registers
             // my loads of the next k-block have landed (the NS-2 blocks after it need not have)
-            if (!VXHIP_PROBE_NO_VMWAIT) wait_vmcnt<(NS - 2) * NLOADS>();
+            wait_vmcnt<(NS - 2) * NLOADS>();
             wg_barrier();
             step(IC<KS - 1>{}, std::true_type{}, IC<0>{}, lds_raw + ((cur + 1) & (NS - 1)) * STAGE_BYTES,
                  IC<NLOADS>{}, kb + NS, cur, kb, parity_tag, stage);
@@ -505,26 +473,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
         k_block(nkb - 1u, std::true_type{}, IC<0>{});
     }
     wait_vmcnt<0>();  // nothing of this workgroup may still be writing LDS when the epilogue reuses it
-    uint64_t probe_loop_end = 0;
-    if (VXHIP_PROBE_CLOCK) {
-        probe_loop_end = __builtin_amdgcn_s_memrealtime();
-        if (blockIdx.x == 8 && threadIdx.x == 0) {
-            // shader cycles and 100 MHz ticks this workgroup's main loop took
-            ((uint64_t*)a.fault)[2] = __builtin_readcyclecounter() - probe_cycles;
-            ((uint64_t*)a.fault)[3] = probe_loop_end - probe_real;
-        }
-    }
-    if (VXHIP_PROBE_NO_EPILOGUE) {
-        int fold = 0;
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int j = 0; j < TM; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) fold ^= acc[i][j][r];
-        if (fold == 0x7fffffff) ((int*)a.y)[0] = 1;
-        return;
-    }
 
     // ---- epilogue ----------------------------------------------------------------
     if constexpr (FAST && !F32OUT) {
@@ -664,15 +612,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
             }
         }
     }
-    if (VXHIP_PROBE_CLOCK && threadIdx.x == 0) {
-        // per workgroup: start, loop begin, loop end, end (100 MHz ticks); the probe build borrows bias_f32
-        __builtin_amdgcn_s_waitcnt(0);
-        uint64_t* o = (uint64_t*)a.bias_f32 + 4 * (size_t)blockIdx.x;
-        o[0] = probe_start;
-        o[1] = probe_real;
-        o[2] = probe_loop_end;
-        o[3] = __builtin_amdgcn_s_memrealtime();
-    }
 }
 
 template <int WN, int WM, int TN, int TM, int MODE, int GK, bool FAST, bool W4, int NS>
@@ -747,9 +686,9 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (forced("t128x128")) pick = 2;
         if (forced("t128x64")) pick = 3;
         if (forced("t64x64")) pick = 4;
-        if (pick == 0 && forced("w4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256w4" : nullptr;
+        if (pick == 0 && forced("wv4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256wv4" : nullptr;
         if (pick == 0) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
-        if (pick == 1 && forced("w4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128w4" : nullptr;
+        if (pick == 1 && forced("wv4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128wv4" : nullptr;
         if (pick == 1) return launch_cfg<2, 4, 4, 1, MODE, GK>(s, a) ? "t256x128" : nullptr;
         // one round of tiles or less: the k loop waits on each k-block's loads in turn; four
         // stages keep three k-blocks in flight (the small tiles leave the LDS for them)

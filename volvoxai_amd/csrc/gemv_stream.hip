@@ -30,13 +30,6 @@
 
 #include <type_traits>
 
-// tuning probe: per-workgroup phase timestamps (100 MHz ticks) through the unused bias_row pointer
-#ifndef VXHIP_GEMV_PROBE
-#define VXHIP_GEMV_PROBE 0
-#endif
-#ifndef VXHIP_GEMV_DEPTH
-#define VXHIP_GEMV_DEPTH 4
-#endif
 
 namespace vxhip {
 
@@ -44,7 +37,7 @@ namespace {
 
 extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
-constexpr int kDepth = VXHIP_GEMV_DEPTH;  // 1 KiB blocks in flight per wave
+constexpr int kDepth = 4;  // 1 KiB blocks in flight per wave
 
 __device__ __forceinline__ v4i load_stream(const int8_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
@@ -70,8 +63,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     static_assert(F || !W4, "four-bit weights exist for the dequantizing epilogue only");
     constexpr int SPB = W4 ? 2 : 1;              // k-steps per 1 KiB block
     constexpr int UNIT = GK > SPB ? GK : SPB;    // a wave's run is a whole number of these
-    uint64_t probe[4] = {0, 0, 0, 0};
-    if (VXHIP_GEMV_PROBE) probe[0] = __builtin_amdgcn_s_memrealtime();
     const int lane = threadIdx.x & 63;
     // wave-uniform, and known to the compiler as such: the bounds of the wave's run and every
     // branch on them are then scalar.  (That is needed, not only cheaper: an MFMA is not
@@ -233,9 +224,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     for (; t < t1; t += ROUND) round(t, std::false_type{});
     if constexpr (!F) park(wave);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (VXHIP_GEMV_PROBE) probe[1] = __builtin_amdgcn_s_memrealtime();
     __syncthreads();
-    if (VXHIP_GEMV_PROBE) probe[2] = __builtin_amdgcn_s_memrealtime();
 
     // Tail: one thread per output, index o = row * CH + channel.  F: sum += f32(dot_g) *
     // (s_a * s_w[n][g]) in ascending group order with separate roundings
@@ -280,14 +269,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
             store_element<MODE>(a, om, on, dot, 0.0f, rs);
         }
     }
-    if (VXHIP_GEMV_PROBE && threadIdx.x == 0) {
-        __builtin_amdgcn_s_waitcnt(0);
-        uint64_t* o = (uint64_t*)a.bias_row + 4 * (size_t)blockIdx.x;
-        o[0] = probe[0];
-        o[1] = probe[1];
-        o[2] = probe[2];
-        o[3] = __builtin_amdgcn_s_memrealtime();
-    }
 }
 
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1>
@@ -323,10 +304,10 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
     const uint32_t panels = (a.n + 31u) / 32u, chunks = ((a.k + 31u) / 32u + UNIT - 1) / UNIT;
     for (int more = waves * 2; more <= 16 && (uint32_t)more <= chunks && panels * (uint32_t)more <= 4096u; more *= 2)
         waves = more;
-    if (force && strstr(force, "w16")) waves = 16;
-    else if (force && strstr(force, "w8")) waves = 8;
-    else if (force && strstr(force, "w4")) waves = 4;
-    else if (force && strstr(force, "w2")) waves = 2;
+    if (force && strstr(force, "wv16")) waves = 16;
+    else if (force && strstr(force, "wv8")) waves = 8;
+    else if (force && strstr(force, "wv4")) waves = 4;
+    else if (force && strstr(force, "wv2")) waves = 2;
     // Fewer panels than half the compute units: two or four workgroups share each panel's
     // channels (only the 8- and 16-wave kernels are built that way; such shapes have them
     // unless K is tiny).
@@ -348,9 +329,9 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
     else if (waves == 4) ok = launch_panel<MODE, GK, 4, W4>(s, a, lds);
     else ok = launch_panel<MODE, GK, 2, W4>(s, a, lds);
     if (!ok) return nullptr;
-    static const char* const names[3][4] = {{"w2", "w4", "w8", "w16"},
-                                            {"w2", "w4", "w8c16", "w16c16"},
-                                            {"w2", "w4", "w8c8", "w16c8"}};
+    static const char* const names[3][4] = {{"wv2", "wv4", "wv8", "wv16"},
+                                            {"wv2", "wv4", "wv8c16", "wv16c16"},
+                                            {"wv2", "wv4", "wv8c8", "wv16c8"}};
     return names[split == 4 ? 2 : split == 2 ? 1 : 0][waves == 16 ? 3 : waves == 8 ? 2 : waves == 4 ? 1 : 0];
 }
 

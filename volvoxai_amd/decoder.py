@@ -1,8 +1,13 @@
 """Decoder-only transformer with every linear routed to the W8A8 PackedLinear
-kernels (28 layers, hidden 1024, 16 query / 8 KV heads of 128, SwiGLU 3072 by default): RMSNorm, rotary embedding, grouped-query attention
-over a KV cache, SwiGLU, residual adds and greedy selection run as PyTorch-ROCm
-f32 ops around them; the linears are `vxhip_packed_linear_forward_f32`
-(DYNAMIC_I8: per-row activation quantization, int8 x int8 MFMA, dequant to f32).
+kernels (28 layers, hidden 1024, 16 query / 8 KV heads of 128, SwiGLU 3072 by
+default).  Everything between the linears -- embedding gather, residual add +
+RMSNorm + activation preparation, rotary embedding + KV-cache append,
+grouped-query attention, SwiGLU + preparation, greedy selection -- runs as HIP
+kernels of the same library (vxhip_*_prepare_i8, vxhip_rope_*, vxhip_gqa_*,
+vxhip_embedding_gather_f32, vxhip_argmax_rows_f32); the linears are
+`vxhip_packed_linear_forward_a8` / `_f32` (DYNAMIC_I8: per-row activation
+quantization, int8 x int8 MFMA, dequant to f32).  PyTorch supplies device
+memory, the stream and the HIP graph, no arithmetic.
 
 The glue follows the reference's definitions: RMSNorm accumulates and scales in
 double (native/src/kernels/softmax_rmsnorm.inc:3-17); the rotary embedding is the
@@ -105,16 +110,14 @@ def rope_tables(cfg: DecoderConfig):
 
 
 class W8A8Decoder:
-    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None, fused=True):
-        """fused=True runs the glue through the library's fused kernels (RMSNorm+prepare,
-        rotary+cache append, attention, SwiGLU+prepare); fused=False through PyTorch ops."""
+    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None):
         import torch
-        self.torch, self.cfg, self.rows, self.fused = torch, cfg, rows, fused
+        self.torch, self.cfg, self.rows = torch, cfg, rows
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
         # prepared activations of up to 32 rows travel between the glue kernels and the GEMVs in
-        # the GEMV's operand order (the fused path only: the other prepares inside each linear)
-        self.ctx.set_activation_layout(fused)
+        # the GEMV's operand order
+        self.ctx.set_activation_layout(True)
         dev = "cuda"
 
         def make(lin):
@@ -124,13 +127,10 @@ class W8A8Decoder:
         self.embedding = torch.from_numpy(weights["embedding"]).to(dev)
         self.layers = []
         for lw in weights["layers"]:
-            self.layers.append({"norm1": torch.from_numpy(lw["norm1"]).to(dev).double(),
-                                "norm2": torch.from_numpy(lw["norm2"]).to(dev).double(),
-                                "gain1": torch.from_numpy(lw["norm1"]).to(dev),
+            self.layers.append({"gain1": torch.from_numpy(lw["norm1"]).to(dev),
                                 "gain2": torch.from_numpy(lw["norm2"]).to(dev),
                                 "qkv": make(lw["qkv"]), "o": make(lw["o"]),
                                 "gate_up": make(lw["gate_up"]), "down": make(lw["down"])})
-        self.norm_f = torch.from_numpy(weights["norm_f"]).to(dev).double()
         self.gain_f = torch.from_numpy(weights["norm_f"]).to(dev)
         self.lm_head = make(weights["lm_head"])
         cos, sin = rope_tables(cfg)
@@ -139,8 +139,8 @@ class W8A8Decoder:
         self.k_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
         self.v_cache = torch.zeros(shape, dtype=torch.float32, device=dev)
         # state of the decode loop, on the device so a captured step advances by itself
-        # (int32 ids on the fused path, as the reference's embedding takes them)
-        self.tokens = torch.zeros(rows, dtype=torch.int32 if fused else torch.int64, device=dev)
+        # (int32 ids, as the reference's embedding takes them)
+        self.tokens = torch.zeros(rows, dtype=torch.int32, device=dev)
         self.position = torch.zeros(1, dtype=torch.int64, device=dev)
         self.history = torch.zeros((cfg.max_seq, rows), dtype=torch.int64, device=dev)
         self.slots = torch.arange(cfg.max_seq, device=dev)
@@ -164,8 +164,8 @@ class W8A8Decoder:
             raise RuntimeError(_library().vxhip_last_error().decode())
         return out
 
-    def _layer_fused(self, li, x2, delta, positions, rows, t):
-        """The same layer through the fused glue kernels.  x2 [rows*t, hidden] is the residual
+    def _layer(self, li, x2, delta, positions, rows, t):
+        """One layer.  x2 [rows*t, hidden] is the residual
         stream, updated in place; delta is the previous layer's MLP output still to be added to it
         (the add rides in the next RMSNorm kernel).  Returns this layer's pending delta."""
         cfg, L = self.cfg, self.layers[li]
@@ -194,7 +194,7 @@ class W8A8Decoder:
         a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
         return self._linear_a8(L["down"], a8, sc)
 
-    def _forward_fused(self, tokens, positions, next_tokens=None, advance=None):
+    def _forward(self, tokens, positions, next_tokens=None, advance=None):
         """tokens int32 [rows, t] -> logits of the last position and their argmax (int32, written
         to `next_tokens` when given; `advance` counters are incremented by the same launch)."""
         cfg = self.cfg
@@ -202,7 +202,7 @@ class W8A8Decoder:
         x2 = vx.embedding_gather(self.ctx, tokens.reshape(-1), self.embedding)
         delta = None
         for li in range(cfg.layers):
-            delta = self._layer_fused(li, x2, delta, positions, rows, t)
+            delta = self._layer(li, x2, delta, positions, rows, t)
         if t > 1:
             x2 = x2.reshape(rows, t, cfg.hidden)[:, -1, :].contiguous()
             delta = delta.reshape(rows, t, cfg.hidden)[:, -1, :].contiguous()
@@ -210,90 +210,40 @@ class W8A8Decoder:
         logits = self._linear_a8(self.lm_head, a8, sc)
         return logits, vx.argmax_rows(self.ctx, logits, out=next_tokens, advance=advance)
 
-    def _rmsnorm(self, x, gain):
-        xd = x.double()
-        inv = 1.0 / self.torch.sqrt((xd * xd).mean(-1, keepdim=True) + self.cfg.eps)
-        return (xd * inv * gain).float()
-
-    def _rope(self, x, cos, sin):
-        # x [rows, t, heads, d]; cos/sin [t, d]
-        half = self.cfg.head_dim // 2
-        partner = self.torch.cat([-x[..., half:], x[..., :half]], dim=-1)
-        return x * cos[None, :, None, :] + partner * sin[None, :, None, :]
-
-    def _layer(self, li, x, cos, sin, write_slots, visible):
-        """x [rows, t, hidden]; write_slots [t] cache positions of these tokens; visible
-        [t, max_seq] bool: which cache slots each of them may attend to."""
-        torch, cfg, L = self.torch, self.cfg, self.layers[li]
-        rows, t, _ = x.shape
-        h = self._rmsnorm(x, L["norm1"])
-        qkv = self._linear(L["qkv"], h.reshape(rows * t, cfg.hidden)).reshape(rows, t, -1)
-        q = qkv[..., :cfg.q_dim].reshape(rows, t, cfg.q_heads, cfg.head_dim)
-        k = qkv[..., cfg.q_dim:cfg.q_dim + cfg.kv_dim].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
-        v = qkv[..., cfg.q_dim + cfg.kv_dim:].reshape(rows, t, cfg.kv_heads, cfg.head_dim)
-        q, k = self._rope(q, cos, sin), self._rope(k, cos, sin)
-        self.k_cache[li].index_copy_(2, write_slots, k.permute(0, 2, 1, 3))
-        self.v_cache[li].index_copy_(2, write_slots, v.permute(0, 2, 1, 3))
-        rep = cfg.q_heads // cfg.kv_heads
-        qg = q.permute(0, 2, 1, 3).reshape(rows, cfg.kv_heads, rep * t, cfg.head_dim)
-        scores = torch.matmul(qg, self.k_cache[li].transpose(-1, -2)) * (1.0 / np.sqrt(cfg.head_dim))
-        scores = scores.reshape(rows, cfg.kv_heads, rep, t, cfg.max_seq)
-        scores = scores.masked_fill(~visible[None, None, None], float("-inf"))
-        probs = torch.softmax(scores, dim=-1).reshape(rows, cfg.kv_heads, rep * t, cfg.max_seq)
-        ctxv = torch.matmul(probs, self.v_cache[li]).reshape(rows, cfg.q_heads, t, cfg.head_dim)
-        attn = ctxv.permute(0, 2, 1, 3).reshape(rows * t, cfg.q_dim)
-        x = x + self._linear(L["o"], attn).reshape(rows, t, cfg.hidden)
-        h = self._rmsnorm(x, L["norm2"])
-        gu = self._linear(L["gate_up"], h.reshape(rows * t, cfg.hidden))
-        act = torch.nn.functional.silu(gu[:, :cfg.inter]) * gu[:, cfg.inter:]
-        return x + self._linear(L["down"], act).reshape(rows, t, cfg.hidden)
-
-    def _head(self, x_last):
-        logits = self._linear(self.lm_head, self._rmsnorm(x_last, self.norm_f))
-        return logits, logits.argmax(dim=-1)
-
     # ---- prefill and decode -----------------------------------------------------------------
     def prefill(self, prompt):
         """prompt int64 [rows, t] on the device; fills the cache and returns the first new tokens."""
         torch, cfg = self.torch, self.cfg
         with torch.cuda.stream(self.stream):
             t = prompt.shape[1]
-            slots = self.slots[:t]
-            visible = self.slots[None, :] <= slots[:, None]
-            if self.fused:
-                self.last_logits, nxt = self._forward_fused(prompt.to(torch.int32).contiguous(), slots)
-            else:
-                x = self.embedding[prompt]
-                for li in range(cfg.layers):
-                    x = self._layer(li, x, self.cos[:t], self.sin[:t], slots, visible)
-                self.last_logits, nxt = self._head(x[:, -1, :])
+            self.last_logits, nxt = self._forward(prompt.to(torch.int32).contiguous(), self.slots[:t])
             self.tokens.copy_(nxt)
             self.position.fill_(t)
             self.history.zero_()
             self.history[0].copy_(nxt)
             self.emitted = 1
+        self._check_faults("prefill")
         return nxt
 
+    def _check_faults(self, what):
+        """Token ids, cache positions and row scales live in device memory, where only the kernels
+        can check them: a raised fault bit means the results of this call are meaningless."""
+        flags = self.ctx.fault_flags()  # synchronises the stream
+        if flags:
+            self.ctx.clear_fault_flags()
+            raise RuntimeError(f"W8A8Decoder.{what}: device fault flags {flags:#x} "
+                               "(1 bad multiplier, 2 token id outside the table, 4 position past the cache)")
+
     def _step(self):
-        torch, cfg = self.torch, self.cfg
-        pos = self.position
-        if self.fused:
-            # the argmax launch writes the next ids over the current ones and advances the position
-            self.last_logits, nxt = self._forward_fused(self.tokens[:, None], pos, next_tokens=self.tokens,
-                                                        advance=self.position)
-            return nxt
-        visible = self.slots[None, :] <= pos[:, None]
-        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        x = self.embedding[self.tokens][:, None, :]
-        for li in range(cfg.layers):
-            x = self._layer(li, x, cos, sin, pos, visible)
-        self.last_logits, nxt = self._head(x[:, 0, :])
-        self.tokens.copy_(nxt)
-        self.position.add_(1)
+        # the argmax launch writes the next ids over the current ones and advances the position
+        self.last_logits, nxt = self._forward(self.tokens[:, None], self.position, next_tokens=self.tokens,
+                                              advance=self.position)
         return nxt
 
     def capture(self):
-        """Capture one decode step in a HIP graph (after a warm-up step has sized every scratch)."""
+        """Capture one decode step in a HIP graph (after a warm-up step has sized every scratch).
+        The graph stays valid when a later, larger call (a longer prompt) grows the context's
+        scratch: the library keeps outgrown scratch blocks alive until the context is destroyed."""
         torch = self.torch
         keep = (self.tokens.clone(), self.position.clone(), self.k_cache.clone(), self.v_cache.clone())
         with torch.cuda.stream(self.stream):
@@ -321,7 +271,7 @@ class W8A8Decoder:
                     nxt = self._step()
                 self.history[self.emitted].copy_(nxt)
                 self.emitted += 1
-        self.stream.synchronize()
+        self._check_faults("decode")
         return self.history[:self.emitted]
 
     def close(self):

@@ -73,6 +73,10 @@ typedef struct PackagePlan {
     /* QuantizeLinear / DequantizeLinear: parameters of the byte side */
     float boundary_scale;
     int32_t boundary_zero_point;
+    /* Aligned copies of the small F32/I32 payloads above (scales, biases): a SafeTensors payload
+     * starts wherever its header ends and may be misaligned for its element type. */
+    void* aligned_copies[4];
+    size_t aligned_count;
     /* mapped files (borrowed) */
     VxstFile** files;
     size_t file_count;
@@ -189,7 +193,10 @@ static VxStatus refuse(Failure* failure, VxStatus status, const char* format, co
 }
 
 static void chain_release(ChainPlan* chain) {
-    for (size_t i = 0; i < chain->count; i++) free(chain->nodes[i].weight_zero_points);
+    for (size_t i = 0; i < chain->count; i++) {
+        free(chain->nodes[i].weight_zero_points);
+        for (size_t c = 0; c < chain->nodes[i].aligned_count; c++) free(chain->nodes[i].aligned_copies[c]);
+    }
     free(chain->nodes);
     for (size_t i = 0; i < chain->file_count; i++) vxst_close(chain->files[i]);
     free(chain->files);
@@ -358,6 +365,17 @@ static VxStatus plan_boundary(PackagePlan* plan, const VxjValue* root, const Vxj
     return VX_STATUS_OK;
 }
 
+/* An aligned copy of `bytes` payload bytes, owned by the plan; NULL when memory runs out. */
+static const void* aligned_payload(PackagePlan* plan, const void* data, size_t bytes) {
+    void* copy;
+    if (plan->aligned_count == sizeof(plan->aligned_copies) / sizeof(plan->aligned_copies[0])) return NULL;
+    copy = malloc(bytes ? bytes : 1);
+    if (!copy) return NULL;
+    memcpy(copy, data, bytes);
+    plan->aligned_copies[plan->aligned_count++] = copy;
+    return copy;
+}
+
 static VxStatus plan_qlinear(PackagePlan* plan, const VxjValue* root, const VxjValue* node, Failure* failure) {
     const VxjValue* node_inputs = vxj_member(node, "inputs");
     const char* weight_name = vxj_member_string(node_inputs, "weight");
@@ -391,16 +409,17 @@ static VxStatus plan_qlinear(PackagePlan* plan, const VxjValue* root, const VxjV
     status = resolve_affine(plan, table, weight_name, plan->weight_dtype == VXHIP_DTYPE_I8 ? VX_DTYPE_I8 : VX_DTYPE_U8,
                             2, plan->d_out, &scale, &zero_point, failure);
     if (status != VX_STATUS_OK) return status;
-    plan->weight_scales = (const float*)(const void*)scale.data;
+    plan->weight_scales = (const float*)aligned_payload(plan, scale.data, sizeof(float) * plan->d_out);
     plan->weight_zero_points = (int32_t*)malloc(sizeof(int32_t) * plan->d_out);
-    if (!plan->weight_zero_points) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
+    if (!plan->weight_scales || !plan->weight_zero_points) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
     for (uint32_t n = 0; n < plan->d_out; n++) plan->weight_zero_points[n] = typed_zero_point(&zero_point, n);
 
     if (bias_name) {
         if (find_tensor(plan, bias_name, &bias) != 1 || strcmp(bias.dtype, "I32") || bias.rank != 1 ||
             bias.shape[0] != (int64_t)plan->d_out)
             return refuse(failure, VX_STATUS_INVALID_GRAPH, "bias '%s' is not a unique I32 [d_out] tensor", bias_name);
-        plan->bias_i32 = (const int32_t*)(const void*)bias.data;
+        plan->bias_i32 = (const int32_t*)aligned_payload(plan, bias.data, sizeof(int32_t) * plan->d_out);
+        if (!plan->bias_i32) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
     }
     plan->kind = PLAN_QLINEAR;
     return VX_STATUS_OK;
@@ -444,13 +463,16 @@ static VxStatus plan_packed(PackagePlan* plan, const VxjValue* node, VxPackedAri
     if (find_tensor(plan, scale_name, &scale) != 1 || strcmp(scale.dtype, "F32") || scale.rank != 2 ||
         scale.shape[0] != (int64_t)plan->d_out || scale.shape[1] != groups)
         return refuse(failure, VX_STATUS_INVALID_GRAPH, "group scales '%s' are not F32 [d_out, groups]", scale_name);
+    /* (the packed words are only ever copied bytewise to the device; they stay in the mapping) */
     plan->packed_words = (const uint32_t*)(const void*)weight.data;
-    plan->group_scales = (const float*)(const void*)scale.data;
+    plan->group_scales = (const float*)aligned_payload(plan, scale.data, sizeof(float) * (size_t)plan->d_out * (size_t)groups);
+    if (!plan->group_scales) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
     if (bias_name) {
         if (find_tensor(plan, bias_name, &bias) != 1 || strcmp(bias.dtype, "F32") || bias.rank != 1 ||
             bias.shape[0] != (int64_t)plan->d_out)
             return refuse(failure, VX_STATUS_INVALID_GRAPH, "bias '%s' is not a unique F32 [d_out] tensor", bias_name);
-        plan->bias_f32 = (const float*)(const void*)bias.data;
+        plan->bias_f32 = (const float*)aligned_payload(plan, bias.data, sizeof(float) * plan->d_out);
+        if (!plan->bias_f32) return refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
     }
     plan->kind = PLAN_PACKED_LINEAR;
     return VX_STATUS_OK;

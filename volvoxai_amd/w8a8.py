@@ -41,12 +41,29 @@ def _hp(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
-def _dp(t):
-    """Device address of a contiguous torch tensor."""
+def _dp(t, name="tensor", dtype=None, shape=None, numel=None, min_numel=None):
+    """Device address of a contiguous torch tensor, after checking what the library cannot: it
+    receives a bare address, so a tensor of the wrong type or extent would be read or written out
+    of bounds on the device.  `dtype` is a torch dtype or a tuple of them."""
     if t is None:
         return None
-    assert t.is_cuda and t.is_contiguous(), "expected a contiguous device tensor"
+    if not (t.is_cuda and t.is_contiguous()):
+        raise ValueError(f"{name}: expected a contiguous device tensor")
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        raise ValueError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+    if numel is not None and t.numel() != numel:
+        raise ValueError(f"{name}: {t.numel()} elements, expected {numel}")
+    if min_numel is not None and t.numel() < min_numel:
+        raise ValueError(f"{name}: {t.numel()} elements, at least {min_numel} are needed")
     return C.c_void_p(t.data_ptr())
+
+
+def _byte_dtype(code, name):
+    if code not in (DTYPE_I8, DTYPE_U8):
+        raise ValueError(f"{name}: dtype id {code} is neither I8 ({DTYPE_I8}) nor U8 ({DTYPE_U8})")
+    return _torch_dtype(code)
 
 
 def _torch_dtype(code):
@@ -104,6 +121,12 @@ class Context:
         _check(library().vxhip_context_fault_flags(self._h, C.byref(v)), "vxhip_context_fault_flags")
         return v.value
 
+    def clear_fault_flags(self):
+        _check(library().vxhip_context_clear_fault_flags(self._h), "vxhip_context_clear_fault_flags")
+
+    def reserve_scratch(self, nbytes: int):
+        _check(library().vxhip_context_reserve_scratch(self._h, int(nbytes)), "vxhip_context_reserve_scratch")
+
     def probe_mfma_rate(self, rounds=128, random_operands=True) -> dict:
         """Register-only MFMA loop: the int8 rate, shader clock and time it reached."""
         tops, mhz, us = C.c_double(0), C.c_double(0), C.c_double(0)
@@ -157,13 +180,17 @@ class QLinear:
                 output_zero_point, input_dtype=DTYPE_I8, output_dtype=DTYPE_I8, out=None,
                 want_accumulators=False, accumulators=None):
         import torch
+        if x.ndim != 2 or x.shape[1] != self.d_in:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.d_in}]")
         rows = x.shape[0]
+        in_t, out_t = _byte_dtype(input_dtype, "input_dtype"), _byte_dtype(output_dtype, "output_dtype")
         if out is None:
-            out = torch.empty((rows, self.d_out), dtype=_torch_dtype(output_dtype), device=x.device)
+            out = torch.empty((rows, self.d_out), dtype=out_t, device=x.device)
         if want_accumulators and accumulators is None:
             accumulators = torch.empty((rows, self.d_out), dtype=torch.int32, device=x.device)
         ok = library().vxhip_qlinear_forward(
-            ctx._h, self._h, _dp(x), _dp(out), _dp(accumulators), rows, float(np.float32(input_scale)),
+            ctx._h, self._h, _dp(x, "x", in_t), _dp(out, "out", out_t, (rows, self.d_out)),
+            _dp(accumulators, "accumulators", torch.int32, (rows, self.d_out)), rows, float(np.float32(input_scale)),
             int(input_zero_point), float(np.float32(output_scale)), int(output_zero_point),
             input_dtype, output_dtype)
         return (ok, out, accumulators) if want_accumulators else (ok, out)
@@ -172,13 +199,18 @@ class QLinear:
                          output_dtype=DTYPE_I8, bias_f32=None, out=None, want_accumulators=False,
                          accumulators=None):
         import torch
+        if x.ndim != 2 or x.shape[1] != self.d_in:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.d_in}]")
         rows = x.shape[0]
+        out_t = _byte_dtype(output_dtype, "output_dtype")
         if out is None:
-            out = torch.empty((rows, self.d_out), dtype=_torch_dtype(output_dtype), device=x.device)
+            out = torch.empty((rows, self.d_out), dtype=out_t, device=x.device)
         if want_accumulators and accumulators is None:
             accumulators = torch.empty((rows, self.d_out), dtype=torch.int32, device=x.device)
         ok = library().vxhip_qlinear_forward_rowscale(
-            ctx._h, self._h, _dp(x), _dp(row_scales), _dp(bias_f32), _dp(out), _dp(accumulators), rows,
+            ctx._h, self._h, _dp(x, "x", torch.int8), _dp(row_scales, "row_scales", torch.float32, numel=rows),
+            _dp(bias_f32, "bias_f32", torch.float32, numel=self.d_out), _dp(out, "out", out_t, (rows, self.d_out)),
+            _dp(accumulators, "accumulators", torch.int32, (rows, self.d_out)), rows,
             float(np.float32(output_scale)), int(output_zero_point), output_dtype)
         return (ok, out, accumulators) if want_accumulators else (ok, out)
 
@@ -213,22 +245,32 @@ class PackedLinear:
 
     def forward_f32(self, ctx: Context, x, out=None):
         import torch
+        if x.ndim != 2 or x.shape[1] != self.k:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.k}]")
         rows = x.shape[0]
         if out is None:
             out = torch.empty((rows, self.n), dtype=torch.float32, device=x.device)
-        st = library().vxhip_packed_linear_forward_f32(ctx._h, self._h, _dp(x), _dp(out), rows)
+        st = library().vxhip_packed_linear_forward_f32(ctx._h, self._h, _dp(x, "x", torch.float32),
+                                                        _dp(out, "out", torch.float32, (rows, self.n)), rows)
         return st, out
 
     def forward_a8(self, ctx: Context, a8, row_scales, out=None, want_accumulators=False,
                    accumulators=None):
         import torch
+        if row_scales.ndim != 1:
+            raise ValueError(f"row_scales: shape {tuple(row_scales.shape)}, expected [rows]")
         rows = row_scales.shape[0]  # (a8 is flat when the context exchanges operand-order activations)
+        need = library().vxhip_context_prepared_bytes(ctx._h, rows, self.k)
+        if a8.ndim == 2 and tuple(a8.shape) != (rows, self.k):
+            raise ValueError(f"a8: shape {tuple(a8.shape)}, expected ({rows}, {self.k}) or the flat operand-order buffer")
         if out is None:
             out = torch.empty((rows, self.n), dtype=torch.float32, device=a8.device)
         if want_accumulators and accumulators is None:
             accumulators = torch.empty((rows, self.n), dtype=torch.int32, device=a8.device)
-        st = library().vxhip_packed_linear_forward_a8(ctx._h, self._h, _dp(a8), _dp(row_scales),
-                                                       _dp(out), _dp(accumulators), rows)
+        st = library().vxhip_packed_linear_forward_a8(
+            ctx._h, self._h, _dp(a8, "a8", torch.int8, numel=need), _dp(row_scales, "row_scales", torch.float32),
+            _dp(out, "out", torch.float32, (rows, self.n)),
+            _dp(accumulators, "accumulators", torch.int32, (rows, self.n)), rows)
         return (st, out, accumulators) if want_accumulators else (st, out)
 
 
@@ -239,8 +281,9 @@ def rmsnorm_prepare_i8(ctx: Context, x, gain, eps, want_normalized=False):
     a8 = ctx.prepared_buffer(rows, d, x.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
     normalized = torch.empty((rows, d), dtype=torch.float32, device=x.device) if want_normalized else None
-    _check(library().vxhip_rmsnorm_prepare_i8(ctx._h, _dp(x), _dp(gain), rows, d, float(eps), _dp(a8), _dp(scales),
-                                              _dp(normalized)), "vxhip_rmsnorm_prepare_i8")
+    _check(library().vxhip_rmsnorm_prepare_i8(ctx._h, _dp(x, "x", torch.float32), _dp(gain, "gain", torch.float32, numel=d),
+                                              rows, d, float(eps), _dp(a8), _dp(scales), _dp(normalized)),
+           "vxhip_rmsnorm_prepare_i8")
     return (a8, scales, normalized) if want_normalized else (a8, scales)
 
 
@@ -250,7 +293,9 @@ def add_rmsnorm_prepare_i8(ctx: Context, residual, delta, gain, eps):
     rows, d = residual.shape
     a8 = ctx.prepared_buffer(rows, d, residual.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=residual.device)
-    _check(library().vxhip_add_rmsnorm_prepare_i8(ctx._h, _dp(residual), _dp(delta), _dp(gain), rows, d, float(eps),
+    _check(library().vxhip_add_rmsnorm_prepare_i8(ctx._h, _dp(residual, "residual", torch.float32),
+                                                  _dp(delta, "delta", torch.float32, (rows, d)),
+                                                  _dp(gain, "gain", torch.float32, numel=d), rows, d, float(eps),
                                                   _dp(a8), _dp(scales)), "vxhip_add_rmsnorm_prepare_i8")
     return a8, scales
 
@@ -259,22 +304,42 @@ def swiglu_prepare_i8(ctx: Context, gate_up, want_activated=False):
     """silu(gate) * up of gate_up [rows, 2*inter], then activation preparation."""
     import torch
     rows, two = gate_up.shape
+    if two % 2:
+        raise ValueError(f"gate_up: shape {tuple(gate_up.shape)}, the last extent must be even")
     inter = two // 2
     a8 = ctx.prepared_buffer(rows, inter, gate_up.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=gate_up.device)
     act = torch.empty((rows, inter), dtype=torch.float32, device=gate_up.device) if want_activated else None
-    _check(library().vxhip_swiglu_prepare_i8(ctx._h, _dp(gate_up), rows, inter, _dp(a8), _dp(scales), _dp(act)),
+    _check(library().vxhip_swiglu_prepare_i8(ctx._h, _dp(gate_up, "gate_up", torch.float32), rows, inter, _dp(a8),
+                                             _dp(scales), _dp(act)),
            "vxhip_swiglu_prepare_i8")
     return (a8, scales, act) if want_activated else (a8, scales)
+
+
+def _check_caches(k_cache, v_cache, cos, sin, rows, kv_heads, head_dim):
+    """Shapes the attention entry points index by: caches [rows, kv_heads, max_seq, head_dim] f32,
+    rotary tables [max_seq, head_dim] f32.  Returns max_seq."""
+    import torch
+    if k_cache.ndim != 4 or tuple(k_cache.shape[:2]) != (rows, kv_heads) or k_cache.shape[3] != head_dim:
+        raise ValueError(f"k_cache: shape {tuple(k_cache.shape)}, expected [{rows}, {kv_heads}, max_seq, {head_dim}]")
+    max_seq = k_cache.shape[2]
+    _dp(k_cache, "k_cache", torch.float32)
+    _dp(v_cache, "v_cache", torch.float32, tuple(k_cache.shape))
+    for name, table in (("cos", cos), ("sin", sin)):
+        if table is not None:
+            _dp(table, name, torch.float32, (max_seq, head_dim))
+    return max_seq
 
 
 def rope_append_kv(ctx: Context, qkv, cos, sin, positions, q_heads, kv_heads, head_dim, k_cache, v_cache):
     """qkv [rows, t, (q+2kv)*d]; caches [rows, kv_heads, max_seq, d] updated in place; returns rotated q."""
     import torch
     rows, t, _ = qkv.shape
+    max_seq = _check_caches(k_cache, v_cache, cos, sin, rows, kv_heads, head_dim)
     q = torch.empty((rows, t, q_heads, head_dim), dtype=torch.float32, device=qkv.device)
-    _check(library().vxhip_rope_append_kv(ctx._h, _dp(qkv), _dp(cos), _dp(sin), _dp(positions), rows, t, q_heads,
-                                          kv_heads, head_dim, k_cache.shape[2], _dp(q), _dp(k_cache), _dp(v_cache)),
+    _check(library().vxhip_rope_append_kv(ctx._h, _dp(qkv, "qkv", torch.float32, (rows, t, (q_heads + 2 * kv_heads) * head_dim)),
+                                          _dp(cos), _dp(sin), _dp(positions, "positions", torch.int64, numel=t), rows, t, q_heads,
+                                          kv_heads, head_dim, max_seq, _dp(q), _dp(k_cache), _dp(v_cache)),
            "vxhip_rope_append_kv")
     return q
 
@@ -283,9 +348,13 @@ def gqa_attention(ctx: Context, q, k_cache, v_cache, positions):
     """q [rows, t, q_heads, d] over caches [rows, kv_heads, max_seq, d]; returns [rows, t, q_heads*d]."""
     import torch
     rows, t, q_heads, head_dim = q.shape
+    if k_cache.ndim != 4:
+        raise ValueError(f"k_cache: shape {tuple(k_cache.shape)}, expected [rows, kv_heads, max_seq, head_dim]")
+    max_seq = _check_caches(k_cache, v_cache, None, None, rows, k_cache.shape[1], head_dim)
     out = torch.empty((rows, t, q_heads * head_dim), dtype=torch.float32, device=q.device)
-    _check(library().vxhip_gqa_attention(ctx._h, _dp(q), _dp(k_cache), _dp(v_cache), _dp(positions), rows, t, q_heads,
-                                         k_cache.shape[1], head_dim, k_cache.shape[2], _dp(out)),
+    _check(library().vxhip_gqa_attention(ctx._h, _dp(q, "q", torch.float32), _dp(k_cache), _dp(v_cache),
+                                         _dp(positions, "positions", torch.int64, numel=t), rows, t, q_heads,
+                                         k_cache.shape[1], head_dim, max_seq, _dp(out)),
            "vxhip_gqa_attention")
     return out
 
@@ -295,9 +364,11 @@ def rope_gqa_attention_decode(ctx: Context, qkv, cos, sin, position, q_heads, kv
     in one launch; returns [rows, q_heads*d]."""
     import torch
     rows = qkv.shape[0]
+    max_seq = _check_caches(k_cache, v_cache, cos, sin, rows, kv_heads, head_dim)
     out = torch.empty((rows, q_heads * head_dim), dtype=torch.float32, device=qkv.device)
-    _check(library().vxhip_rope_gqa_attention_decode(ctx._h, _dp(qkv), _dp(cos), _dp(sin), _dp(position), rows, q_heads,
-                                                     kv_heads, head_dim, k_cache.shape[2], _dp(k_cache), _dp(v_cache),
+    _check(library().vxhip_rope_gqa_attention_decode(ctx._h, _dp(qkv, "qkv", torch.float32, (rows, (q_heads + 2 * kv_heads) * head_dim)),
+                                                     _dp(cos), _dp(sin), _dp(position, "position", torch.int64, min_numel=1),
+                                                     rows, q_heads, kv_heads, head_dim, max_seq, _dp(k_cache), _dp(v_cache),
                                                      _dp(out)),
            "vxhip_rope_gqa_attention_decode")
     return out
@@ -310,7 +381,9 @@ def embedding_gather(ctx: Context, tokens_i32, table, out=None):
     vocab, d = table.shape
     if out is None:
         out = torch.empty((count, d), dtype=torch.float32, device=table.device)
-    _check(library().vxhip_embedding_gather_f32(ctx._h, _dp(tokens_i32), _dp(table), count, d, vocab, _dp(out)),
+    _check(library().vxhip_embedding_gather_f32(ctx._h, _dp(tokens_i32, "tokens", torch.int32),
+                                                _dp(table, "table", torch.float32), count, d, vocab,
+                                                _dp(out, "out", torch.float32, numel=count * d)),
            "vxhip_embedding_gather_f32")
     return out
 
@@ -322,7 +395,10 @@ def argmax_rows(ctx: Context, x, out=None, advance=None):
     rows, n = x.shape
     if out is None:
         out = torch.empty((rows,), dtype=torch.int32, device=x.device)
-    _check(library().vxhip_argmax_rows_f32(ctx._h, _dp(x), rows, n, _dp(out), _dp(advance),
+    if advance is not None and advance.numel() > 64:
+        raise ValueError("advance: at most 64 counters")
+    _check(library().vxhip_argmax_rows_f32(ctx._h, _dp(x, "x", torch.float32), rows, n,
+                                           _dp(out, "out", torch.int32, numel=rows), _dp(advance, "advance", torch.int64),
                                            0 if advance is None else advance.numel()),
            "vxhip_argmax_rows_f32")
     return out
@@ -349,7 +425,7 @@ def packed_prepare_i8(ctx: Context, x):
     rows, k = x.shape
     a8 = ctx.prepared_buffer(rows, k, x.device)
     scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
-    _check(library().vxhip_packed_prepare_i8(ctx._h, _dp(x), rows, k, _dp(a8), _dp(scales)),
+    _check(library().vxhip_packed_prepare_i8(ctx._h, _dp(x, "x", torch.float32), rows, k, _dp(a8), _dp(scales)),
            "vxhip_packed_prepare_i8")
     return a8, scales
 
