@@ -36,15 +36,17 @@ class DecoderRef:
         partner = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
         return (x * cos[None, :, None, :] + partner * sin[None, :, None, :]).astype(np.float32)
 
-    def forward(self, tokens, start, k_cache, v_cache):
+    def forward(self, tokens, start, k_cache, v_cache, trace=None):
         """tokens [rows, t] at positions start..start+t-1; caches [layers][rows, kvh, seq, d] lists
-        grown in place.  Returns the logits of the last position."""
+        grown in place.  Returns the logits of the last position.  `trace` (a list) receives one
+        dict per layer with every intermediate tensor, for stage-by-stage comparisons."""
         cfg = self.cfg
         rows, t = tokens.shape
         x = self.w["embedding"][tokens]
         cos, sin = self.cos[start:start + t], self.sin[start:start + t]
         rep = cfg.q_heads // cfg.kv_heads
         for li, L in enumerate(self.w["layers"]):
+            x_in = x
             h = self.rmsnorm(x, L["norm1"])
             qkv = self.linear((li, "qkv"), L["qkv"], h.reshape(rows * t, -1)).reshape(rows, t, -1)
             q = self.rope(qkv[..., :cfg.q_dim].reshape(rows, t, cfg.q_heads, cfg.head_dim), cos, sin)
@@ -70,12 +72,16 @@ class DecoderRef:
             else:
                 ctxv = np.einsum("bgrts,bgsd->bgrtd", p, v_cache[li]).astype(np.float32)
             attn = ctxv.reshape(rows, cfg.q_heads, t, cfg.head_dim).transpose(0, 2, 1, 3).reshape(rows * t, cfg.q_dim)
-            x = x + self.linear((li, "o"), L["o"], attn).reshape(rows, t, -1)
+            o = self.linear((li, "o"), L["o"], attn)
+            x = x + o.reshape(rows, t, -1)
             h = self.rmsnorm(x, L["norm2"])
             gu = self.linear((li, "gu"), L["gate_up"], h.reshape(rows * t, -1))
             gate, up = gu[:, :cfg.inter], gu[:, cfg.inter:]
             act = (gate / (1.0 + np.exp(-gate.astype(np.float64)))).astype(np.float32) * up
-            x = x + self.linear((li, "down"), L["down"], act).reshape(rows, t, -1)
+            down = self.linear((li, "down"), L["down"], act)
+            if trace is not None:
+                trace.append(dict(x_in=x_in, qkv=qkv, attn=attn, o=o, x_mid=x, gu=gu, act=act, down=down))
+            x = x + down.reshape(rows, t, -1)
         return self.linear("head", self.w["lm_head"], self.rmsnorm(x[:, -1, :], self.w["norm_f"]))
 
     def generate(self, prompt, new_tokens):
