@@ -336,6 +336,24 @@ int vxhip_packed_linear_forward_f32(VxHipContext* context,
                                     const float* input_dev, float* output_dev,
                                     uint32_t rows);
 
+/* vxhip_packed_linear_forward_f32 for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): it has no counterpart in the reference.  Same arguments, same
+ * arithmetic, same output bits; the prepared activations are staged in a fixed
+ * 4 MiB array inside the library's device code instead of the context's
+ * grow-only scratch, and the call makes no hipMalloc/hipFree.  The staging needs
+ * 256 + 4 * rows (rounded up to 256) + max(rows, 32 when rows <= 32) * ceil16(k)
+ * bytes; a call that needs more returns -1 with vxhip_last_error saying so
+ * (for example rows = 256 at k = 14336 fits, rows = 2048 does not).  Each device
+ * has one such array, shared by every context on it and keeping the last call's
+ * contents: calls that overlap on one device (two streams, two threads) race.
+ * The array's address is looked up when the first context on a device is
+ * created, so the entry point itself performs no set-up. */
+int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* context,
+                                            const VxHipPackedLinear* linear,
+                                            const float* input_dev,
+                                            float* output_dev, uint32_t rows);
+
 /* Same arithmetic from already prepared activations (the x[4]/x[5] form of
  * src/kernels/llm_ops.h:30-32): int8 codes [rows,k] and one f32 scale per
  * row; a NaN scale marks a non-finite row (whole output row NaN).

@@ -86,6 +86,43 @@ struct Carver {
     }
 };
 
+// ---- scratch of the entry point that allocates nothing ---------------------------------------
+// vxhip_packed_linear_forward_f32_noalloc stages its prepared activations (one f32 scale per row,
+// then the int8 codes) here instead of in a context's grow-only scratch.  The array lives in every
+// device's copy of the code object, at an address of its own on each device: host code never uses
+// the array's name as a pointer, only the per-device address looked up once, with that device
+// current, when the first context on the device is created.
+constexpr size_t kNoAllocScratchBytes = 4u << 20;
+static __device__ __align__(256) unsigned char g_no_alloc_scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::mutex g_no_alloc_mutex;
+static void* g_no_alloc_ptr[kMaxDevices] = {};
+static hipError_t g_no_alloc_status[kMaxDevices] = {};
+static bool g_no_alloc_looked_up[kMaxDevices] = {};
+
+// Looks the array's address up on `device`, which must be current.  Returns null on failure (the
+// error text is set); the failure is remembered, so the entry point reports it instead of trying
+// again at a time when the caller may not allocate.
+static void* no_alloc_scratch(int device) {
+    if (device < 0 || device >= kMaxDevices) {
+        set_error("device ordinal %d is outside the table of %d", device, kMaxDevices);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_no_alloc_mutex);
+    if (!g_no_alloc_looked_up[device]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_no_alloc_scratch));
+        if (e != hipSuccess) (void)hipGetLastError();
+        g_no_alloc_status[device] = e;
+        g_no_alloc_ptr[device] = e == hipSuccess ? ptr : nullptr;
+        g_no_alloc_looked_up[device] = true;
+    }
+    if (!g_no_alloc_ptr[device])
+        set_error("hipGetSymbolAddress(no-alloc scratch) failed on device %d: %s", device,
+                  hipGetErrorString(g_no_alloc_status[device]));
+    return g_no_alloc_ptr[device];
+}
+
 static bool use_device(int device) {
     if (hipSetDevice(device) != hipSuccess) {
         set_error("hipSetDevice(%d) failed", device);
@@ -181,6 +218,9 @@ VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags, V
     VxHipContext* ctx = new (std::nothrow) VxHipContext();
     if (!ctx) return VXHIP_OUT_OF_MEMORY;
     ctx->device = device;
+    // set-up of the entry point that allocates nothing: this device's address of its scratch array
+    // (a failure is reported by that entry point, not here)
+    ctx->no_alloc_scratch = no_alloc_scratch(device);
     ctx->cu_count = prop.multiProcessorCount;
     if (flags == VXHIP_CONTEXT_BORROW_STREAM) {
         ctx->stream = (hipStream_t)stream;
@@ -811,6 +851,46 @@ int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* 
     const int st = packed_run_a8(ctx, pl, prepared, ld, operand_order, row_scales, output_dev, nullptr, nullptr, rows);
     if (st != -2) return st;
     // no GEMV takes the shape (or a GEMM tile is forced): once more, as rows, for the GEMM
+    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, 0u}, row_scales) != VXHIP_OK)
+        return -1;
+    return packed_run_a8(ctx, pl, prepared, ld, false, row_scales, output_dev, nullptr, nullptr, rows);
+}
+
+int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,
+                                            float* output_dev, uint32_t rows) {
+    if (!ctx || !pl || !input_dev || !output_dev) {
+        set_error("packed_linear_forward_f32_noalloc: null handle or tensor");
+        return -1;
+    }
+    if (!rows) return 0;
+    if (!same_device(ctx, pl->device, "packed_linear_forward_f32_noalloc") || !use_device(ctx->device)) return -1;
+    if (!ctx->no_alloc_scratch) {
+        (void)no_alloc_scratch(ctx->device);  // sets the error text of the failed set-up
+        return -1;
+    }
+    const uint32_t k = pl->w.k;
+    const uint32_t ld = (k + 15u) / 16u * 16u;
+    const bool operand_order = rows <= kOperandOrderRows;
+    const size_t prepared_rows = operand_order ? kOperandOrderRows : rows;
+    // the same carving as vxhip_packed_linear_forward_f32, out of the fixed array
+    Carver sizes{nullptr};
+    sizes.take<float>(rows);
+    sizes.take<int8_t>(prepared_rows * ld);
+    if (sizes.off > kNoAllocScratchBytes) {
+        set_error("packed_linear_forward_f32_noalloc: rows=%u k=%u need %zu bytes of staging, the fixed scratch "
+                  "holds %zu (use vxhip_packed_linear_forward_f32, which sizes its own)",
+                  rows, k, sizes.off, kNoAllocScratchBytes);
+        return -1;
+    }
+    Carver c{(char*)ctx->no_alloc_scratch};
+    float* row_scales = c.take<float>(rows);
+    int8_t* prepared = c.take<int8_t>(prepared_rows * ld);
+    // every byte the linear reads is written by the preparation first: nothing has to start at zero
+    if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, operand_order ? 1u : 0u},
+                          row_scales) != VXHIP_OK)
+        return -1;
+    const int st = packed_run_a8(ctx, pl, prepared, ld, operand_order, row_scales, output_dev, nullptr, nullptr, rows);
+    if (st != -2) return st;
     if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, 0u}, row_scales) != VXHIP_OK)
         return -1;
     return packed_run_a8(ctx, pl, prepared, ld, false, row_scales, output_dev, nullptr, nullptr, rows);

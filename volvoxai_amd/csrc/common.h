@@ -73,6 +73,7 @@ struct VxHipContext {
     void* retired[kRetiredSlots] = {};
     int retired_count = 0;
     uint32_t* fault_dev = nullptr;
+    void* no_alloc_scratch = nullptr;  // this device's address of the fixed scratch array (api.hip), or null
     // Exhaustive exactness proofs of the short division sequences, one pair of mismatch
     // counters per divisor seen (the output scales of the calls made on this context).
     static constexpr int kDivisorSlots = 16;

@@ -243,15 +243,19 @@ class PackedLinear:
     def resident_bytes(self) -> int:
         return int(library().vxhip_packed_linear_resident_bytes(self._h))
 
-    def forward_f32(self, ctx: Context, x, out=None):
+    def forward_f32(self, ctx: Context, x, out=None, no_alloc=False):
+        """no_alloc=True takes the entry point that stages in the library's fixed scratch array and
+        allocates nothing (`out` must then be given)."""
         import torch
         if x.ndim != 2 or x.shape[1] != self.k:
             raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.k}]")
         rows = x.shape[0]
         if out is None:
+            if no_alloc:
+                raise ValueError("out: the entry point that allocates nothing needs the output tensor from its caller")
             out = torch.empty((rows, self.n), dtype=torch.float32, device=x.device)
-        st = library().vxhip_packed_linear_forward_f32(ctx._h, self._h, _dp(x, "x", torch.float32),
-                                                        _dp(out, "out", torch.float32, (rows, self.n)), rows)
+        entry = library().vxhip_packed_linear_forward_f32_noalloc if no_alloc else library().vxhip_packed_linear_forward_f32
+        st = entry(ctx._h, self._h, _dp(x, "x", torch.float32), _dp(out, "out", torch.float32, (rows, self.n)), rows)
         return st, out
 
     def forward_a8(self, ctx: Context, a8, row_scales, out=None, want_accumulators=False,
