@@ -25,56 +25,16 @@
 #include "common.h"
 #include "device_math.h"
 #include "epilogue.h"
+#include "gemm_tile.h"
 
 #include <stdio.h>
 #include <string.h>
-
-#include <type_traits>
-#include <utility>
 
 namespace vxhip {
 
 namespace {
 
 extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-__device__ __forceinline__ void wg_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
-__device__ __forceinline__ void load_to_lds16(const void* gptr, void* lptr) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
-                                     (__attribute__((address_space(3))) void*)lptr, 16, 0, 0);
-}
-
-__device__ __forceinline__ void load_to_lds4(const void* gptr, void* lptr) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
-                                     (__attribute__((address_space(3))) void*)lptr, 4, 0, 0);
-}
-
-struct GemmParams {
-    LinearArgs a;
-    uint32_t tiles_n, tiles_m;
-};
-
-template <int V>
-using IC = std::integral_constant<int, V>;
-template <int... I, class F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
-    (f(IC<I>{}), ...);
-}
-// f(IC<0>{}), f(IC<1>{}), ... f(IC<N-1>{}): a loop whose index is a compile-time constant
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-    static_for_impl(std::make_integer_sequence<int, N>{}, f);
-}
 
 constexpr int KS = 4;  // k-steps of 32 per stage: 128 bytes of k, one cache line per activation row
 
@@ -121,23 +81,13 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_mfma_kernel(const GemmParams
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int wave_n = wave % WN, wave_m = wave / WN;
 
-    // ---- workgroup -> tile, XCD aware ------------------------------------
-    // Consecutive workgroup ids land on different XCDs (8 of them, each with
-    // its own L2).  Give XCD x the x-th contiguous run of tiles, and order
-    // tiles so a run is a compact block of the output: that block's operand
-    // slices are then shared through one L2 instead of being fetched by all.
-    const uint32_t total = p.tiles_n * p.tiles_m;
-    const uint32_t per_xcd = (total + 7u) / 8u;
-    const uint32_t lin = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-    if (lin >= total) return;
-    constexpr uint32_t GROUP_M = 4;
-    const uint32_t band = lin / (GROUP_M * p.tiles_n);
-    const uint32_t band_first = band * GROUP_M;
-    const uint32_t band_rows = min(GROUP_M, p.tiles_m - band_first);
-    const uint32_t in_band = lin - band * GROUP_M * p.tiles_n;
-    const uint32_t tile_m = band_first + in_band % band_rows;
-    const uint32_t tile_n = in_band / band_rows;
-    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    uint32_t m0, n0;
+    {
+        const TileOrigin t = tile_of_workgroup<BN, BM>(p);
+        if (!t.valid) return;
+        m0 = t.m0;
+        n0 = t.n0;
+    }
 
     // ---- per-lane load sources ---------------------------------------------
     // Weights: block b = wave + t*NWAVES of the stage is (panel b/KB, block b%KB); its address is
@@ -686,6 +636,11 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (forced("t128x128")) pick = 2;
         if (forced("t128x64")) pick = 3;
         if (forced("t64x64")) pick = 4;
+        // The two large tiles run on the 16x16x64 MFMA (gemm_k64.hip) when the straight-line epilogue
+        // applies; a forced tile name without "k64" keeps the 32x32x32 kernel of this file.
+        const bool fast_ok = (a.n % 16u) == 0u && a.y && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u;
+        const bool named = forced("t256x") || forced("t128x") || forced("t64x");
+        if (pick <= 1 && fast_ok && (forced("k64") || !named)) return launch_gemm_k64(s, a, pick);
         if (pick == 0 && forced("wv4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256wv4" : nullptr;
         if (pick == 0) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
         if (pick == 1 && forced("wv4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128wv4" : nullptr;
