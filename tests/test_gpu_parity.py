@@ -192,7 +192,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
     seen = set()
     try:
         for force in ("gemv.wv2", "gemv.wv16c32", "gemv.wv16c8", "gemv.wv8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
-                      "a8-mfma.t64x64", "a8-mfma.t128x128p"):
+                      "a8-mfma.t64x64", "a8-mfma.t128x128p", "a8-mfma.t128x128k64", "a8-mfma.t128x256k64s3"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -202,7 +202,7 @@ def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):
         vx.force_variant(None)
     # one scale group per k-step has no eight-wave tile: that request runs the four-wave one
     # (the pipelined 128x128 tile exists for one group per k-block only, i.e. G = 128)
-    assert len(seen) == (7 if group == 32 else 9 if group == 128 else 8), seen
+    assert len(seen) == (7 if group == 32 else 11 if group == 128 else 10), seen
     pl.close()
 
 
@@ -260,7 +260,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
     seen = set()
     try:
         for force in ("gemv.wv2", "gemv.wv16c32", "gemv.wv16c8", "gemv.wv8c16", "a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128",
-                      "a8-mfma.t64x64", "a8-mfma.t128x128p"):
+                      "a8-mfma.t64x64", "a8-mfma.t128x128p", "a8-mfma.t128x128k64", "a8-mfma.t128x256k64s3"):
             vx.force_variant(force)
             st, y = pl.forward_f32(ctx, xd)
             ctx.synchronize()
@@ -268,7 +268,7 @@ def test_gemv_and_gemm_agree_packed_w4(ctx, oracle, rows, k, n, group):
             seen.add(ctx.last_variant)
     finally:
         vx.force_variant(None)
-    assert all("w4a8" in v for v in seen) and len(seen) == (7 if group == 32 else 9 if group == 128 else 8), seen
+    assert all("w4a8" in v for v in seen) and len(seen) == (7 if group == 32 else 10 if group == 128 else 9), seen
     pl.close()
 
 
@@ -687,7 +687,7 @@ def test_every_tile_and_stage_variant_on_ragged_shapes(ctx, oracle):
     import volvoxai_amd as vx
     rng = np.random.default_rng(31)
     packed_variants = ("a8-mfma.t128x128", "a8-mfma.t256x256", "a8-mfma.t64x128", "a8-mfma.t64x64",
-                       "a8-mfma.t128x128p")
+                       "a8-mfma.t128x128p", "a8-mfma.t128x128k64", "a8-mfma.t128x256k64s3")
     for trial in range(24):
         rows = int(rng.choice([3, 33, 65, 128, 200, 257]))
         k = int(rng.choice([31, 64, 129, 384, 640, 1153]))

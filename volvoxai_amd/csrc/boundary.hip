@@ -102,11 +102,85 @@ __global__ __launch_bounds__(1024) void prepare_i8_kernel(
     if (threadIdx.x == 0) scales[row] = bad ? __builtin_nanf("") : scale;
 }
 
+// The same rule for many rows in row-major layout (k % 4 == 0, 16-byte aligned rows): a workgroup
+// per row, 16 bytes per lane and load, four codes per store, and the whole row kept in registers
+// between the two passes when it has at most 256 * 4 * kKeptChunks elements -- the row is then read
+// from HBM once and the kernel runs at the speed of that read.
+template <int kKeptChunks>
+__global__ __launch_bounds__(256) void prepare_i8_rows_kernel(const float* __restrict__ x, uint32_t k,
+                                                              int8_t* __restrict__ prepared, uint32_t ld,
+                                                              float* __restrict__ scales) {
+    __shared__ float slot_max[4];
+    __shared__ uint32_t slot_bad[4];
+    const uint32_t row = blockIdx.x;
+    const v4f* src = reinterpret_cast<const v4f*>(x + (size_t)row * k);
+    const uint32_t chunks = k / 4u;
+    float maximum = 0.0f;
+    uint32_t bad = 0u;
+    v4f kept[kKeptChunks];
+#pragma unroll
+    for (int i = 0; i < kKeptChunks; i++) {
+        const uint32_t c = threadIdx.x + i * 256u;
+        kept[i] = c < chunks ? __builtin_nontemporal_load(src + c) : v4f{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < kKeptChunks; i++) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            bad |= finite_f32(kept[i][e]) ? 0u : 1u;
+            maximum = fmaxf(maximum, fabsf(kept[i][e]));  // fmaxf ignores a NaN operand; `bad` records it
+        }
+    }
+    for (uint32_t c = threadIdx.x + kKeptChunks * 256u; c < chunks; c += 256u) {
+        const v4f v = src[c];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            bad |= finite_f32(v[e]) ? 0u : 1u;
+            maximum = fmaxf(maximum, fabsf(v[e]));
+        }
+    }
+    maximum = wave_max(maximum);
+    bad = __builtin_amdgcn_ballot_w64(bad != 0u) != 0ull ? 1u : 0u;
+    if ((threadIdx.x & 63u) == 0u) {
+        slot_max[threadIdx.x >> 6] = maximum;
+        slot_bad[threadIdx.x >> 6] = bad;
+    }
+    __syncthreads();
+    maximum = fmaxf(fmaxf(slot_max[0], slot_max[1]), fmaxf(slot_max[2], slot_max[3]));
+    bad = slot_bad[0] | slot_bad[1] | slot_bad[2] | slot_bad[3];
+    float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+    if (scale < 0x1p-126f) scale = 0x1p-126f;
+    uint32_t* dst = reinterpret_cast<uint32_t*>(prepared + (size_t)row * ld);
+    auto codes = [&](const v4f v) {
+        if (bad) return 0u;
+        return pack4_bytes(packed_round_i8(__fdiv_rn(v[0], scale)), packed_round_i8(__fdiv_rn(v[1], scale)),
+                           packed_round_i8(__fdiv_rn(v[2], scale)), packed_round_i8(__fdiv_rn(v[3], scale)));
+    };
+#pragma unroll
+    for (int i = 0; i < kKeptChunks; i++) {
+        const uint32_t c = threadIdx.x + i * 256u;
+        if (c < chunks) dst[c] = codes(kept[i]);
+    }
+    for (uint32_t c = threadIdx.x + kKeptChunks * 256u; c < chunks; c += 256u) dst[c] = codes(src[c]);
+    for (uint32_t c = chunks + threadIdx.x; c < ld / 4u; c += 256u) dst[c] = 0u;  // the padding of the row
+    if (threadIdx.x == 0) scales[row] = bad ? __builtin_nanf("") : scale;
+}
+
 VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint32_t k,
                               int8_t* prepared, ActivationLayout layout, float* scales) {
     // (operand order has room for 32 rows, and its rows are whole 16-byte chunks)
     if (layout.operand_order && (rows > kOperandOrderRows || layout.ld != (k + 15u) / 16u * 16u))
         return VXHIP_INVALID_ARGUMENT;
+    // many rows: the vectorized kernel (rows that fit its registers are read once)
+    if (!layout.operand_order && rows > 64u && (k % 4u) == 0u && (layout.ld % 4u) == 0u && ((uintptr_t)x % 16u) == 0u &&
+        ((uintptr_t)prepared % 4u) == 0u) {
+        if (k <= 4096u)
+            hipLaunchKernelGGL(prepare_i8_rows_kernel<4>, dim3(rows), dim3(256), 0, s, x, k, prepared, layout.ld, scales);
+        else
+            hipLaunchKernelGGL(prepare_i8_rows_kernel<14>, dim3(rows), dim3(256), 0, s, x, k, prepared, layout.ld, scales);
+        VXHIP_TRY(hipGetLastError());
+        return VXHIP_OK;
+    }
     // few long rows: latency bound, give each row a full workgroup
     const uint32_t block = rows <= 256u && k >= 1024u ? 1024u : 256u;
     hipLaunchKernelGGL(prepare_i8_kernel, dim3(rows), dim3(block), 0, s, x, k, prepared, layout, scales);

@@ -304,6 +304,218 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
     else run(IC<0>{});
 }
 
+// ---- the dequantizing form (PackedLinear under DYNAMIC_I8) ----------------------------------------
+// sum += f32(dot_g) * (s_a * s_w[n][g]) in ascending group order with every product and sum rounded
+// on its own (packed_linear_ops.inc:1498-1504): four VALU operations per output and group against
+// 2 * group_size matrix operations, so the kernel is bound by the vector pipe, not by the MFMAs.
+// It therefore runs small wave tiles (64 channels x 32 rows) at four waves per SIMD and leaves the
+// overlap of one wave's fold with the other waves' MFMAs to the hardware: two workgroups of
+// 128 x 128 per compute unit, each with its own barrier.  GK: 64-wide MFMA steps per scale group
+// (1, 2 or 4).  W4: four-bit weights; a 1 KiB block then holds the block pair of one MFMA step, low
+// nibbles for its first 32 k, high nibbles for the rest, and a lane shifts its half into place.
+// The scales of the groups that end in a k-block travel as the tail of that k-block's LDS stage.
+template <int GK, bool W4, int WM, int NS>
+__global__ __launch_bounds__(WM * 128, 4) void gemm_k64_f32_kernel(const GemmParams p) {
+    constexpr int WN = 2, TN = 4, TM = 2, NWAVES = WN * WM;
+    constexpr int BN = WN * TN * 16, BM = WM * TM * 16;  // 128 channels x 128 or 256 rows
+    constexpr int KS = 4, KB = W4 ? 2 : 4;  // 32-byte k-steps and 1 KiB weight blocks per panel and stage
+    constexpr int WBLK = (BN / 32) * KB, XBLK = BM / 8;
+    constexpr int WLOADS = WBLK / NWAVES, XLOADS = XBLK / NWAVES;
+    static_assert(WBLK % NWAVES == 0 && XBLK % NWAVES == 0, "blocks must divide over waves");
+    constexpr int GPB = GK == 1 ? 2 : 1;  // scale groups that end in a k-block (GK == 4: every second block)
+    constexpr int SCALE_OFF = (WBLK + XBLK) * 1024;
+    constexpr int STAGE_BYTES = SCALE_OFF + GPB * BN * 4;
+    constexpr int NLOADS = WLOADS + XLOADS;
+    const LinearArgs& a = p.a;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wave_n = wave % WN, wave_m = wave / WN;
+    uint32_t m0, n0;
+    {
+        const TileOrigin t = tile_of_workgroup<BN, BM, 8>(p);
+        if (!t.valid) return;
+        m0 = t.m0;
+        n0 = t.n0;
+    }
+
+    const uint32_t w_lane = lane * 16u;
+    const uint32_t panel_bytes = a.ksteps * 1024u;
+    const int8_t* const w_tile = a.w + (size_t)(n0 / 32u) * panel_bytes;
+    const uint32_t last_chunk = (a.k - 1u) / 16u;
+    const uint32_t my_chunk = (lane & 7) ^ ((lane >> 3) & 7);
+    uint32_t xrow[XLOADS];
+#pragma unroll
+    for (int i = 0; i < XLOADS; i++) {
+        const int b = wave + i * NWAVES;
+        uint32_t row = m0 + b * 8 + (lane >> 3);
+        row = min(row, a.rows - 1u);
+        xrow[i] = row * a.ldx;
+    }
+    const uint32_t ksteps_real = (a.k + 31u) / 32u;
+    const uint32_t nkb = (ksteps_real + KS - 1) / KS;
+    auto issue_block = [&](uint32_t kb, int stage) {
+        char* base = lds_raw + stage * STAGE_BYTES;
+        // the scales of the groups that end in this k-block: 64 channels per wavefront, 4 bytes per lane
+        if (wave < GPB * (BN / 64)) {
+            const uint32_t slot = wave / (BN / 64), half = wave % (BN / 64);
+            const uint32_t g = min(GK == 1 ? kb * 2u + slot : GK == 2 ? kb : kb / 2u, a.groups - 1u);
+            load_to_lds4(a.scales_t + (size_t)g * a.n_pad + n0 + half * 64 + lane,
+                         base + SCALE_OFF + (slot * BN + half * 64) * 4);
+        }
+        static_for<NLOADS>([&](auto t_tag) {
+            constexpr int t = decltype(t_tag)::value;
+            if constexpr (t < WLOADS) {
+                const uint32_t b = wave + t * NWAVES;
+                const int8_t* src = w_tile + (size_t)(b / KB) * panel_bytes + (size_t)(kb * KB + b % KB) * 1024u;
+                load_to_lds16(src + w_lane, base + b * 1024);
+            } else {
+                const uint32_t chunk16 = min(kb * 8u + my_chunk, last_chunk) * 16u;
+                const uint32_t b = wave + (t - WLOADS) * NWAVES;
+                load_to_lds16(a.x + (xrow[t - WLOADS] + chunk16), base + (WBLK + b) * 1024);
+            }
+        });
+    };
+
+    v4i acc[TN][TM];
+    v4f fsum[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++) {
+            acc[i][j] = v4i{0, 0, 0, 0};
+            fsum[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+    float row_scale[TM];
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const uint32_t m = min(m0 + (wave_m * TM + j) * 16 + (lane & 15), a.rows - 1u);
+        row_scale[j] = a.row_scale[m];
+    }
+
+    // fragment addressing (see the requantizing kernel); four-bit weights: one block per MFMA step,
+    // the lane's 16-byte slot is the same for both halves of the step
+    const uint32_t a_frag = W4 ? (uint32_t)(wave_n * (TN / 2) * KB) * 1024u + (uint32_t)((lane & 15) + 32 * ((lane >> 4) & 1)) * 16u
+                               : (uint32_t)(wave_n * (TN / 2) * KB) * 1024u + (uint32_t)(lane >> 5) * 1024u +
+                                     (uint32_t)((lane & 15) + 32 * ((lane >> 4) & 1)) * 16u;
+    const uint32_t nib_shift = lane < 32 ? 4u : 0u;
+    const uint32_t x_row = WBLK * 1024u + ((uint32_t)(wave_m * TM * 16) + (lane & 15)) * 128u;
+    uint32_t x_slot[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) x_slot[s] = (((4u * s + (lane >> 4)) ^ (lane & 7u)) << 4);
+    const uint32_t sw_lane = SCALE_OFF + (uint32_t)(wave_n * TN * 16 + (lane >> 4) * 4) * 4u;
+
+    // fold of scale-group slot `slot` of the stage: every tile of the wave
+    auto fold = [&](const char* stage, int slot) {
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const v4f sw = *reinterpret_cast<const v4f*>(stage + sw_lane + (slot * BN + i * 16) * 4);
+#pragma unroll
+            for (int j = 0; j < TM; j++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float gs = __fmul_rn(row_scale[j], sw[e]);
+                    // four-bit operands carry a factor 16; the dot is exact, so is the shift
+                    const float term = __fmul_rn((float)(acc[i][j][e] >> (W4 ? 4 : 0)), gs);
+                    fsum[i][j][e] = __fadd_rn(fsum[i][j][e], term);
+                }
+            }
+        }
+    };
+
+    // NS stages: k-blocks kb+1 .. kb+NS-1 are in flight while k-block kb is consumed.  One barrier per
+    // k-block, at its top: behind it every wave's loads of the block have landed and every wave is done
+    // with the previous block, whose stage is refilled at once.  (Blocks past the end are clamped to the
+    // last one, so the count of loads in flight is the same in every iteration.)
+    static_for<NS - 1>([&](auto b_tag) { issue_block(min((uint32_t)decltype(b_tag)::value, nkb - 1u), decltype(b_tag)::value); });
+    int cur = 0, refill = NS - 1;
+    for (uint32_t kb = 0; kb < nkb; kb++) {
+        wait_vmcnt<(NS - 2) * NLOADS>();  // (waves that also carry a scale load wait for one load more than they must)
+        wg_barrier();
+        issue_block(min(kb + NS - 1u, nkb - 1u), refill);
+        const char* stage = lds_raw + cur * STAGE_BYTES;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            v4i af[TN], bf[TM];
+#pragma unroll
+            for (int j = 0; j < TM; j++) bf[j] = *reinterpret_cast<const v4i*>(stage + x_row + j * 16 * 128 + x_slot[s]);
+#pragma unroll
+            for (int i = 0; i < TN; i++) {
+                if constexpr (W4) {
+                    const v4i raw = *reinterpret_cast<const v4i*>(stage + a_frag + ((i / 2) * KB + s) * 1024 + (i & 1) * 256);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) af[i][d] = (raw[d] << nib_shift) & (int)0xf0f0f0f0u;
+                } else {
+                    af[i] = *reinterpret_cast<const v4i*>(stage + a_frag + ((i / 2) * KB + 2 * s) * 1024 + (i & 1) * 256);
+                }
+            }
+            // first MFMA step of a scale group: accumulate onto zero instead of clearing registers
+            const bool fresh = GK == 1 || (GK == 2 && s == 0) || (GK == 4 && s == 0 && (kb & 1u) == 0u);
+            const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[i], bf[j], fresh ? zero : acc[i][j], 0, 0, 0);
+            // last MFMA step of a scale group (or of the row): fold it.  A group that starts past the
+            // end of k does not exist (its dot would be zero, but adding +0.0 can flip a -0.0 sum).
+            if constexpr (GK == 1) {
+                if (kb * 2u + s < a.groups) fold(stage, s);
+            } else if constexpr (GK == 2) {
+                if (s == 1) fold(stage, 0);
+            } else {
+                if (s == 1 && ((kb & 1u) == 1u || kb + 1u == nkb)) fold(stage, 0);
+            }
+        }
+        refill = cur;
+        cur = cur + 1 == NS ? 0 : cur + 1;
+    }
+    wait_vmcnt<0>();
+
+    // ---- epilogue: + bias, 16-byte stores (a lane owns row l%16 and four consecutive channels) ----
+    const bool vec_ok = (a.n % 4u) == 0u;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const uint32_t m = m0 + (wave_m * TM + j) * 16 + (lane & 15);
+        if (m >= a.rows) continue;
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const uint32_t n = n0 + (wave_n * TN + i) * 16 + (lane >> 4) * 4;
+            if (n >= a.n) continue;
+            const v4f b = *reinterpret_cast<const v4f*>(a.bias_f32 + n);
+            v4f out;
+#pragma unroll
+            for (int e = 0; e < 4; e++) out[e] = __fadd_rn(fsum[i][j][e], b[e]);
+            float* y = (float*)a.y + (size_t)m * a.n + n;
+            if (vec_ok) {
+                *reinterpret_cast<v4f*>(y) = out;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < a.n) y[e] = out[e];
+            }
+        }
+    }
+}
+
+template <int GK, bool W4, int WM, int NS>
+bool launch_f32(hipStream_t s, const LinearArgs& a) {
+    constexpr int BN = 128, BM = WM * 32;
+    constexpr int LDS = NS * (((BN / 32) * (W4 ? 2 : 4) + BM / 8) * 1024 + (GK == 1 ? 2 : 1) * BN * 4);
+    static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
+    static std::atomic<uint64_t> configured{0};
+    auto kern = gemm_k64_f32_kernel<GK, W4, WM, NS>;
+    if (!raise_lds_limit((const void*)kern, LDS, configured)) return false;
+    GemmParams p;
+    p.a = a;
+    p.tiles_n = (a.n + BN - 1) / BN;
+    p.tiles_m = (a.rows + BM - 1) / BM;
+    const uint32_t total = p.tiles_n * p.tiles_m;
+    const uint32_t grid = ((total + 7u) / 8u) * 8u;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * 128), LDS, s, p);
+    return hipGetLastError() == hipSuccess;
+}
+
 template <int WN, int WM, int TN, int TM, int MODE>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 16, BM = WM * TM * 16;
@@ -337,6 +549,38 @@ const char* launch_gemm_k64(hipStream_t s, const LinearArgs& a, int tile) {
     }
     const bool ok = row ? launch_one<2, 4, 8, 2, R>(s, a) : launch_one<2, 4, 8, 2, T>(s, a);
     return ok ? "t256x128k64" : nullptr;
+}
+
+// The dequantizing GEMM on 16x16x64 MFMAs; group sizes 64, 128 and 256.  deep: one workgroup of
+// sixteen waves per compute unit on a 128 x 256 tile with three LDS stages (eight-bit weights only),
+// else two workgroups of eight waves on 128 x 128 tiles with two stages each.
+const char* launch_gemm_k64_f32(hipStream_t s, const LinearArgs& a, bool deep) {
+    if (a.mode != Epilogue::DequantF32 || a.acc_out || !a.y) return nullptr;
+    bool ok = false;
+    if (a.weight_bits == 4u) {
+        deep = false;
+        switch (a.group_size) {
+            case 64: ok = launch_f32<1, true, 4, 2>(s, a); break;
+            case 128: ok = launch_f32<2, true, 4, 2>(s, a); break;
+            case 256: ok = launch_f32<4, true, 4, 2>(s, a); break;
+            default: return nullptr;
+        }
+    } else if (deep) {
+        switch (a.group_size) {
+            case 64: ok = launch_f32<1, false, 8, 3>(s, a); break;
+            case 128: ok = launch_f32<2, false, 8, 3>(s, a); break;
+            case 256: ok = launch_f32<4, false, 8, 3>(s, a); break;
+            default: return nullptr;
+        }
+    } else {
+        switch (a.group_size) {
+            case 64: ok = launch_f32<1, false, 4, 2>(s, a); break;
+            case 128: ok = launch_f32<2, false, 4, 2>(s, a); break;
+            case 256: ok = launch_f32<4, false, 4, 2>(s, a); break;
+            default: return nullptr;
+        }
+    }
+    return !ok ? nullptr : deep ? "t128x256k64s3" : "t128x128k64";
 }
 
 }  // namespace vxhip

@@ -608,6 +608,13 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         const uint64_t enough = (uint64_t)cu_count * 3 / 4;
         int pick = a.rows <= 64u ? 3 : tiles(128, 256) >= enough && GK > 1 ? 0 : tiles(128, 128) >= enough ? 1
                    : tiles(64, 128) >= enough ? 2 : 3;
+        // Enough 128 x 128 tiles for every compute unit to hold its two workgroups, or most of them: the
+        // 16x16x64 kernel of gemm_k64.hip (group sizes of 64 and more), unless a tile of this file is named.
+        const bool named = forced("t256x") || forced("t128x") || forced("t64x");
+        if (a.group_size >= 64u && (forced("k64") || (!named && tiles(128, 128) >= enough))) {
+            const char* t = launch_gemm_k64_f32(s, a, forced("t128x256k64"));
+            if (t) return t;
+        }
         if (forced("t256x256")) pick = GK > 1 ? 0 : 1;
         if (forced("t128x128")) pick = 1;
         if (forced("t64x128")) pick = 2;

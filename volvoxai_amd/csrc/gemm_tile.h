@@ -72,5 +72,6 @@ __device__ __forceinline__ TileOrigin tile_of_workgroup(const GemmParams& p) {
 
 // gemm_k64.hip
 const char* launch_gemm_k64(hipStream_t s, const LinearArgs& a, int tile);
+const char* launch_gemm_k64_f32(hipStream_t s, const LinearArgs& a, bool deep);
 
 }  // namespace vxhip
