@@ -462,7 +462,11 @@ def main():
             "same_mfma_count_random_operands": ctx.probe_mfma_rate(128, True),
             "same_mfma_count_constant_operands": ctx.probe_mfma_rate(128, False),
             "sustained_random_operands": ctx.probe_mfma_rate(2000, True),
-            "sustained_constant_operands": ctx.probe_mfma_rate(2000, False)}
+            "sustained_constant_operands": ctx.probe_mfma_rate(2000, False),
+            # the instruction the benchmarked tile runs on
+            "k64_same_mfma_count_random_operands": ctx.probe_mfma_rate(128, True, k64=True),
+            "k64_sustained_random_operands": ctx.probe_mfma_rate(2000, True, k64=True),
+            "k64_sustained_constant_operands": ctx.probe_mfma_rate(2000, False, k64=True)}
         # spot parity on the benchmarked output itself
         orc = Oracle()
         ridx, cidx = np.arange(0, M, 257)[:12], np.arange(3, N, 131)[:24]

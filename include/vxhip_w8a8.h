@@ -202,12 +202,14 @@ VxHipStatus vxhip_argmax_rows_f32(VxHipContext* context, const float* input_dev,
 /* Measurement aid with no counterpart in the reference: runs a register-only
  * v_mfma_i32_32x32x32_i8 loop (16 accumulators per wave, one wave per SIMD,
  * `rounds` x 16 MFMAs per wave) and reports the int8 rate it reached, the
- * shader clock it ran at and the launch time.  random_operands != 0 feeds
- * random 8-bit operand bytes instead of constants; the clock the device then
- * sustains is the ceiling of any int8 GEMM on such data.  Synchronises the
- * context's stream. */
+ * shader clock it ran at and the launch time.  flags bit 0 feeds random 8-bit
+ * operand bytes instead of constants; the clock the device then sustains is
+ * the ceiling of any int8 GEMM on such data.  flags bit 1 runs the loop on
+ * v_mfma_i32_16x16x64_i8 instead (64 accumulators of four registers, the same
+ * operations per round), the instruction of the large GEMM tiles.
+ * Synchronises the context's stream. */
 VxHipStatus vxhip_probe_mfma_rate(VxHipContext* context, uint32_t rounds,
-                                  uint32_t random_operands, double* tops,
+                                  uint32_t flags, double* tops,
                                   double* shader_mhz, double* microseconds);
 /* Its HBM counterpart, also without a counterpart in the reference: `launches`
  * launches of a kernel that only reads, each one whole buffer of bytes_each

@@ -739,6 +739,8 @@ def test_ceiling_probes_report_rates(ctx):
     from volvoxai_amd.w8a8 import VxHipError
     m = ctx.probe_mfma_rate(32, True)
     assert 100.0 < m["tops"] < 6000.0 and 300.0 < m["shader_mhz"] < 3500.0
+    m = ctx.probe_mfma_rate(32, True, k64=True)
+    assert 100.0 < m["tops"] < 6000.0 and 300.0 < m["shader_mhz"] < 3500.0
     bufs = [torch.zeros((1 << 20) + 48, dtype=torch.uint8, device="cuda") for _ in range(3)]
     r = ctx.probe_stream_read(bufs, launches=9)
     assert r["bytes"] == (1 << 20) + 48 and r["GBs"] > 1.0 and r["microseconds"] > 0.0

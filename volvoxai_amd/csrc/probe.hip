@@ -1,6 +1,8 @@
 // Hardware-ceiling probe for the MFMA roofline: how fast do the matrix pipes run when they
 // are fed without a single stall?  Every wave keeps 16 independent 32x32 accumulators in
-// registers and issues v_mfma_i32_32x32x32_i8 back to back -- no memory, no LDS, no barrier.
+// registers and issues v_mfma_i32_32x32x32_i8 back to back -- no memory, no LDS, no barrier --
+// or, in the second form, 64 independent 16x16 accumulators and v_mfma_i32_16x16x64_i8 (the same
+// operations per round), which is the instruction the large GEMM tiles run on.
 // With constant operands the device holds its clock; with random 8-bit operands (what a GEMM
 // on uniform +-127 data feeds them) the datapath toggles fully and the power manager lowers
 // the shader clock, which bounds what any int8 GEMM can reach on such data.
@@ -16,9 +18,10 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kAccumulators = 16;
 
+template <bool K64>
 __global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i* __restrict__ operands, uint32_t rounds,
                                                         uint64_t* __restrict__ clocks, int* sink) {
-    v16i acc[kAccumulators];
+    v16i acc[kAccumulators];  // as 64 tiles of four registers in the 16x16x64 form
 #pragma unroll
     for (int i = 0; i < kAccumulators; i++)
 #pragma unroll
@@ -31,9 +34,21 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i* __restrict__ 
     }
     const uint64_t c0 = __builtin_readcyclecounter(), t0 = __builtin_amdgcn_s_memrealtime();
     for (uint32_t it = 0; it < rounds; it++) {
+        if constexpr (K64) {
 #pragma unroll
-        for (int i = 0; i < kAccumulators; i++)
-            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
+            for (int i = 0; i < kAccumulators; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i c = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
+                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i & 3], b[q], c, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[i][4 * q + e] = c[e];
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kAccumulators; i++)
+                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
+        }
     }
     int fold = 0;
 #pragma unroll
@@ -122,8 +137,9 @@ extern "C" VxHipStatus vxhip_probe_stream_read(VxHipContext* ctx, const void* co
     return st;
 }
 
-extern "C" VxHipStatus vxhip_probe_mfma_rate(VxHipContext* ctx, uint32_t rounds, uint32_t random_operands,
+extern "C" VxHipStatus vxhip_probe_mfma_rate(VxHipContext* ctx, uint32_t rounds, uint32_t flags,
                                              double* tops, double* shader_mhz, double* microseconds) {
+    const bool random_operands = (flags & 1u) != 0u, k64 = (flags & 2u) != 0u;
     if (!ctx || !rounds || !tops) {
         set_error("probe_mfma_rate: null context/result or zero rounds");
         return VXHIP_INVALID_ARGUMENT;
@@ -158,10 +174,11 @@ extern "C" VxHipStatus vxhip_probe_mfma_rate(VxHipContext* ctx, uint32_t rounds,
     const int groups = ctx->cu_count > 0 ? ctx->cu_count : 256;
     float ms = 0.0f;
     if (st == VXHIP_OK) {
-        hipLaunchKernelGGL(mfma_rate_kernel, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
+        auto kern = k64 ? mfma_rate_kernel<true> : mfma_rate_kernel<false>;
+        hipLaunchKernelGGL(kern, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
         check(hipStreamSynchronize(ctx->stream), "warm-up launch");
         check(hipEventRecord(e0, ctx->stream), "record");
-        hipLaunchKernelGGL(mfma_rate_kernel, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
+        hipLaunchKernelGGL(kern, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
         check(hipGetLastError(), "launch");
         check(hipEventRecord(e1, ctx->stream), "record");
         check(hipEventSynchronize(e1), "sync");

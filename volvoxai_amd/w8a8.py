@@ -127,10 +127,11 @@ class Context:
     def reserve_scratch(self, nbytes: int):
         _check(library().vxhip_context_reserve_scratch(self._h, int(nbytes)), "vxhip_context_reserve_scratch")
 
-    def probe_mfma_rate(self, rounds=128, random_operands=True) -> dict:
-        """Register-only MFMA loop: the int8 rate, shader clock and time it reached."""
+    def probe_mfma_rate(self, rounds=128, random_operands=True, k64=False) -> dict:
+        """Register-only MFMA loop: the int8 rate, shader clock and time it reached (k64: on the
+        16x16x64 instruction instead of the 32x32x32 one)."""
         tops, mhz, us = C.c_double(0), C.c_double(0), C.c_double(0)
-        _check(library().vxhip_probe_mfma_rate(self._h, int(rounds), 1 if random_operands else 0, C.byref(tops),
+        _check(library().vxhip_probe_mfma_rate(self._h, int(rounds), (1 if random_operands else 0) | (2 if k64 else 0), C.byref(tops),
                                                C.byref(mhz), C.byref(us)), "vxhip_probe_mfma_rate")
         return {"tops": tops.value, "shader_mhz": mhz.value, "microseconds": us.value}
 
