@@ -133,7 +133,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
     // kb+2, every request placed behind a fixed MFMA so that LDS reads, global loads and MFMAs
     // issue evenly mixed.
     constexpr int RB = 2;
-    static_assert(TN > RB + 1, "rows before the barrier");
+    static_assert(TN - RB >= TM && TN >= TM, "every activation fragment needs a row to be re-read behind");
     static_for<NLOADS>([&](auto t) { issue_one(t, 0u, 0); });
 
     float* lds_f0 = reinterpret_cast<float*>(lds_raw + 2 * STAGE_BYTES);
