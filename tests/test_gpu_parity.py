@@ -731,6 +731,33 @@ def test_every_tile_and_stage_variant_on_ragged_shapes(ctx, oracle):
     assert ctx.fault_flags() == 0
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [64, 128, 256])
+def test_uniform_group_scales_take_the_hoisted_fold(ctx, oracle, group, bits):
+    """One scale per channel replicated over the groups (what per-channel quantization exports): the
+    16x16x64 tiles then form s_a * s_w once per output.  Same products, so the oracle's bits, on
+    ragged shapes, special rows included; the general kernels on the same package agree."""
+    import volvoxai_amd as vx
+    for trial, (rows, k, n) in enumerate([(130, 1000, 144), (257, 4608, 72), (300, 384, 300), (65, 4096 + 64, 130)]):
+        c = cases.packed_case(rows, k, n, group, 700 + trial, with_bias=bool(trial % 2), special_rows=True)
+        scales = np.repeat(c["scales"][:, :1], c["scales"].shape[1], axis=1).copy()
+        w = c["w"] if bits == 8 else cases.four_bit(c["w"])
+        words = oracle.pack_w8_words(w) if bits == 8 else oracle.pack_w4_words(w)
+        _, want = oracle.packed_linear(c["x"], words, scales, c["bias"], n, group, bits=bits)
+        pl = vx.PackedLinear(words, scales, c["bias"], k, n, group, weight_bits=bits)
+        xd = dev(c["x"])
+        fam = "a8-mfma" if bits == 8 else "w4a8-mfma"
+        try:
+            for force in (f"{fam}.t128x128k64", f"{fam}.t128x256k64s3", f"{fam}.t128x128", None):
+                vx.force_variant(force)
+                st, y = pl.forward_f32(ctx, xd)
+                ctx.synchronize()
+                assert st == 0 and same_f32(host(y), want), (rows, k, n, group, bits, ctx.last_variant)
+        finally:
+            vx.force_variant(None)
+        pl.close()
+
+
 def test_ceiling_probes_report_rates(ctx):
     """The two measurement aids: a register-only MFMA loop and a read-only kernel.  Rates are
     machine facts, so only their sanity is checked, and that bad arguments are refused."""

@@ -660,9 +660,11 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
     const uint32_t groups = (k + group_size - 1u) / group_size;
     const uint32_t n_pad = ((n + 31u) / 32u + kPanelPad - 1) / kPanelPad * kPanelPad * 32u;
     std::vector<float> st((size_t)groups * n_pad, 1.0f), hb(n_pad, 0.0f);
+    bool uniform_scales = true;
     for (uint32_t o = 0; o < n; o++) {
         for (uint32_t g = 0; g < groups; g++) {
             const float s = scales[(size_t)o * groups + g];
+            if (memcmp(&s, &scales[(size_t)o * groups], sizeof s) != 0) uniform_scales = false;
             if (!isfinite(s)) {
                 set_error("packed_linear_create: scale [%u][%u] is not finite", o, g);
                 return VXHIP_INVALID_ARGUMENT;
@@ -676,6 +678,7 @@ VxHipStatus vxhip_packed_linear_create(const uint32_t* packed_words, const float
     pl->device = device;
     pl->group_size = group_size;
     pl->groups = groups;
+    pl->uniform_scales = uniform_scales;
     uint8_t* raw = nullptr;
     const size_t raw_bytes = (size_t)n * words * 4u;
     auto fail = [&](VxHipStatus s) {
@@ -741,6 +744,7 @@ static int packed_run_a8(VxHipContext* ctx, const VxHipPackedLinear* pl, const i
     a.bias_f32 = pl->bias;
     a.group_size = pl->group_size;
     a.groups = pl->groups;
+    a.uniform_group_scales = pl->uniform_scales;
     a.n_pad = pl->w.panels * 32u;
     a.y = y;
     a.fault = ctx->fault_dev;

@@ -106,6 +106,7 @@ struct VxHipPackedLinear {
     uint32_t group_size = 0, groups = 0;
     float* scales_t = nullptr;  // [groups][n_pad], transposed so 4 channels are contiguous
     float* bias = nullptr;      // [n_pad] (zeros when the node has no bias)
+    bool uniform_scales = false; // every channel's group scales are bit-equal (a per-channel scale replicated over the groups)
     uint64_t resident = 0;
 };
 
@@ -192,6 +193,7 @@ struct LinearArgs {
     const float* scales_t;  // [groups][n_pad]
     const float* bias_f32;  // [n_pad]
     uint32_t group_size, groups, n_pad;
+    bool uniform_group_scales;  // scales_t[g][n] is the same for every g: a kernel may form s_a * s_w once
     // outputs
     void* y;                // int8/uint8 [rows][n] or float [rows][n]; may be null with acc_out
     int32_t* acc_out;       // optional int32 [rows][n]

@@ -132,7 +132,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
     // and from there on reads the next stage's step 0 and refills the current stage for k-block
     // kb+2, every request placed behind a fixed MFMA so that LDS reads, global loads and MFMAs
     // issue evenly mixed.
-    constexpr int RB = 2;
+    constexpr int RB = 1;
     static_assert(TN - RB >= TM && TN >= TM, "every activation fragment needs a row to be re-read behind");
     static_for<NLOADS>([&](auto t) { issue_one(t, 0u, 0); });
 
@@ -314,7 +314,10 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
 // (1, 2 or 4).  W4: four-bit weights; a 1 KiB block then holds the block pair of one MFMA step, low
 // nibbles for its first 32 k, high nibbles for the rest, and a lane shifts its half into place.
 // The scales of the groups that end in a k-block travel as the tail of that k-block's LDS stage.
-template <int GK, bool W4, int WM, int NS>
+// UNI: every channel has one scale for all its groups (a per-channel scale replicated, which is what
+// per-channel quantization exports); s_a * s_w is then formed once per output instead of once per
+// output and group -- the same products, so the same bits -- and the fold is three operations.
+template <int GK, bool W4, int WM, int NS, bool UNI>
 __global__ __launch_bounds__(WM * 128, 4) void gemm_k64_f32_kernel(const GemmParams p) {
     constexpr int WN = 2, TN = 4, TM = 2, NWAVES = WN * WM;
     constexpr int BN = WN * TN * 16, BM = WM * TM * 16;  // 128 channels x 128 or 256 rows
@@ -357,7 +360,7 @@ __global__ __launch_bounds__(WM * 128, 4) void gemm_k64_f32_kernel(const GemmPar
     auto issue_block = [&](uint32_t kb, int stage) {
         char* base = lds_raw + stage * STAGE_BYTES;
         // the scales of the groups that end in this k-block: 64 channels per wavefront, 4 bytes per lane
-        if (wave < GPB * (BN / 64)) {
+        if (!UNI && wave < GPB * (BN / 64)) {
             const uint32_t slot = wave / (BN / 64), half = wave % (BN / 64);
             const uint32_t g = min(GK == 1 ? kb * 2u + slot : GK == 2 ? kb : kb / 2u, a.groups - 1u);
             load_to_lds4(a.scales_t + (size_t)g * a.n_pad + n0 + half * 64 + lane,
@@ -405,16 +408,29 @@ __global__ __launch_bounds__(WM * 128, 4) void gemm_k64_f32_kernel(const GemmPar
     for (int s = 0; s < 2; s++) x_slot[s] = (((4u * s + (lane >> 4)) ^ (lane & 7u)) << 4);
     const uint32_t sw_lane = SCALE_OFF + (uint32_t)(wave_n * TN * 16 + (lane >> 4) * 4) * 4u;
 
+    // UNI: the products s_a * s_w of the lane's outputs
+    float gs_all[UNI ? TN : 1][UNI ? TM : 1][4];
+    if constexpr (UNI) {
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+            const v4f sw = *reinterpret_cast<const v4f*>(a.scales_t + n0 + (wave_n * TN + i) * 16 + (lane >> 4) * 4);
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) gs_all[i][j][e] = __fmul_rn(row_scale[j], sw[e]);
+        }
+    }
     // fold of scale-group slot `slot` of the stage: every tile of the wave
     auto fold = [&](const char* stage, int slot) {
 #pragma unroll
         for (int i = 0; i < TN; i++) {
-            const v4f sw = *reinterpret_cast<const v4f*>(stage + sw_lane + (slot * BN + i * 16) * 4);
+            v4f sw = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (!UNI) sw = *reinterpret_cast<const v4f*>(stage + sw_lane + (slot * BN + i * 16) * 4);
 #pragma unroll
             for (int j = 0; j < TM; j++) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const float gs = __fmul_rn(row_scale[j], sw[e]);
+                    const float gs = UNI ? gs_all[UNI ? i : 0][UNI ? j : 0][e] : __fmul_rn(row_scale[j], sw[e]);
                     // four-bit operands carry a factor 16; the dot is exact, so is the shift
                     const float term = __fmul_rn((float)(acc[i][j][e] >> (W4 ? 4 : 0)), gs);
                     fsum[i][j][e] = __fadd_rn(fsum[i][j][e], term);
@@ -498,13 +514,27 @@ __global__ __launch_bounds__(WM * 128, 4) void gemm_k64_f32_kernel(const GemmPar
     }
 }
 
+template <int GK, bool W4, int WM, int NS, bool UNI>
+bool launch_f32_as(hipStream_t s, const LinearArgs& a);
+
 template <int GK, bool W4, int WM, int NS>
 bool launch_f32(hipStream_t s, const LinearArgs& a) {
+    // (the instances listed keep the products in registers without spilling at four waves per SIMD;
+    // the others would lose more to scratch traffic than the fourth operation costs)
+    constexpr bool kUniformFits = GK == 1 || (GK == 2 && (W4 || WM == 8));
+    if constexpr (kUniformFits) {
+        if (a.uniform_group_scales) return launch_f32_as<GK, W4, WM, NS, true>(s, a);
+    }
+    return launch_f32_as<GK, W4, WM, NS, false>(s, a);
+}
+
+template <int GK, bool W4, int WM, int NS, bool UNI>
+bool launch_f32_as(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = 128, BM = WM * 32;
     constexpr int LDS = NS * (((BN / 32) * (W4 ? 2 : 4) + BM / 8) * 1024 + (GK == 1 ? 2 : 1) * BN * 4);
     static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_k64_f32_kernel<GK, W4, WM, NS>;
+    auto kern = gemm_k64_f32_kernel<GK, W4, WM, NS, UNI>;
     if (!raise_lds_limit((const void*)kern, LDS, configured)) return false;
     GemmParams p;
     p.a = a;

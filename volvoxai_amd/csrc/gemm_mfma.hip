@@ -612,7 +612,11 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         // 16x16x64 kernel of gemm_k64.hip (group sizes of 64 and more), unless a tile of this file is named.
         const bool named = forced("t256x") || forced("t128x") || forced("t64x");
         if (a.group_size >= 64u && (forced("k64") || (!named && tiles(128, 128) >= enough))) {
-            const char* t = launch_gemm_k64_f32(s, a, forced("t128x256k64"));
+            // long rows with one scale per channel: sixteen waves on a 128 x 256 tile, three stages
+            // (K = 14336, N = 4096, 2048 rows: 211 against 232 us; short rows favour the small tile)
+            const bool deep = forced("t128x256k64") || (!forced("k64") && a.uniform_group_scales && a.weight_bits == 8u &&
+                                                        a.group_size <= 128u && a.k >= 4096u && tiles(128, 256) >= enough);
+            const char* t = launch_gemm_k64_f32(s, a, deep);
             if (t) return t;
         }
         if (forced("t256x256")) pick = GK > 1 ? 0 : 1;
