@@ -134,7 +134,9 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
     // issue evenly mixed.
     constexpr int RB = 1;
     static_assert(TN - RB >= TM && TN >= TM, "every activation fragment needs a row to be re-read behind");
+    // both stages are requested at once: the second k-block's latency then runs beside the first's
     static_for<NLOADS>([&](auto t) { issue_one(t, 0u, 0); });
+    static_for<NLOADS>([&](auto t) { issue_one(t, 1u, 1); });
 
     float* lds_f0 = reinterpret_cast<float*>(lds_raw + 2 * STAGE_BYTES);
     int32_t* lds_cb = reinterpret_cast<int32_t*>(lds_f0 + BN);
@@ -160,7 +162,6 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
 
     wait_vmcnt<0>();
     wg_barrier();
-    static_for<NLOADS>([&](auto t) { issue_one(t, 1u, 1); });
     static_for<TM>([&](auto j) { read_b(j, lds_raw, IC<0>{}); });
     static_for<TN>([&](auto i) { read_a(i, lds_raw, IC<0>{}); });
 
