@@ -205,8 +205,9 @@ VxHipStatus vxhip_argmax_rows_f32(VxHipContext* context, const float* input_dev,
  * shader clock it ran at and the launch time.  flags bit 0 feeds random 8-bit
  * operand bytes instead of constants; the clock the device then sustains is
  * the ceiling of any int8 GEMM on such data.  flags bit 1 runs the loop on
- * v_mfma_i32_16x16x64_i8 instead (64 accumulators of four registers, the same
- * operations per round), the instruction of the large GEMM tiles.
+ * v_mfma_i32_16x16x64_i8 instead (two waves per SIMD with 16 accumulators of
+ * four registers each: the same operations per round and SIMD), the
+ * instruction of the large GEMM tiles.
  * Synchronises the context's stream. */
 VxHipStatus vxhip_probe_mfma_rate(VxHipContext* context, uint32_t rounds,
                                   uint32_t flags, double* tops,

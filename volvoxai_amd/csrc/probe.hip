@@ -1,13 +1,15 @@
 // Hardware-ceiling probe for the MFMA roofline: how fast do the matrix pipes run when they
 // are fed without a single stall?  Every wave keeps 16 independent 32x32 accumulators in
 // registers and issues v_mfma_i32_32x32x32_i8 back to back -- no memory, no LDS, no barrier --
-// or, in the second form, 64 independent 16x16 accumulators and v_mfma_i32_16x16x64_i8 (the same
-// operations per round), which is the instruction the large GEMM tiles run on.
+// or, in the second form, two waves per SIMD with 16 independent 16x16 accumulators each and
+// v_mfma_i32_16x16x64_i8 (the same operations per round and SIMD), which is the instruction and the
+// occupancy of the large GEMM tiles.
 // With constant operands the device holds its clock; with random 8-bit operands (what a GEMM
 // on uniform +-127 data feeds them) the datapath toggles fully and the power manager lowers
 // the shader clock, which bounds what any int8 GEMM can reach on such data.
 #include "common.h"
 
+#include <type_traits>
 #include <vector>
 
 namespace vxhip {
@@ -19,42 +21,38 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kAccumulators = 16;
 
 template <bool K64>
-__global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i* __restrict__ operands, uint32_t rounds,
+__global__ __launch_bounds__(K64 ? 512 : 256) void mfma_rate_kernel(const v4i* __restrict__ operands, uint32_t rounds,
                                                         uint64_t* __restrict__ clocks, int* sink) {
-    v16i acc[kAccumulators];  // as 64 tiles of four registers in the 16x16x64 form
+    // 16 tiles per wave either way; the 16x16x64 form runs two waves per SIMD (as the GEMM does), so
+    // a round is the same number of operations per SIMD in both forms
+    constexpr int kTiles = kAccumulators;
+    using Tile = typename std::conditional<K64, v4i, v16i>::type;
+    Tile acc[kTiles];
 #pragma unroll
-    for (int i = 0; i < kAccumulators; i++)
+    for (int i = 0; i < kTiles; i++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+        for (int r = 0; r < (K64 ? 4 : 16); r++) acc[i][r] = 0;
     v4i a[4], b[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        a[i] = operands[i * 256 + threadIdx.x];
-        b[i] = operands[(i + 4) * 256 + threadIdx.x];
+        a[i] = operands[i * 256 + (threadIdx.x & 255u)];
+        b[i] = operands[(i + 4) * 256 + (threadIdx.x & 255u)];
     }
     const uint64_t c0 = __builtin_readcyclecounter(), t0 = __builtin_amdgcn_s_memrealtime();
     for (uint32_t it = 0; it < rounds; it++) {
-        if constexpr (K64) {
 #pragma unroll
-            for (int i = 0; i < kAccumulators; i++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    v4i c = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
-                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i & 3], b[q], c, 0, 0, 0);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) acc[i][4 * q + e] = c[e];
-                }
-        } else {
-#pragma unroll
-            for (int i = 0; i < kAccumulators; i++)
+        for (int i = 0; i < kTiles; i++) {
+            if constexpr (K64)
+                acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[(i >> 2) & 3], b[i & 3], acc[i], 0, 0, 0);
+            else
                 acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
         }
     }
     int fold = 0;
 #pragma unroll
-    for (int i = 0; i < kAccumulators; i++)
+    for (int i = 0; i < kTiles; i++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) fold ^= acc[i][r];
+        for (int r = 0; r < (K64 ? 4 : 16); r++) fold ^= acc[i][r];
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         clocks[0] = __builtin_readcyclecounter() - c0;       // shader cycles
         clocks[1] = __builtin_amdgcn_s_memrealtime() - t0;   // 100 MHz ticks
@@ -170,15 +168,16 @@ extern "C" VxHipStatus vxhip_probe_mfma_rate(VxHipContext* ctx, uint32_t rounds,
         check(hipMemcpyAsync(operands, host.data(), host.size() * 4, hipMemcpyHostToDevice, ctx->stream), "copy");
         check(hipStreamSynchronize(ctx->stream), "sync");
     }
-    // one workgroup of four waves per compute unit: one wave on every SIMD
+    // one workgroup per compute unit: one wave on every SIMD (two in the 16x16x64 form)
     const int groups = ctx->cu_count > 0 ? ctx->cu_count : 256;
     float ms = 0.0f;
     if (st == VXHIP_OK) {
         auto kern = k64 ? mfma_rate_kernel<true> : mfma_rate_kernel<false>;
-        hipLaunchKernelGGL(kern, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
+        const int threads = k64 ? 512 : 256;
+        hipLaunchKernelGGL(kern, dim3(groups), dim3(threads), 0, ctx->stream, operands, rounds, clocks, sink);
         check(hipStreamSynchronize(ctx->stream), "warm-up launch");
         check(hipEventRecord(e0, ctx->stream), "record");
-        hipLaunchKernelGGL(kern, dim3(groups), dim3(256), 0, ctx->stream, operands, rounds, clocks, sink);
+        hipLaunchKernelGGL(kern, dim3(groups), dim3(threads), 0, ctx->stream, operands, rounds, clocks, sink);
         check(hipGetLastError(), "launch");
         check(hipEventRecord(e1, ctx->stream), "record");
         check(hipEventSynchronize(e1), "sync");
