@@ -14,31 +14,32 @@ constexpr int kQuantizeLinear = 0, kDequantizeLinear = 0;  // boundary ops carry
     {id, 0, kQMatMul, entry, pred, feat, prio}
 
 const VxHipKernelVariant kVariants[] = {
-    QROWS("hip.qlinear.mfma-i8", "gemm_mfma_kernel<RequantTensor>",
+    // (tile suffixes ending in k64 are gemm_k64_kernel, the 16x16x64 form of the large tiles)
+    QROWS("hip.qlinear.mfma-i8", "gemm_mfma_kernel<RequantTensor>|gemm_k64_kernel<RequantTensor>",
           "hip.qlinear.canonical-resident-int32-bound-rows-gt32-any-k-tail",
-          "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300),
-    QROWS("hip.qlinear.mfma-i8-rowscale", "gemm_mfma_kernel<RequantRow>",
+          "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300),
+    QROWS("hip.qlinear.mfma-i8-rowscale", "gemm_mfma_kernel<RequantRow>|gemm_k64_kernel<RequantRow>",
           "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-gt32",
-          "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300),
+          "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300),
     QROWS("hip.qlinear.gemv-mfma", "gemv_panel_kernel<RequantTensor>",
           "hip.qlinear.canonical-resident-int32-bound-rows-le32",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400),
     QROWS("hip.qlinear.gemv-mfma-rowscale", "gemv_panel_kernel<RequantRow>",
           "hip.qlinear.per-row-input-scale-i8-zero-input-zp-int32-bound-rows-le32",
           "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400),
-    {"hip.packed-linear.a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32>",
+    {"hip.packed-linear.a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32>|gemm_k64_f32_kernel",
      "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-gt32",
-     "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300},
+     "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300},
     {"hip.packed-linear.a8-gemv-mfma", 0, kPackedLinear, "gemv_panel_kernel<DequantF32>",
      "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-le32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400},
-    {"hip.packed-linear.w4a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32, W4>",
+    {"hip.packed-linear.w4a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32, W4>|gemm_k64_f32_kernel<W4>",
      "hip.packed-linear.w4-dynamic-i8-g32-64-128-256-rows-gt32",
-     "hip.gfx950-mfma-i32-32x32x32-i8,hip.global-load-lds-b128", 300},
+     "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300},
     {"hip.packed-linear.w4a8-gemv-mfma", 0, kPackedLinear, "gemv_panel_kernel<DequantF32, W4>",
      "hip.packed-linear.w4-dynamic-i8-g32-64-128-256-rows-le32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400},
-    {"hip.packed-linear.prepare-i8", 0, kPackedLinear, "prepare_i8_kernel",
+    {"hip.packed-linear.prepare-i8", 0, kPackedLinear, "prepare_i8_kernel|prepare_i8_rows_kernel",
      "hip.packed-linear.dynamic-i8-row-absmax", "", 100},
 };
 }  // namespace
