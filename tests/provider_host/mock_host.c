@@ -498,3 +498,216 @@ done:
     if (runtime) g_provider.runtime_destroy(runtime);
     return run->status = status;
 }
+
+/* Row decode through the decode callbacks (native/include/volvoxai_backend.h:214-232), the way the
+ * reference's Generate loop drives a provider context created with decode rows enabled
+ * (native/src/runtime/public_api_execute_result.inc:563-576): one prefill at the last prompt
+ * position, then one step per new token, the host feeding each step's ids back into the id rows.
+ * Also holds the provider to the state rules: a step that is not at the next position is refused
+ * and changes nothing; after a reset the same prefill gives the same ids. */
+typedef struct MockDecode {
+    /* in */
+    const char* graph_path;
+    const char* weight_path;
+    const char* input_name;
+    const char* ids_name;
+    const char* logits_name; /* NULL: the graph declares the ids only */
+    int32_t slots, capacity, vocab, prompt_len, steps;
+    int32_t* token_ids;   /* [slots, capacity]: the prompt, generated ids are written behind it */
+    int32_t* generated;   /* out [steps + 1, slots] */
+    float* first_logits;  /* out [slots, vocab] when logits_name is set */
+    /* out */
+    int32_t status, failed_stage, writes, sink_mismatch;
+    int32_t wrong_step_refused, reset_repeats, attested;
+    char message[VX_REPORT_MESSAGE_CAPACITY];
+    char compile_route[VX_REPORT_ROUTE_CAPACITY];
+    char execute_route[VX_REPORT_ROUTE_CAPACITY];
+} MockDecode;
+
+typedef struct DecodeSink {
+    MockDecode* run;
+    int32_t* ids;
+    float* logits;
+    int32_t ids_written, logits_written;
+} DecodeSink;
+
+static VxStatus decode_write(void* user, const char* name, VxDataType dtype, const int64_t* shape, uint32_t rank,
+                             const void* data, size_t bytes) {
+    DecodeSink* sink = (DecodeSink*)user;
+    MockDecode* run = sink->run;
+    run->writes++;
+    if (name && !strcmp(name, run->ids_name) && dtype == VX_DTYPE_I32 && rank == 1 && shape[0] == run->slots && data &&
+        bytes == (size_t)run->slots * 4u && !sink->ids_written) {
+        memcpy(sink->ids, data, bytes);
+        sink->ids_written = 1;
+        return VX_STATUS_OK;
+    }
+    if (name && run->logits_name && !strcmp(name, run->logits_name) && dtype == VX_DTYPE_F32 && rank == 2 &&
+        shape[0] == run->slots && shape[1] == run->vocab && data && bytes == (size_t)run->slots * run->vocab * 4u &&
+        !sink->logits_written) {
+        if (sink->logits) memcpy(sink->logits, data, bytes);
+        sink->logits_written = 1;
+        return VX_STATUS_OK;
+    }
+    run->sink_mismatch = 1;
+    return VX_STATUS_INVALID_ARGUMENT;
+}
+
+static void fixed_spec(VxTensorSpec* spec, const char* name, VxDataType dtype, uint32_t rank, int64_t d0, int64_t d1) {
+    memset(spec, 0, sizeof(*spec));
+    spec->struct_size = sizeof(*spec);
+    spec->name = name;
+    spec->dtype = dtype;
+    spec->rank = rank;
+    spec->location = VX_MEMORY_HOST;
+    for (uint32_t a = 0; a < rank; a++) {
+        VxDimensionConstraint* d = &spec->dimensions[a];
+        d->struct_size = sizeof(*d);
+        d->kind = VX_DIMENSION_FIXED;
+        d->multiple_of = 1;
+        d->min = d->max = a ? d1 : d0;
+    }
+}
+
+int32_t mock_host_run_decode(MockDecode* run) {
+    static const char fingerprint[] = "sha256:mock-graph-fingerprint";
+    static const char proof[] = "sha256:mock-shape-domain-proof";
+    VxRuntimeOptions runtime_options = VX_RUNTIME_OPTIONS_INIT;
+    VxContextOptions context_options = VX_CONTEXT_OPTIONS_INIT;
+    VxReport report = VX_REPORT_INIT;
+    VxModelSource source = VX_MODEL_SOURCE_INIT;
+    VxBackendCompileInput input = VX_BACKEND_COMPILE_INPUT_INIT;
+    VxBackendShapeDomainAttestation attestation = VX_BACKEND_SHAPE_DOMAIN_ATTESTATION_INIT;
+    VxBackendPolicy policy = VX_BACKEND_POLICY_INIT;
+    VxTensorSpec in_spec, out_specs[2];
+    VxTensorBinding binding = VX_TENSOR_BINDING_INIT;
+    DecodeSink state = {run, NULL, NULL, 0, 0};
+    VxBackendOutputSink sink = {sizeof(VxBackendOutputSink), &state, decode_write};
+    const char* weights[1];
+    const char* wanted[1];
+    const char* decode_inputs[1];
+    void *runtime = NULL, *compiled = NULL, *context = NULL;
+    int32_t* again = NULL;
+    const int32_t expected_writes = run->logits_name ? 2 : 1;
+    VxStatus status;
+    if (!g_registered) return run->status = VX_STATUS_NOT_FOUND;
+    if (!g_provider.context_decode_prefill || !g_provider.context_decode_step || !g_provider.context_decode_reset)
+        return run->status = VX_STATUS_BACKEND_UNSUPPORTED;
+    run->writes = run->sink_mismatch = run->wrong_step_refused = run->reset_repeats = run->attested = 0;
+    status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
+    run->failed_stage = VX_STAGE_RUNTIME_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+    weights[0] = run->weight_path;
+    source.graph_path = run->graph_path;
+    source.weight_paths = weights;
+    source.weight_path_count = 1;
+    fixed_spec(&in_spec, run->input_name, VX_DTYPE_I32, 2, run->slots, run->capacity);
+    fixed_spec(&out_specs[0], run->ids_name, VX_DTYPE_I32, 1, run->slots, 0);
+    if (run->logits_name) fixed_spec(&out_specs[1], run->logits_name, VX_DTYPE_F32, 2, run->slots, run->vocab);
+    input.source = &source;
+    input.graph_fingerprint = fingerprint;
+    input.shape_domain_proof_identity = proof;
+    input.inputs = &in_spec;
+    input.input_count = 1;
+    input.outputs = out_specs;
+    input.output_count = (size_t)expected_writes;
+    input.packed_arithmetic = VX_PACKED_ARITHMETIC_DYNAMIC_I8;
+    wanted[0] = g_name;
+    policy.mode = VX_BACKEND_REQUIRE;
+    policy.operator_fallback = VX_OPERATOR_FALLBACK_FORBID;
+    policy.backends = wanted;
+    policy.backend_count = 1;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.compile(runtime, &input, &policy, &compiled, &attestation, &report);
+    run->failed_stage = VX_STAGE_COMPILE;
+    if (status != VX_STATUS_OK) {
+        if (compiled) status = VX_STATUS_INTERNAL;
+        goto done;
+    }
+    snprintf(run->compile_route, sizeof(run->compile_route), "%s", report.route_evidence);
+    run->attested = report.route_attested && !report.operator_fallback_used && attestation.graph_fingerprint &&
+                    !strcmp(attestation.graph_fingerprint, fingerprint) &&
+                    attestation.packed_arithmetic == VX_PACKED_ARITHMETIC_DYNAMIC_I8;
+
+    decode_inputs[0] = run->input_name;
+    context_options.decode_row_mode = VX_DECODE_ROW_REQUIRED;
+    context_options.require_incremental = 1;
+    context_options.decode_slots = (uint32_t)run->slots;
+    context_options.decode_inputs = decode_inputs;
+    context_options.decode_input_count = 1;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_create(compiled, &context_options, &context, &report);
+    run->failed_stage = VX_STAGE_CONTEXT_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+
+    binding.name = run->input_name;
+    binding.dtype = VX_DTYPE_I32;
+    binding.rank = 2;
+    binding.shape[0] = run->slots;
+    binding.shape[1] = run->capacity;
+    binding.data = run->token_ids;
+    binding.byte_size = (size_t)run->slots * run->capacity * 4u;
+    binding.location = VX_MEMORY_HOST;
+    run->failed_stage = VX_STAGE_EXECUTE;
+
+    /* prefill: rows 0 .. prompt_len-1 */
+    state.ids = run->generated;
+    state.logits = run->first_logits;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_decode_prefill(context, run->prompt_len - 1, &binding, 1, &sink, &report);
+    if (status == VX_STATUS_OK && (run->writes != expected_writes || run->sink_mismatch)) status = VX_STATUS_EXECUTION_FAILED;
+    if (status != VX_STATUS_OK) goto done;
+    run->attested = run->attested && report.route_attested && report.route_evidence[0];
+    snprintf(run->execute_route, sizeof(run->execute_route), "%s", report.route_evidence);
+    /* a step that skips a position is refused and leaves the state alone */
+    {
+        DecodeSink scratch_state = {run, (int32_t*)calloc((size_t)run->slots, 4u), NULL, 0, 0};
+        VxBackendOutputSink scratch = {sizeof(VxBackendOutputSink), &scratch_state, decode_write};
+        const int32_t before = run->writes;
+        VxReport r2 = VX_REPORT_INIT;
+        VxStatus refused = g_provider.context_decode_step(context, run->prompt_len + 1, &binding, 1, &scratch, &r2);
+        run->wrong_step_refused = refused == VX_STATUS_INVALID_ARGUMENT && run->writes == before;
+        free(scratch_state.ids);
+    }
+    for (int32_t i = 1; i <= run->steps && status == VX_STATUS_OK; i++) {
+        const int32_t position = run->prompt_len + i - 1; /* the column of the token generated last */
+        const int32_t before = run->writes;
+        if (position >= run->capacity) {
+            status = VX_STATUS_INVALID_ARGUMENT;
+            break;
+        }
+        for (int32_t r = 0; r < run->slots; r++)
+            run->token_ids[(size_t)r * run->capacity + position] = run->generated[(size_t)(i - 1) * run->slots + r];
+        state.ids = run->generated + (size_t)i * run->slots;
+        state.logits = NULL;
+        state.ids_written = state.logits_written = 0;
+        report = (VxReport)VX_REPORT_INIT;
+        status = g_provider.context_decode_step(context, position, &binding, 1, &sink, &report);
+        if (status == VX_STATUS_OK && (run->writes != before + expected_writes || run->sink_mismatch))
+            status = VX_STATUS_EXECUTION_FAILED;
+    }
+    if (status != VX_STATUS_OK) goto done;
+    /* reset, then the same prefill again: the same first ids */
+    again = (int32_t*)calloc((size_t)run->slots, 4u);
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_decode_reset(context, &report);
+    if (status == VX_STATUS_OK) {
+        state.ids = again;
+        state.logits = NULL;
+        state.ids_written = state.logits_written = 0;
+        report = (VxReport)VX_REPORT_INIT;
+        status = g_provider.context_decode_prefill(context, run->prompt_len - 1, &binding, 1, &sink, &report);
+        run->reset_repeats = status == VX_STATUS_OK && !memcmp(again, run->generated, (size_t)run->slots * 4u);
+    }
+    if (status == VX_STATUS_OK) run->failed_stage = VX_STAGE_NONE;
+done:
+    snprintf(run->message, sizeof(run->message), "%s", report.message);
+    free(again);
+    if (context) {
+        if (g_provider.context_close) (void)g_provider.context_close(context, &report);
+        g_provider.context_destroy(context);
+    }
+    if (compiled) g_provider.compiled_destroy(compiled);
+    if (runtime) g_provider.runtime_destroy(runtime);
+    return run->status = status;
+}

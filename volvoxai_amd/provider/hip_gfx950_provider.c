@@ -106,8 +106,12 @@ typedef struct HipStage {
     int32_t input_zero_point, output_zero_point;
 } HipStage;
 
+struct DecoderModel;
+struct DecoderState;
+
 typedef struct HipCompiled {
     HipRuntime* runtime;
+    struct DecoderModel* decoder; /* set for a decoder graph (decoder_route.inc); stages are then unused */
     HipStage* stages;
     size_t stage_count;
     uint64_t widest_row_bytes; /* of any tensor of the chain, graph input and output included */
@@ -131,6 +135,7 @@ typedef struct HipCompiled {
 typedef struct HipContext {
     HipCompiled* compiled;
     VxHipContext* ctx;
+    struct DecoderState* decode; /* decoder graphs: the cache and work buffers of this context */
     void* work_dev[2]; /* a node reads one and writes the other */
     void* output_host;
     size_t work_capacity[2], host_capacity;
@@ -645,6 +650,8 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
     return status;
 }
 
+#include "decoder_route.inc"
+
 /* ---- SPI callbacks ---------------------------------------------------------------- */
 
 static VxStatus hip_runtime_create(void* user_data, const VxRuntimeOptions* options, void** out_runtime,
@@ -684,6 +691,7 @@ static int policy_names(const VxBackendPolicy* policy, const char* name) {
 static void hip_compiled_destroy(void* compiled_instance) {
     HipCompiled* compiled = (HipCompiled*)compiled_instance;
     if (!compiled) return;
+    decoder_model_release(compiled->decoder);
     for (size_t i = 0; i < compiled->stage_count; i++) {
         if (compiled->stages[i].qlinear) vxhip_qlinear_destroy(compiled->stages[i].qlinear);
         if (compiled->stages[i].packed) vxhip_packed_linear_destroy(compiled->stages[i].packed);
@@ -733,6 +741,75 @@ static int specs_match(const VxBackendCompileInput* input, const ChainPlan* plan
     return 1;
 }
 
+/* A graph whose first node is an Embedding is a decoder graph: read it, open the weight files and
+ * compile the decoder route.  *is_decoder = 0 leaves everything to the chain reader. */
+static VxStatus try_decoder(const VxModelSource* source, VxPackedArithmetic arithmetic, int32_t device, int* is_decoder,
+                            DecoderModel** out, Failure* failure) {
+    size_t length = 0, opened = 0;
+    const char* json_error = NULL;
+    char* text = read_text_file(source->graph_path, &length);
+    VxjValue* root;
+    VxstFile** files;
+    VxStatus status = VX_STATUS_OK;
+    *is_decoder = 0;
+    *out = NULL;
+    if (!text) return VX_STATUS_OK; /* the chain reader reports what is wrong with the document */
+    root = vxj_parse(text, length, &json_error);
+    free(text);
+    if (!root) return VX_STATUS_OK;
+    if (!graph_is_decoder(root)) {
+        vxj_free(root);
+        return VX_STATUS_OK;
+    }
+    *is_decoder = 1;
+    files = (VxstFile**)calloc(source->weight_path_count ? source->weight_path_count : 1, sizeof(VxstFile*));
+    if (!files) status = refuse(failure, VX_STATUS_OUT_OF_MEMORY, "out of memory%s", "");
+    {
+        const char* format = vxj_member_string(root, "format");
+        if (status == VX_STATUS_OK && (!format || strcmp(format, "volvox-graph/v1")))
+            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph format is not volvox-graph/v1%s", "");
+    }
+    for (size_t i = 0; i < source->weight_path_count && status == VX_STATUS_OK; i++) {
+        char error[VX_REPORT_MESSAGE_CAPACITY];
+        if (vxst_open(source->weight_paths[i], &files[opened], error, sizeof(error)) != 0)
+            status = refuse(failure, VX_STATUS_IO_ERROR, "%s", error);
+        else
+            opened++;
+    }
+    if (status == VX_STATUS_OK) status = decoder_compile(root, files, opened, device, arithmetic, out, failure);
+    for (size_t i = 0; i < opened; i++) vxst_close(files[i]);
+    free(files);
+    vxj_free(root);
+    return status;
+}
+
+/* The logical specifications of a decoder graph: the id rows in, ids and/or logits out. */
+static int decoder_specs_match(const VxBackendCompileInput* input, const DecoderModel* m) {
+    const size_t want_outputs = (size_t)(m->publish_ids + m->publish_logits);
+    const VxTensorSpec* in;
+    if (input->input_count != 1 || input->output_count != want_outputs || !input->inputs || !input->outputs) return 0;
+    in = &input->inputs[0];
+    if (in->struct_size != sizeof(*in) || !in->name || strcmp(in->name, m->input_name) || in->dtype != VX_DTYPE_I32 ||
+        in->rank != 2 || in->location != VX_MEMORY_HOST || in->dimensions[0].kind != VX_DIMENSION_FIXED ||
+        in->dimensions[0].min != (int64_t)m->slots || in->dimensions[1].kind != VX_DIMENSION_FIXED ||
+        in->dimensions[1].min != (int64_t)m->capacity)
+        return 0;
+    for (size_t i = 0; i < input->output_count; i++) {
+        const VxTensorSpec* o = &input->outputs[i];
+        if (o->struct_size != sizeof(*o) || !o->name || o->location != VX_MEMORY_HOST) return 0;
+        if (m->publish_ids && !strcmp(o->name, m->ids_name)) {
+            if (o->dtype != VX_DTYPE_I32 || o->rank != 1 || o->dimensions[0].min != (int64_t)m->slots) return 0;
+        } else if (m->publish_logits && !strcmp(o->name, m->logits_name)) {
+            if (o->dtype != VX_DTYPE_F32 || o->rank != 2 || o->dimensions[0].min != (int64_t)m->slots ||
+                o->dimensions[1].min != (int64_t)m->vocab)
+                return 0;
+        } else {
+            return 0;
+        }
+    }
+    return 1;
+}
+
 static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput* input, const VxBackendPolicy* policy,
                             void** out_compiled, VxBackendShapeDomainAttestation* attestation, VxReport* report) {
     HipRuntime* runtime = (HipRuntime*)runtime_instance;
@@ -754,6 +831,54 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
                     "DYNAMIC_I4 packed arithmetic is not offered");
         return VX_STATUS_BACKEND_UNSUPPORTED;
+    }
+    {
+        /* decoder graphs take their own route (decoder_route.inc) */
+        int is_decoder = 0;
+        DecoderModel* decoder = NULL;
+        status = try_decoder(input->source, input->packed_arithmetic, runtime->device, &is_decoder, &decoder, &failure);
+        if (is_decoder) {
+            char route[64];
+            if (status != VX_STATUS_OK) {
+                fill_report(report, runtime, status, VX_STAGE_COMPILE, code_for(status), failure.message);
+                return status;
+            }
+            if (!decoder_specs_match(input, decoder)) {
+                decoder_model_release(decoder);
+                fill_report(report, runtime, VX_STATUS_INVALID_ARGUMENT, VX_STAGE_COMPILE, VX_CODE_INVALID_ARGUMENT,
+                            "logical tensor specifications do not describe the decoder's ids and outputs");
+                return VX_STATUS_INVALID_ARGUMENT;
+            }
+            compiled = (HipCompiled*)calloc(1, sizeof(*compiled));
+            if (!compiled) {
+                decoder_model_release(decoder);
+                return VX_STATUS_OUT_OF_MEMORY;
+            }
+            compiled->runtime = runtime;
+            compiled->decoder = decoder;
+            snprintf(compiled->route, sizeof(compiled->route), "hip.decoder.w8a8-packed-linear.layers%u", decoder->layers);
+            attestation->graph_fingerprint = input->graph_fingerprint;
+            attestation->shape_domain_proof_identity = input->shape_domain_proof_identity;
+            {
+                const uint64_t rows = (uint64_t)decoder->slots * decoder->capacity;
+                const uint64_t kv = (uint64_t)decoder->kv_heads * decoder->head_dim, q = (uint64_t)decoder->q_heads * decoder->head_dim;
+                const uint64_t widest = 2u * (uint64_t)decoder->inter > q + 2u * kv ? 2u * (uint64_t)decoder->inter : q + 2u * kv;
+                const uint64_t logits = (uint64_t)decoder->slots * decoder->vocab * 4u;
+                attestation->maximum_tensor_bytes = rows * widest * 4u > logits ? rows * widest * 4u : logits;
+                /* weights; per context the two caches and the work buffers of one full-length call */
+                attestation->maximum_resident_bytes =
+                    decoder->resident_bytes + 2u * (uint64_t)decoder->layers * rows * kv * 4u +
+                    rows * (4u * (uint64_t)decoder->hidden + 3u * q + 2u * kv + 2u * (uint64_t)decoder->inter + 4u) * 4u + 2u * logits;
+            }
+            attestation->resource_limit_bytes = 0;
+            attestation->has_resource_limit = 0;
+            attestation->packed_arithmetic = VX_PACKED_ARITHMETIC_DYNAMIC_I8;
+            *out_compiled = compiled;
+            fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE, "W8A8 decoder compiled");
+            snprintf(route, sizeof(route), "%s", compiled->route);
+            attest(report, decoder->node_count, route);
+            return VX_STATUS_OK;
+        }
     }
     if (input->input_count != 1 || input->output_count != 1 || !input->inputs || !input->outputs) {
         fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
@@ -871,6 +996,7 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
 static void hip_context_destroy(void* context_instance) {
     HipContext* context = (HipContext*)context_instance;
     if (!context) return;
+    decoder_state_release(context->decode);
     if (context->work_dev[0]) vxhip_device_free(context->work_dev[0]);
     if (context->work_dev[1]) vxhip_device_free(context->work_dev[1]);
     free(context->output_host);
@@ -886,7 +1012,10 @@ static VxStatus hip_context_create(void* compiled_instance, const VxContextOptio
     if (!out_context) return VX_STATUS_INVALID_ARGUMENT;
     *out_context = NULL;
     if (!compiled || !options || options->struct_size != sizeof(*options)) return VX_STATUS_INVALID_ARGUMENT;
-    if (options->decode_row_mode != VX_DECODE_ROW_DISABLED) return VX_STATUS_BACKEND_UNSUPPORTED;
+    /* row decode is what a decoder graph offers; a chain of linears has no rows to keep */
+    if (options->decode_row_mode != VX_DECODE_ROW_DISABLED &&
+        (!compiled->decoder || (options->decode_slots > 1u && options->decode_slots != compiled->decoder->slots)))
+        return VX_STATUS_BACKEND_UNSUPPORTED;
     context = (HipContext*)calloc(1, sizeof(*context));
     if (!context) return VX_STATUS_OUT_OF_MEMORY;
     context->compiled = compiled;
@@ -896,6 +1025,15 @@ static VxStatus hip_context_create(void* compiled_instance, const VxContextOptio
                     vxhip_last_error());
         hip_context_destroy(context);
         return status;
+    }
+    if (compiled->decoder) {
+        status = decoder_state_create(compiled->decoder, context->ctx, &context->decode);
+        if (status != VX_STATUS_OK) {
+            fill_report(report, compiled->runtime, status, VX_STAGE_CONTEXT_CREATE, VX_CODE_BACKEND_CONTEXT_CREATE_FAILED,
+                        status == VX_STATUS_OUT_OF_MEMORY ? "the decoder's cache and work buffers do not fit" : vxhip_last_error());
+            hip_context_destroy(context);
+            return status;
+        }
     }
     *out_context = context;
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_CONTEXT_CREATE, VX_CODE_NONE, "context created");
@@ -994,6 +1132,89 @@ static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, 
     return status;
 }
 
+/* ---- decoder graphs: execute and the decode callbacks ------------------------------------- */
+
+/* The one binding of a decoder graph: the id rows [slots, capacity]. */
+static const int32_t* decoder_ids(const DecoderModel* m, const VxTensorBinding* inputs, size_t input_count) {
+    const VxTensorBinding* b = inputs;
+    if (!inputs || input_count != 1 || b->struct_size != sizeof(*b) || !b->name || strcmp(b->name, m->input_name) ||
+        b->dtype != VX_DTYPE_I32 || b->rank != 2 || b->location != VX_MEMORY_HOST || !b->data ||
+        b->shape[0] != (int64_t)m->slots || b->shape[1] != (int64_t)m->capacity ||
+        b->byte_size != (size_t)m->slots * m->capacity * 4u)
+        return NULL;
+    return (const int32_t*)b->data;
+}
+
+static VxStatus decoder_publish(HipContext* context, const VxBackendOutputSink* sink, VxReport* report, const char* what) {
+    const DecoderModel* m = context->compiled->decoder;
+    const DecoderState* s = context->decode;
+    VxStatus status = VX_STATUS_OK;
+    if (m->publish_ids) {
+        const int64_t shape[1] = {(int64_t)m->slots};
+        status = sink->write(sink->user_data, m->ids_name, VX_DTYPE_I32, shape, 1, s->ids_host, (size_t)m->slots * 4u);
+    }
+    if (status == VX_STATUS_OK && m->publish_logits) {
+        const int64_t shape[2] = {(int64_t)m->slots, (int64_t)m->vocab};
+        status = sink->write(sink->user_data, m->logits_name, VX_DTYPE_F32, shape, 2, s->logits_host,
+                             (size_t)m->slots * m->vocab * 4u);
+    }
+    if (status != VX_STATUS_OK) return status;
+    fill_report(report, context->compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, what);
+    attest(report, m->node_count, vxhip_context_last_variant(context->ctx));
+    return VX_STATUS_OK;
+}
+
+/* Rows first..last through the decoder, then the outputs of row `last`; on success the cache holds
+ * rows 0..last.  Everything is validated before the device is touched. */
+static VxStatus decoder_rows(HipContext* context, const VxTensorBinding* inputs, size_t input_count, int64_t first,
+                             int64_t last, const VxBackendOutputSink* sink, VxReport* report, const char* what) {
+    const DecoderModel* m;
+    const int32_t* ids;
+    VxStatus status;
+    if (!context || context->closed || !context->compiled->decoder || !context->decode || !sink ||
+        sink->struct_size != sizeof(*sink) || !sink->write)
+        return VX_STATUS_INVALID_ARGUMENT;
+    m = context->compiled->decoder;
+    ids = decoder_ids(m, inputs, input_count);
+    if (!ids || first < 0 || last < first || last >= (int64_t)m->capacity) return VX_STATUS_INVALID_ARGUMENT;
+    status = decoder_run(m, context->decode, context->ctx, ids, (uint32_t)first, (uint32_t)last);
+    if (status != VX_STATUS_OK) {
+        context->decode->filled = 0; /* the cache may hold part of the failed call */
+        fill_report(report, context->compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status),
+                    status == VX_STATUS_INVALID_ARGUMENT ? "a token id lies outside the embedding table" : vxhip_last_error());
+        return status;
+    }
+    context->decode->filled = (int32_t)last + 1;
+    return decoder_publish(context, sink, report, what);
+}
+
+/* Prefill at `position`: rows 0..position of every slot (native/include/volvoxai_backend.h:214-221). */
+static VxStatus hip_context_decode_prefill(void* context_instance, int32_t position, const VxTensorBinding* inputs,
+                                           size_t input_count, const VxBackendOutputSink* sink, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    if (!context || !context->compiled->decoder) return VX_STATUS_BACKEND_UNSUPPORTED;
+    return decoder_rows(context, inputs, input_count, 0, position, sink, report, "W8A8 decoder prefill executed");
+}
+
+/* One step: row `position` against the cached rows 0..position-1; the position must be the next
+ * unfilled cache slot, else the decode state would no longer describe the rows before it. */
+static VxStatus hip_context_decode_step(void* context_instance, int32_t position, const VxTensorBinding* inputs,
+                                        size_t input_count, const VxBackendOutputSink* sink, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    if (!context || !context->compiled->decoder) return VX_STATUS_BACKEND_UNSUPPORTED;
+    if (!context->decode || position < 1 || position != context->decode->filled) return VX_STATUS_INVALID_ARGUMENT;
+    return decoder_rows(context, inputs, input_count, position, position, sink, report, "W8A8 decoder step executed");
+}
+
+static VxStatus hip_context_decode_reset(void* context_instance, VxReport* report) {
+    HipContext* context = (HipContext*)context_instance;
+    if (!context || context->closed) return VX_STATUS_INVALID_ARGUMENT;
+    if (!context->compiled->decoder) return VX_STATUS_BACKEND_UNSUPPORTED;
+    context->decode->filled = 0;
+    fill_report(report, context->compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "decode state reset");
+    return VX_STATUS_OK;
+}
+
 static VxStatus hip_context_execute(void* context_instance, const VxTensorBinding* inputs, size_t input_count,
                                     const VxBackendOutputSink* sink, VxReport* report) {
     HipContext* context = (HipContext*)context_instance;
@@ -1005,6 +1226,14 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
         !sink->write)
         return VX_STATUS_INVALID_ARGUMENT;
     compiled = context->compiled;
+    if (compiled->decoder) {
+        /* the stateless evaluation of a decoder graph: every row, the outputs of the last; no decode
+         * state survives it */
+        status = decoder_rows(context, inputs, input_count, 0, (int64_t)compiled->decoder->capacity - 1, sink, report,
+                              "W8A8 decoder executed");
+        context->decode->filled = 0;
+        return status;
+    }
     /* the complete batch is validated before anything is mutated */
     if (!binding_admitted(compiled, &inputs[0], &rows, shape)) return VX_STATUS_INVALID_ARGUMENT;
     status = run_rows(context, inputs[0].data, rows, report);
@@ -1034,7 +1263,7 @@ static VxStatus hip_compiled_batch_contract(void* compiled_instance, VxBackendBa
     contract->device_epoch = 0;
     contract->graph_fingerprint = NULL;
     contract->independent_batch_proof_identity = NULL;
-    if (compiled->batch_capable) {
+    if (compiled->batch_capable && !compiled->decoder) {
         contract->graph_fingerprint = compiled->graph_fingerprint;
         contract->independent_batch_proof_identity = compiled->batch_proof_identity;
         contract->max_batch = compiled->lead_max[0] > 65536 ? 65536u : (uint32_t)compiled->lead_max[0];
@@ -1058,6 +1287,10 @@ static VxStatus hip_context_execute_batch(void* context_instance, const VxBacken
         !invocation->lane_output_sinks || invocation->lane_output_sink_count != invocation->batch_size)
         return VX_STATUS_INVALID_ARGUMENT;
     compiled = context->compiled;
+    if (compiled->decoder) /* the slots of a decoder are its batch: one invocation, one lane */
+        return invocation->batch_size == 1 ? hip_context_execute(context_instance, invocation->stacked_inputs, 1,
+                                                                 &invocation->lane_output_sinks[0], report)
+                                           : VX_STATUS_BACKEND_UNSUPPORTED;
     if (invocation->batch_size > 1 && !compiled->batch_capable) return VX_STATUS_BACKEND_UNSUPPORTED;
     if (!binding_admitted(compiled, &invocation->stacked_inputs[0], &rows, shape) ||
         shape[0] != (int64_t)invocation->batch_size)
@@ -1108,6 +1341,9 @@ VxStatus volvoxai_hip_gfx950_backend_register(VxReport* report) {
         .context_execute_batch = hip_context_execute_batch,
         .context_create = hip_context_create,
         .context_execute = hip_context_execute,
+        .context_decode_prefill = hip_context_decode_prefill,
+        .context_decode_step = hip_context_decode_step,
+        .context_decode_reset = hip_context_decode_reset,
         .context_close = hip_context_close,
         .context_destroy = hip_context_destroy,
         .exact_contract_marker = VX_BACKEND_PROVIDER_EXACT_CONTRACT_MARKER,
@@ -1125,6 +1361,17 @@ VxStatus volvoxai_hip_gfx950_inspect_package(const VxModelSource* source, VxPack
     Failure failure = {VX_STATUS_OK, {0}};
     VxStatus status;
     if (!source || source->struct_size != sizeof(*source)) return VX_STATUS_INVALID_ARGUMENT;
+    {
+        /* a decoder graph is read by its own route; without a device only the reading is done */
+        int is_decoder = 0;
+        DecoderModel* unused = NULL;
+        status = try_decoder(source, arithmetic, -1, &is_decoder, &unused, &failure);
+        if (is_decoder) {
+            if (message && message_capacity) snprintf(message, message_capacity, "%s", failure.message);
+            if (status == VX_STATUS_OK && is_packed_linear) *is_packed_linear = 1;
+            return status;
+        }
+    }
     status = plan_package(source, arithmetic, &plan, &failure);
     if (message && message_capacity) snprintf(message, message_capacity, "%s", failure.message);
     if (status == VX_STATUS_OK) {
