@@ -711,3 +711,204 @@ done:
     if (runtime) g_provider.runtime_destroy(runtime);
     return run->status = status;
 }
+
+/* A graph with several inputs and outputs: every input bound by name in one context_execute (or
+ * one context_execute_batch over `batch` lanes stacked along axis 0), every declared output
+ * written exactly once (per lane) with its own name, dtype and shape. */
+typedef struct MockPort {
+    const char* name;
+    int32_t dtype;
+    int64_t last; /* last extent */
+    void* data;   /* input bytes, or the buffer an output is copied into */
+    uint64_t bytes;
+    int32_t written;
+} MockPort;
+
+typedef struct MockGraphRun {
+    /* in */
+    const char* graph_path;
+    const char* weight_path;
+    int32_t packed_arithmetic;
+    uint32_t rank;
+    int64_t lead[VX_MAX_TENSOR_RANK]; /* the leading extents of every tensor */
+    int64_t lead_max0;                /* > 0: axis 0 is symbolic, bounded 1..lead_max0 */
+    int32_t batch;                    /* > 0: run as one scheduler batch of lead[0] lanes */
+    int32_t input_count, output_count;
+    MockPort inputs[8], outputs[8];
+    /* out */
+    int32_t status, failed_stage, writes, sink_mismatch;
+    char message[VX_REPORT_MESSAGE_CAPACITY];
+    char execute_route[VX_REPORT_ROUTE_CAPACITY];
+} MockGraphRun;
+
+typedef struct GraphLane {
+    MockGraphRun* run;
+    int32_t lane; /* -1: the whole tensor */
+    int32_t written[8];
+} GraphLane;
+
+static VxStatus graph_write(void* user, const char* name, VxDataType dtype, const int64_t* shape, uint32_t rank,
+                            const void* data, size_t bytes) {
+    GraphLane* lane = (GraphLane*)user;
+    MockGraphRun* run = lane->run;
+    run->writes++;
+    for (int32_t k = 0; name && k < run->output_count; k++) {
+        MockPort* port = &run->outputs[k];
+        const size_t lanes = lane->lane < 0 ? 1u : (size_t)run->lead[0];
+        int ok = !strcmp(name, port->name) && (int32_t)dtype == port->dtype && rank == run->rank && data &&
+                 bytes == (size_t)port->bytes / lanes && shape[rank - 1] == port->last && !lane->written[k];
+        if (strcmp(name, port->name)) continue;
+        for (uint32_t a = 0; ok && a + 1 < rank; a++)
+            if (shape[a] != (a == 0 && lane->lane >= 0 ? 1 : run->lead[a])) ok = 0;
+        if (!ok) break;
+        memcpy((unsigned char*)port->data + (lane->lane < 0 ? 0u : (size_t)lane->lane * bytes), data, bytes);
+        lane->written[k] = 1;
+        port->written++;
+        return VX_STATUS_OK;
+    }
+    run->sink_mismatch = 1;
+    return VX_STATUS_INVALID_ARGUMENT;
+}
+
+static void port_spec(VxTensorSpec* spec, const MockGraphRun* run, const MockPort* port) {
+    memset(spec, 0, sizeof(*spec));
+    spec->struct_size = sizeof(*spec);
+    spec->name = port->name;
+    spec->dtype = (VxDataType)port->dtype;
+    spec->rank = run->rank;
+    spec->location = VX_MEMORY_HOST;
+    for (uint32_t a = 0; a < run->rank; a++) {
+        VxDimensionConstraint* d = &spec->dimensions[a];
+        d->struct_size = sizeof(*d);
+        d->multiple_of = 1;
+        if (a == 0 && run->rank > 1 && run->lead_max0 > 0) {
+            d->kind = VX_DIMENSION_SYMBOLIC;
+            d->symbol = "rows";
+            d->min = 1;
+            d->max = run->lead_max0;
+        } else {
+            d->kind = VX_DIMENSION_FIXED;
+            d->min = d->max = a + 1 < run->rank ? run->lead[a] : port->last;
+        }
+    }
+}
+
+int32_t mock_host_run_graph(MockGraphRun* run) {
+    static const char fingerprint[] = "sha256:mock-graph-fingerprint";
+    static const char proof[] = "sha256:mock-shape-domain-proof";
+    static const char batch_proof[] = "sha256:mock-independent-batch-proof";
+    VxRuntimeOptions runtime_options = VX_RUNTIME_OPTIONS_INIT;
+    VxContextOptions context_options = VX_CONTEXT_OPTIONS_INIT;
+    VxReport report = VX_REPORT_INIT;
+    VxModelSource source = VX_MODEL_SOURCE_INIT;
+    VxBackendCompileInput input = VX_BACKEND_COMPILE_INPUT_INIT;
+    VxBackendShapeDomainAttestation attestation = VX_BACKEND_SHAPE_DOMAIN_ATTESTATION_INIT;
+    VxBackendPolicy policy = VX_BACKEND_POLICY_INIT;
+    VxTensorSpec in_specs[8], out_specs[8];
+    VxTensorBinding bindings[8];
+    const char* weights[1];
+    const char* wanted[1];
+    void *runtime = NULL, *compiled = NULL, *context = NULL;
+    VxStatus status;
+    if (!g_registered || run->input_count < 1 || run->input_count > 8 || run->output_count < 1 || run->output_count > 8)
+        return run->status = VX_STATUS_INVALID_ARGUMENT;
+    run->writes = run->sink_mismatch = 0;
+    for (int32_t k = 0; k < run->output_count; k++) run->outputs[k].written = 0;
+    status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
+    run->failed_stage = VX_STAGE_RUNTIME_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+    weights[0] = run->weight_path;
+    source.graph_path = run->graph_path;
+    source.weight_paths = weights;
+    source.weight_path_count = 1;
+    for (int32_t k = 0; k < run->input_count; k++) port_spec(&in_specs[k], run, &run->inputs[k]);
+    for (int32_t k = 0; k < run->output_count; k++) port_spec(&out_specs[k], run, &run->outputs[k]);
+    input.source = &source;
+    input.graph_fingerprint = fingerprint;
+    input.shape_domain_proof_identity = proof;
+    input.inputs = in_specs;
+    input.input_count = (size_t)run->input_count;
+    input.outputs = out_specs;
+    input.output_count = (size_t)run->output_count;
+    input.packed_arithmetic = (VxPackedArithmetic)run->packed_arithmetic;
+    if (run->batch > 0) {
+        input.independent_batch_proof_protocol = VX_BACKEND_INDEPENDENT_BATCH_PROOF_PROTOCOL;
+        input.independent_batch_proof_identity = batch_proof;
+    }
+    wanted[0] = g_name;
+    policy.mode = VX_BACKEND_REQUIRE;
+    policy.operator_fallback = VX_OPERATOR_FALLBACK_FORBID;
+    policy.backends = wanted;
+    policy.backend_count = 1;
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.compile(runtime, &input, &policy, &compiled, &attestation, &report);
+    run->failed_stage = VX_STAGE_COMPILE;
+    if (status != VX_STATUS_OK) {
+        if (compiled) status = VX_STATUS_INTERNAL;
+        goto done;
+    }
+    report = (VxReport)VX_REPORT_INIT;
+    status = g_provider.context_create(compiled, &context_options, &context, &report);
+    run->failed_stage = VX_STAGE_CONTEXT_CREATE;
+    if (status != VX_STATUS_OK) goto done;
+    /* the bindings in reverse order of the declaration: a provider finds them by name */
+    for (int32_t k = 0; k < run->input_count; k++) {
+        VxTensorBinding* b = &bindings[run->input_count - 1 - k];
+        *b = (VxTensorBinding)VX_TENSOR_BINDING_INIT;
+        b->name = run->inputs[k].name;
+        b->dtype = (VxDataType)run->inputs[k].dtype;
+        b->rank = run->rank;
+        for (uint32_t a = 0; a + 1 < run->rank; a++) b->shape[a] = run->lead[a];
+        b->shape[run->rank - 1] = run->inputs[k].last;
+        b->data = run->inputs[k].data;
+        b->byte_size = (size_t)run->inputs[k].bytes;
+        b->location = VX_MEMORY_HOST;
+    }
+    run->failed_stage = VX_STAGE_EXECUTE;
+    report = (VxReport)VX_REPORT_INIT;
+    if (run->batch > 0) {
+        const uint32_t batch = (uint32_t)run->lead[0];
+        VxBackendBatchContract contract = VX_BACKEND_BATCH_CONTRACT_INIT;
+        VxBackendBatchInvocation invocation = VX_BACKEND_BATCH_INVOCATION_INIT;
+        VxBackendOutputSink* sinks = (VxBackendOutputSink*)calloc(batch, sizeof(*sinks));
+        GraphLane* lanes = (GraphLane*)calloc(batch, sizeof(*lanes));
+        status = g_provider.compiled_batch_contract(compiled, &contract, &report);
+        if (status == VX_STATUS_OK && batch > contract.max_batch) status = VX_STATUS_BACKEND_UNSUPPORTED;
+        for (uint32_t i = 0; i < batch; i++) {
+            lanes[i].run = run;
+            lanes[i].lane = (int32_t)i;
+            sinks[i].struct_size = sizeof(sinks[i]);
+            sinks[i].user_data = &lanes[i];
+            sinks[i].write = graph_write;
+        }
+        invocation.stacked_inputs = bindings;
+        invocation.stacked_input_count = (size_t)run->input_count;
+        invocation.batch_size = batch;
+        invocation.lane_output_sinks = sinks;
+        invocation.lane_output_sink_count = batch;
+        report = (VxReport)VX_REPORT_INIT;
+        if (status == VX_STATUS_OK) status = g_provider.context_execute_batch(context, &invocation, &report);
+        for (int32_t k = 0; status == VX_STATUS_OK && k < run->output_count; k++)
+            if (run->outputs[k].written != (int32_t)batch) status = VX_STATUS_EXECUTION_FAILED;
+        free(sinks);
+        free(lanes);
+    } else {
+        GraphLane whole = {run, -1, {0}};
+        VxBackendOutputSink sink = {sizeof(VxBackendOutputSink), &whole, graph_write};
+        status = g_provider.context_execute(context, bindings, (size_t)run->input_count, &sink, &report);
+        for (int32_t k = 0; status == VX_STATUS_OK && k < run->output_count; k++)
+            if (run->outputs[k].written != 1) status = VX_STATUS_EXECUTION_FAILED;
+    }
+    if (status == VX_STATUS_OK && run->sink_mismatch) status = VX_STATUS_EXECUTION_FAILED;
+    snprintf(run->execute_route, sizeof(run->execute_route), "%s", report.route_evidence);
+    if (status == VX_STATUS_OK) run->failed_stage = VX_STAGE_NONE;
+done:
+    snprintf(run->message, sizeof(run->message), "%s", report.message);
+    if (context) {
+        if (g_provider.context_close) (void)g_provider.context_close(context, &report);
+        g_provider.context_destroy(context);
+    }
+    if (compiled) g_provider.compiled_destroy(compiled);
+    if (runtime) g_provider.runtime_destroy(runtime);
+    return run->status = status;
+}

@@ -290,7 +290,7 @@ def _drop(path):
 
 @pytest.mark.parametrize("name,mutate,status", [
     ("format", lambda g, t: g.__setitem__("format", "volvox-graph/v0"), -5),
-    ("two nodes", lambda g, t: g["nodes"].append(dict(g["nodes"][0], id="again")), -7),
+    ("two writers of one tensor", lambda g, t: g["nodes"].append(dict(g["nodes"][0], id="again")), -5),
     ("other op", lambda g, t: g["nodes"][0].__setitem__("opType", "Linear"), -7),
     ("no table", _drop(["quantization"]), -5),
     ("table extra field", lambda g, t: g["quantization"].__setitem__("scales", [1.0]), -5),
@@ -355,13 +355,28 @@ def test_reads_node_chains(registered, tmp_path):
     (g, w), d_out = sandwich(tmp_path / "ok", (4, 48), c1, c2)
     assert inspect(registered, g, w)[:4] == (0, 48, 10, 0)
 
-    # the second linear reads the first node's output instead of the one before it: not a chain
+    # a node may read any earlier tensor, but the weight it names must fit what it reads: the second
+    # linear (24 inputs) on the quantized graph input (48 wide) is refused for its shapes
     (g, w), _ = sandwich(tmp_path / "dag", (4, 48), c1, c2)
     doc = json.loads(g.read_text())
     doc["nodes"][2]["inputs"]["input"] = "xq"
     g.write_text(json.dumps(doc))
+    assert inspect(registered, g, w)[0] == -5
+    # a node that reads a tensor nobody provides, or one a LATER node writes
+    doc["nodes"][2]["inputs"]["input"] = "nowhere"
+    g.write_text(json.dumps(doc))
     st, *_, msg = inspect(registered, g, w)
-    assert st == -7 and "chain" in msg
+    assert st == -5 and "neither a graph input nor an earlier node" in msg
+    doc["nodes"][2]["inputs"]["input"] = doc["nodes"][3]["outputs"]["out"]["tensor"]
+    g.write_text(json.dumps(doc))
+    assert inspect(registered, g, w)[0] == -5
+    # a graph output no node writes
+    (g, w), _ = sandwich(tmp_path / "out", (4, 48), c1, c2)
+    doc = json.loads(g.read_text())
+    doc["outputs"] = ["xq", "missing"]
+    g.write_text(json.dumps(doc))
+    st, *_, msg = inspect(registered, g, w)
+    assert st == -5 and "missing" in msg
 
     def other_parameters(nodes, tensors, affine):  # the node and the table disagree about the input's scale
         tensors["in.s2"] = np.array([0.5], np.float32)
@@ -643,3 +658,145 @@ def test_bindings_are_validated_before_anything_runs(registered, tmp_path):
     assert r.status == -1 and r.writes == 0
     r, _ = run(registered, g, w, k["x"], "other", "i8", "projected_q", "i8", 4)
     assert r.status == -1 and r.writes == 0
+
+
+# ---- graphs that are not chains ----------------------------------------------------------------
+
+class MockPort(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("dtype", C.c_int32), ("last", C.c_int64), ("data", C.c_void_p),
+                ("bytes", C.c_uint64), ("written", C.c_int32)]
+
+
+class MockGraphRun(C.Structure):
+    _fields_ = [("graph_path", C.c_char_p), ("weight_path", C.c_char_p), ("packed_arithmetic", C.c_int32),
+                ("rank", C.c_uint32), ("lead", C.c_int64 * 8), ("lead_max0", C.c_int64), ("batch", C.c_int32),
+                ("input_count", C.c_int32), ("output_count", C.c_int32), ("inputs", MockPort * 8),
+                ("outputs", MockPort * 8),
+                ("status", C.c_int32), ("failed_stage", C.c_int32), ("writes", C.c_int32), ("sink_mismatch", C.c_int32),
+                ("message", C.c_char * 256), ("execute_route", C.c_char * 512)]
+
+
+def forked_package(tmp, lead, a, b, c, q, rows_symbol=False):
+    """Two inputs, three outputs: x -> PackedLinear A -> ya;  x -> PackedLinear B -> h -> PackedLinear C
+    -> yc (x is read twice);  u -> QuantizeLinear -> uq -> QLinear -> vq (an independent branch)."""
+    lead = list(lead)
+    shape = lambda d: lead + [d]
+
+    def packed(node_id, fed, out_name, case, prefix):
+        return {"id": node_id, "opType": "PackedLinear",
+                "inputs": {"input": fed, "weight": prefix + ".w", "scale": prefix + ".s", "bias": prefix + ".b"},
+                "outputs": {"out": {"tensor": out_name, "shape": shape(case["n"]), "dtype": "float32"}},
+                "params": {"group_size": case["group"], "weight_bits": 8}}
+
+    nodes = [packed("A", "x", "ya", a, "a"), packed("B", "x", "h", b, "b"),
+             {"id": "quant", "opType": "QuantizeLinear", "inputs": {"input": "u", "scale": "u.s", "zero_point": "u.z"},
+              "outputs": {"out": {"tensor": "uq", "shape": shape(q["w"].shape[1]), "dtype": "int8"}}, "params": {}},
+             packed("C", "h", "yc", c, "c"),
+             {"id": "fc", "opType": "QLinear", "inputs": {"input": "uq", "weight": "q.w", "bias": "q.b"},
+              "outputs": {"out": {"tensor": "vq", "shape": shape(q["w"].shape[0]), "dtype": "int8"}}, "params": {}}]
+    graph = {"format": "volvox-graph/v1", "dimensions": {"rows": {"min": 1, "max": 64}} if rows_symbol else {},
+             "inputs": {"x": {"shape": shape(a["k"]), "dtype": "float32"},
+                        "u": {"shape": shape(q["w"].shape[1]), "dtype": "float32"}},
+             "nodes": nodes, "outputs": ["yc", "vq", "ya"],
+             "quantization": {"format": "volvox-affine-safetensors/v1", "tensors": {
+                 "uq": {"scheme": "per_tensor", "scale_tensor": "u.s", "zero_point_tensor": "u.z"},
+                 "q.w": {"scheme": "per_axis", "axis": 0, "scale_tensor": "q.w.s", "zero_point_tensor": "q.w.z"},
+                 "vq": {"scheme": "per_tensor", "scale_tensor": "v.s", "zero_point_tensor": "v.z"}}}}
+    from oracle.pyoracle import Oracle
+    orc = Oracle()
+    tensors = {"u.s": np.array([q["s_in"]], np.float32), "u.z": np.array([q["zp_in"]], np.int8),
+               "q.w": q["w"], "q.b": q["bias"], "q.w.s": q["scales"], "q.w.z": q["zps"].astype(np.int8),
+               "v.s": np.array([q["s_out"]], np.float32), "v.z": np.array([q["zp_out"]], np.int8)}
+    for prefix, case in (("a", a), ("b", b), ("c", c)):
+        tensors[prefix + ".w#as_i32"] = orc.pack_w8_words(case["w"])
+        tensors[prefix + ".s"], tensors[prefix + ".b"] = case["scales"], case["bias"]
+    tmp.mkdir(parents=True, exist_ok=True)
+    (tmp / "graph.json").write_text(json.dumps(graph, separators=(",", ":")))
+    write_safetensors(tmp / "model.safetensors", tensors)
+    return tmp / "graph.json", tmp / "model.safetensors"
+
+
+def forked_cases(rows):
+    a = cases.packed_case(rows, 384, 200, 128, 31)
+    b = cases.packed_case(rows, 384, 130, 64, 32)
+    c = cases.packed_case(rows, 130, 72, 32, 33)
+    q = cases.qlinear_random_case(rows, 96, 40, 34, I8, I8, I8, False)
+    u = np.random.default_rng(35).normal(0, 20, (rows, 96)).astype(np.float32)
+    return a, b, c, q, u
+
+
+def forked_expectation(oracle, a, b, c, q, u):
+    _, ya = oracle.packed_linear(a["x"], oracle.pack_w8_words(a["w"]), a["scales"], a["bias"], a["n"], a["group"])
+    _, h = oracle.packed_linear(a["x"], oracle.pack_w8_words(b["w"]), b["scales"], b["bias"], b["n"], b["group"])
+    _, yc = oracle.packed_linear(h, oracle.pack_w8_words(c["w"]), c["scales"], c["bias"], c["n"], c["group"])
+    _, uq = oracle.quantize(u, q["s_in"], q["zp_in"], I8)
+    ok, vq = oracle.qlinear(uq, q["w"], q["bias"], q["scales"], q["zps"], q["s_in"], q["zp_in"], q["s_out"], q["zp_out"],
+                            I8, I8, I8)
+    assert ok == 1
+    return ya, yc, vq
+
+
+def run_forked(host, g, w, lead, a, q, u, batch=0, lead_max0=0):
+    mock, _, _ = host
+    rows = int(np.prod(lead))
+    x = np.ascontiguousarray(a["x"])
+    outs = {"yc": np.zeros((rows, 72), np.float32), "vq": np.zeros((rows, 40), np.int8), "ya": np.zeros((rows, 200), np.float32)}
+    r = MockGraphRun()
+    r.graph_path, r.weight_path, r.packed_arithmetic = str(g).encode(), str(w).encode(), ARITH["dynamic_i8"]
+    r.rank = len(lead) + 1
+    for i, e in enumerate(lead):
+        r.lead[i] = e
+    r.lead_max0, r.batch = lead_max0, batch
+    r.input_count, r.output_count = 2, 3
+    r.inputs[0] = MockPort(b"x", DT["f32"], 384, x.ctypes.data, x.nbytes, 0)
+    r.inputs[1] = MockPort(b"u", DT["f32"], 96, u.ctypes.data, u.nbytes, 0)
+    for k, (name, dt) in enumerate((("ya", "f32"), ("yc", "f32"), ("vq", "i8"))):
+        r.outputs[k] = MockPort(name.encode(), DT[dt], outs[name].shape[1], outs[name].ctypes.data, outs[name].nbytes, 0)
+    mock.mock_host_run_graph.argtypes = [C.POINTER(MockGraphRun)]
+    mock.mock_host_run_graph(C.byref(r))
+    return r, outs
+
+
+def test_reads_graphs_with_branches_and_several_ports(registered, tmp_path):
+    a, b, c, q, _ = forked_cases(6)
+    g, w = forked_package(tmp_path / "fork", (6,), a, b, c, q)
+    assert inspect(registered, g, w, "dynamic_i8")[:4] == (0, 384, 72, 1)  # first input, first output
+    doc = json.loads(g.read_text())
+    doc["inputs"]["u"]["shape"] = [7, 96]  # another row count than x
+    g.write_text(json.dumps(doc))
+    st, *_, msg = inspect(registered, g, w, "dynamic_i8")
+    assert st == -7 and "leading extents" in msg
+
+
+@pytest.mark.gpu
+def test_forked_graph_two_inputs_three_outputs(registered, oracle, tmp_path):
+    """A graph that is not a chain: one input read by two linears, a second input with its own
+    branch, three outputs declared in another order than they are computed; every output equals the
+    oracle's composition of its branch, and each is written once under its own name and type."""
+    rows = 37
+    a, b, c, q, u = forked_cases(rows)
+    g, w = forked_package(tmp_path / "fork", (rows,), a, b, c, q)
+    r, outs = run_forked(registered, g, w, (rows,), a, q, u)
+    assert r.status == 0 and r.failed_stage == 0, (r.status, r.failed_stage, r.message)
+    ya, yc, vq = forked_expectation(oracle, a, b, c, q, u)
+    assert (outs["ya"].view(np.uint32) == ya.view(np.uint32)).all()
+    assert (outs["yc"].view(np.uint32) == yc.view(np.uint32)).all()
+    assert (outs["vq"] == vq).all()
+    assert r.writes == 3 and b"nodes=5" in r.execute_route
+
+
+@pytest.mark.gpu
+def test_forked_graph_as_one_scheduler_batch(registered, oracle, tmp_path):
+    """The same graph with a symbolic axis 0: five requests of [1, 3, d] stacked into one
+    invocation, every lane's sink receiving its slice of each of the three outputs."""
+    batch, inner = 5, 3
+    rows = batch * inner
+    a, b, c, q, u = forked_cases(rows)
+    g, w = forked_package(tmp_path / "fork", (1, inner), a, b, c, q)
+    r, outs = run_forked(registered, g, w, (batch, inner), a, q, u, batch=1, lead_max0=16)
+    assert r.status == 0 and r.failed_stage == 0, (r.status, r.failed_stage, r.message)
+    ya, yc, vq = forked_expectation(oracle, a, b, c, q, u)
+    assert (outs["ya"].view(np.uint32) == ya.view(np.uint32)).all()
+    assert (outs["yc"].view(np.uint32) == yc.view(np.uint32)).all()
+    assert (outs["vq"] == vq).all()
+    assert r.writes == 3 * batch

@@ -46,6 +46,8 @@ typedef enum PlanKind {
 } PlanKind;
 
 #define MAX_CHAIN_NODES 64u
+#define MAX_GRAPH_PORTS 8u                           /* graph inputs, and graph outputs */
+#define MAX_GRAPH_TENSORS (MAX_CHAIN_NODES + MAX_GRAPH_PORTS) /* every graph input and node output */
 
 /* Host-side result of reading one node; tensor pointers borrow the mapped weight files, which
  * belong to the ChainPlan. */
@@ -56,6 +58,7 @@ typedef struct PackagePlan {
     char output_name[NAME_CAPACITY];
     uint32_t d_in, d_out;
     VxDataType input_dtype, output_dtype;
+    uint32_t input_slot, output_slot; /* the tensors it reads and writes, as indices of the graph's tensor table */
     /* QLinear */
     const void* weight;
     uint32_t weight_dtype;
@@ -82,12 +85,27 @@ typedef struct PackagePlan {
     size_t file_count;
 } PackagePlan;
 
-/* The whole graph: its nodes in execution order and the files they read. */
+/* A tensor of the graph: a graph input or the output of a node.  All share their leading extents
+ * (the rows); name, element type and last extent tell them apart. */
+typedef struct PlanTensor {
+    char name[NAME_CAPACITY];
+    VxDataType dtype;
+    uint32_t d;
+} PlanTensor;
+
+/* The whole graph: its nodes in execution order (every node reads a graph input or the output of
+ * an earlier node -- a chain, a tree with shared prefixes, several independent branches), the
+ * tensors between them and the files they read.  input_name .. output_dtype describe the first
+ * graph input and the first graph output. */
 typedef struct ChainPlan {
     PackagePlan* nodes;
     size_t count;
     VxstFile** files;
     size_t file_count;
+    PlanTensor tensors[MAX_GRAPH_TENSORS];
+    size_t tensor_count;
+    uint32_t input_slots[MAX_GRAPH_PORTS], output_slots[MAX_GRAPH_PORTS];
+    size_t input_count, output_count;
     char input_name[NAME_CAPACITY];
     char output_name[NAME_CAPACITY];
     uint32_t d_in, d_out;
@@ -98,6 +116,7 @@ typedef struct ChainPlan {
 /* One compiled node. */
 typedef struct HipStage {
     PlanKind kind;
+    uint32_t input_slot, output_slot;
     uint32_t d_in, d_out;
     VxDataType input_dtype, output_dtype;
     VxHipQLinear* qlinear;
@@ -114,13 +133,14 @@ typedef struct HipCompiled {
     struct DecoderModel* decoder; /* set for a decoder graph (decoder_route.inc); stages are then unused */
     HipStage* stages;
     size_t stage_count;
-    uint64_t widest_row_bytes; /* of any tensor of the chain, graph input and output included */
-    char input_name[NAME_CAPACITY];
-    char output_name[NAME_CAPACITY];
-    uint32_t d_in, d_out;
-    VxDataType input_dtype, output_dtype;
-    size_t input_element_bytes, output_element_bytes;
-    uint32_t rank;                        /* of input and output alike */
+    PlanTensor tensors[MAX_GRAPH_TENSORS]; /* graph inputs and node outputs; a context holds one device buffer each */
+    size_t tensor_count;
+    uint32_t input_slots[MAX_GRAPH_PORTS], output_slots[MAX_GRAPH_PORTS];
+    size_t input_count, output_count;
+    uint64_t widest_row_bytes;  /* of any tensor of the graph */
+    uint64_t all_rows_bytes;    /* of one row of every tensor together */
+    uint64_t widest_float_row;  /* elements of the widest PackedLinear input (its int8 staging) */
+    uint32_t rank;                        /* of every input and output alike */
     int64_t lead_min[VX_MAX_TENSOR_RANK]; /* bounds of the leading dimensions */
     int64_t lead_max[VX_MAX_TENSOR_RANK];
     int64_t lead_multiple[VX_MAX_TENSOR_RANK];
@@ -136,9 +156,10 @@ typedef struct HipContext {
     HipCompiled* compiled;
     VxHipContext* ctx;
     struct DecoderState* decode; /* decoder graphs: the cache and work buffers of this context */
-    void* work_dev[2]; /* a node reads one and writes the other */
-    void* output_host;
-    size_t work_capacity[2], host_capacity;
+    void* tensor_dev[MAX_GRAPH_TENSORS]; /* one buffer per tensor of the graph, grown to the rows of a call */
+    size_t tensor_capacity[MAX_GRAPH_TENSORS];
+    void* output_host[MAX_GRAPH_PORTS];
+    size_t host_capacity[MAX_GRAPH_PORTS];
     int closed;
 } HipContext;
 
@@ -516,45 +537,62 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
         const VxjValue* inputs = vxj_member(root, "inputs");
         const VxjValue* nodes = vxj_member(root, "nodes");
         const VxjValue* outputs = vxj_member(root, "outputs");
-        const VxjValue* graph_input = inputs && inputs->kind == VXJ_OBJECT ? inputs->first : NULL;
-        const VxjValue* in_shape = vxj_member(graph_input, "shape");
-        const VxjValue* declared_output = vxj_item(outputs, 0);
-        /* the tensor the next node must read */
-        char current[NAME_CAPACITY];
-        VxDataType current_dtype;
-        uint32_t current_d;
+        const VxjValue* first_input = inputs && inputs->kind == VXJ_OBJECT ? inputs->first : NULL;
+        const VxjValue* in_shape = vxj_member(first_input, "shape");
         if (!format || strcmp(format, "volvox-graph/v1")) {
             status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph format is not volvox-graph/v1%s", "");
             break;
         }
         /* representations v1 retired: an artifact that carries one is not a v1 package
          * (docs/w8a8-safetensors.md:176-188) */
-        if (vxj_member(root, "weights_quantization") || vxj_member(root, "weights_quantization_storage") ||
-            (graph_input && graph_input->kind == VXJ_OBJECT && vxj_member(graph_input, "quantization"))) {
+        if (vxj_member(root, "weights_quantization") || vxj_member(root, "weights_quantization_storage")) {
             status = refuse(failure, VX_STATUS_INVALID_GRAPH,
                             "the graph carries a retired quantization field (weights_quantization, "
                             "weights_quantization_storage or an inline input quantization)%s", "");
             break;
         }
+        for (const VxjValue* in = first_input; in; in = in->next)
+            if (in->kind == VXJ_OBJECT && vxj_member(in, "quantization")) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                "the graph carries a retired quantization field (weights_quantization, "
+                                "weights_quantization_storage or an inline input quantization)%s", "");
+                break;
+            }
+        if (status != VX_STATUS_OK) break;
         if (!nodes || nodes->kind != VXJ_ARRAY || !nodes->count || nodes->count > MAX_CHAIN_NODES || !inputs ||
-            inputs->count != 1 || !outputs || outputs->kind != VXJ_ARRAY || outputs->count != 1) {
+            inputs->kind != VXJ_OBJECT || !inputs->count || inputs->count > MAX_GRAPH_PORTS || !outputs ||
+            outputs->kind != VXJ_ARRAY || !outputs->count || outputs->count > MAX_GRAPH_PORTS) {
             status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
-                            "this provider compiles chains of up to 64 nodes with one input and one output%s", "");
+                            "this provider compiles graphs of up to 64 nodes with up to 8 inputs and 8 outputs%s", "");
             break;
         }
-        if (!copy_name(chain->input_name, graph_input->key) ||
-            !graph_dtype(vxj_member_string(graph_input, "dtype"), &chain->input_dtype) || !in_shape ||
-            in_shape->kind != VXJ_ARRAY || !in_shape->count || declared_output->kind != VXJ_STRING ||
-            !copy_name(chain->output_name, declared_output->string)) {
+        if (!in_shape || in_shape->kind != VXJ_ARRAY || !in_shape->count) {
             status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph input or output declaration is incomplete%s", "");
             break;
         }
-        /* dense on the last axis: that extent is a number in every declaration */
-        chain->d_in = fixed_extent(vxj_item(in_shape, in_shape->count - 1));
-        if (!chain->d_in) {
-            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the input's last extent must be a fixed d_in%s", "");
-            break;
+        /* the graph inputs: dense on the last axis (that extent is a number in every declaration),
+         * one set of leading extents -- the rows -- for all of them */
+        for (const VxjValue* in = first_input; in && status == VX_STATUS_OK; in = in->next) {
+            PlanTensor* t = &chain->tensors[chain->tensor_count];
+            const VxjValue* shape = vxj_member(in, "shape");
+            if (!copy_name(t->name, in->key) || !graph_dtype(vxj_member_string(in, "dtype"), &t->dtype) || !shape ||
+                shape->kind != VXJ_ARRAY || shape->count != in_shape->count) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH, "graph input or output declaration is incomplete%s", "");
+                break;
+            }
+            for (size_t axis = 0; axis + 1 < in_shape->count; axis++)
+                if (!same_extent(vxj_item(in_shape, axis), vxj_item(shape, axis)))
+                    status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED,
+                                    "graph input '%s' does not share the leading extents of the first input", t->name);
+            t->d = fixed_extent(vxj_item(shape, shape->count - 1));
+            if (status == VX_STATUS_OK && !t->d)
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the input's last extent must be a fixed d_in%s", "");
+            chain->input_slots[chain->input_count++] = (uint32_t)chain->tensor_count++;
         }
+        if (status != VX_STATUS_OK) break;
+        memcpy(chain->input_name, chain->tensors[0].name, sizeof(chain->input_name));
+        chain->input_dtype = chain->tensors[0].dtype;
+        chain->d_in = chain->tensors[0].d;
         chain->files = (VxstFile**)calloc(source->weight_path_count ? source->weight_path_count : 1, sizeof(VxstFile*));
         chain->nodes = (PackagePlan*)calloc(nodes->count, sizeof(PackagePlan));
         if (!chain->files || !chain->nodes) {
@@ -577,15 +615,14 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
         }
         if (status != VX_STATUS_OK) break;
 
-        memcpy(current, chain->input_name, sizeof(current));
-        current_dtype = chain->input_dtype;
-        current_d = chain->d_in;
         for (const VxjValue* node = nodes->first; node && status == VX_STATUS_OK; node = node->next) {
             PackagePlan* plan = &chain->nodes[chain->count];
             const char* op = vxj_member_string(node, "opType");
             const VxjValue* out = vxj_member(vxj_member(node, "outputs"), "out");
             const VxjValue* out_shape = vxj_member(out, "shape");
             const char* fed = vxj_member_string(vxj_member(node, "inputs"), "input");
+            PlanTensor* written = &chain->tensors[chain->tensor_count];
+            size_t reads = chain->tensor_count;
             chain->count++;
             if (node->kind == VXJ_OBJECT && vxj_member(node, "outputs_quantization")) {
                 status = refuse(failure, VX_STATUS_INVALID_GRAPH,
@@ -601,21 +638,30 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
                 status = refuse(failure, VX_STATUS_INVALID_GRAPH, "node or tensor declaration is incomplete%s", "");
                 break;
             }
-            if (!fed || strcmp(fed, current)) {
-                status = refuse(failure, nodes->count == 1 ? VX_STATUS_INVALID_GRAPH : VX_STATUS_BACKEND_UNSUPPORTED,
-                                "node '%s' does not read the tensor before it: only chains are compiled",
+            /* a node reads a graph input or what an earlier node wrote, and writes a new tensor */
+            for (size_t t = 0; fed && t < chain->tensor_count; t++)
+                if (!strcmp(chain->tensors[t].name, fed)) reads = t;
+            if (reads == chain->tensor_count) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH,
+                                "node '%s' reads a tensor that neither a graph input nor an earlier node provides",
                                 plan->node_id);
                 break;
             }
+            for (size_t t = 0; t < chain->tensor_count; t++)
+                if (!strcmp(chain->tensors[t].name, plan->output_name))
+                    status = refuse(failure, VX_STATUS_INVALID_GRAPH, "node '%s' writes a tensor that already exists",
+                                    plan->node_id);
             /* rows pass through unchanged: the leading extents are the graph input's */
-            for (size_t axis = 0; axis + 1 < in_shape->count; axis++)
+            for (size_t axis = 0; axis + 1 < in_shape->count && status == VX_STATUS_OK; axis++)
                 if (!same_extent(vxj_item(in_shape, axis), vxj_item(out_shape, axis)))
                     status = refuse(failure, VX_STATUS_INVALID_GRAPH,
                                     "node '%s' changes a leading extent", plan->node_id);
             if (status != VX_STATUS_OK) break;
-            memcpy(plan->input_name, current, sizeof(current));
-            plan->input_dtype = current_dtype;
-            plan->d_in = current_d;
+            memcpy(plan->input_name, chain->tensors[reads].name, sizeof(plan->input_name));
+            plan->input_dtype = chain->tensors[reads].dtype;
+            plan->d_in = chain->tensors[reads].d;
+            plan->input_slot = (uint32_t)reads;
+            plan->output_slot = (uint32_t)chain->tensor_count;
             plan->d_out = fixed_extent(vxj_item(out_shape, out_shape->count - 1));
             if (!plan->d_out) {
                 status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the last extent of '%s' must be fixed",
@@ -632,18 +678,30 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
                 status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "operator '%s' is not offered by this provider",
                                 op);
             if (plan->kind == PLAN_PACKED_LINEAR) chain->any_packed = 1;
-            memcpy(current, plan->output_name, sizeof(current));
-            current_dtype = plan->output_dtype;
-            current_d = plan->d_out;
+            memcpy(written->name, plan->output_name, sizeof(written->name));
+            written->dtype = plan->output_dtype;
+            written->d = plan->d_out;
+            chain->tensor_count++;
         }
         if (status != VX_STATUS_OK) break;
-        if (strcmp(current, chain->output_name)) {
-            status = refuse(failure, VX_STATUS_INVALID_GRAPH, "the last node must write the graph output '%s'",
-                            chain->output_name);
-            break;
+        /* the graph outputs: distinct tensors written by nodes */
+        for (const VxjValue* o = outputs->first; o && status == VX_STATUS_OK; o = o->next) {
+            size_t slot = chain->tensor_count;
+            for (size_t t = chain->input_count; o->kind == VXJ_STRING && t < chain->tensor_count; t++)
+                if (!strcmp(chain->tensors[t].name, o->string)) slot = t;
+            for (size_t k = 0; k < chain->output_count; k++)
+                if (chain->output_slots[k] == slot) slot = chain->tensor_count;
+            if (slot == chain->tensor_count) {
+                status = refuse(failure, VX_STATUS_INVALID_GRAPH, "no node writes the graph output '%s' (or it is listed twice)",
+                                o->kind == VXJ_STRING ? o->string : "(not a name)");
+                break;
+            }
+            chain->output_slots[chain->output_count++] = (uint32_t)slot;
         }
-        chain->output_dtype = current_dtype;
-        chain->d_out = current_d;
+        if (status != VX_STATUS_OK) break;
+        memcpy(chain->output_name, chain->tensors[chain->output_slots[0]].name, sizeof(chain->output_name));
+        chain->output_dtype = chain->tensors[chain->output_slots[0]].dtype;
+        chain->d_out = chain->tensors[chain->output_slots[0]].d;
     } while (0);
     vxj_free(root);
     if (status != VX_STATUS_OK) chain_release(chain);
@@ -700,34 +758,47 @@ static void hip_compiled_destroy(void* compiled_instance) {
     free(compiled);
 }
 
-/* The logical specifications the core hands over must describe the same tensors as the graph. */
+/* The logical specifications the core hands over must describe the same tensors as the graph:
+ * every graph input and output by name, with its element type, a fixed last extent and one common
+ * set of leading dimensions. */
+static const VxTensorSpec* spec_named(const VxTensorSpec* specs, size_t count, const char* name) {
+    for (size_t i = 0; specs && i < count; i++)
+        if (specs[i].struct_size == sizeof(specs[i]) && specs[i].name && !strcmp(specs[i].name, name)) return &specs[i];
+    return NULL;
+}
+
 static int specs_match(const VxBackendCompileInput* input, const ChainPlan* plan, HipCompiled* compiled) {
-    const VxTensorSpec* in = &input->inputs[0];
-    const VxTensorSpec* out = &input->outputs[0];
-    if (in->struct_size != sizeof(*in) || out->struct_size != sizeof(*out) || !in->name || !out->name ||
-        strcmp(in->name, plan->input_name) || strcmp(out->name, plan->output_name) || in->dtype != plan->input_dtype ||
-        out->dtype != plan->output_dtype || in->rank != out->rank || in->rank < 1 || in->rank > VX_MAX_TENSOR_RANK ||
-        in->location != VX_MEMORY_HOST || out->location != VX_MEMORY_HOST)
+    const VxTensorSpec* first = spec_named(input->inputs, input->input_count, plan->tensors[plan->input_slots[0]].name);
+    int symbolic_rows = 1;
+    if (input->input_count != plan->input_count || input->output_count != plan->output_count || !first ||
+        first->rank < 1 || first->rank > VX_MAX_TENSOR_RANK)
         return 0;
-    const VxDimensionConstraint* last_in = &in->dimensions[in->rank - 1];
-    const VxDimensionConstraint* last_out = &out->dimensions[out->rank - 1];
-    if (last_in->kind != VX_DIMENSION_FIXED || last_in->min != (int64_t)plan->d_in || last_in->max != last_in->min ||
-        last_out->kind != VX_DIMENSION_FIXED || last_out->min != (int64_t)plan->d_out || last_out->max != last_out->min)
-        return 0;
-    compiled->rank = in->rank;
-    for (uint32_t axis = 0; axis + 1 < in->rank; axis++) {
-        const VxDimensionConstraint* a = &in->dimensions[axis];
-        const VxDimensionConstraint* b = &out->dimensions[axis];
-        if (a->min < 1 || a->max < a->min || a->multiple_of < 1 || a->min != b->min || a->max != b->max ||
-            a->multiple_of != b->multiple_of)
-            return 0;
-        compiled->lead_min[axis] = a->min;
-        compiled->lead_max[axis] = a->max;
-        compiled->lead_multiple[axis] = a->multiple_of;
+    compiled->rank = first->rank;
+    for (size_t k = 0; k < plan->input_count + plan->output_count; k++) {
+        const int is_input = k < plan->input_count;
+        const PlanTensor* t = &plan->tensors[is_input ? plan->input_slots[k] : plan->output_slots[k - plan->input_count]];
+        const VxTensorSpec* spec = is_input ? spec_named(input->inputs, input->input_count, t->name)
+                                            : spec_named(input->outputs, input->output_count, t->name);
+        const VxDimensionConstraint* last;
+        if (!spec || spec->dtype != t->dtype || spec->rank != first->rank || spec->location != VX_MEMORY_HOST) return 0;
+        last = &spec->dimensions[spec->rank - 1];
+        if (last->kind != VX_DIMENSION_FIXED || last->min != (int64_t)t->d || last->max != last->min) return 0;
+        for (uint32_t axis = 0; axis + 1 < first->rank; axis++) {
+            const VxDimensionConstraint* a = &first->dimensions[axis];
+            const VxDimensionConstraint* b = &spec->dimensions[axis];
+            if (a->min < 1 || a->max < a->min || a->multiple_of < 1 || a->min != b->min || a->max != b->max ||
+                a->multiple_of != b->multiple_of)
+                return 0;
+        }
+        if (spec->dimensions[0].kind != VX_DIMENSION_SYMBOLIC) symbolic_rows = 0;
     }
-    compiled->batch_capable = in->rank >= 2 && in->dimensions[0].kind == VX_DIMENSION_SYMBOLIC &&
-                              out->dimensions[0].kind == VX_DIMENSION_SYMBOLIC && in->dimensions[0].min <= 1 &&
-                              in->dimensions[0].multiple_of == 1 && input->independent_batch_proof_protocol &&
+    for (uint32_t axis = 0; axis + 1 < first->rank; axis++) {
+        compiled->lead_min[axis] = first->dimensions[axis].min;
+        compiled->lead_max[axis] = first->dimensions[axis].max;
+        compiled->lead_multiple[axis] = first->dimensions[axis].multiple_of;
+    }
+    compiled->batch_capable = first->rank >= 2 && symbolic_rows && first->dimensions[0].min <= 1 &&
+                              first->dimensions[0].multiple_of == 1 && input->independent_batch_proof_protocol &&
                               !strcmp(input->independent_batch_proof_protocol,
                                       VX_BACKEND_INDEPENDENT_BATCH_PROOF_PROTOCOL) &&
                               input->independent_batch_proof_identity &&
@@ -880,10 +951,10 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
             return VX_STATUS_OK;
         }
     }
-    if (input->input_count != 1 || input->output_count != 1 || !input->inputs || !input->outputs) {
-        fill_report(report, runtime, VX_STATUS_BACKEND_UNSUPPORTED, VX_STAGE_COMPILE, VX_CODE_BACKEND_UNSUPPORTED,
-                    "this provider compiles graphs with one input and one output");
-        return VX_STATUS_BACKEND_UNSUPPORTED;
+    if (!input->input_count || !input->output_count || !input->inputs || !input->outputs) {
+        fill_report(report, runtime, VX_STATUS_INVALID_ARGUMENT, VX_STAGE_COMPILE, VX_CODE_INVALID_ARGUMENT,
+                    "the compile input names no input or no output");
+        return VX_STATUS_INVALID_ARGUMENT;
     }
     status = plan_package(input->source, input->packed_arithmetic, &plan, &failure);
     if (status != VX_STATUS_OK) {
@@ -905,27 +976,31 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         return VX_STATUS_INVALID_ARGUMENT;
     }
     compiled->runtime = runtime;
-    memcpy(compiled->input_name, plan.input_name, sizeof(compiled->input_name));
-    memcpy(compiled->output_name, plan.output_name, sizeof(compiled->output_name));
-    compiled->d_in = plan.d_in;
-    compiled->d_out = plan.d_out;
-    compiled->input_dtype = plan.input_dtype;
-    compiled->output_dtype = plan.output_dtype;
-    compiled->input_element_bytes = plan.input_dtype == VX_DTYPE_F32 ? 4u : 1u;
-    compiled->output_element_bytes = plan.output_dtype == VX_DTYPE_F32 ? 4u : 1u;
-    compiled->widest_row_bytes = (uint64_t)plan.d_in * compiled->input_element_bytes;
+    memcpy(compiled->tensors, plan.tensors, sizeof(compiled->tensors));
+    compiled->tensor_count = plan.tensor_count;
+    memcpy(compiled->input_slots, plan.input_slots, sizeof(compiled->input_slots));
+    memcpy(compiled->output_slots, plan.output_slots, sizeof(compiled->output_slots));
+    compiled->input_count = plan.input_count;
+    compiled->output_count = plan.output_count;
+    for (size_t t = 0; t < plan.tensor_count; t++) {
+        const uint64_t row_bytes = (uint64_t)plan.tensors[t].d * (plan.tensors[t].dtype == VX_DTYPE_F32 ? 4u : 1u);
+        if (row_bytes > compiled->widest_row_bytes) compiled->widest_row_bytes = row_bytes;
+        compiled->all_rows_bytes += row_bytes;
+    }
 
     for (size_t i = 0; i < plan.count && status == VX_STATUS_OK; i++) {
         const PackagePlan* node = &plan.nodes[i];
         HipStage* stage = &compiled->stages[compiled->stage_count++];
         const char* family = "";
-        const uint64_t row_bytes = (uint64_t)node->d_out * (node->output_dtype == VX_DTYPE_F32 ? 4u : 1u);
         stage->kind = node->kind;
+        stage->input_slot = node->input_slot;
+        stage->output_slot = node->output_slot;
         stage->d_in = node->d_in;
         stage->d_out = node->d_out;
         stage->input_dtype = node->input_dtype;
         stage->output_dtype = node->output_dtype;
-        if (row_bytes > compiled->widest_row_bytes) compiled->widest_row_bytes = row_bytes;
+        if (node->kind == PLAN_PACKED_LINEAR && node->d_in > compiled->widest_float_row)
+            compiled->widest_float_row = node->d_in;
         if (node->kind == PLAN_QLINEAR) {
             stage->input_scale = node->input_scale;
             stage->output_scale = node->output_scale;
@@ -980,15 +1055,15 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
     attestation->graph_fingerprint = input->graph_fingerprint;
     attestation->shape_domain_proof_identity = input->shape_domain_proof_identity;
     attestation->maximum_tensor_bytes = rows_max * compiled->widest_row_bytes;
-    /* weights plus, per context, the two work buffers, the int8 staging of a PackedLinear call
-     * (at most one byte per float of its input) and row scales */
-    attestation->maximum_resident_bytes = resident + rows_max * (3u * compiled->widest_row_bytes + 8u);
+    /* weights plus, per context, one buffer per tensor of the graph, the int8 staging of a
+     * PackedLinear call (one byte per float of its input, rows padded to 16) and row scales */
+    attestation->maximum_resident_bytes = resident + rows_max * (compiled->all_rows_bytes + compiled->widest_float_row + 24u);
     attestation->resource_limit_bytes = 0;
     attestation->has_resource_limit = 0;
     attestation->packed_arithmetic = any_packed ? VX_PACKED_ARITHMETIC_DYNAMIC_I8 : input->packed_arithmetic;
     *out_compiled = compiled;
     fill_report(report, runtime, VX_STATUS_OK, VX_STAGE_COMPILE, VX_CODE_NONE,
-                node_count == 1 ? "single-node W8A8 package compiled" : "W8A8 node chain compiled");
+                node_count == 1 ? "single-node W8A8 package compiled" : "W8A8 node graph compiled");
     attest(report, compiled->stage_count, compiled->route);
     return VX_STATUS_OK;
 }
@@ -997,9 +1072,9 @@ static void hip_context_destroy(void* context_instance) {
     HipContext* context = (HipContext*)context_instance;
     if (!context) return;
     decoder_state_release(context->decode);
-    if (context->work_dev[0]) vxhip_device_free(context->work_dev[0]);
-    if (context->work_dev[1]) vxhip_device_free(context->work_dev[1]);
-    free(context->output_host);
+    for (size_t t = 0; t < MAX_GRAPH_TENSORS; t++)
+        if (context->tensor_dev[t]) vxhip_device_free(context->tensor_dev[t]);
+    for (size_t k = 0; k < MAX_GRAPH_PORTS; k++) free(context->output_host[k]);
     if (context->ctx) vxhip_context_destroy(context->ctx);
     free(context);
 }
@@ -1052,51 +1127,75 @@ static VxStatus grow_device(void** buffer, size_t* capacity, size_t bytes) {
     return VX_STATUS_OK;
 }
 
-/* Checks one binding against the compiled contract; on success the row count and output shape. */
-static int binding_admitted(const HipCompiled* compiled, const VxTensorBinding* binding, uint64_t* rows,
-                            int64_t* shape) {
-    *rows = 1;
-    if (binding->struct_size != sizeof(*binding) || !binding->name || strcmp(binding->name, compiled->input_name) ||
-        binding->dtype != compiled->input_dtype || binding->rank != compiled->rank ||
-        binding->location != VX_MEMORY_HOST || !binding->data ||
-        binding->shape[compiled->rank - 1] != (int64_t)compiled->d_in)
-        return 0;
-    for (uint32_t axis = 0; axis + 1 < compiled->rank; axis++) {
-        const int64_t extent = binding->shape[axis];
-        if (extent < compiled->lead_min[axis] || extent > compiled->lead_max[axis] ||
-            extent % compiled->lead_multiple[axis] != 0)
-            return 0;
-        *rows *= (uint64_t)extent;
-        shape[axis] = extent;
-    }
-    shape[compiled->rank - 1] = (int64_t)compiled->d_out;
-    return binding->byte_size == (size_t)*rows * compiled->d_in * compiled->input_element_bytes;
+static size_t element_bytes(VxDataType dtype) {
+    return dtype == VX_DTYPE_F32 ? 4u : 1u;
 }
 
-/* Upload, every node over all rows (each reads one work buffer and writes the other), download
- * into the context's host buffer. */
-static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, VxReport* report) {
+/* Checks the bindings of a call against the compiled contract: every graph input bound exactly
+ * once, by name, with its element type, rank, last extent and byte size, all with the same leading
+ * extents.  On success the row count, the leading extents and the data pointer of every input. */
+static int bindings_admitted(const HipCompiled* compiled, const VxTensorBinding* bindings, size_t binding_count,
+                             uint64_t* rows, int64_t* lead, const void** data) {
+    *rows = 1;
+    if (!bindings || binding_count != compiled->input_count) return 0;
+    for (size_t k = 0; k < compiled->input_count; k++) {
+        const PlanTensor* t = &compiled->tensors[compiled->input_slots[k]];
+        const VxTensorBinding* binding = NULL;
+        uint64_t binding_rows = 1;
+        for (size_t b = 0; b < binding_count; b++)
+            if (bindings[b].struct_size == sizeof(bindings[b]) && bindings[b].name && !strcmp(bindings[b].name, t->name)) {
+                if (binding) return 0; /* bound twice */
+                binding = &bindings[b];
+            }
+        if (!binding || binding->dtype != t->dtype || binding->rank != compiled->rank ||
+            binding->location != VX_MEMORY_HOST || !binding->data ||
+            binding->shape[compiled->rank - 1] != (int64_t)t->d)
+            return 0;
+        for (uint32_t axis = 0; axis + 1 < compiled->rank; axis++) {
+            const int64_t extent = binding->shape[axis];
+            if (extent < compiled->lead_min[axis] || extent > compiled->lead_max[axis] ||
+                extent % compiled->lead_multiple[axis] != 0 || (k && extent != lead[axis]))
+                return 0;
+            binding_rows *= (uint64_t)extent;
+            lead[axis] = extent;
+        }
+        if (binding->byte_size != (size_t)binding_rows * t->d * element_bytes(t->dtype)) return 0;
+        *rows = binding_rows;
+        data[k] = binding->data;
+    }
+    return 1;
+}
+
+/* Upload every input, run every node over all rows (each reads the buffer of its input tensor and
+ * writes the buffer of its output tensor), download every graph output into the context's host
+ * buffers. */
+static VxStatus run_rows(HipContext* context, const void* const* inputs, uint64_t rows, VxReport* report) {
     const HipCompiled* compiled = context->compiled;
-    const size_t input_bytes = (size_t)rows * compiled->d_in * compiled->input_element_bytes;
-    const size_t output_bytes = (size_t)rows * compiled->d_out * compiled->output_element_bytes;
-    const size_t work_bytes = (size_t)rows * (size_t)compiled->widest_row_bytes;
-    VxStatus status;
-    status = grow_device(&context->work_dev[0], &context->work_capacity[0], work_bytes);
-    if (status == VX_STATUS_OK) status = grow_device(&context->work_dev[1], &context->work_capacity[1], work_bytes);
-    if (status == VX_STATUS_OK && output_bytes > context->host_capacity) {
-        void* fresh = realloc(context->output_host, output_bytes);
-        if (!fresh) status = VX_STATUS_OUT_OF_MEMORY;
-        else {
-            context->output_host = fresh;
-            context->host_capacity = output_bytes;
+    VxStatus status = VX_STATUS_OK;
+    for (size_t t = 0; t < compiled->tensor_count && status == VX_STATUS_OK; t++)
+        status = grow_device(&context->tensor_dev[t], &context->tensor_capacity[t],
+                             (size_t)rows * compiled->tensors[t].d * element_bytes(compiled->tensors[t].dtype));
+    for (size_t k = 0; k < compiled->output_count && status == VX_STATUS_OK; k++) {
+        const PlanTensor* t = &compiled->tensors[compiled->output_slots[k]];
+        const size_t bytes = (size_t)rows * t->d * element_bytes(t->dtype);
+        if (bytes > context->host_capacity[k]) {
+            void* fresh = realloc(context->output_host[k], bytes);
+            if (!fresh) status = VX_STATUS_OUT_OF_MEMORY;
+            else {
+                context->output_host[k] = fresh;
+                context->host_capacity[k] = bytes;
+            }
         }
     }
-    if (status == VX_STATUS_OK)
-        status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->work_dev[0], input, input_bytes);
+    for (size_t k = 0; k < compiled->input_count && status == VX_STATUS_OK; k++) {
+        const PlanTensor* t = &compiled->tensors[compiled->input_slots[k]];
+        status = (VxStatus)vxhip_memcpy_to_device(context->ctx, context->tensor_dev[compiled->input_slots[k]], inputs[k],
+                                                  (size_t)rows * t->d * element_bytes(t->dtype));
+    }
     for (size_t i = 0; i < compiled->stage_count && status == VX_STATUS_OK; i++) {
         const HipStage* stage = &compiled->stages[i];
-        const void* from = context->work_dev[i & 1u];
-        void* to = context->work_dev[(i + 1u) & 1u];
+        const void* from = context->tensor_dev[stage->input_slot];
+        void* to = context->tensor_dev[stage->output_slot];
         const uint64_t elements = rows * stage->d_in;
         int handled = 0;
         switch (stage->kind) {
@@ -1124,9 +1223,12 @@ static VxStatus run_rows(HipContext* context, const void* input, uint64_t rows, 
         }
         if (!handled) status = VX_STATUS_EXECUTION_FAILED;
     }
-    if (status == VX_STATUS_OK)
-        status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host,
-                                                context->work_dev[compiled->stage_count & 1u], output_bytes);
+    for (size_t k = 0; k < compiled->output_count && status == VX_STATUS_OK; k++) {
+        const PlanTensor* t = &compiled->tensors[compiled->output_slots[k]];
+        status = (VxStatus)vxhip_memcpy_to_host(context->ctx, context->output_host[k],
+                                                context->tensor_dev[compiled->output_slots[k]],
+                                                (size_t)rows * t->d * element_bytes(t->dtype));
+    }
     if (status != VX_STATUS_OK)
         fill_report(report, compiled->runtime, status, VX_STAGE_EXECUTE, code_for(status), vxhip_last_error());
     return status;
@@ -1220,9 +1322,10 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
     HipContext* context = (HipContext*)context_instance;
     const HipCompiled* compiled;
     int64_t shape[VX_MAX_TENSOR_RANK];
+    const void* data[MAX_GRAPH_PORTS];
     uint64_t rows;
     VxStatus status;
-    if (!context || context->closed || !inputs || input_count != 1 || !sink || sink->struct_size != sizeof(*sink) ||
+    if (!context || context->closed || !inputs || !input_count || !sink || sink->struct_size != sizeof(*sink) ||
         !sink->write)
         return VX_STATUS_INVALID_ARGUMENT;
     compiled = context->compiled;
@@ -1235,12 +1338,16 @@ static VxStatus hip_context_execute(void* context_instance, const VxTensorBindin
         return status;
     }
     /* the complete batch is validated before anything is mutated */
-    if (!binding_admitted(compiled, &inputs[0], &rows, shape)) return VX_STATUS_INVALID_ARGUMENT;
-    status = run_rows(context, inputs[0].data, rows, report);
+    if (!bindings_admitted(compiled, inputs, input_count, &rows, shape, data)) return VX_STATUS_INVALID_ARGUMENT;
+    status = run_rows(context, data, rows, report);
     if (status != VX_STATUS_OK) return status;
-    status = sink->write(sink->user_data, compiled->output_name, compiled->output_dtype, shape, compiled->rank,
-                         context->output_host, (size_t)rows * compiled->d_out * compiled->output_element_bytes);
-    if (status != VX_STATUS_OK) return status;
+    for (size_t k = 0; k < compiled->output_count; k++) {
+        const PlanTensor* t = &compiled->tensors[compiled->output_slots[k]];
+        shape[compiled->rank - 1] = (int64_t)t->d;
+        status = sink->write(sink->user_data, t->name, t->dtype, shape, compiled->rank, context->output_host[k],
+                             (size_t)rows * t->d * element_bytes(t->dtype));
+        if (status != VX_STATUS_OK) return status;
+    }
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear executed");
     attest(report, compiled->stage_count, vxhip_context_last_variant(context->ctx));
     return VX_STATUS_OK;
@@ -1279,35 +1386,40 @@ static VxStatus hip_context_execute_batch(void* context_instance, const VxBacken
     HipContext* context = (HipContext*)context_instance;
     const HipCompiled* compiled;
     int64_t shape[VX_MAX_TENSOR_RANK];
+    const void* data[MAX_GRAPH_PORTS];
     uint64_t rows;
-    size_t lane_bytes;
     VxStatus status;
     if (!context || context->closed || !invocation || invocation->struct_size != sizeof(*invocation) ||
-        !invocation->stacked_inputs || invocation->stacked_input_count != 1 || !invocation->batch_size ||
+        !invocation->stacked_inputs || !invocation->stacked_input_count || !invocation->batch_size ||
         !invocation->lane_output_sinks || invocation->lane_output_sink_count != invocation->batch_size)
         return VX_STATUS_INVALID_ARGUMENT;
     compiled = context->compiled;
     if (compiled->decoder) /* the slots of a decoder are its batch: one invocation, one lane */
-        return invocation->batch_size == 1 ? hip_context_execute(context_instance, invocation->stacked_inputs, 1,
+        return invocation->batch_size == 1 ? hip_context_execute(context_instance, invocation->stacked_inputs,
+                                                                 invocation->stacked_input_count,
                                                                  &invocation->lane_output_sinks[0], report)
                                            : VX_STATUS_BACKEND_UNSUPPORTED;
     if (invocation->batch_size > 1 && !compiled->batch_capable) return VX_STATUS_BACKEND_UNSUPPORTED;
-    if (!binding_admitted(compiled, &invocation->stacked_inputs[0], &rows, shape) ||
+    if (!bindings_admitted(compiled, invocation->stacked_inputs, invocation->stacked_input_count, &rows, shape, data) ||
         shape[0] != (int64_t)invocation->batch_size)
         return VX_STATUS_INVALID_ARGUMENT;
     for (uint32_t lane = 0; lane < invocation->batch_size; lane++) {
         const VxBackendOutputSink* sink = &invocation->lane_output_sinks[lane];
         if (sink->struct_size != sizeof(*sink) || !sink->write) return VX_STATUS_INVALID_ARGUMENT;
     }
-    status = run_rows(context, invocation->stacked_inputs[0].data, rows, report);
+    status = run_rows(context, data, rows, report);
     if (status != VX_STATUS_OK) return status;
-    lane_bytes = (size_t)(rows / invocation->batch_size) * compiled->d_out * compiled->output_element_bytes;
     shape[0] = 1;
     for (uint32_t lane = 0; lane < invocation->batch_size; lane++) {
         const VxBackendOutputSink* sink = &invocation->lane_output_sinks[lane];
-        status = sink->write(sink->user_data, compiled->output_name, compiled->output_dtype, shape, compiled->rank,
-                             (const unsigned char*)context->output_host + (size_t)lane * lane_bytes, lane_bytes);
-        if (status != VX_STATUS_OK) return status;
+        for (size_t k = 0; k < compiled->output_count; k++) {
+            const PlanTensor* t = &compiled->tensors[compiled->output_slots[k]];
+            const size_t lane_bytes = (size_t)(rows / invocation->batch_size) * t->d * element_bytes(t->dtype);
+            shape[compiled->rank - 1] = (int64_t)t->d;
+            status = sink->write(sink->user_data, t->name, t->dtype, shape, compiled->rank,
+                                 (const unsigned char*)context->output_host[k] + (size_t)lane * lane_bytes, lane_bytes);
+            if (status != VX_STATUS_OK) return status;
+        }
     }
     fill_report(report, compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, "W8A8 linear batch executed");
     attest(report, compiled->stage_count, vxhip_context_last_variant(context->ctx));
