@@ -429,18 +429,20 @@ def test_rowscale_epilogue_levels_and_divisors(ctx, oracle, s_out_bits, zp_out, 
     bias_f32 = (c["bias_f32"] * (s_out / np.float32(0.05))).astype(np.float32)
     bias_i32 = np.random.default_rng(5).integers(-5000, 5000, n).astype(np.int32) if int_bias else None
     lin = vx.QLinear(c["w"], scales, c["zps"], bias_i32, I8)
-    vx.force_variant("mfma-i8")
-    try:
-        ok, y = lin.forward_rowscale(ctx, dev(c["x"]), dev(c["row_scales"]), s_out, zp_out, bias_f32=dev(bias_f32))
-        ctx.synchronize()
-    finally:
-        vx.force_variant(None)
     ok2, want, _ = oracle.qlinear_rowscale(c["x"], c["w"], scales, c["zps"], c["row_scales"], s_out, zp_out,
                                            bias_i32=bias_i32, bias_f32=bias_f32)
-    assert ok == ok2 == 1 and "mfma-i8-rowscale" in ctx.last_variant
-    y = host(y)
-    assert (y == want).all()
-    assert ((y == 127) | (y == -128)).mean() < 0.5
+    # the 32x32x32 tile the shape picks by itself, and both 16x16x64 tiles (their own epilogue code)
+    for force in ("mfma-i8", "mfma-i8-rowscale.t256x256k64", "mfma-i8-rowscale.t256x128k64"):
+        vx.force_variant(force)
+        try:
+            ok, y = lin.forward_rowscale(ctx, dev(c["x"]), dev(c["row_scales"]), s_out, zp_out, bias_f32=dev(bias_f32))
+            ctx.synchronize()
+        finally:
+            vx.force_variant(None)
+        assert ok == ok2 == 1 and "mfma-i8-rowscale" in ctx.last_variant and ("k64" in force) == ("k64" in ctx.last_variant)
+        y = host(y)
+        assert (y == want).all(), ctx.last_variant
+        assert ((y == 127) | (y == -128)).mean() < 0.5
     assert ctx.fault_flags() == 0
     lin.close()
 
@@ -522,7 +524,9 @@ def test_device_side_faults_are_raised_and_cleared(oracle):
     import torch
     import volvoxai_amd as vx
     own = vx.Context(0, torch.cuda.current_stream())  # fault bits are sticky: not the shared context
-    for rows, bad_row in ((8, 3), (160, 77)):         # the streaming GEMV and the MFMA GEMM
+    # the streaming GEMV, the 32x32x32 GEMM and (named) the 16x16x64 GEMM
+    for rows, bad_row, force in ((8, 3, None), (160, 77, None), (160, 77, "mfma-i8-rowscale.t256x128k64")):
+        vx.force_variant(force)
         c = cases.rowscale_case(rows, 256, 64, 5)
         lin = vx.QLinear(c["w"], c["scales"], c["zps"], None, I8)
         xd, bd = dev(c["x"]), dev(c["bias_f32"])
@@ -549,7 +553,9 @@ def test_device_side_faults_are_raised_and_cleared(oracle):
         _, want, _ = oracle.qlinear_rowscale(c["x"], c["w"], c["scales"], c["zps"], c["row_scales"], c["s_out"], 0,
                                              bias_f32=c["bias_f32"])
         assert ok == 1 and own.fault_flags() == 0 and (host(y) == want).all()
+        assert force is None or "k64" in own.last_variant
         lin.close()
+    vx.force_variant(None)
     own.close()
 
 
