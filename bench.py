@@ -44,8 +44,8 @@ PEAK_HBM_GBS = 8000.0     # HBM3E, MI355X
 # profiles/ (each counter scaled by what it reads for a 512 MiB copy kernel).  A counter run
 # cannot share a process with the timed run, so the measured values are carried here.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_4096x4096x4096": 101_159_415 + 16_923_819,
-    "gemv_1x4096x14336": 60_757_529 + 57_344,
+    "gemm_4096x4096x4096": 101_190_827 + 16_860_089,
+    "gemv_1x4096x14336": 60_759_162 + 57_344,
 }
 
 
@@ -449,7 +449,7 @@ def main():
         out["roofline"] = {"bound": "mfma", "achieved": ops / (wall_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS,
                            "unit": "TOP/s", "frac": ops / (wall_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                            "traffic": MEASURED_TRAFFIC_BYTES["gemm_4096x4096x4096"],
-                           "traffic_source": "profiles/gemm_mfma_rowscale_4096x4096x4096.md (FETCH_SIZE + WRITE_SIZE runs)",
+                           "traffic_source": "profiles/gemm_k64_rowscale_4096x4096x4096.md (FETCH_SIZE + WRITE_SIZE runs)",
                            "kernel": ctx.last_variant, "ops_per_launch": ops,
                            "avg_kernel_ms": wall_ms, "fastest_replay_kernel_ms": reg["graph_min_ms"],
                            "event_pair_per_launch_ms": {"mean": ev_mean, "median": ev_med, "min": ev_min},
