@@ -430,6 +430,35 @@ def test_readers_survive_mutated_documents_under_sanitizers(tmp_path):
     assert "parsed" in r.stdout and "refused" in r.stdout
 
 
+def test_package_reading_survives_mutated_graphs_under_sanitizers(tmp_path):
+    """The whole package reading -- planner, ports, fused linears, the decoder route -- built from the
+    provider's sources with AddressSanitizer and UBSan (host code only; no device is touched) and fed
+    truncations, byte pokes, digit and name edits and random corruptions of three valid graph
+    documents: a graph with branches and several ports, a boundary/linear chain, a decoder.  Every
+    mutant is accepted or refused; the program aborts on the first finding."""
+    import os
+    import subprocess
+    import test_provider_decode as decode_tests
+    from volvoxai_amd.decoder import DecoderConfig, init_weights
+    here = Path(__file__).parent / "provider_host"
+    built = subprocess.run(["make", "-C", str(here), "planner_mutations"], capture_output=True, text=True)
+    if built.returncode != 0:
+        pytest.skip("sanitizer build unavailable: " + built.stderr[-200:])
+    a, b, c, q, _ = forked_cases(3)
+    packages = [("dynamic_i8",) + tuple(forked_package(tmp_path / "forked", [3], a, b, c, q))]
+    (g, w), _ = sandwich(tmp_path / "chain", (3, 96), cases.qlinear_random_case(3, 96, 40, 34, I8, I8, I8, False))
+    packages.append(("f32", g, w))
+    cfg = DecoderConfig(layers=2, hidden=128, q_heads=2, kv_heads=1, head_dim=64, inter=128, vocab=40, group=64, max_seq=16)
+    packages.append(("dynamic_i8",) + tuple(decode_tests.decoder_package(tmp_path / "decoder", cfg, init_weights(cfg, 3), 2, 8)))
+    # (leak checking needs ptrace, which a sandbox may refuse; out-of-bounds and use-after-free checks do not)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    for arithmetic, graph, weights in packages:
+        r = subprocess.run([str(here / "planner_mutations"), str(ARITH[arithmetic]), str(tmp_path / "mutant.json"),
+                            str(graph), str(weights)], capture_output=True, text=True, timeout=300, env=env)
+        assert r.returncode == 0, (str(graph), r.stderr[-2000:])
+        assert "accepted" in r.stdout and "refused" in r.stdout
+
+
 def test_malformed_documents_are_refused(registered, tmp_path):
     k = KAT
     g, w = qlinear_package(tmp_path / "q", k["x"].shape, k["w"], k["scales"], k["zps"], k["bias"], k["s_in"], k["zp_in"],
