@@ -272,6 +272,26 @@ int vxhip_qlinear_forward(VxHipContext* context, const VxHipQLinear* linear,
                           float output_scale, int32_t output_zero_point,
                           uint32_t input_dtype, uint32_t output_dtype);
 
+/* QLinear followed by the DequantizeLinear that reads its output, in one launch:
+ * output_f32_dev [rows,d_out] = f32((q - dequant_zero_point) * dequant_scale) for
+ * the byte q that vxhip_qlinear_forward writes (DequantizeLinear,
+ * src/kernels/quantize_linear_ops.inc:9-16, applied in the linear's epilogue) --
+ * the Q -> QLinear -> DQ sandwich of an exported W8A8 graph without the byte
+ * tensor's round trip and its launch.  output_dev (optional) also receives the
+ * bytes, for a graph in which another node reads them.  The dequantization
+ * parameters are those of the DequantizeLinear node (in a valid package they
+ * equal the tensor's output_scale / output_zero_point); a scale that is not
+ * finite and positive or a zero point outside output_dtype declines.  The f32
+ * values are bit-identical to vxhip_qlinear_forward + vxhip_dequantize_forward.
+ * Returns 1 handled / 0 declined. */
+int vxhip_qlinear_forward_dequantized(VxHipContext* context, const VxHipQLinear* linear,
+                                      const void* input_dev, float* output_f32_dev,
+                                      void* output_dev, uint32_t rows,
+                                      float input_scale, int32_t input_zero_point,
+                                      float output_scale, int32_t output_zero_point,
+                                      uint32_t input_dtype, uint32_t output_dtype,
+                                      float dequant_scale, int32_t dequant_zero_point);
+
 /* Per-token activation scales: row m behaves as its own canonical QLinear
  * call with input_scale = row_scales_dev[m], input zero point 0, I8 input.
  * bias_f32_dev (optional, [d_out]) is an extension with no reference

@@ -606,6 +606,37 @@ def test_quantize_dequantize_match_oracle(oracle):
         assert ok == 1 and same_f32(d, wd)
 
 
+@pytest.mark.parametrize("rows,k,n", [(1, 96, 40), (17, 4096, 300), (32, 1024, 1024), (33, 200, 72), (200, 777, 130),
+                                      (600, 1024, 512)])
+@pytest.mark.parametrize("idt,odt", [(I8, I8), (U8, U8), (I8, U8)])
+def test_qlinear_dequantized_equals_the_two_nodes(ctx, oracle, rows, k, n, idt, odt):
+    """QLinear with the DequantizeLinear behind it folded into its epilogue
+    (native/src/kernels/quantize_linear_ops.inc:9-16 applied to each byte where it is made): the f32
+    values are those of the two operators one after the other, the bytes (asked for as well) too;
+    dequantization parameters other than the output's own are honoured; a bad one declines."""
+    import volvoxai_amd as vx
+    c = cases.qlinear_random_case(rows, k, n, 4100 + rows + n, idt, I8, odt, zero_weight_zp=(rows % 2 == 0))
+    ok, q = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"],
+                           idt, I8, odt)
+    assert ok == 1
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], c["bias"], I8)
+    xd = dev(c["x"])
+    for dq_scale, dq_zp in ((None, None), (np.float32(0.37), 3)):
+        s, z = (c["s_out"], c["zp_out"]) if dq_scale is None else (dq_scale, dq_zp)
+        _, want = oracle.dequantize(q, s, z, odt)
+        got = lin.forward_dequantized(ctx, xd, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, dequant_scale=dq_scale,
+                                      dequant_zero_point=dq_zp, want_bytes=True)
+        assert got[0] == 1 and same_f32(got[1].cpu().numpy(), want) and (got[2].cpu().numpy() == q).all(), ctx.last_variant
+        ok2, only = lin.forward_dequantized(ctx, xd, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt,
+                                            dequant_scale=dq_scale, dequant_zero_point=dq_zp)
+        assert ok2 == 1 and same_f32(only.cpu().numpy(), want)
+    for bad_scale, bad_zp in ((0.0, 0), (float("nan"), 0), (0.1, 300), (0.1, -129 if odt == I8 else -1)):
+        assert lin.forward_dequantized(ctx, xd, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt,
+                                       dequant_scale=bad_scale, dequant_zero_point=bad_zp)[0] == 0
+    assert ctx.fault_flags() == 0
+    lin.close()
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

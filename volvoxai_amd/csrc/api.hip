@@ -498,8 +498,9 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
                        const float* row_scales_dev, const float* bias_f32_dev, void* output_dev,
                        int32_t* acc_dev, uint32_t rows, float input_scale, int32_t input_zp,
                        float output_scale, int32_t output_zp, uint32_t input_dtype,
-                       uint32_t output_dtype, bool per_row) {
-    if (!ctx || !lin || !input_dev || (!output_dev && !acc_dev) || !rows) {
+                       uint32_t output_dtype, bool per_row, float* dq_dev = nullptr, float dq_scale = 0.0f,
+                       int32_t dq_zp = 0) {
+    if (!ctx || !lin || !input_dev || (!output_dev && !acc_dev && !dq_dev) || !rows) {
         set_error("qlinear_forward: null handle/tensor or zero rows");
         return 0;
     }
@@ -560,6 +561,9 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     a.n_pad = n_pad;
     a.y = output_dev;
     a.acc_out = acc_dev;
+    a.dq_out = dq_dev;
+    a.dq_scale = dq_scale;
+    a.dq_zp = dq_zp;
     a.fault = ctx->fault_dev;
     const char* id = run_linear(ctx, a);
     if (!id) {
@@ -576,6 +580,26 @@ int vxhip_qlinear_forward(VxHipContext* ctx, const VxHipQLinear* lin, const void
                           uint32_t input_dtype, uint32_t output_dtype) {
     return qlinear_run(ctx, lin, input_dev, nullptr, nullptr, output_dev, acc_dev, rows, input_scale,
                        input_zp, output_scale, output_zp, input_dtype, output_dtype, false);
+}
+
+int vxhip_qlinear_forward_dequantized(VxHipContext* ctx, const VxHipQLinear* lin, const void* input_dev,
+                                      float* output_f32_dev, void* output_dev, uint32_t rows, float input_scale,
+                                      int32_t input_zp, float output_scale, int32_t output_zp, uint32_t input_dtype,
+                                      uint32_t output_dtype, float dequant_scale, int32_t dequant_zp) {
+    if (!output_f32_dev) {
+        set_error("qlinear_forward_dequantized: null f32 output");
+        return 0;
+    }
+    // the parameters a typed DequantizeLinear is given (native/src/kernels/w8a8_affine.h:46-65): a finite positive scale and a
+    // zero point inside the byte type it reads; then q - zero_point is exact in f32 as well
+    if (!byte_dtype(output_dtype) || !scale_ok(dequant_scale) || !zero_point_ok(dequant_zp, output_dtype)) {
+        set_error("qlinear_forward_dequantized: dequantization scale %g / zero point %d not admissible", (double)dequant_scale,
+                  dequant_zp);
+        return 0;
+    }
+    return qlinear_run(ctx, lin, input_dev, nullptr, nullptr, output_dev, nullptr, rows, input_scale, input_zp,
+                       output_scale, output_zp, input_dtype, output_dtype, false, output_f32_dev, dequant_scale,
+                       dequant_zp);
 }
 
 int vxhip_qlinear_forward_rowscale(VxHipContext* ctx, const VxHipQLinear* lin, const int8_t* input_dev,

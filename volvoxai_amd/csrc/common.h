@@ -195,8 +195,13 @@ struct LinearArgs {
     uint32_t group_size, groups, n_pad;
     bool uniform_group_scales;  // scales_t[g][n] is the same for every g: a kernel may form s_a * s_w once
     // outputs
-    void* y;                // int8/uint8 [rows][n] or float [rows][n]; may be null with acc_out
+    void* y;                // int8/uint8 [rows][n] or float [rows][n]; may be null with acc_out or dq_out
     int32_t* acc_out;       // optional int32 [rows][n]
+    // requant: optional float [rows][n], the requantized value dequantized again with the parameters
+    // of the DequantizeLinear that reads it, f32((q - dq_zp) * dq_scale)
+    float* dq_out;
+    float dq_scale;
+    int32_t dq_zp;
     uint32_t* fault;
 };
 

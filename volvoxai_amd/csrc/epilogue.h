@@ -72,6 +72,14 @@ __device__ __forceinline__ int32_t requant_one(const LinearArgs& a, int32_t dot,
     return requantize(t, (float)a.out_lo, (float)a.out_hi, a.out_zp);
 }
 
+// The DequantizeLinear that reads a requantized value, applied where the value is made:
+// f32((double)(q - zp) * (double)s) (native/src/kernels/quantize_linear_ops.inc:9-16).  q - zp has at
+// most nine bits, so its product with an f32 is exact in double and rounds once: the single f32
+// multiplication below gives the same bits.
+__device__ __forceinline__ float dequantized(const LinearArgs& a, int32_t q) {
+    return __fmul_rn((float)(q - a.dq_zp), a.dq_scale);
+}
+
 // One output element (split-K tail, where a thread owns one element).
 template <int MODE>
 __device__ __forceinline__ void store_element(const LinearArgs& a, uint32_t m, uint32_t n,
@@ -86,6 +94,7 @@ __device__ __forceinline__ void store_element(const LinearArgs& a, uint32_t m, u
         const int32_t q = requant_one<MODE>(a, dot, c, row_scale, rsum, &total);
         if (a.y) ((uint8_t*)a.y)[(size_t)m * a.n + n] = (uint8_t)q;
         if (a.acc_out) a.acc_out[(size_t)m * a.n + n] = total;
+        if (a.dq_out) a.dq_out[(size_t)m * a.n + n] = dequantized(a, q);
     }
 }
 
@@ -129,6 +138,17 @@ __device__ __forceinline__ void store_quad(const LinearArgs& a, uint32_t m, uint
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 if (n + e < a.n) ao[e] = total[e];
+        }
+        if (a.dq_out) {
+            float* dq = a.dq_out + (size_t)m * a.n + n;
+            if (vec_ok) {
+                *reinterpret_cast<v4f*>(dq) = v4f{dequantized(a, q[0]), dequantized(a, q[1]), dequantized(a, q[2]),
+                                                  dequantized(a, q[3])};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (n + e < a.n) dq[e] = dequantized(a, q[e]);
+            }
         }
     }
 }

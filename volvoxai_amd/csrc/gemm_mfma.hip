@@ -587,7 +587,7 @@ bool launch_one(hipStream_t s, const LinearArgs& a) {
 template <int WN, int WM, int TN, int TM, int MODE, int GK, bool W4 = false, int NS = 2>
 bool launch_cfg(hipStream_t s, const LinearArgs& a) {
     if constexpr (MODE != (int)Epilogue::DequantF32) {
-        if ((a.n % 16u) == 0u && a.y && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u)
+        if ((a.n % 16u) == 0u && a.y && !a.acc_out && !a.dq_out && ((uintptr_t)a.y % 16u) == 0u)
             return launch_one<WN, WM, TN, TM, MODE, GK, true, false, NS>(s, a);
     }
     return launch_one<WN, WM, TN, TM, MODE, GK, false, W4, NS>(s, a);
@@ -649,7 +649,7 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (forced("t64x64")) pick = 4;
         // The two large tiles run on the 16x16x64 MFMA (gemm_k64.hip) when the straight-line epilogue
         // applies; a forced tile name without "k64" keeps the 32x32x32 kernel of this file.
-        const bool fast_ok = (a.n % 16u) == 0u && a.y && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u;
+        const bool fast_ok = (a.n % 16u) == 0u && a.y && !a.acc_out && !a.dq_out && ((uintptr_t)a.y % 16u) == 0u;
         const bool named = forced("t256x") || forced("t128x") || forced("t64x");
         if (pick <= 1 && fast_ok && (forced("k64") || !named)) return launch_gemm_k64(s, a, pick);
         if (pick == 0 && forced("wv4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256wv4" : nullptr;

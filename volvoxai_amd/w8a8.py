@@ -196,6 +196,27 @@ class QLinear:
             input_dtype, output_dtype)
         return (ok, out, accumulators) if want_accumulators else (ok, out)
 
+    def forward_dequantized(self, ctx: Context, x, input_scale, input_zero_point, output_scale, output_zero_point,
+                            input_dtype=DTYPE_I8, output_dtype=DTYPE_I8, dequant_scale=None, dequant_zero_point=None,
+                            out=None, want_bytes=False):
+        """QLinear and the DequantizeLinear behind it in one launch: returns (ok, f32 [rows, d_out][, bytes]).
+        The dequantization parameters default to the output's own."""
+        import torch
+        if x.ndim != 2 or x.shape[1] != self.d_in:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.d_in}]")
+        rows = x.shape[0]
+        in_t, out_t = _byte_dtype(input_dtype, "input_dtype"), _byte_dtype(output_dtype, "output_dtype")
+        if out is None:
+            out = torch.empty((rows, self.d_out), dtype=torch.float32, device=x.device)
+        q = torch.empty((rows, self.d_out), dtype=out_t, device=x.device) if want_bytes else None
+        ok = library().vxhip_qlinear_forward_dequantized(
+            ctx._h, self._h, _dp(x, "x", in_t), _dp(out, "out", torch.float32, (rows, self.d_out)),
+            _dp(q, "bytes", out_t, (rows, self.d_out)), rows, float(np.float32(input_scale)), int(input_zero_point),
+            float(np.float32(output_scale)), int(output_zero_point), input_dtype, output_dtype,
+            float(np.float32(output_scale if dequant_scale is None else dequant_scale)),
+            int(output_zero_point if dequant_zero_point is None else dequant_zero_point))
+        return (ok, out, q) if want_bytes else (ok, out)
+
     def forward_rowscale(self, ctx: Context, x, row_scales, output_scale, output_zero_point=0,
                          output_dtype=DTYPE_I8, bias_f32=None, out=None, want_accumulators=False,
                          accumulators=None):
