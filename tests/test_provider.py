@@ -595,7 +595,8 @@ def test_packed_linear_w4_package_matches_oracle(registered, oracle, tmp_path, r
 @pytest.mark.parametrize("rows,two", [(3, False), (40, True), (1, True)])
 def test_quantize_linear_dequantize_chain_matches_oracle(registered, oracle, tmp_path, rows, two):
     """QuantizeLinear -> QLinear (-> QGemm) -> DequantizeLinear in one compiled model: every node's
-    bytes are the oracle's, and the intermediate tensors never leave the device."""
+    bytes are the oracle's, and the intermediate tensors never leave the device (the bytes in front
+    of the DequantizeLinear are never stored at all)."""
     c1 = cases.qlinear_random_case(rows, 200, 96, 15, I8, I8, I8, False)
     c2 = cases.qlinear_random_case(rows, 96, 36, 16, I8, I8, I8, False) if two else None
     x = np.random.default_rng(3).normal(0, 40 * c1["s_in"], (rows, 200)).astype(np.float32)
@@ -618,6 +619,9 @@ def test_quantize_linear_dequantize_chain_matches_oracle(registered, oracle, tmp
     _, want = oracle.dequantize(h, last["s_out"], last["zp_out"], I8)
     assert (y.view(np.uint32) == want.view(np.uint32)).all()
     assert (b"nodes=4" if two else b"nodes=3") in r.execute_route
+    # the last QLinear and the DequantizeLinear behind it are one launch: nobody else reads its bytes
+    assert r.compile_route.endswith(b">hip.qlinear+dequantize-linear") and r.compile_route.count(b"hip.qlinear") == (2 if two else 1)
+    assert b"route=hip.qlinear." in r.execute_route  # the last launch of the execution is the linear's own
 
 
 @pytest.mark.gpu

@@ -123,6 +123,13 @@ typedef struct HipStage {
     VxHipPackedLinear* packed;
     float input_scale, output_scale; /* QLinear; the byte side of a boundary node in input_scale */
     int32_t input_zero_point, output_zero_point;
+    /* A QLinear whose bytes only a DequantizeLinear reads runs both in one launch and writes that
+     * node's f32 tensor (dequantized_slot); the DequantizeLinear stage is then marked absorbed. */
+    int dequantizes, absorbed;
+    const char* family; /* of the launch, for the route string */
+    uint32_t dequantized_slot;
+    float dequantize_scale;
+    int32_t dequantize_zero_point;
 } HipStage;
 
 struct DecoderModel;
@@ -1029,9 +1036,38 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
             stage->input_zero_point = node->boundary_zero_point;
             family = node->kind == PLAN_QUANTIZE ? "hip.quantize-linear" : "hip.dequantize-linear";
         }
+        stage->family = family;
+    }
+    /* QLinear -> DequantizeLinear with no other reader of the bytes (the tail of a Q / QLinear / DQ
+     * sandwich): one launch, no byte tensor */
+    for (size_t i = 0; i < compiled->stage_count && status == VX_STATUS_OK; i++) {
+        HipStage* linear = &compiled->stages[i];
+        size_t readers = 0, reader = 0;
+        if (linear->kind != PLAN_QLINEAR) continue;
+        for (size_t j = 0; j < compiled->stage_count; j++)
+            if (compiled->stages[j].input_slot == linear->output_slot) {
+                readers++;
+                reader = j;
+            }
+        for (size_t k = 0; k < compiled->output_count; k++)
+            if (compiled->output_slots[k] == linear->output_slot) readers += 2; /* the caller reads the bytes */
+        if (readers != 1 || reader <= i || compiled->stages[reader].kind != PLAN_DEQUANTIZE ||
+            compiled->stages[reader].input_dtype != linear->output_dtype)
+            continue;
+        linear->dequantizes = 1;
+        linear->dequantized_slot = compiled->stages[reader].output_slot;
+        linear->dequantize_scale = compiled->stages[reader].input_scale;
+        linear->dequantize_zero_point = compiled->stages[reader].input_zero_point;
+        compiled->stages[reader].absorbed = 1;
+        linear->family = "hip.qlinear+dequantize-linear";
+    }
+    /* the route names the launches of an execution, in order */
+    for (size_t i = 0; i < compiled->stage_count; i++) {
+        const HipStage* stage = &compiled->stages[i];
+        if (stage->absorbed || !stage->family) continue;
         if (route_used + 1 < sizeof(compiled->route))
             route_used += (size_t)snprintf(compiled->route + route_used, sizeof(compiled->route) - route_used, "%s%s",
-                                           i ? ">" : "", family);
+                                           route_used ? ">" : "", stage->family);
         if (route_used >= sizeof(compiled->route)) route_used = sizeof(compiled->route) - 1u;
     }
     const int any_packed = plan.any_packed;
@@ -1198,12 +1234,20 @@ static VxStatus run_rows(HipContext* context, const void* const* inputs, uint64_
         void* to = context->tensor_dev[stage->output_slot];
         const uint64_t elements = rows * stage->d_in;
         int handled = 0;
+        if (stage->absorbed) continue; /* ran inside the QLinear in front of it */
         switch (stage->kind) {
             case PLAN_QLINEAR:
-                handled = vxhip_qlinear_forward(context->ctx, stage->qlinear, from, to, NULL, (uint32_t)rows,
-                                                stage->input_scale, stage->input_zero_point, stage->output_scale,
-                                                stage->output_zero_point, (uint32_t)stage->input_dtype,
-                                                (uint32_t)stage->output_dtype);
+                if (stage->dequantizes)
+                    handled = vxhip_qlinear_forward_dequantized(
+                        context->ctx, stage->qlinear, from, (float*)context->tensor_dev[stage->dequantized_slot], NULL,
+                        (uint32_t)rows, stage->input_scale, stage->input_zero_point, stage->output_scale,
+                        stage->output_zero_point, (uint32_t)stage->input_dtype, (uint32_t)stage->output_dtype,
+                        stage->dequantize_scale, stage->dequantize_zero_point);
+                else
+                    handled = vxhip_qlinear_forward(context->ctx, stage->qlinear, from, to, NULL, (uint32_t)rows,
+                                                    stage->input_scale, stage->input_zero_point, stage->output_scale,
+                                                    stage->output_zero_point, (uint32_t)stage->input_dtype,
+                                                    (uint32_t)stage->output_dtype);
                 break;
             case PLAN_PACKED_LINEAR:
                 handled = vxhip_packed_linear_forward_f32(context->ctx, stage->packed, (const float*)from, (float*)to,
