@@ -353,6 +353,10 @@ VxHipStatus vxhip_packed_prepare_i8(VxHipContext* context,
 
 /* vx_packed_linear_forward with normalize==8, groups in {8, 4, 3, 2}
  * (src/kernels/packed_linear_ops.inc:1545-1621) on resident f32 rows.
+ * One or two rows (the reference's single-row route, :1471-1535, which prepares
+ * the row and multiplies in one call) run as one launch: the streaming kernel
+ * prepares the rows itself (route id ends in "-prep"); more rows are prepared
+ * by a launch of their own first.  The bits are the same either way.
  * Returns 0 on success, -1 on a rejected descriptor (reference convention). */
 int vxhip_packed_linear_forward_f32(VxHipContext* context,
                                     const VxHipPackedLinear* linear,

@@ -637,6 +637,40 @@ def test_qlinear_dequantized_equals_the_two_nodes(ctx, oracle, rows, k, n, idt, 
     lin.close()
 
 
+@pytest.mark.parametrize("rows", [1, 2, 3, 4])
+@pytest.mark.parametrize("k,n,group,bits", [(4096, 14336, 128, 8), (1000, 200, 32, 8), (129, 40, 64, 8), (4096, 1024, 128, 4),
+                                            (2048, 4096, 256, 8), (1024, 6144, 128, 3), (3072, 1024, 64, 2)])
+def test_few_f32_rows_are_prepared_inside_the_gemv(ctx, oracle, rows, k, n, group, bits):
+    """PackedLinear on one or two f32 rows is one launch: the streaming kernel quantizes the rows itself
+    (the reference's single-row route does both in one call, packed_linear_ops.inc:1471-1535).  Same
+    bits as the oracle and as the two launches, special rows included (all zero, denormal, huge, NaN)."""
+    import volvoxai_amd as vx
+    c = cases.packed_case(max(rows, 5), k, n, group, 8800 + rows + n, special_rows=True)
+    x = c["x"][[0, 3, 1, 2][:rows]] if rows > 1 else c["x"][:1]
+    x = np.ascontiguousarray(x)
+    if rows % 2 == 0:
+        x[rows - 1, k // 2] = np.nan   # a row that holds a NaN: every output of the row is NaN
+    w = c["w"] if bits == 8 else cases.low_bit(c["w"], bits)
+    words = oracle.pack_w8_words(w) if bits == 8 else oracle.pack_low_bit_words(w, bits)
+    _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group, bits=bits)
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=bits)
+    st, y = pl.forward_f32(ctx, dev(x))
+    ctx.synchronize()
+    # (more rows, or a K too short for eight wavefronts per workgroup, keep the two launches)
+    assert st == 0 and ctx.last_variant.endswith("-prep") == (k >= 1000 and rows <= 2) and "gemv-mfma" in ctx.last_variant, ctx.last_variant
+    assert same_f32(y.cpu().numpy(), want)
+    vx.force_variant("gemv.noprep")
+    try:
+        st2, y2 = pl.forward_f32(ctx, dev(x))
+        ctx.synchronize()
+        assert st2 == 0 and not ctx.last_variant.endswith("-prep")
+    finally:
+        vx.force_variant(None)
+    assert same_f32(y2.cpu().numpy(), want)
+    assert ctx.fault_flags() == 0
+    pl.close()
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

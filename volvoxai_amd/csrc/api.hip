@@ -853,6 +853,36 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
                          zeros, rows);
 }
 
+// Few f32 rows: one launch, the GEMV preparing the rows itself (gemv_stream.hip, PREP).  0: ran; -2: no
+// such kernel takes the call (shape, forced variant) and nothing was launched.
+static int packed_run_f32_rows(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* x, float* y, uint32_t rows) {
+    const char* force = forced_variant();
+    if (rows > kMaxPrepRows || (force && (!strstr(force, "gemv") || strstr(force, "noprep")))) return -2;
+    LinearArgs a{};
+    a.mode = Epilogue::DequantF32;
+    a.x_f32 = x;
+    a.ldx = pl->w.k;
+    a.rows = rows;
+    a.n = pl->w.n;
+    a.k = pl->w.k;
+    a.w = pl->w.data;
+    a.panels = pl->w.panels;
+    a.ksteps = pl->w.ksteps;
+    a.weight_bits = pl->w.bits;
+    a.scales_t = pl->scales_t;
+    a.bias_f32 = pl->bias;
+    a.group_size = pl->group_size;
+    a.groups = pl->groups;
+    a.uniform_group_scales = pl->uniform_scales;
+    a.n_pad = pl->w.panels * 32u;
+    a.y = y;
+    a.fault = ctx->fault_dev;
+    const char* id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
+    if (!id) return -2;
+    set_last_variant(ctx, id);
+    return 0;
+}
+
 int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,
                                     float* output_dev, uint32_t rows) {
     if (!ctx || !pl || !input_dev || !output_dev) {
@@ -862,6 +892,7 @@ int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* 
     if (!rows) return 0;
     if (!same_device(ctx, pl->device, "packed_linear_forward_f32") || !use_device(ctx->device)) return -1;
     const uint32_t k = pl->w.k;
+    if (packed_run_f32_rows(ctx, pl, input_dev, output_dev, rows) == 0) return 0;
     const uint32_t ld = (k + 15u) / 16u * 16u;
     // the prepared rows never leave this call: up to 32 rows go to the GEMV in its operand order
     const bool operand_order = rows <= kOperandOrderRows;
@@ -896,6 +927,7 @@ int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* ctx, const VxHipPacked
         (void)no_alloc_scratch(ctx->device);  // sets the error text of the failed set-up
         return -1;
     }
+    if (packed_run_f32_rows(ctx, pl, input_dev, output_dev, rows) == 0) return 0;
     const uint32_t k = pl->w.k;
     const uint32_t ld = (k + 15u) / 16u * 16u;
     const bool operand_order = rows <= kOperandOrderRows;

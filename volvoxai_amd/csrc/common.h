@@ -50,6 +50,7 @@ struct PackedWeight {
 
 constexpr uint32_t kPanelRows = 32, kStepK = 32, kPanelPad = 8, kStepPad = 4;
 constexpr uint32_t kMaxGemvRows = 32;  // the MFMA operand has 32 row slots
+constexpr uint32_t kMaxPrepRows = 2;   // f32 rows a GEMV workgroup prepares by itself (every workgroup repeats them; measured: one and two rows are faster that way than as two launches, four are not)
 
 enum FaultBits : uint32_t {
     kFaultBadMultiplier = 1u,   // a requantization multiplier was not finite and positive
@@ -165,6 +166,7 @@ enum class Epilogue : int { RequantTensor = 0, RequantRow = 1, DequantF32 = 2 };
 struct LinearArgs {
     Epilogue mode;
     const int8_t* x;        // signed activations [rows][ldx], or in operand order (GEMV only)
+    const float* x_f32;     // instead of x (DequantF32 GEMV, rows <= kMaxPrepRows): f32 rows of ldx elements, prepared in the kernel
     uint32_t ldx;
     uint32_t x_operand_order;  // see ActivationLayout; rows <= 32
     uint32_t rows, n, k;

@@ -24,6 +24,7 @@
 #include "common.h"
 #include "device_math.h"
 #include "epilogue.h"
+#include "wave_ops.h"
 
 #include <stdio.h>
 #include <string.h>
@@ -38,6 +39,7 @@ namespace {
 extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
 constexpr int kDepth = 4;  // 1 KiB blocks in flight per wave
+constexpr int kPrepPerThread = 8;  // f32 elements of a row that a thread of a preparing kernel holds
 
 __device__ __forceinline__ v4i load_stream(const int8_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
@@ -55,9 +57,19 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 // lanes are pointed at the same lines, so nothing in the stream becomes conditional, the MFMA runs
 // on a full operand whose other rows repeat the workgroup's own, and only the accumulator quads of
 // the workgroup's channels are parked, folded and stored.
-template <int MODE, int GK, int WAVES, bool W4, int SPLIT>
+//
+// PREP: the activations arrive as f32 rows (a.x_f32, at most kMaxPrepRows of them) and the workgroup
+// prepares them itself, exactly as prepare_i8_kernel does (boundary.hip): per row scale = max|x| / 127
+// with a true division, floored at 2^-126, 1 for a zero row; codes = ties-to-even(x / scale) clamped to
+// +-127; a row holding NaN or Inf gets zero codes and a NaN scale.  The codes live in LDS, where the
+// MFMA's activation operand is then read from.  Every workgroup repeats this for all rows -- a few
+// 16 KiB reads that hit L2, issued behind the first weight requests -- and the linear is one launch
+// instead of two: the single-row route of the reference (packed_linear_ops.inc:1471-1535) also
+// quantizes the row and multiplies in one call.
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT, bool PREP>
 __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
+    static_assert(F || !PREP, "f32 activations exist for the dequantizing epilogue only");
     constexpr int CH = 32 / SPLIT;     // channels of this workgroup
     constexpr int QUADS = 4 / SPLIT;   // accumulator quads (8 channels each) of this workgroup
     static_assert(F || !W4, "four-bit weights exist for the dequantizing epilogue only");
@@ -87,7 +99,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
     // row-major rows, or operand order: the row's 16-byte chunks 512 bytes apart (see
     // ActivationLayout), which makes the 64 lanes' loads of a k-step one contiguous KiB
-    const int8_t* xp = a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
+    const int8_t* xp = PREP ? nullptr : a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
     const uint32_t x_chunk_pitch = a.x_operand_order ? 16u * kOperandOrderRows : 16u;
     const uint32_t half = lane >> 5;
     const uint32_t last_chunk = (a.k - 1u) / 16u;
@@ -101,16 +113,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     v4i wbuf[kDepth], xbuf[kDepth][SPB];
     auto issue = [&](int slot, uint32_t t) {
         wbuf[slot] = load_stream(wp + (size_t)(t / SPB) * 1024u);
+        if constexpr (!PREP) {
 #pragma unroll
-        for (int h = 0; h < SPB; h++) {
-            const uint32_t chunk = min((t + h) * 2u + half, last_chunk);
-            xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
+            for (int h = 0; h < SPB; h++) {
+                const uint32_t chunk = min((t + h) * 2u + half, last_chunk);
+                xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
+            }
         }
     };
 
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
+
+    // PREP: the f32 rows are requested first of all (loads return in order: behind the weight stream
+    // they would arrive with it, in front of it they are L2 hits whose preparation then runs while the
+    // first weight blocks are on their way) and stay in registers for the two passes.
+    constexpr int PREP_ROWS = PREP ? (int)kMaxPrepRows : 1, PREP_KEPT = PREP ? kPrepPerThread : 1;
+    float xrows[PREP_ROWS][PREP_KEPT];
+    if constexpr (PREP) {
+#pragma unroll
+        for (int r = 0; r < PREP_ROWS; r++) {
+            const float* src = a.x_f32 + (size_t)min((uint32_t)r, rows - 1u) * a.ldx;
+#pragma unroll
+            for (int i = 0; i < PREP_KEPT; i++) {
+                const uint32_t j = threadIdx.x + i * WAVES * 64;
+                xrows[r][i] = ((uint32_t)r < rows && j < a.k) ? src[j] : 0.0f;
+            }
+        }
+    }
 
     // The tail's per-output operands (activation scale, bias) are requested now, so that their
     // latency hides behind the stream instead of following it.
@@ -120,7 +151,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
         for (int it = 0; it < TAIL_ITERS; it++) {
             const uint32_t o = threadIdx.x + it * WAVES * 64;
-            tail_rs[it] = a.row_scale[min(o / CH, rows - 1u)];
+            tail_rs[it] = PREP ? 0.0f : a.row_scale[min(o / CH, rows - 1u)];
             tail_bias[it] = a.bias_f32[ch0 + o % CH];  // padded to whole panels
         }
     }
@@ -166,6 +197,55 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
         }
     };
 
+    // PREP: the rows' codes [rows][ldk] and scales [rows] behind the group dots and group scales
+    __shared__ float slot_max[PREP_ROWS][WAVES];
+    __shared__ uint32_t slot_bad[PREP_ROWS][WAVES];
+    const uint32_t ldk = (a.k + 15u) / 16u * 16u;
+    int8_t* prep_codes = reinterpret_cast<int8_t*>(gemv_lds) + (size_t)a.groups * (rows + 1u) * CH * 4u;
+    float* prep_scale = reinterpret_cast<float*>(prep_codes + (size_t)rows * ldk);
+    auto prepare_rows = [&]() {
+        if constexpr (PREP) {
+#pragma unroll
+            for (int r = 0; r < PREP_ROWS; r++) {
+                float maximum = 0.0f;
+                uint32_t bad = 0u;
+#pragma unroll
+                for (int i = 0; i < PREP_KEPT; i++) {
+                    bad |= finite_f32(xrows[r][i]) ? 0u : 1u;
+                    maximum = fmaxf(maximum, fabsf(xrows[r][i]));  // fmaxf ignores a NaN operand; `bad` records it
+                }
+                maximum = wave_max(maximum);
+                bad = __builtin_amdgcn_ballot_w64(bad != 0u) != 0ull ? 1u : 0u;
+                if (lane == 0) {
+                    slot_max[r][wave] = maximum;
+                    slot_bad[r][wave] = bad;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < PREP_ROWS; r++) {
+                if ((uint32_t)r >= rows) break;
+                float maximum = slot_max[r][0];
+                uint32_t bad = slot_bad[r][0];
+#pragma unroll
+                for (int w = 1; w < WAVES; w++) {
+                    maximum = fmaxf(maximum, slot_max[r][w]);
+                    bad |= slot_bad[r][w];
+                }
+                float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+                if (scale < 0x1p-126f) scale = 0x1p-126f;
+#pragma unroll
+                for (int i = 0; i < PREP_KEPT; i++) {
+                    const uint32_t j = threadIdx.x + i * WAVES * 64;
+                    // (elements past k were loaded as zeros: the padding of the last 16-byte chunk)
+                    if (j < ldk) prep_codes[(size_t)r * ldk + j] = (int8_t)(bad ? 0 : packed_round_i8(__fdiv_rn(xrows[r][i], scale)));
+                }
+                if (threadIdx.x == 0) prep_scale[r] = bad ? __builtin_nanf("") : scale;
+            }
+            __syncthreads();  // every wave reads every row's codes
+        }
+    };
+
     auto stash_scales = [&]() {
         if constexpr (F) {
 #pragma unroll
@@ -194,7 +274,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
                         for (int d = 0; d < 4; d++)
                             wop[d] = (h == 0 ? wbuf[i][d] << 4 : wbuf[i][d]) & (int)0xf0f0f0f0u;
                     }
-                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, xbuf[i][h], acc, 0, 0, 0);
+                    v4i xop;
+                    if constexpr (PREP) {
+                        const uint32_t chunk = min(tt * 2u + half, last_chunk);
+                        xop = *reinterpret_cast<const v4i*>(prep_codes + (size_t)m * ldk + chunk * 16u);
+                    } else {
+                        xop = xbuf[i][h];
+                    }
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, xop, acc, 0, 0, 0);
                     if constexpr (F) {
                         // a group closes after GK steps (t0 is group aligned) or at the row end
                         if ((tt + 1) % GK == 0 || (!STEADY && tt + 1 == t1)) {
@@ -214,12 +301,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
         for (int i = 0; i < kDepth; i++) issue(i, t0 + i * SPB);
         stash_scales();
+        prepare_rows();
         for (; t + 2 * ROUND <= t1; t += ROUND) round(t, std::true_type{});
     } else {
 #pragma unroll
         for (int i = 0; i < kDepth; i++)
             if (t0 + i * SPB < t1) issue(i, t0 + i * SPB);
         stash_scales();
+        prepare_rows();
     }
     for (; t < t1; t += ROUND) round(t, std::false_type{});
     if constexpr (!F) park(wave);
@@ -237,7 +326,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
             const uint32_t o = threadIdx.x + it * WAVES * 64;
             if (o >= rows * CH) break;
             const uint32_t om = o / CH, on = ch0 + o % CH;
-            const float rs = tail_rs[it];
+            const float rs = PREP ? prep_scale[om] : tail_rs[it];
             float sum = 0.0f;
             const int32_t* dp = parts + o;
             const float* sp = lds_scales + o % CH;
@@ -271,9 +360,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     }
 }
 
-template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1>
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, bool PREP = false>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
-    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT>;
+    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT, PREP>;
     if (lds > 64u * 1024u) {
         static std::atomic<uint64_t> configured{0};
         if (!raise_lds_limit((const void*)kern, 160 * 1024, configured)) return false;
@@ -282,11 +371,11 @@ bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int MODE, int GK, int WAVES, bool W4>
+template <int MODE, int GK, int WAVES, bool W4, bool PREP = false>
 bool launch_split(hipStream_t s, const LinearArgs& a, size_t lds, int split) {
-    if (split == 4) return launch_panel<MODE, GK, WAVES, W4, 4>(s, a, lds);
-    if (split == 2) return launch_panel<MODE, GK, WAVES, W4, 2>(s, a, lds);
-    return launch_panel<MODE, GK, WAVES, W4, 1>(s, a, lds);
+    if (split == 4) return launch_panel<MODE, GK, WAVES, W4, 4, PREP>(s, a, lds);
+    if (split == 2) return launch_panel<MODE, GK, WAVES, W4, 2, PREP>(s, a, lds);
+    return launch_panel<MODE, GK, WAVES, W4, 1, PREP>(s, a, lds);
 }
 
 template <int MODE, int GK, bool W4 = false>
@@ -319,11 +408,31 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
         else if (force && strstr(force, "c32")) split = 1;
     }
     const size_t ch_bytes = 128u / (size_t)split;  // one row of the workgroup's channels, int32 or f32
-    const size_t lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * (a.rows + 1u) * ch_bytes
-                                                          : (size_t)waves * a.rows * ch_bytes;
+    size_t lds = MODE == (int)Epilogue::DequantF32 ? (size_t)a.groups * (a.rows + 1u) * ch_bytes
+                                                    : (size_t)waves * a.rows * ch_bytes;
+    // f32 activations: the kernel prepares them itself (codes and scales in LDS behind the rest)
+    const bool prep = a.x_f32 != nullptr;
+    if (prep) {
+        // (a thread keeps kPrepPerThread elements of every row in registers between the two passes)
+        if (MODE != (int)Epilogue::DequantF32 || a.rows > kMaxPrepRows || waves < 8 ||
+            a.k > (uint32_t)kPrepPerThread * (uint32_t)waves * 64u)
+            return nullptr;
+        lds += (size_t)a.rows * ((a.k + 15u) / 16u * 16u) + (size_t)a.rows * 4u + 16u;
+    }
     // the MFMA GEMM takes shapes whose group dots or scales do not fit
     if (lds > 156u * 1024u) return nullptr;
     bool ok = false;
+    if constexpr (MODE == (int)Epilogue::DequantF32) {
+        if (prep) {
+            ok = waves == 16 ? launch_split<MODE, GK, 16, W4, true>(s, a, lds, split)
+                             : launch_split<MODE, GK, 8, W4, true>(s, a, lds, split);
+            if (!ok) return nullptr;
+            static const char* const prep_names[3][2] = {{"wv8-prep", "wv16-prep"},
+                                                         {"wv8c16-prep", "wv16c16-prep"},
+                                                         {"wv8c8-prep", "wv16c8-prep"}};
+            return prep_names[split == 4 ? 2 : split == 2 ? 1 : 0][waves == 16 ? 1 : 0];
+        }
+    }
     if (waves == 16) ok = launch_split<MODE, GK, 16, W4>(s, a, lds, split);
     else if (waves == 8) ok = launch_split<MODE, GK, 8, W4>(s, a, lds, split);
     else if (waves == 4) ok = launch_panel<MODE, GK, 4, W4>(s, a, lds);
@@ -339,8 +448,13 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (cu_count <= 0) cu_count = 256;
-    if (a.rows == 0u || a.rows > kMaxGemvRows || ((uintptr_t)a.x % 16u) != 0u) return nullptr;
-    if (!a.x_operand_order && (a.ldx < 16u || (a.ldx % 16u) != 0u)) return nullptr;
+    if (a.rows == 0u || a.rows > kMaxGemvRows) return nullptr;
+    if (a.x_f32) {
+        if (a.ldx < a.k) return nullptr;  // f32 rows of ldx elements
+    } else {
+        if (((uintptr_t)a.x % 16u) != 0u) return nullptr;
+        if (!a.x_operand_order && (a.ldx < 16u || (a.ldx % 16u) != 0u)) return nullptr;
+    }
     static_assert(kMaxGemvRows <= kOperandOrderRows, "an operand-order buffer holds every row of a GEMV");
     if (a.weight_bits != 8u && !(a.weight_bits == 4u && a.mode == Epilogue::DequantF32)) return nullptr;
     const char* kind = nullptr;
