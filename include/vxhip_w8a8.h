@@ -292,6 +292,25 @@ int vxhip_qlinear_forward_dequantized(VxHipContext* context, const VxHipQLinear*
                                       uint32_t input_dtype, uint32_t output_dtype,
                                       float dequant_scale, int32_t dequant_zero_point);
 
+/* The whole QuantizeLinear -> QLinear -> DequantizeLinear sandwich on resident f32
+ * rows: input_f32_dev [rows,d_in] is quantized with the QLinear's own input
+ * parameters (input_scale, input_zero_point, input_dtype: QuantizeLinear,
+ * src/kernels/quantize_linear_ops.inc:156-169), multiplied, and written as
+ * bytes (output_dev, optional) and / or dequantized f32 (output_f32_dev,
+ * optional; parameters as in vxhip_qlinear_forward_dequantized) -- at least one
+ * of the two.  One or two rows against weights without zero points run as one
+ * launch (the streaming kernel quantizes the rows itself, route id ending in
+ * "-prep"); otherwise the quantization is a launch of its own first.  The
+ * results are bit-identical to the three operators in turn.
+ * Returns 1 handled / 0 declined. */
+int vxhip_qlinear_forward_f32(VxHipContext* context, const VxHipQLinear* linear,
+                              const float* input_f32_dev, float* output_f32_dev,
+                              void* output_dev, uint32_t rows,
+                              float input_scale, int32_t input_zero_point,
+                              float output_scale, int32_t output_zero_point,
+                              uint32_t input_dtype, uint32_t output_dtype,
+                              float dequant_scale, int32_t dequant_zero_point);
+
 /* Per-token activation scales: row m behaves as its own canonical QLinear
  * call with input_scale = row_scales_dev[m], input zero point 0, I8 input.
  * bias_f32_dev (optional, [d_out]) is an extension with no reference

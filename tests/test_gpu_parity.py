@@ -671,6 +671,37 @@ def test_few_f32_rows_are_prepared_inside_the_gemv(ctx, oracle, rows, k, n, grou
     pl.close()
 
 
+@pytest.mark.parametrize("rows,k,n", [(1, 4096, 4096), (2, 1024, 300), (1, 1000, 72), (2, 96, 40), (3, 4096, 512), (40, 777, 130),
+                                      (300, 256, 64)])
+@pytest.mark.parametrize("idt,odt", [(I8, I8), (U8, U8), (U8, I8)])
+def test_qlinear_on_f32_rows_equals_the_three_nodes(ctx, oracle, rows, k, n, idt, odt):
+    """QuantizeLinear -> QLinear -> DequantizeLinear through one entry point: one launch for one or two
+    rows (the streaming kernel quantizes the rows itself), the quantization as a launch of its own
+    otherwise; bytes and f32 are those of the three operators in turn, NaN, infinities and
+    half-way values in the input included; weight zero points keep the separate launches."""
+    import volvoxai_amd as vx
+    for zero_weight_zp in (True, False):
+        c = cases.qlinear_random_case(rows, k, n, 5200 + rows + n, idt, I8, odt, zero_weight_zp=zero_weight_zp)
+        rng = np.random.default_rng(rows * 7 + n)
+        x = rng.normal(0, 40 * c["s_in"], (rows, k)).astype(np.float32)
+        x[0, :6] = [np.nan, np.inf, -np.inf, 0.5 * c["s_in"], 1.5 * c["s_in"], -2.5 * c["s_in"]]
+        ok, xq = oracle.quantize(x, c["s_in"], c["zp_in"], idt)
+        ok1, q = oracle.qlinear(xq, c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"],
+                                idt, I8, odt)
+        assert ok == 1 and ok1 == 1
+        _, want = oracle.dequantize(q, c["s_out"], c["zp_out"], odt)
+        lin = vx.QLinear(c["w"], c["scales"], c["zps"], c["bias"], I8)
+        got = lin.forward_f32(ctx, dev(x), c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, want_bytes=True)
+        assert got[0] == 1 and (got[2].cpu().numpy() == q).all() and same_f32(got[1].cpu().numpy(), want), ctx.last_variant
+        inside = rows <= 2 and k >= 1000 and zero_weight_zp
+        assert ctx.last_variant.endswith("-prep") == inside, ctx.last_variant
+        ok2, only_bytes = lin.forward_f32(ctx, dev(x), c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, want_f32=False,
+                                          want_bytes=True)[::2]
+        assert ok2 == 1 and (only_bytes.cpu().numpy() == q).all()
+        lin.close()
+    assert ctx.fault_flags() == 0
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

@@ -619,8 +619,9 @@ def test_quantize_linear_dequantize_chain_matches_oracle(registered, oracle, tmp
     _, want = oracle.dequantize(h, last["s_out"], last["zp_out"], I8)
     assert (y.view(np.uint32) == want.view(np.uint32)).all()
     assert (b"nodes=4" if two else b"nodes=3") in r.execute_route
-    # the last QLinear and the DequantizeLinear behind it are one launch: nobody else reads its bytes
-    assert r.compile_route.endswith(b">hip.qlinear+dequantize-linear") and r.compile_route.count(b"hip.qlinear") == (2 if two else 1)
+    # the boundary nodes ride in the linears next to them (nobody else reads those bytes): one launch per QLinear
+    assert r.compile_route.endswith(b"route=hip.quantize-linear+qlinear>hip.qlinear+dequantize-linear" if two else
+                                    b"route=hip.quantize-linear+qlinear+dequantize-linear")
     assert b"route=hip.qlinear." in r.execute_route  # the last launch of the execution is the linear's own
 
 

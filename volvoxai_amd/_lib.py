@@ -88,6 +88,7 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_qlinear_admits": (C.c_int, [vp, f32, i32, f32, i32, u32, u32]),
         "vxhip_qlinear_forward": (C.c_int, [vp, vp, vp, vp, vp, u32, f32, i32, f32, i32, u32, u32]),
         "vxhip_qlinear_forward_dequantized": (C.c_int, [vp, vp, vp, vp, vp, u32, f32, i32, f32, i32, u32, u32, f32, i32]),
+        "vxhip_qlinear_forward_f32": (C.c_int, [vp, vp, vp, vp, vp, u32, f32, i32, f32, i32, u32, u32, f32, i32]),
         "vxhip_qlinear_forward_rowscale": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u32, f32, i32, u32]),
         "vxhip_qlinear_i8u8": (C.c_int, [vp, vp, vp, vp, vp, vp, u32, u32, u32, f32, i32, f32, i32,
                                          u32, u32, u32]),

@@ -499,8 +499,9 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
                        int32_t* acc_dev, uint32_t rows, float input_scale, int32_t input_zp,
                        float output_scale, int32_t output_zp, uint32_t input_dtype,
                        uint32_t output_dtype, bool per_row, float* dq_dev = nullptr, float dq_scale = 0.0f,
-                       int32_t dq_zp = 0) {
-    if (!ctx || !lin || !input_dev || (!output_dev && !acc_dev && !dq_dev) || !rows) {
+                       int32_t dq_zp = 0, const float* input_f32_dev = nullptr) {
+    // input_f32_dev (instead of input_dev): the rows before the QuantizeLinear that feeds this QLinear
+    if (!ctx || !lin || (!input_dev && !input_f32_dev) || (!output_dev && !acc_dev && !dq_dev) || !rows) {
         set_error("qlinear_forward: null handle/tensor or zero rows");
         return 0;
     }
@@ -511,26 +512,32 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     if (!same_device(ctx, lin->device, "qlinear_forward") || !use_device(ctx->device)) return 0;
 
     const bool flip = input_dtype == VXHIP_DTYPE_U8;
-    const bool stage = flip || (k % 16u) != 0u || ((uintptr_t)input_dev % 16u) != 0u;
+    const char* force = forced_variant();
+    // One or two f32 rows and weights without zero points: the streaming kernel quantizes the rows
+    // itself (gemv_stream.hip, PREP) and the QuantizeLinear costs no launch.  Otherwise, or when no such
+    // kernel takes the shape, it runs first, into the scratch.
+    bool quantize_inside = input_f32_dev && !per_row && rows <= kMaxPrepRows && !lin->any_zero_point && !acc_dev &&
+                           !(force && (!strstr(force, "gemv") || strstr(force, "noprep")));
+    if (input_f32_dev && (uint64_t)rows * k > UINT32_MAX) {
+        set_error("qlinear_forward: rows * k beyond 2^32 elements");
+        return 0;
+    }
+    // bytes are staged when they need flipping, padding to whole 16-byte chunks, or alignment
+    const bool stage = flip || (k % 16u) != 0u || (!input_f32_dev && ((uintptr_t)input_dev % 16u) != 0u);
     const uint32_t ld = stage ? (k + 15u) / 16u * 16u : k;
     const uint32_t n_pad = lin->w.panels * 32u;
     Carver sizes{nullptr};
     sizes.take<int32_t>(rows);
     sizes.take<int8_t>(stage ? (size_t)rows * ld : 0);
+    sizes.take<int8_t>(input_f32_dev ? (size_t)rows * k : 0);
     if (ensure_scratch(ctx, sizes.off + 256u) != VXHIP_OK) return 0;
     Carver c{(char*)ctx->scratch};
     int32_t* rowsum = c.take<int32_t>(rows);
     int8_t* staged = c.take<int8_t>(stage ? (size_t)rows * ld : 0);
+    int8_t* quantized = c.take<int8_t>(input_f32_dev ? (size_t)rows * k : 0);
 
-    if (stage || lin->any_zero_point) {
-        if (launch_stage_activations(ctx->stream, input_dev, rows, k, flip, stage ? staged : nullptr, ld,
-                                     lin->any_zero_point ? rowsum : nullptr) != VXHIP_OK)
-            return 0;
-    }
     LinearArgs a{};
     a.mode = per_row ? Epilogue::RequantRow : Epilogue::RequantTensor;
-    a.x = stage ? staged : (const int8_t*)input_dev;
-    a.ldx = ld;
     a.rows = rows;
     a.n = n;
     a.k = k;
@@ -565,7 +572,31 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
     a.dq_scale = dq_scale;
     a.dq_zp = dq_zp;
     a.fault = ctx->fault_dev;
-    const char* id = run_linear(ctx, a);
+
+    const char* id = nullptr;
+    if (quantize_inside) {
+        a.x_f32 = input_f32_dev;
+        a.x_f32_unsigned = flip ? 1u : 0u;
+        a.ldx = k;
+        id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
+        a.x_f32 = nullptr;
+    }
+    if (!id) {
+        if (input_f32_dev) {
+            if (launch_quantize(ctx->stream, input_f32_dev, rows * k, quantized, input_scale, input_zp,
+                                input_dtype == VXHIP_DTYPE_I8) != VXHIP_OK)
+                return 0;
+            input_dev = quantized;
+        }
+        if (stage || lin->any_zero_point) {
+            if (launch_stage_activations(ctx->stream, input_dev, rows, k, flip, stage ? staged : nullptr, ld,
+                                         lin->any_zero_point ? rowsum : nullptr) != VXHIP_OK)
+                return 0;
+        }
+        a.x = stage ? staged : (const int8_t*)input_dev;
+        a.ldx = ld;
+        id = run_linear(ctx, a);
+    }
     if (!id) {
         set_error("qlinear_forward: no kernel variant accepts rows=%u k=%u n=%u", rows, k, n);
         return 0;
@@ -600,6 +631,26 @@ int vxhip_qlinear_forward_dequantized(VxHipContext* ctx, const VxHipQLinear* lin
     return qlinear_run(ctx, lin, input_dev, nullptr, nullptr, output_dev, nullptr, rows, input_scale, input_zp,
                        output_scale, output_zp, input_dtype, output_dtype, false, output_f32_dev, dequant_scale,
                        dequant_zp);
+}
+
+int vxhip_qlinear_forward_f32(VxHipContext* ctx, const VxHipQLinear* lin, const float* input_f32_dev,
+                              float* output_f32_dev, void* output_dev, uint32_t rows, float input_scale,
+                              int32_t input_zp, float output_scale, int32_t output_zp, uint32_t input_dtype,
+                              uint32_t output_dtype, float dequant_scale, int32_t dequant_zp) {
+    if (!input_f32_dev || (!output_f32_dev && !output_dev)) {
+        set_error("qlinear_forward_f32: null input, or neither output");
+        return 0;
+    }
+    if (output_f32_dev &&
+        (!byte_dtype(output_dtype) || !scale_ok(dequant_scale) || !zero_point_ok(dequant_zp, output_dtype))) {
+        set_error("qlinear_forward_f32: dequantization scale %g / zero point %d not admissible", (double)dequant_scale,
+                  dequant_zp);
+        return 0;
+    }
+    // (the QuantizeLinear's own parameters are the QLinear's input scale and zero point, which its admission checks)
+    return qlinear_run(ctx, lin, nullptr, nullptr, nullptr, output_dev, nullptr, rows, input_scale, input_zp,
+                       output_scale, output_zp, input_dtype, output_dtype, false, output_f32_dev, dequant_scale,
+                       dequant_zp, input_f32_dev);
 }
 
 int vxhip_qlinear_forward_rowscale(VxHipContext* ctx, const VxHipQLinear* lin, const int8_t* input_dev,

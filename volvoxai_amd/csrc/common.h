@@ -166,7 +166,11 @@ enum class Epilogue : int { RequantTensor = 0, RequantRow = 1, DequantF32 = 2 };
 struct LinearArgs {
     Epilogue mode;
     const int8_t* x;        // signed activations [rows][ldx], or in operand order (GEMV only)
-    const float* x_f32;     // instead of x (DequantF32 GEMV, rows <= kMaxPrepRows): f32 rows of ldx elements, prepared in the kernel
+    // instead of x (GEMV, rows <= kMaxPrepRows): f32 rows of ldx elements which the kernel turns into codes
+    // itself -- DequantF32: the dynamic per-row preparation; RequantTensor: the QuantizeLinear in front
+    // of the QLinear (input_scale, input_zp; x_f32_unsigned: that node writes U8)
+    const float* x_f32;
+    uint32_t x_f32_unsigned;
     uint32_t ldx;
     uint32_t x_operand_order;  // see ActivationLayout; rows <= 32
     uint32_t rows, n, k;

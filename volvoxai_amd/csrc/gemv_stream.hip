@@ -69,7 +69,7 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT, bool PREP>
 __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
-    static_assert(F || !PREP, "f32 activations exist for the dequantizing epilogue only");
+    static_assert(MODE != (int)Epilogue::RequantRow || !PREP, "f32 activations: PackedLinear, or QLinear behind a QuantizeLinear");
     constexpr int CH = 32 / SPLIT;     // channels of this workgroup
     constexpr int QUADS = 4 / SPLIT;   // accumulator quads (8 channels each) of this workgroup
     static_assert(F || !W4, "four-bit weights exist for the dequantizing epilogue only");
@@ -201,10 +201,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     __shared__ float slot_max[PREP_ROWS][WAVES];
     __shared__ uint32_t slot_bad[PREP_ROWS][WAVES];
     const uint32_t ldk = (a.k + 15u) / 16u * 16u;
-    int8_t* prep_codes = reinterpret_cast<int8_t*>(gemv_lds) + (size_t)a.groups * (rows + 1u) * CH * 4u;
+    int8_t* prep_codes = reinterpret_cast<int8_t*>(gemv_lds) +
+                         (F ? (size_t)a.groups * (rows + 1u) * CH * 4u : (size_t)WAVES * rows * CH * 4u);
     float* prep_scale = reinterpret_cast<float*>(prep_codes + (size_t)rows * ldk);
     auto prepare_rows = [&]() {
-        if constexpr (PREP) {
+        if constexpr (PREP && !F) {
+            // QuantizeLinear in front of a QLinear: q = saturate(ties-to-even(f32(x / s) + f32(zp))), NaN -> zp
+            // (native/src/kernels/quantize_linear_ops.inc:156-169), stored as the signed byte the MFMA takes
+            // (an unsigned type's bytes have their top bit flipped, as input_zp already is)
+            const int32_t shift = a.x_f32_unsigned ? 128 : 0;
+            const float zp_f = (float)(a.input_zp + shift), lo_f = (float)(a.x_f32_unsigned ? 0 : -128),
+                        hi_f = (float)(a.x_f32_unsigned ? 255 : 127);
+#pragma unroll
+            for (int r = 0; r < PREP_ROWS; r++) {
+                if ((uint32_t)r >= rows) break;
+#pragma unroll
+                for (int i = 0; i < PREP_KEPT; i++) {
+                    const uint32_t j = threadIdx.x + i * WAVES * 64;
+                    const float v = xrows[r][i];
+                    int32_t q = a.input_zp + shift;
+                    if (v == v) {
+                        const float t = __fadd_rn(__fdiv_rn(v, a.input_scale), zp_f);
+                        q = t <= lo_f ? (int32_t)lo_f : t >= hi_f ? (int32_t)hi_f : (int32_t)__builtin_rintf(t);
+                    }
+                    if (j < ldk) prep_codes[(size_t)r * ldk + j] = (int8_t)(q - shift);
+                }
+            }
+            __syncthreads();  // every wave reads every row's codes
+        }
+        if constexpr (PREP && F) {
 #pragma unroll
             for (int r = 0; r < PREP_ROWS; r++) {
                 float maximum = 0.0f;
@@ -414,15 +439,15 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
     const bool prep = a.x_f32 != nullptr;
     if (prep) {
         // (a thread keeps kPrepPerThread elements of every row in registers between the two passes)
-        if (MODE != (int)Epilogue::DequantF32 || a.rows > kMaxPrepRows || waves < 8 ||
-            a.k > (uint32_t)kPrepPerThread * (uint32_t)waves * 64u)
+        if (MODE == (int)Epilogue::RequantRow || a.rows > kMaxPrepRows || waves < 8 ||
+            a.k > (uint32_t)kPrepPerThread * (uint32_t)waves * 64u || (MODE != (int)Epilogue::DequantF32 && a.zw))
             return nullptr;
         lds += (size_t)a.rows * ((a.k + 15u) / 16u * 16u) + (size_t)a.rows * 4u + 16u;
     }
     // the MFMA GEMM takes shapes whose group dots or scales do not fit
     if (lds > 156u * 1024u) return nullptr;
     bool ok = false;
-    if constexpr (MODE == (int)Epilogue::DequantF32) {
+    if constexpr (MODE != (int)Epilogue::RequantRow) {
         if (prep) {
             ok = waves == 16 ? launch_split<MODE, GK, 16, W4, true>(s, a, lds, split)
                              : launch_split<MODE, GK, 8, W4, true>(s, a, lds, split);

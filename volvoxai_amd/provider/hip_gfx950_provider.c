@@ -126,6 +126,10 @@ typedef struct HipStage {
     /* A QLinear whose bytes only a DequantizeLinear reads runs both in one launch and writes that
      * node's f32 tensor (dequantized_slot); the DequantizeLinear stage is then marked absorbed. */
     int dequantizes, absorbed;
+    /* ... and one whose input bytes only it reads, written by a QuantizeLinear with the linear's own input
+     * parameters, starts from that node's f32 tensor (quantized_slot; the QuantizeLinear is absorbed) */
+    int quantizes;
+    uint32_t quantized_slot;
     const char* family; /* of the launch, for the route string */
     uint32_t dequantized_slot;
     float dequantize_scale;
@@ -1061,6 +1065,27 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
         compiled->stages[reader].absorbed = 1;
         linear->family = "hip.qlinear+dequantize-linear";
     }
+    /* QuantizeLinear -> QLinear, the bytes read by nobody else and quantized with the linear's input parameters */
+    for (size_t i = 0; i < compiled->stage_count && status == VX_STATUS_OK; i++) {
+        HipStage* linear = &compiled->stages[i];
+        size_t readers = 0, writer = compiled->stage_count;
+        if (linear->kind != PLAN_QLINEAR) continue;
+        for (size_t j = 0; j < compiled->stage_count; j++) {
+            if (compiled->stages[j].input_slot == linear->input_slot) readers++;
+            if (compiled->stages[j].output_slot == linear->input_slot) writer = j;
+        }
+        for (size_t k = 0; k < compiled->output_count; k++)
+            if (compiled->output_slots[k] == linear->input_slot) readers += 2;
+        if (readers != 1 || writer >= i || compiled->stages[writer].kind != PLAN_QUANTIZE ||
+            compiled->stages[writer].output_dtype != linear->input_dtype ||
+            memcmp(&compiled->stages[writer].input_scale, &linear->input_scale, sizeof(float)) ||
+            compiled->stages[writer].input_zero_point != linear->input_zero_point)
+            continue;
+        linear->quantizes = 1;
+        linear->quantized_slot = compiled->stages[writer].input_slot;
+        compiled->stages[writer].absorbed = 1;
+        linear->family = linear->dequantizes ? "hip.quantize-linear+qlinear+dequantize-linear" : "hip.quantize-linear+qlinear";
+    }
     /* the route names the launches of an execution, in order */
     for (size_t i = 0; i < compiled->stage_count; i++) {
         const HipStage* stage = &compiled->stages[i];
@@ -1237,7 +1262,14 @@ static VxStatus run_rows(HipContext* context, const void* const* inputs, uint64_
         if (stage->absorbed) continue; /* ran inside the QLinear in front of it */
         switch (stage->kind) {
             case PLAN_QLINEAR:
-                if (stage->dequantizes)
+                if (stage->quantizes)
+                    handled = vxhip_qlinear_forward_f32(
+                        context->ctx, stage->qlinear, (const float*)context->tensor_dev[stage->quantized_slot],
+                        stage->dequantizes ? (float*)context->tensor_dev[stage->dequantized_slot] : NULL,
+                        stage->dequantizes ? NULL : to, (uint32_t)rows, stage->input_scale, stage->input_zero_point,
+                        stage->output_scale, stage->output_zero_point, (uint32_t)stage->input_dtype,
+                        (uint32_t)stage->output_dtype, stage->dequantize_scale, stage->dequantize_zero_point);
+                else if (stage->dequantizes)
                     handled = vxhip_qlinear_forward_dequantized(
                         context->ctx, stage->qlinear, from, (float*)context->tensor_dev[stage->dequantized_slot], NULL,
                         (uint32_t)rows, stage->input_scale, stage->input_zero_point, stage->output_scale,

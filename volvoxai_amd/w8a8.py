@@ -217,6 +217,25 @@ class QLinear:
             int(output_zero_point if dequant_zero_point is None else dequant_zero_point))
         return (ok, out, q) if want_bytes else (ok, out)
 
+    def forward_f32(self, ctx: Context, x, input_scale, input_zero_point, output_scale, output_zero_point,
+                    input_dtype=DTYPE_I8, output_dtype=DTYPE_I8, want_f32=True, want_bytes=False):
+        """QuantizeLinear -> QLinear [-> DequantizeLinear] on f32 rows x [rows, d_in]:
+        returns (ok, f32 or None, bytes or None)."""
+        import torch
+        if x.ndim != 2 or x.shape[1] != self.d_in:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.d_in}]")
+        rows = x.shape[0]
+        _byte_dtype(input_dtype, "input_dtype")
+        out_t = _byte_dtype(output_dtype, "output_dtype")
+        y = torch.empty((rows, self.d_out), dtype=torch.float32, device=x.device) if want_f32 else None
+        q = torch.empty((rows, self.d_out), dtype=out_t, device=x.device) if want_bytes else None
+        ok = library().vxhip_qlinear_forward_f32(
+            ctx._h, self._h, _dp(x, "x", torch.float32), _dp(y, "out", torch.float32, (rows, self.d_out)),
+            _dp(q, "bytes", out_t, (rows, self.d_out)), rows, float(np.float32(input_scale)), int(input_zero_point),
+            float(np.float32(output_scale)), int(output_zero_point), input_dtype, output_dtype,
+            float(np.float32(output_scale)), int(output_zero_point))
+        return ok, y, q
+
     def forward_rowscale(self, ctx: Context, x, row_scales, output_scale, output_zero_point=0,
                          output_dtype=DTYPE_I8, bias_f32=None, out=None, want_accumulators=False,
                          accumulators=None):
