@@ -581,6 +581,16 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
         id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
         a.x_f32 = nullptr;
     }
+    // Unsigned bytes in whole aligned 16-byte chunks, few rows, no row sums wanted: the streaming kernel
+    // flips the top bits itself and the staging launch is saved.
+    if (!id && !input_f32_dev && flip && rows <= kMaxGemvRows && (k % 16u) == 0u && ((uintptr_t)input_dev % 16u) == 0u &&
+        !lin->any_zero_point && !(force && !strstr(force, "gemv"))) {
+        a.x = (const int8_t*)input_dev;
+        a.ldx = k;
+        a.x_flip_mask = 0x80808080u;
+        id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
+        a.x_flip_mask = 0u;
+    }
     if (!id) {
         if (input_f32_dev) {
             if (launch_quantize(ctx->stream, input_f32_dev, rows * k, quantized, input_scale, input_zp,

@@ -173,6 +173,7 @@ struct LinearArgs {
     uint32_t x_f32_unsigned;
     uint32_t ldx;
     uint32_t x_operand_order;  // see ActivationLayout; rows <= 32
+    uint32_t x_flip_mask;      // GEMV only: 0x80808080 when x holds unsigned bytes (the kernel flips their top bits), else 0
     uint32_t rows, n, k;
     const int8_t* w;        // packed
     uint32_t panels, ksteps;

@@ -304,7 +304,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
                         const uint32_t chunk = min(tt * 2u + half, last_chunk);
                         xop = *reinterpret_cast<const v4i*>(prep_codes + (size_t)m * ldk + chunk * 16u);
                     } else {
-                        xop = xbuf[i][h];
+                        // (unsigned activation bytes become the signed operand here: one XOR per dword, in a
+                        // kernel that waits for memory)
+                        xop = xbuf[i][h] ^ (int)a.x_flip_mask;
                     }
                     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, xop, acc, 0, 0, 0);
                     if constexpr (F) {
