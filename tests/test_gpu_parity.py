@@ -180,6 +180,29 @@ def test_gemv_and_gemm_agree_qlinear(ctx, oracle, rows, k, n):
     assert len(seen) == (14 if n % 16 == 0 else 12), seen
 
 
+@pytest.mark.parametrize("rows,k,n", [(1, 256, 64), (9, 4096, 96), (32, 1000, 48), (40, 512, 64), (300, 1040, 272), (129, 777, 80)])
+def test_unsigned_activation_bytes_flipped_in_the_kernels(ctx, oracle, rows, k, n):
+    """U8 activations: the streaming kernel and the 16x16x64 tiles flip the bytes' top bits themselves
+    when the rows are whole aligned 16-byte chunks; other row lengths and other tiles get them staged
+    first.  The bytes are the oracle's on every route, with and without weight zero points."""
+    import volvoxai_amd as vx
+    for zero_weight_zp in (True, False):
+        c = cases.qlinear_random_case(rows, k, n, 6100 + rows, U8, I8, U8, zero_weight_zp=zero_weight_zp)
+        ok, want = oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
+                                  c["zp_out"], U8, I8, U8)
+        assert ok == 1
+        try:
+            for force in (None, "gemv", "mfma-i8.t256x256k64", "mfma-i8.t256x128k64", "mfma-i8.t128x128s4"):
+                if force == "gemv" and rows > 32:
+                    continue
+                vx.force_variant(force)
+                (ok, y), variant = run_resident_qlinear(vx, ctx, c)
+                assert ok == 1 and (y == want).all(), (variant, zero_weight_zp)
+        finally:
+            vx.force_variant(None)
+    assert ctx.fault_flags() == 0
+
+
 @pytest.mark.parametrize("group", [32, 64, 128, 256])
 @pytest.mark.parametrize("rows,k,n", [(1, 4096, 48), (5, 1000, 36), (16, 1536, 130), (32, 1024, 40), (27, 1024, 96)])
 def test_gemv_and_gemm_agree_packed(ctx, oracle, rows, k, n, group):

@@ -591,6 +591,15 @@ static int qlinear_run(VxHipContext* ctx, const VxHipQLinear* lin, const void* i
         id = launch_gemv_stream(ctx->stream, a, ctx->cu_count, force);
         a.x_flip_mask = 0u;
     }
+    // ... and so do the large-tile GEMM kernels (gemm_k64.hip, FLIP) for more rows
+    if (!id && !input_f32_dev && flip && rows > kMaxGemvRows && (k % 16u) == 0u && ((uintptr_t)input_dev % 16u) == 0u &&
+        !lin->any_zero_point && !per_row && !(force && strstr(force, "gemv"))) {
+        a.x = (const int8_t*)input_dev;
+        a.ldx = k;
+        a.x_flip_mask = 0x80808080u;
+        id = launch_gemm_mfma(ctx->stream, a, ctx->cu_count, force);
+        a.x_flip_mask = 0u;
+    }
     if (!id) {
         if (input_f32_dev) {
             if (launch_quantize(ctx->stream, input_f32_dev, rows * k, quantized, input_scale, input_zp,

@@ -31,7 +31,9 @@ extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
 
 // WN x WM wavefronts, each owning TN x TM result tiles of 16 channels x 16 rows.  MODE is the
 // requantizing Epilogue.  Two LDS stages of 128 k-bytes, i.e. two 64-wide MFMA steps each.
-template <int WN, int WM, int TN, int TM, int MODE>
+// FLIP: the activation bytes are unsigned; each activation fragment has its top bits flipped (one XOR per
+// dword) in front of the first MFMA row of the step that uses it, so that a U8 input needs no pass of its own.
+template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false>
 __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams p) {
     static_assert(MODE != (int)Epilogue::DequantF32, "requantizing epilogues only");
     static_assert(TN % 4 == 0, "the epilogue transposes four channel tiles at a time");
@@ -154,6 +156,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
         constexpr int i = decltype(i_tag)::value, s = decltype(s_tag)::value;
         static_for<TM>([&](auto j_tag) {
             constexpr int j = decltype(j_tag)::value;
+            if constexpr (FLIP && i == 0) bf[s][j] ^= (int)0x80808080u;
             acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[i], bf[s][j], acc[i][j], 0, 0, 0);
             after(j_tag);
             __builtin_amdgcn_sched_barrier(0);
@@ -547,13 +550,13 @@ bool launch_f32_as(hipStream_t s, const LinearArgs& a) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int WN, int WM, int TN, int TM, int MODE>
+template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 16, BM = WM * TM * 16;
     constexpr int LDS = 2 * ((BN / 32) * 4 + BM / 8) * 1024 + BN * 16;
     static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_k64_kernel<WN, WM, TN, TM, MODE>;
+    auto kern = gemm_k64_kernel<WN, WM, TN, TM, MODE, FLIP>;
     if (!raise_lds_limit((const void*)kern, LDS, configured)) return false;
     GemmParams p;
     p.a = a;
@@ -574,6 +577,12 @@ const char* launch_gemm_k64(hipStream_t s, const LinearArgs& a, int tile) {
     const bool row = a.mode == Epilogue::RequantRow;
     if (a.mode == Epilogue::DequantF32) return nullptr;
     constexpr int T = (int)Epilogue::RequantTensor, R = (int)Epilogue::RequantRow;
+    if (a.x_flip_mask) {
+        // unsigned activation bytes, flipped in the kernel (the per-tensor form only: per-token scales come with I8 rows)
+        if (row) return nullptr;
+        if (tile == 0) return launch_one<2, 4, 8, 4, T, true>(s, a) ? "t256x256k64" : nullptr;
+        return launch_one<2, 4, 8, 2, T, true>(s, a) ? "t256x128k64" : nullptr;
+    }
     if (tile == 0) {
         const bool ok = row ? launch_one<2, 4, 8, 4, R>(s, a) : launch_one<2, 4, 8, 4, T>(s, a);
         return ok ? "t256x256k64" : nullptr;

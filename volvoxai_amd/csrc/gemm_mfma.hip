@@ -652,6 +652,7 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         const bool fast_ok = (a.n % 16u) == 0u && a.y && !a.acc_out && !a.dq_out && ((uintptr_t)a.y % 16u) == 0u;
         const bool named = forced("t256x") || forced("t128x") || forced("t64x");
         if (pick <= 1 && fast_ok && (forced("k64") || !named)) return launch_gemm_k64(s, a, pick);
+        if (a.x_flip_mask) return nullptr;  // only those kernels flip unsigned bytes themselves: the caller stages them
         if (pick == 0 && forced("wv4")) return launch_cfg<2, 2, 4, 4, MODE, GK>(s, a) ? "t256x256wv4" : nullptr;
         if (pick == 0) return launch_cfg<2, 4, 4, 2, MODE, GK>(s, a) ? "t256x256" : nullptr;
         if (pick == 1 && forced("wv4")) return launch_cfg<2, 2, 4, 2, MODE, GK>(s, a) ? "t256x128wv4" : nullptr;
