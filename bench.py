@@ -264,6 +264,13 @@ def bench_other_configs(torch, vx, cases, ctx):
                                            "variant": octx.last_variant, "activations": "operand order",
                                            "ms_with_row_major_activations": ms_rows,
                                            "same_bits_either_way": bool(torch.equal(y.view(torch.int32), y_rows.view(torch.int32)))}
+    # one f32 row through the reference's own call shape (the row is quantized inside the call:
+    # vx_packed_linear_forward, packed_linear_ops.inc:1545-1621): one launch, the GEMV preparing the row
+    x1 = torch.from_numpy((d["a8"][:1].astype(np.float32) * d["row_scales"][:1, None]).astype(np.float32)).cuda()
+    y1 = torch.empty((1, Ng), dtype=torch.float32, device="cuda")
+    ms = region_ms(lambda i: pls[i % copies].forward_f32(ctx, x1, out=y1), 100, torch)
+    res["packed_linear_f32_row_M1_K4096_N14336"] = {"ms": ms, "variant": ctx.last_variant,
+                                                    "includes": "activation preparation, in the same launch"}
     for p in pls:
         p.close()
     # the same decode shape with four-bit weights: half the weight bytes, same scales and output
@@ -305,6 +312,15 @@ def bench_other_configs(torch, vx, cases, ctx):
         res[f"gemm_M{m}_K4096_N4096"] = {"ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12, "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                                           "variant": ctx.last_variant}
     lin.close()
+    # QuantizeLinear -> QLinear -> DequantizeLinear on one f32 row (static scales), as one call
+    q = cases.qlinear_random_case(1, 4096, 4096, 4097, vx.DTYPE_I8, vx.DTYPE_I8, vx.DTYPE_I8, True)
+    lins = [vx.QLinear(q["w"], q["scales"], q["zps"], q["bias"], vx.DTYPE_I8) for _ in range(24)]  # 24 x 16 MiB: past the Infinity Cache
+    xq = torch.from_numpy(np.random.default_rng(9).normal(0, 40 * q["s_in"], (1, 4096)).astype(np.float32)).cuda()
+    ms = region_ms(lambda i: lins[i % 24].forward_f32(ctx, xq, q["s_in"], q["zp_in"], q["s_out"], q["zp_out"]), 96, torch)
+    res["qlinear_sandwich_f32_row_M1_K4096_N4096"] = {"ms": ms, "variant": ctx.last_variant,
+                                                      "includes": "QuantizeLinear and DequantizeLinear, in the same launch"}
+    for l in lins:
+        l.close()
     # outlier-heavy large-K GEMM: f32 activations, dynamic per-token quantization, f32 out
     rows, k, n = 2048, 14336, 4096
     rng = np.random.default_rng(55)
