@@ -75,6 +75,19 @@ def test_qlinear_wrappers_refuse_wrong_tensors():
         lin.forward_rowscale(ctx, x8, fake(5), 0.05, bias_f32=fake(31), out=y8)
     with pytest.raises(ValueError, match="x: dtype"):
         lin.forward_rowscale(ctx, fake(5, 64, dtype=torch.uint8), fake(5), 0.05, out=y8)
+    # the forms that carry their boundary operators
+    with pytest.raises(ValueError, match=r"expected \[rows, 64\]"):
+        lin.forward_dequantized(ctx, fake(5, 48, dtype=torch.int8), 0.1, 0, 0.1, 0)
+    with pytest.raises(ValueError, match="x: dtype"):
+        lin.forward_dequantized(ctx, fake(5, 64), 0.1, 0, 0.1, 0, out=fake(5, 32))    # f32 rows where bytes are due
+    with pytest.raises(ValueError, match="out: shape"):
+        lin.forward_dequantized(ctx, x8, 0.1, 0, 0.1, 0, out=fake(5, 16))
+    with pytest.raises(ValueError, match="out: dtype"):
+        lin.forward_dequantized(ctx, x8, 0.1, 0, 0.1, 0, out=y8)                      # the output is f32
+    with pytest.raises(ValueError, match=r"expected \[rows, 64\]"):
+        lin.forward_f32(ctx, fake(5, 63), 0.1, 0, 0.1, 0)
+    with pytest.raises(ValueError, match="neither I8"):
+        lin.forward_f32(ctx, fake(5, 64), 0.1, 0, 0.1, 0, input_dtype=3)
 
 
 def test_packed_linear_wrappers_refuse_wrong_tensors():
