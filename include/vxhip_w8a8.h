@@ -447,6 +447,28 @@ int vxhip_dequantize_forward(VxHipContext* context, const void* input_dev,
                              int32_t zero_point, uint32_t input_dtype,
                              float* output_dev);
 
+/* RequantizeLinear, the byte-to-byte bridge between two per-tensor descriptors:
+ * the VxCopyI8U8Fn slot `requantize_linear_i8u8` of VxW8A8Ops
+ * (src/backends/w8a8_device_ops.h:33-34,116), arithmetic of
+ * requantize_linear_i8u8 (src/kernels/portable_inference_kernels.inc:2437-2463):
+ * multiplier = f32(input_scale / output_scale), then a rounded product, a
+ * rounded sum with the output zero point, ties to even, saturation.  Declines
+ * what the reference declines (dtypes, scales, zero points, a multiplier that is
+ * not finite and positive) and, like its device forms
+ * (src/backends/cuda/host/cuda_graph_quantized_boundary_shape_host.inc:246-281),
+ * unequal counts and overlapping buffers.  HOST pointers, synchronous,
+ * 1 handled / 0 declined; then the resident form. */
+int vxhip_requantize_linear_i8u8(const void* input, uint32_t input_elements,
+                                 void* output, uint32_t output_elements,
+                                 float input_scale, int32_t input_zero_point,
+                                 float output_scale, int32_t output_zero_point,
+                                 uint32_t input_dtype, uint32_t output_dtype);
+int vxhip_requantize_forward(VxHipContext* context, const void* input_dev,
+                             uint32_t elements, void* output_dev,
+                             float input_scale, int32_t input_zero_point,
+                             float output_scale, int32_t output_zero_point,
+                             uint32_t input_dtype, uint32_t output_dtype);
+
 /* ---- kernel-variant table --------------------------------------------- */
 
 /* Same record shape as VxKernelVariantRegistration

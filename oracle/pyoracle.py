@@ -92,6 +92,9 @@ class Oracle:
         L.vxo_quantize_linear.restype = C.c_int
         L.vxo_quantize_linear.argtypes = [
             _f32p, C.c_uint32, C.c_void_p, C.c_float, C.c_int32, C.c_uint32]
+        L.vxo_requantize_linear.restype = C.c_int
+        L.vxo_requantize_linear.argtypes = [C.c_void_p, C.c_uint32, C.c_float, C.c_int32, C.c_float, C.c_int32,
+                                            C.c_uint32, C.c_uint32, C.c_void_p]
         L.vxo_dequantize_linear.restype = C.c_int
         L.vxo_dequantize_linear.argtypes = [
             C.c_void_p, C.c_uint32, C.c_float, C.c_int32, C.c_uint32, _f32p]
@@ -223,6 +226,12 @@ class Oracle:
                                             int(zp), dtype, _ptr(out, _f32p))
         return int(ok), out
 
+    def requantize_linear(self, q, s_in, zp_in, s_out, zp_out, in_dtype, out_dtype):
+        out = np.zeros(q.shape, dtype=np_dtype(out_dtype))
+        ok = self.lib.vxo_requantize_linear(_ptr(q), q.size, _f(s_in), int(zp_in), _f(s_out), int(zp_out),
+                                            in_dtype, out_dtype, _ptr(out))
+        return int(ok), out
+
     def ptq_symmetric_scale(self, x):
         s = C.c_float(0)
         st = self.lib.vxo_ptq_symmetric_scale(_ptr(x, _f32p), x.size, C.byref(s))
@@ -346,6 +355,9 @@ class Reference:
         L.dequantize_linear_typed.restype = C.c_int
         L.dequantize_linear_typed.argtypes = [C.c_void_p, C.c_int, _f32p, C.c_void_p,
                                               C.c_int, _f32p, C.c_int]
+        L.requantize_linear_i8u8.restype = C.c_int
+        L.requantize_linear_i8u8.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_float, C.c_int32, C.c_float,
+                                             C.c_int32, C.c_uint32, C.c_uint32]
         L.vx_kernel_thread_pool_create.restype = C.c_void_p
         L.vx_kernel_thread_pool_create.argtypes = [C.c_int]
         L.vx_kernel_thread_pool_destroy.argtypes = [C.c_void_p]
@@ -405,6 +417,13 @@ class Reference:
     def qlinear_packed(self, x, packed, bias, w_scales, w_zps, *rest):
         return self._qcall(self.lib.vx_qlinear_i8u8_packed, x, packed, bias,
                            w_scales, w_zps, *rest)
+
+    def requantize_linear(self, q, s_in, zp_in, s_out, zp_out, in_dtype, out_dtype):
+        """requantize_linear_i8u8 of the reference build (portable_inference_kernels.inc:2437-2463)."""
+        out = np.zeros(q.shape, dtype=np_dtype(out_dtype))
+        ok = self.lib.requantize_linear_i8u8(_ptr(q), _ptr(out), q.size, _f(s_in), int(zp_in), _f(s_out), int(zp_out),
+                                             in_dtype, out_dtype)
+        return int(ok), out
 
     def packed_preferred(self, rows, k, n, w_dtype, zero_zp):
         return int(self.lib.vx_packed_q8_preferred_for_native_w8a8(

@@ -371,6 +371,31 @@ int vxo_dequantize_linear(const void* input, uint32_t elements, float scale,
     return 1;
 }
 
+/* RequantizeLinear: a byte tensor moved from one per-tensor descriptor to another
+ * (native/src/kernels/portable_inference_kernels.inc:2437-2463).  multiplier = f32(s_in / s_out);
+ * q' = saturate(ties-to-even(f32(f32(f32(q - zp_in) * multiplier) + f32(zp_out)))): the product and
+ * the sum are rounded separately.  Declines a scale that is not finite and positive, a zero point
+ * outside its type, and a multiplier that is not finite and positive. */
+int vxo_requantize_linear(const void* input, uint32_t elements, float input_scale,
+                          int32_t input_zero_point, float output_scale, int32_t output_zero_point,
+                          uint32_t input_dtype, uint32_t output_dtype, void* output) {
+    if (!input || !output || !elements || !byte_dtype(input_dtype) || !byte_dtype(output_dtype) ||
+        !scale_ok(input_scale) || !scale_ok(output_scale) || !zero_point_ok(input_zero_point, input_dtype) ||
+        !zero_point_ok(output_zero_point, output_dtype))
+        return 0;
+    const volatile float multiplier = input_scale / output_scale;
+    if (!scale_ok(multiplier)) return 0;
+    const int32_t lo = output_dtype == VXO_DTYPE_I8 ? -128 : 0;
+    const int32_t hi = output_dtype == VXO_DTYPE_I8 ? 127 : 255;
+    for (uint32_t i = 0; i < elements; i++) {
+        const float centered = (float)(load_byte(input, input_dtype, i) - input_zero_point);
+        const volatile float scaled = centered * multiplier;
+        const volatile float transformed = scaled + (float)output_zero_point;
+        store_byte(output, output_dtype, i, vxo_requantize(transformed, lo, hi, output_zero_point));
+    }
+    return 1;
+}
+
 /* ---- PTQ rules used to synthesise inputs ------------------------------ */
 
 static double round_ties_even_f64(double v) {

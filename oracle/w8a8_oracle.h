@@ -127,6 +127,10 @@ int vxo_quantize_linear(const float* input, uint32_t elements, void* output,
 /* src/kernels/quantize_linear_ops.inc:9-16, :95-128 */
 int vxo_dequantize_linear(const void* input, uint32_t elements, float scale,
                           int32_t zero_point, uint32_t dtype, float* output);
+/* RequantizeLinear (portable_inference_kernels.inc:2437-2463): 1 done / 0 declined. */
+int vxo_requantize_linear(const void* input, uint32_t elements, float input_scale,
+                          int32_t input_zero_point, float output_scale, int32_t output_zero_point,
+                          uint32_t input_dtype, uint32_t output_dtype, void* output);
 
 /* src/training/quantization.c:142-160: symmetric per-tensor activation scale
  * s = f32(max|x| / 127.0) computed in double; 1.0 for an all-zero tensor. */

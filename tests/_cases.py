@@ -141,6 +141,17 @@ def rowscale_case(rows, d_in, d_out, seed, with_bias=True):
                 bias_f32=bias, s_out=np.float32(0.05), zp_out=0)
 
 
+def requantize_case(elements, seed, input_dtype=DTYPE_I8, output_dtype=DTYPE_I8):
+    """RequantizeLinear inputs: every byte value in random order, two descriptors whose ratio puts a
+    good part of the outputs into saturation."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 256, elements).astype(np.uint8).view(np.int8 if input_dtype == DTYPE_I8 else np.uint8)
+    s_in, s_out = np.float32(rng.uniform(0.005, 0.08)), np.float32(rng.uniform(0.005, 0.08))
+    zp_in = int(rng.integers(-40, 40)) if input_dtype == DTYPE_I8 else int(rng.integers(90, 170))
+    zp_out = int(rng.integers(-40, 40)) if output_dtype == DTYPE_I8 else int(rng.integers(90, 170))
+    return dict(x=x, s_in=s_in, zp_in=zp_in, s_out=s_out, zp_out=zp_out, in_dtype=input_dtype, out_dtype=output_dtype)
+
+
 def packed_case(rows, k, n, group, seed, with_bias=True, special_rows=False):
     """PackedLinear inputs: f32 activations, W8 codes, group scales."""
     rng = np.random.default_rng(seed)

@@ -4,7 +4,7 @@ Run in a container that has the reference tree:  the kernels are compiled from
 their sources by `make -C oracle ref` into oracle/_ref/libvxref.so, and every
 expected value below is an output of those kernels (qlinear_i8u8,
 vx_qlinear_i8u8_native, vx_qlinear_i8u8_packed, vx_llm_forward_f32,
-volvoxai_ptq_pack_bias_i32) on the seeded inputs of tests/_cases.py.  Large
+volvoxai_ptq_pack_bias_i32, requantize_linear_i8u8) on the seeded inputs of tests/_cases.py.  Large
 outputs are stored as a SHA-256 plus a leading slice; small ones whole.
 
     python tests/golden/make_reference_vectors.py
@@ -76,6 +76,10 @@ PACKED_CASES = [dict(rows=r, k=k, n=n, group=g, seed=s, with_bias=b, special_row
     (200, 768, 136, 256, 44, True, True)]]
 
 
+REQUANTIZE_CASES = [dict(elements=e, seed=s, input_dtype=i, output_dtype=o) for (e, s, i, o) in [
+    (4096, 51, I8, I8), (4096, 52, I8, U8), (4096, 53, U8, I8), (4096, 54, U8, U8), (100003, 55, I8, I8), (7, 56, U8, I8)]]
+
+
 def build_case(kind, params):
     if kind == "isa_parity":
         return cases.isa_parity_case(**params)
@@ -89,7 +93,8 @@ def main():
     orc = Oracle()
     out = {"_comment": "Outputs of the reference's C kernels on the seeded inputs of tests/_cases.py; "
                        "written by tests/golden/make_reference_vectors.py.",
-           "qlinear": [], "rowscale": [], "packed": [], "packed_w4": [], "packed_w3": [], "packed_w2": []}
+           "qlinear": [], "rowscale": [], "packed": [], "packed_w4": [], "packed_w3": [], "packed_w2": [],
+           "requantize": []}
     for kind, params in QLINEAR_CASES:
         c = build_case(kind, params)
         args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
@@ -129,6 +134,11 @@ def main():
             st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
             assert st == 0
             out[f"packed_w{bits}"].append({"params": params, "expected": digest(y)})
+    for params in REQUANTIZE_CASES:
+        c = cases.requantize_case(**params)
+        ok, y = ref.requantize_linear(c["x"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"], c["out_dtype"])
+        assert ok == 1
+        out["requantize"].append({"params": params, "expected": digest(y)})
     path = Path(__file__).with_name("reference_vectors.json")
     path.write_text(json.dumps(out, indent=1) + "\n")
     print("wrote", path, path.stat().st_size, "bytes")

@@ -725,6 +725,43 @@ def test_qlinear_on_f32_rows_equals_the_three_nodes(ctx, oracle, rows, k, n, idt
     assert ctx.fault_flags() == 0
 
 
+@pytest.mark.parametrize("entry", VECTORS["requantize"], ids=lambda e: "x".join(str(v) for v in e["params"].values()))
+def test_requantize_reference_vectors(ctx, oracle, entry):
+    """RequantizeLinear: the bytes of the reference's own kernel (committed digests), through the host-pointer
+    drop-in and the resident entry, on aligned and on unaligned tensors."""
+    import volvoxai_amd as vx
+    c = cases.requantize_case(**entry["params"])
+    args = (c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"], c["out_dtype"])
+    ok, y = vx.requantize_linear_i8u8(c["x"], *args)
+    assert ok == 1 and sha(y) == entry["expected"]["sha256"]
+    ok2, want = oracle.requantize_linear(c["x"], *args)
+    assert ok2 == 1 and (y == want).all()
+    xd = dev(np.concatenate([np.zeros(3, c["x"].dtype), c["x"]]))[3:]   # three bytes off a 16-byte boundary
+    ok3, yd = vx.requantize_forward(ctx, xd.contiguous() if False else xd, *args)
+    ctx.synchronize()
+    assert ok3 == 1 and (host(yd) == want).all() and ctx.last_variant == "hip.requantize-linear.elementwise"
+    ok4, ya = vx.requantize_forward(ctx, dev(c["x"]), *args)
+    ctx.synchronize()
+    assert ok4 == 1 and (host(ya) == want).all()
+
+
+def test_requantize_declines(oracle):
+    import volvoxai_amd as vx
+    x = np.arange(-8, 8).astype(np.int8)
+    for args in ((0.0, 0, 1.0, 0, I8, I8), (1.0, 0, float("nan"), 0, I8, I8), (1.0, 128, 1.0, 0, I8, I8),
+                 (1.0, 0, 1.0, -1, I8, U8), (3e38, 0, 1e-38, 0, I8, I8), (1e-38, 0, 3e38, 0, I8, I8), (1.0, 0, 1.0, 0, 3, I8)):
+        assert oracle.requantize_linear(x, *args)[0] == 0
+        ok, y = vx.requantize_linear_i8u8(x, *args)
+        assert ok == 0 and not y.any(), args   # declined, output untouched
+    # unequal counts and overlapping buffers, as the reference's device forms refuse them
+    lib = vx.library()
+    buf = np.zeros(64, np.int8)
+    p = buf.ctypes.data
+    import ctypes as C
+    call = lambda a, na, b, nb: lib.vxhip_requantize_linear_i8u8(C.c_void_p(a), na, C.c_void_p(b), nb, 1.0, 0, 0.5, 0, I8, I8)
+    assert call(p, 16, p + 32, 8) == 0 and call(p, 16, p + 8, 16) == 0 and call(p, 16, p + 16, 16) == 1
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

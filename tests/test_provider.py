@@ -625,6 +625,69 @@ def test_quantize_linear_dequantize_chain_matches_oracle(registered, oracle, tmp
     assert b"route=hip.qlinear." in r.execute_route  # the last launch of the execution is the linear's own
 
 
+def requantize_chain(tmp, rows, mutate=None):
+    """QuantizeLinear -> QLinear -> RequantizeLinear (I8 -> U8, other scale) -> QLinear -> DequantizeLinear."""
+    c1 = cases.qlinear_random_case(rows, 128, 64, 41, I8, I8, I8, True)
+    c2 = cases.qlinear_random_case(rows, 64, 48, 42, U8, I8, I8, True)
+    tensors = {"in.s": np.array([c1["s_in"]], np.float32), "in.z": np.array([c1["zp_in"]], np.int8),
+               "w1": c1["w"], "w1.s": c1["scales"], "w1.z": c1["zps"].astype(np.int8), "b1": c1["bias"],
+               "h.s": np.array([c1["s_out"]], np.float32), "h.z": np.array([c1["zp_out"]], np.int8),
+               "r.s": np.array([c2["s_in"]], np.float32), "r.z": np.array([c2["zp_in"]], np.uint8),
+               "w2": c2["w"], "w2.s": c2["scales"], "w2.z": c2["zps"].astype(np.int8), "b2": c2["bias"],
+               "y.s": np.array([c2["s_out"]], np.float32), "y.z": np.array([c2["zp_out"]], np.int8)}
+    affine = {"xq": ("in.s", "in.z"), "w1": ("w1.s", "w1.z", 0), "hq": ("h.s", "h.z"), "rq": ("r.s", "r.z"),
+              "w2": ("w2.s", "w2.z", 0), "yq": ("y.s", "y.z")}
+    nodes = [("q", "QuantizeLinear", {"scale": "in.s", "zero_point": "in.z"}, "xq", 128, "int8", {}),
+             ("fc1", "QLinear", {"weight": "w1", "bias": "b1"}, "hq", 64, "int8", {}),
+             ("bridge", "RequantizeLinear", {}, "rq", 64, "uint8", {}),
+             ("fc2", "QLinear", {"weight": "w2", "bias": "b2"}, "yq", 48, "int8", {}),
+             ("dq", "DequantizeLinear", {"scale": "y.s", "zero_point": "y.z"}, "y", 48, "float32", {})]
+    if mutate:
+        mutate(nodes, tensors, affine)
+    return chain_package(tmp, (rows, 128), "x", "float32", nodes, tensors, affine), c1, c2
+
+
+def test_reads_requantize_nodes(registered, tmp_path):
+    """RequantizeLinear between two QLinear nodes is read with the descriptors of its two byte tensors; a
+    float side, a changed width or a missing descriptor is refused."""
+    (g, w), _, _ = requantize_chain(tmp_path / "ok", 3)
+    assert inspect(registered, g, w)[0] == 0
+
+    def to_float(nodes, tensors, affine):
+        nodes[2] = nodes[2][:5] + ("float32",) + nodes[2][6:]
+
+    def widen(nodes, tensors, affine):
+        nodes[2] = nodes[2][:4] + (80,) + nodes[2][5:]
+
+    def undescribed(nodes, tensors, affine):
+        del affine["rq"]
+
+    for name, mutate in (("float", to_float), ("wide", widen), ("bare", undescribed)):
+        (g, w), _, _ = requantize_chain(tmp_path / name, 3, mutate)
+        assert inspect(registered, g, w)[0] == -5, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [1, 37])
+def test_requantize_chain_matches_oracle(registered, oracle, tmp_path, rows):
+    """The five-node chain through the provider: the f32 rows are those of the oracle's five operators in
+    turn (the bridge changes type, scale and zero point between the two linears)."""
+    (g, w), c1, c2 = requantize_chain(tmp_path / "c", rows)
+    x = np.random.default_rng(5).normal(0, 40 * c1["s_in"], (rows, 128)).astype(np.float32)
+    r, y = run(registered, g, w, x, "x", "f32", "y", "f32", 48)
+    assert r.status == 0, r.message
+    _, xq = oracle.quantize(x, c1["s_in"], c1["zp_in"], I8)
+    ok1, h = oracle.qlinear(xq, c1["w"], c1["bias"], c1["scales"], c1["zps"], c1["s_in"], c1["zp_in"], c1["s_out"], c1["zp_out"],
+                            I8, I8, I8)
+    ok2, rq = oracle.requantize_linear(h, c1["s_out"], c1["zp_out"], c2["s_in"], c2["zp_in"], I8, U8)
+    ok3, q = oracle.qlinear(rq, c2["w"], c2["bias"], c2["scales"], c2["zps"], c2["s_in"], c2["zp_in"], c2["s_out"], c2["zp_out"],
+                            U8, I8, I8)
+    assert ok1 == ok2 == ok3 == 1
+    _, want = oracle.dequantize(q, c2["s_out"], c2["zp_out"], I8)
+    assert (y.view(np.uint32) == want.view(np.uint32)).all()
+    assert b"hip.requantize-linear" in r.compile_route and b"nodes=5" in r.execute_route
+
+
 @pytest.mark.gpu
 def test_packed_linear_chain_matches_oracle(registered, oracle, tmp_path):
     """Two PackedLinear nodes (W8 then W4) back to back: the f32 rows of the first are what the second

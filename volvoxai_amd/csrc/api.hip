@@ -1081,6 +1081,57 @@ int vxhip_dequantize_forward(VxHipContext* ctx, const void* input_dev, uint32_t 
                              output_dev) == VXHIP_OK;
 }
 
+// the descriptor checks of requantize_linear_i8u8 (portable_inference_kernels.inc:2441-2449); the multiplier on success
+static bool requantize_admission(float input_scale, int32_t input_zp, float output_scale, int32_t output_zp,
+                                 uint32_t input_dtype, uint32_t output_dtype, float* multiplier) {
+    if (!byte_dtype(input_dtype) || !byte_dtype(output_dtype) || !scale_ok(input_scale) || !scale_ok(output_scale) ||
+        !zero_point_ok(input_zp, input_dtype) || !zero_point_ok(output_zp, output_dtype))
+        return false;
+    volatile float m = input_scale / output_scale;
+    *multiplier = m;
+    return scale_ok(m);
+}
+
+int vxhip_requantize_forward(VxHipContext* ctx, const void* input_dev, uint32_t elements, void* output_dev,
+                             float input_scale, int32_t input_zp, float output_scale, int32_t output_zp,
+                             uint32_t input_dtype, uint32_t output_dtype) {
+    float multiplier = 0.0f;
+    if (!ctx || !input_dev || !output_dev || !elements ||
+        !requantize_admission(input_scale, input_zp, output_scale, output_zp, input_dtype, output_dtype, &multiplier))
+        return 0;
+    if (!use_device(ctx->device)) return 0;
+    set_last_variant(ctx, "hip.requantize-linear.elementwise");
+    return launch_requantize(ctx->stream, input_dev, elements, output_dev, multiplier, input_zp, output_zp,
+                             input_dtype == VXHIP_DTYPE_I8, output_dtype == VXHIP_DTYPE_I8) == VXHIP_OK;
+}
+
+int vxhip_requantize_linear_i8u8(const void* input, uint32_t input_elements, void* output, uint32_t output_elements,
+                                 float input_scale, int32_t input_zp, float output_scale, int32_t output_zp,
+                                 uint32_t input_dtype, uint32_t output_dtype) {
+    float multiplier = 0.0f;
+    // (the device form's own refusals as well: equal counts, no overlap --
+    // cuda_graph_quantized_boundary_shape_host.inc:257-265)
+    if (!input || !output || !input_elements || input_elements != output_elements ||
+        !requantize_admission(input_scale, input_zp, output_scale, output_zp, input_dtype, output_dtype, &multiplier))
+        return 0;
+    const uintptr_t a = (uintptr_t)input, b = (uintptr_t)output;
+    if (a < b + output_elements && b < a + input_elements) return 0;
+    VxHipContext* ctx = default_context();
+    if (!ctx) return 0;
+    void *xd = nullptr, *yd = nullptr;
+    int ok = 0;
+    if (hipMalloc(&xd, input_elements) == hipSuccess && hipMalloc(&yd, output_elements) == hipSuccess &&
+        vxhip_memcpy_to_device(ctx, xd, input, input_elements) == VXHIP_OK) {
+        ok = vxhip_requantize_forward(ctx, xd, input_elements, yd, input_scale, input_zp, output_scale, output_zp,
+                                      input_dtype, output_dtype);
+        if (ok && vxhip_memcpy_to_host(ctx, output, yd, output_elements) != VXHIP_OK) ok = 0;
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    if (xd) (void)hipFree(xd);
+    if (yd) (void)hipFree(yd);
+    return ok;
+}
+
 int vxhip_quantize_typed_f32_i8u8(const float* input, uint32_t elements, void* output, float scale,
                                   int32_t zp, uint32_t dtype) {
     if (!input || !output || !byte_dtype(dtype) || !scale_ok(scale) || !zero_point_ok(zp, dtype)) return 0;

@@ -282,6 +282,51 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
     y[i] = (float)((double)(q - zp) * (double)scale);
 }
 
+// RequantizeLinear: q' = saturate(ties-to-even(f32(f32(f32(q - zp_in) * m) + f32(zp_out)))), m = f32(s_in / s_out)
+// formed by the host (native/src/kernels/portable_inference_kernels.inc:2437-2463); 16 bytes per thread
+// where the tensors allow it.
+__device__ __forceinline__ uint32_t requantize_byte(uint32_t byte, uint32_t in_i8, int32_t zp_in, float m, float zp_out_f,
+                                                    float lo_f, float hi_f) {
+    const int32_t q = in_i8 ? (int32_t)(int8_t)byte : (int32_t)byte;
+    const float t = __fadd_rn(__fmul_rn((float)(q - zp_in), m), zp_out_f);
+    // (t is finite: a byte difference times a finite multiplier plus a byte)
+    return (uint32_t)(int32_t)__builtin_rintf(fminf(fmaxf(t, lo_f), hi_f)) & 255u;
+}
+__global__ __launch_bounds__(256) void requantize_kernel(const uint8_t* __restrict__ x, uint32_t n, uint8_t* __restrict__ y,
+                                                         float m, int32_t zp_in, int32_t zp_out, uint32_t in_i8,
+                                                         uint32_t out_i8, uint32_t vectors) {
+    const float zp_out_f = (float)zp_out, lo_f = out_i8 ? -128.0f : 0.0f, hi_f = out_i8 ? 127.0f : 255.0f;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < vectors) {
+        const uint4 v = reinterpret_cast<const uint4*>(x)[i];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            o[d] = 0u;
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                o[d] |= requantize_byte((w[d] >> (8 * b)) & 255u, in_i8, zp_in, m, zp_out_f, lo_f, hi_f) << (8 * b);
+        }
+        reinterpret_cast<uint4*>(y)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        const uint32_t e = vectors * 16u + (i - vectors);  // the tail (or everything, for unaligned tensors) byte by byte
+        if (e < n) y[e] = (uint8_t)requantize_byte(x[e], in_i8, zp_in, m, zp_out_f, lo_f, hi_f);
+    }
+}
+
+VxHipStatus launch_requantize(hipStream_t s, const void* x, uint32_t n, void* y, float multiplier, int32_t zp_in,
+                              int32_t zp_out, bool in_i8, bool out_i8) {
+    if (!n) return VXHIP_OK;
+    const bool aligned = ((uintptr_t)x % 16u) == 0u && ((uintptr_t)y % 16u) == 0u;
+    const uint32_t vectors = aligned ? n / 16u : 0u;
+    const uint32_t threads = vectors + (n - vectors * 16u);
+    hipLaunchKernelGGL(requantize_kernel, dim3((threads + 255u) / 256u), dim3(256), 0, s, (const uint8_t*)x, n,
+                       (uint8_t*)y, multiplier, zp_in, zp_out, in_i8 ? 1u : 0u, out_i8 ? 1u : 0u, vectors);
+    VXHIP_TRY(hipGetLastError());
+    return VXHIP_OK;
+}
+
 VxHipStatus launch_quantize(hipStream_t s, const float* x, uint32_t n, void* y, float scale,
                             int32_t zp, bool is_i8) {
     if (!n) return VXHIP_OK;

@@ -151,6 +151,8 @@ VxHipStatus launch_prepare_i8(hipStream_t s, const float* x, uint32_t rows, uint
 // operand-order activations (rows <= 32, k codes each) back to row-major rows of ld bytes
 VxHipStatus launch_unblock_activations(hipStream_t s, const int8_t* blocked, uint32_t rows, uint32_t k,
                                        int8_t* row_major, uint32_t ld);
+VxHipStatus launch_requantize(hipStream_t s, const void* x, uint32_t n, void* y, float multiplier, int32_t zp_in,
+                              int32_t zp_out, bool in_i8, bool out_i8);
 VxHipStatus launch_fill_u32(hipStream_t s, uint32_t* p, uint32_t count, uint32_t value);
 // Counts, over every f32 mantissa of the dividend, where the one- and the two-correction
 // division by `divisor` differ from IEEE division: counters[0] and counters[1].

@@ -42,7 +42,8 @@ typedef enum PlanKind {
     PLAN_QLINEAR = 1,
     PLAN_PACKED_LINEAR = 2,
     PLAN_QUANTIZE = 3,
-    PLAN_DEQUANTIZE = 4
+    PLAN_DEQUANTIZE = 4,
+    PLAN_REQUANTIZE = 5
 } PlanKind;
 
 #define MAX_CHAIN_NODES 64u
@@ -402,6 +403,36 @@ static VxStatus plan_boundary(PackagePlan* plan, const VxjValue* root, const Vxj
     return VX_STATUS_OK;
 }
 
+/* RequantizeLinear: int8/uint8 -> int8/uint8 between the central per-tensor descriptors of its input
+ * and its output; the node itself names no parameter tensors
+ * (native/src/runtime/engine_runtime_w8a8.inc:3470-3481). */
+static VxStatus plan_requantize(PackagePlan* plan, const VxjValue* root, Failure* failure) {
+    const VxjValue* table = quantization_table(root, failure);
+    VxstTensor scale, zero_point;
+    VxStatus status;
+    if (!table) return failure->status;
+    if (plan->input_dtype == VX_DTYPE_F32 || plan->output_dtype == VX_DTYPE_F32 || plan->d_in != plan->d_out)
+        return refuse(failure, VX_STATUS_INVALID_GRAPH, "node '%s' must convert between int8/uint8 tensors of one shape",
+                      plan->node_id);
+    status = resolve_affine(plan, table, plan->input_name, plan->input_dtype, 2, 0, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    memcpy(&plan->input_scale, scale.data, 4);
+    plan->input_zero_point = typed_zero_point(&zero_point, 0);
+    status = resolve_affine(plan, table, plan->output_name, plan->output_dtype, 2, 0, &scale, &zero_point, failure);
+    if (status != VX_STATUS_OK) return status;
+    memcpy(&plan->output_scale, scale.data, 4);
+    plan->output_zero_point = typed_zero_point(&zero_point, 0);
+    {
+        /* the operator's own contract: the ratio of the scales is a positive finite f32 */
+        volatile float multiplier = plan->input_scale / plan->output_scale;
+        if (!(multiplier > 0.0f) || !isfinite(multiplier))
+            return refuse(failure, VX_STATUS_INVALID_GRAPH, "the scales of node '%s' have no finite positive ratio",
+                          plan->node_id);
+    }
+    plan->kind = PLAN_REQUANTIZE;
+    return VX_STATUS_OK;
+}
+
 /* An aligned copy of `bytes` payload bytes, owned by the plan; NULL when memory runs out. */
 static const void* aligned_payload(PackagePlan* plan, const void* data, size_t bytes) {
     void* copy;
@@ -685,6 +716,8 @@ static VxStatus plan_package(const VxModelSource* source, VxPackedArithmetic ari
                 status = plan_packed(plan, node, arithmetic, failure);
             else if (!strcmp(op, "QuantizeLinear") || !strcmp(op, "DequantizeLinear"))
                 status = plan_boundary(plan, root, node, op[0] == 'Q', failure);
+            else if (!strcmp(op, "RequantizeLinear"))
+                status = plan_requantize(plan, root, failure);
             else
                 status = refuse(failure, VX_STATUS_BACKEND_UNSUPPORTED, "operator '%s' is not offered by this provider",
                                 op);
@@ -1035,6 +1068,12 @@ static VxStatus hip_compile(void* runtime_instance, const VxBackendCompileInput*
                                                           &stage->packed);
             if (status == VX_STATUS_OK) resident += vxhip_packed_linear_resident_bytes(stage->packed);
             family = "hip.packed-linear";
+        } else if (node->kind == PLAN_REQUANTIZE) {
+            stage->input_scale = node->input_scale;
+            stage->output_scale = node->output_scale;
+            stage->input_zero_point = node->input_zero_point;
+            stage->output_zero_point = node->output_zero_point;
+            family = "hip.requantize-linear";
         } else {
             stage->input_scale = node->boundary_scale;
             stage->input_zero_point = node->boundary_zero_point;
@@ -1290,6 +1329,13 @@ static VxStatus run_rows(HipContext* context, const void* const* inputs, uint64_
                           vxhip_quantize_forward(context->ctx, (const float*)from, (uint32_t)elements, to,
                                                  stage->input_scale, stage->input_zero_point,
                                                  (uint32_t)stage->output_dtype);
+                break;
+            case PLAN_REQUANTIZE:
+                handled = elements <= UINT32_MAX &&
+                          vxhip_requantize_forward(context->ctx, from, (uint32_t)elements, to, stage->input_scale,
+                                                   stage->input_zero_point, stage->output_scale,
+                                                   stage->output_zero_point, (uint32_t)stage->input_dtype,
+                                                   (uint32_t)stage->output_dtype);
                 break;
             case PLAN_DEQUANTIZE:
                 handled = elements <= UINT32_MAX &&

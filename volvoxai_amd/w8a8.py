@@ -523,6 +523,30 @@ def dequantize_typed_i8u8_f32(input, scale, zero_point, input_dtype):
     return int(ok), out
 
 
+def requantize_linear_i8u8(input, input_scale, input_zero_point, output_scale, output_zero_point, input_dtype,
+                           output_dtype):
+    """RequantizeLinear on host arrays (the drop-in slot): (ok, bytes)."""
+    q = _np(input)
+    out = np.zeros(q.shape, dtype=np.int8 if output_dtype == DTYPE_I8 else np.uint8)
+    ok = library().vxhip_requantize_linear_i8u8(_hp(q), q.size, _hp(out), out.size, float(np.float32(input_scale)),
+                                                int(input_zero_point), float(np.float32(output_scale)),
+                                                int(output_zero_point), input_dtype, output_dtype)
+    return int(ok), out
+
+
+def requantize_forward(ctx: Context, x, input_scale, input_zero_point, output_scale, output_zero_point, input_dtype,
+                       output_dtype, out=None):
+    """RequantizeLinear on a resident byte tensor: (ok, bytes)."""
+    import torch
+    in_t, out_t = _byte_dtype(input_dtype, "input_dtype"), _byte_dtype(output_dtype, "output_dtype")
+    if out is None:
+        out = torch.empty(x.shape, dtype=out_t, device=x.device)
+    ok = library().vxhip_requantize_forward(ctx._h, _dp(x, "x", in_t), x.numel(), _dp(out, "out", out_t, tuple(x.shape)),
+                                            float(np.float32(input_scale)), int(input_zero_point),
+                                            float(np.float32(output_scale)), int(output_zero_point), input_dtype, output_dtype)
+    return int(ok), out
+
+
 class _Variant(C.Structure):
     _fields_ = [("id", C.c_char_p), ("backend", C.c_int32), ("operator_kind", C.c_int32),
                 ("entrypoint_id", C.c_char_p), ("predicate_id", C.c_char_p),
