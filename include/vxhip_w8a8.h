@@ -329,7 +329,9 @@ int vxhip_qlinear_forward_rowscale(VxHipContext* context,
 
 /* Drop-in for the VxW8A8Ops.qlinear_i8u8 slot: identical argument order and
  * meaning to VxQLinearI8U8Fn (src/backends/w8a8_device_ops.h:15-17), HOST
- * pointers, synchronous.  Packs, uploads, runs and downloads on device 0.
+ * pointers, synchronous, on device 0.  The packed weight stays resident
+ * between calls (see vxhip_resident_weights_clear); a call uploads the
+ * activations, runs and downloads the outputs.
  * Returns 1 handled / 0 declined before any side effect. */
 int vxhip_qlinear_i8u8(const void* input, const void* weight,
                        const float* weight_scales,
@@ -417,13 +419,27 @@ int vxhip_packed_linear_forward_a8(VxHipContext* context,
  * entry takes the same values as plain arguments: x=input f32 [rows,k],
  * packed_weight, scale, bias (optional), y=out [rows,n], key_dim=k,
  * value_dim=n, rate=group_size, groups=weight_bits (8, 4, 3 or 2; 0 means 4
- * as in the reference), normalize=8.
+ * as in the reference), normalize=8.  The packed weight stays resident
+ * between calls (see vxhip_resident_weights_clear).
  * Returns 0 / -1 like vx_llm_forward_f32 (src/kernels/llm_ops.inc:41-56). */
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
                             const float* scale, const float* bias,
                             float* output, uint64_t rows, int32_t key_dim,
                             int32_t value_dim, int32_t rate, int32_t groups,
                             int32_t normalize);
+
+/* The host-pointer entry points (vxhip_qlinear_i8u8, vxhip_packed_linear_f32) keep
+ * the weights they are given resident on the device -- prepacked, with scales,
+ * zero points and bias -- keyed by the host pointers, shape and type, as the
+ * reference's device routes keep immutable inputs resident by host pointer
+ * (src/backends/cuda/host/cuda_graph_quantized_linear_conv_host.inc:74-77), plus a
+ * fingerprint of the bytes (the per-channel arrays whole, the weight's ends and a
+ * few hundred samples), so a buffer that is refilled is packed again.  A caller
+ * that rewrites individual weights in place clears the set.  Entries are dropped
+ * least recently used first beyond 256 entries or VXHIP_RESIDENT_WEIGHT_BYTES
+ * bytes (environment, default 4 GiB).  No counterpart in the reference's ABI. */
+void vxhip_resident_weights_clear(void);
+uint64_t vxhip_resident_weights_bytes(void);
 
 /* ---- F32 <-> byte boundaries ------------------------------------------ */
 

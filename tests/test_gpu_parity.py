@@ -762,6 +762,40 @@ def test_requantize_declines(oracle):
     assert call(p, 16, p + 32, 8) == 0 and call(p, 16, p + 8, 16) == 0 and call(p, 16, p + 16, 16) == 1
 
 
+def test_host_pointer_entry_points_keep_weights_resident(oracle):
+    """vxhip_qlinear_i8u8 / vxhip_packed_linear_f32 pack a weight once per (pointers, shape, type,
+    fingerprint) and reuse it: the second call adds nothing to the resident set, refilling the
+    buffer in place is noticed (the bytes are the new weight's), clearing empties the set."""
+    import volvoxai_amd as vx
+    lib = vx.library()
+    lib.vxhip_resident_weights_clear()
+    c = cases.qlinear_random_case(9, 512, 160, 91, I8, I8, I8, False)
+    w = np.ascontiguousarray(c["w"])
+    args = lambda: (c["x"], w, c["scales"], c["zps"], c["bias"], 9, 512, 160, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"],
+                    I8, I8, I8)
+    ok, y = vx.qlinear_i8u8(*args())
+    _, want = oracle.qlinear(c["x"], w, c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], I8, I8, I8)
+    held = lib.vxhip_resident_weights_bytes()
+    assert ok == 1 and (y == want).all() and held > 0
+    ok, y = vx.qlinear_i8u8(*args())
+    assert ok == 1 and (y == want).all() and lib.vxhip_resident_weights_bytes() == held      # reused
+    w[:] = np.roll(w, 1, axis=0)                                                              # same buffer, new weight
+    _, want2 = oracle.qlinear(c["x"], w, c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], I8, I8, I8)
+    ok, y = vx.qlinear_i8u8(*args())
+    assert ok == 1 and (y == want2).all() and not (want2 == want).all()
+    assert lib.vxhip_resident_weights_bytes() == 2 * held                                     # packed again, beside the old entry
+    p = cases.packed_case(3, 256, 40, 64, 92)
+    words = oracle.pack_w8_words(p["w"])
+    st, z = vx.packed_linear_f32(p["x"], words, p["scales"], p["bias"], 256, 40, 64)
+    _, zwant = oracle.packed_linear(p["x"], words, p["scales"], p["bias"], 40, 64)
+    grown = lib.vxhip_resident_weights_bytes()
+    assert st == 0 and same_f32(z, zwant) and grown > 2 * held
+    st, z = vx.packed_linear_f32(p["x"], words, p["scales"], p["bias"], 256, 40, 64)
+    assert st == 0 and same_f32(z, zwant) and lib.vxhip_resident_weights_bytes() == grown
+    lib.vxhip_resident_weights_clear()
+    assert lib.vxhip_resident_weights_bytes() == 0
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

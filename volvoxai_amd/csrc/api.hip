@@ -10,6 +10,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -133,6 +134,122 @@ static bool use_device(int device) {
 
 // The context of the host-pointer entry points: device 0, one per thread.  Its device is made
 // current on every use, because the handles those entry points create live on the current device.
+// ---- weights of the host-pointer entry points, kept resident --------------------------------------
+// vxhip_qlinear_i8u8 and vxhip_packed_linear_f32 receive their weights as host pointers on every call,
+// as the VxW8A8Ops slots do.  The reference's device routes keep such immutable inputs resident, keyed
+// by the host pointer (graph_ensure_input(ptr, bytes, 1),
+// native/src/backends/cuda/host/cuda_graph_quantized_linear_conv_host.inc:74-77); so does this one: the
+// prepacked weight with its scales, zero points and bias is built once per (pointers, shape, type) and
+// reused.  On top of the reference's rule a fingerprint of the bytes is part of the key (all of the
+// per-channel arrays, and of the weight its ends and a few hundred samples), so that a buffer that was
+// refilled in place is packed again rather than served stale -- a caller that rewrites single weights
+// calls vxhip_resident_weights_clear.  Least recently used entries go when the entry or byte limit is
+// reached (VXHIP_RESIDENT_WEIGHT_BYTES, default 4 GiB).  An entry in use by another thread outlives
+// its eviction.
+struct ResidentWeights {
+    VxHipQLinear* qlinear = nullptr;
+    VxHipPackedLinear* packed = nullptr;
+    ~ResidentWeights() {
+        if (qlinear) vxhip_qlinear_destroy(qlinear);
+        if (packed) vxhip_packed_linear_destroy(packed);
+    }
+};
+struct ResidentKey {
+    const void* pointers[4];
+    uint32_t extents[4];
+    uint64_t fingerprint;
+    bool operator==(const ResidentKey& o) const { return memcmp(this, &o, sizeof(*this)) == 0; }
+};
+struct ResidentSlot {
+    ResidentKey key;
+    std::shared_ptr<ResidentWeights> weights;
+    uint64_t last_use;
+    size_t bytes;
+};
+static std::mutex g_resident_mutex;
+// never destroyed: at process exit the runtime may already be gone when static destructors run
+static std::vector<ResidentSlot>& g_resident = *new std::vector<ResidentSlot>();
+static uint64_t g_resident_clock = 0;
+constexpr size_t kResidentMaxEntries = 256;
+
+static size_t resident_limit_bytes() {
+    const char* text = getenv("VXHIP_RESIDENT_WEIGHT_BYTES");
+    if (text && *text) return (size_t)strtoull(text, nullptr, 10);
+    return (size_t)4 << 30;
+}
+
+static uint64_t fnv1a(uint64_t h, const void* data, size_t bytes) {
+    const unsigned char* p = (const unsigned char*)data;
+    size_t i = 0;
+    for (; i + 8u <= bytes; i += 8u) {  // eight bytes a step: this runs on every call
+        uint64_t word;
+        memcpy(&word, p + i, 8u);
+        h = (h ^ word) * 0x100000001b3ull;
+        h ^= h >> 29;
+    }
+    for (; i < bytes; i++) h = (h ^ p[i]) * 0x100000001b3ull;
+    return h;
+}
+// all of a small array; of a large one both ends and 512 samples of 8 bytes spread evenly
+static uint64_t fingerprint(uint64_t h, const void* data, size_t bytes) {
+    if (!data) return fnv1a(h, "null", 4);
+    h = fnv1a(h, &bytes, sizeof bytes);
+    if (bytes <= 65536u) return fnv1a(h, data, bytes);
+    const unsigned char* p = (const unsigned char*)data;
+    h = fnv1a(h, p, 8192u);
+    h = fnv1a(h, p + bytes - 8192u, 8192u);
+    const size_t stride = (bytes - 16384u) / 512u;
+    for (size_t i = 0; i < 512u; i++) h = fnv1a(h, p + 8192u + i * stride, 8u);
+    return h;
+}
+
+static std::shared_ptr<ResidentWeights> resident_find(const ResidentKey& key) {
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    for (ResidentSlot& slot : g_resident)
+        if (slot.key == key) {
+            slot.last_use = ++g_resident_clock;
+            return slot.weights;
+        }
+    return nullptr;
+}
+
+static void resident_insert(const ResidentKey& key, const std::shared_ptr<ResidentWeights>& weights, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    const size_t limit = resident_limit_bytes();
+    if (bytes > limit) return;  // used for this call only
+    size_t held = bytes;
+    for (const ResidentSlot& slot : g_resident) held += slot.bytes;
+    while (!g_resident.empty() && (held > limit || g_resident.size() >= kResidentMaxEntries)) {
+        size_t oldest = 0;
+        for (size_t i = 1; i < g_resident.size(); i++)
+            if (g_resident[i].last_use < g_resident[oldest].last_use) oldest = i;
+        held -= g_resident[oldest].bytes;
+        g_resident.erase(g_resident.begin() + (long)oldest);
+    }
+    g_resident.push_back(ResidentSlot{key, weights, ++g_resident_clock, bytes});
+}
+
+// device staging of a host-pointer call's activations and outputs, grown as needed and kept by the context
+static bool io_staging(VxHipContext* ctx, size_t in_bytes, size_t out_bytes) {
+    if (in_bytes > ctx->io_in_bytes) {
+        (void)hipStreamSynchronize(ctx->stream);
+        if (ctx->io_in) (void)hipFree(ctx->io_in);
+        ctx->io_in = nullptr;
+        ctx->io_in_bytes = 0;
+        if (hipMalloc(&ctx->io_in, in_bytes) != hipSuccess) return false;
+        ctx->io_in_bytes = in_bytes;
+    }
+    if (out_bytes > ctx->io_out_bytes) {
+        (void)hipStreamSynchronize(ctx->stream);
+        if (ctx->io_out) (void)hipFree(ctx->io_out);
+        ctx->io_out = nullptr;
+        ctx->io_out_bytes = 0;
+        if (hipMalloc(&ctx->io_out, out_bytes) != hipSuccess) return false;
+        ctx->io_out_bytes = out_bytes;
+    }
+    return true;
+}
+
 static VxHipContext* default_context() {
     static thread_local VxHipContext* ctx = nullptr;
     if (!ctx && vxhip_context_create(0, nullptr, VXHIP_CONTEXT_OWN_STREAM, &ctx) != VXHIP_OK) ctx = nullptr;
@@ -252,6 +369,8 @@ void vxhip_context_destroy(VxHipContext* ctx) {
     for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
     if (ctx->fault_dev) (void)hipFree(ctx->fault_dev);
     if (ctx->div_proof_dev) (void)hipFree(ctx->div_proof_dev);
+    if (ctx->io_in) (void)hipFree(ctx->io_in);
+    if (ctx->io_out) (void)hipFree(ctx->io_out);
     if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -694,24 +813,36 @@ int vxhip_qlinear_i8u8(const void* input, const void* weight, const float* weigh
     }
     VxHipContext* ctx = default_context();
     if (!ctx) return 0;
-    VxHipQLinear* lin = nullptr;
-    if (vxhip_qlinear_create(weight, weight_scales, weight_zero_points, bias, d_in, d_out, weight_dtype,
-                             &lin) != VXHIP_OK)
-        return 0;
+    ResidentKey key{};
+    key.pointers[0] = weight;
+    key.pointers[1] = weight_scales;
+    key.pointers[2] = weight_zero_points;
+    key.pointers[3] = bias;
+    key.extents[0] = d_in;
+    key.extents[1] = d_out;
+    key.extents[2] = weight_dtype;
+    key.extents[3] = 1u;  // a QLinear
+    key.fingerprint = fingerprint(0xcbf29ce484222325ull, weight, (size_t)d_in * d_out);
+    key.fingerprint = fingerprint(key.fingerprint, weight_scales, (size_t)d_out * 4u);
+    key.fingerprint = fingerprint(key.fingerprint, weight_zero_points, (size_t)d_out * 4u);
+    key.fingerprint = fingerprint(key.fingerprint, bias, (size_t)d_out * 4u);
+    std::shared_ptr<ResidentWeights> held = resident_find(key);
+    if (!held) {
+        held = std::make_shared<ResidentWeights>();
+        if (vxhip_qlinear_create(weight, weight_scales, weight_zero_points, bias, d_in, d_out, weight_dtype,
+                                 &held->qlinear) != VXHIP_OK)
+            return 0;
+        resident_insert(key, held, (size_t)vxhip_qlinear_resident_bytes(held->qlinear));
+    }
     const size_t in_bytes = (size_t)rows * d_in, out_bytes = (size_t)rows * d_out;
-    void *xd = nullptr, *yd = nullptr;
     int ok = 0;
-    if (hipMalloc(&xd, in_bytes) == hipSuccess && hipMalloc(&yd, out_bytes) == hipSuccess &&
-        vxhip_memcpy_to_device(ctx, xd, input, in_bytes) == VXHIP_OK) {
-        ok = vxhip_qlinear_forward(ctx, lin, xd, yd, nullptr, rows, input_scale, input_zp, output_scale,
-                                   output_zp, input_dtype, output_dtype);
+    if (io_staging(ctx, in_bytes, out_bytes) && vxhip_memcpy_to_device(ctx, ctx->io_in, input, in_bytes) == VXHIP_OK) {
+        ok = vxhip_qlinear_forward(ctx, held->qlinear, ctx->io_in, ctx->io_out, nullptr, rows, input_scale, input_zp,
+                                   output_scale, output_zp, input_dtype, output_dtype);
         // the caller's output is written only after the whole launch succeeded
-        if (ok && vxhip_memcpy_to_host(ctx, output, yd, out_bytes) != VXHIP_OK) ok = 0;
+        if (ok && vxhip_memcpy_to_host(ctx, output, ctx->io_out, out_bytes) != VXHIP_OK) ok = 0;
     }
     (void)hipStreamSynchronize(ctx->stream);
-    if (xd) (void)hipFree(xd);
-    if (yd) (void)hipFree(yd);
-    vxhip_qlinear_destroy(lin);
     return ok;
 }
 
@@ -1040,22 +1171,35 @@ int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, c
     }
     VxHipContext* ctx = default_context();
     if (!ctx) return -1;
-    VxHipPackedLinear* pl = nullptr;
-    if (vxhip_packed_linear_create(packed_weight, scale, bias, (uint32_t)key_dim, (uint32_t)value_dim,
-                                   (uint32_t)rate, bits, &pl) != VXHIP_OK)
-        return -1;
+    if (rate <= 0) return -1;
+    const uint32_t k = (uint32_t)key_dim, n = (uint32_t)value_dim;
+    const size_t row_words = (size_t)(k / 32u) * bits + ((size_t)(k % 32u) * bits + 31u) / 32u;
+    const size_t group_count = ((size_t)k + (size_t)rate - 1u) / (size_t)rate;
+    ResidentKey key{};
+    key.pointers[0] = packed_weight;
+    key.pointers[1] = scale;
+    key.pointers[2] = bias;
+    key.extents[0] = k;
+    key.extents[1] = n;
+    key.extents[2] = (uint32_t)rate * 16u + bits;
+    key.extents[3] = 2u;  // a PackedLinear
+    key.fingerprint = fingerprint(0xcbf29ce484222325ull, packed_weight, (size_t)n * row_words * 4u);
+    key.fingerprint = fingerprint(key.fingerprint, scale, (size_t)n * group_count * 4u);
+    key.fingerprint = fingerprint(key.fingerprint, bias, (size_t)n * 4u);
+    std::shared_ptr<ResidentWeights> held = resident_find(key);
+    if (!held) {
+        held = std::make_shared<ResidentWeights>();
+        if (vxhip_packed_linear_create(packed_weight, scale, bias, k, n, (uint32_t)rate, bits, &held->packed) != VXHIP_OK)
+            return -1;
+        resident_insert(key, held, (size_t)vxhip_packed_linear_resident_bytes(held->packed));
+    }
     const size_t in_bytes = (size_t)rows * key_dim * 4u, out_bytes = (size_t)rows * value_dim * 4u;
-    void *xd = nullptr, *yd = nullptr;
     int st = -1;
-    if (hipMalloc(&xd, in_bytes) == hipSuccess && hipMalloc(&yd, out_bytes) == hipSuccess &&
-        vxhip_memcpy_to_device(ctx, xd, input, in_bytes) == VXHIP_OK) {
-        st = vxhip_packed_linear_forward_f32(ctx, pl, (const float*)xd, (float*)yd, (uint32_t)rows);
-        if (st == 0 && vxhip_memcpy_to_host(ctx, output, yd, out_bytes) != VXHIP_OK) st = -1;
+    if (io_staging(ctx, in_bytes, out_bytes) && vxhip_memcpy_to_device(ctx, ctx->io_in, input, in_bytes) == VXHIP_OK) {
+        st = vxhip_packed_linear_forward_f32(ctx, held->packed, (const float*)ctx->io_in, (float*)ctx->io_out, (uint32_t)rows);
+        if (st == 0 && vxhip_memcpy_to_host(ctx, output, ctx->io_out, out_bytes) != VXHIP_OK) st = -1;
     }
     (void)hipStreamSynchronize(ctx->stream);
-    if (xd) (void)hipFree(xd);
-    if (yd) (void)hipFree(yd);
-    vxhip_packed_linear_destroy(pl);
     return st;
 }
 
@@ -1168,6 +1312,18 @@ int vxhip_dequantize_typed_i8u8_f32(const void* input, uint32_t elements, float 
     if (xd) (void)hipFree(xd);
     if (yd) (void)hipFree(yd);
     return ok;
+}
+
+void vxhip_resident_weights_clear(void) {
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    g_resident.clear();
+}
+
+uint64_t vxhip_resident_weights_bytes(void) {
+    std::lock_guard<std::mutex> lock(g_resident_mutex);
+    uint64_t held = 0;
+    for (const ResidentSlot& slot : g_resident) held += slot.bytes;
+    return held;
 }
 
 }  // extern "C"

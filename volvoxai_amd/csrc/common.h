@@ -84,6 +84,10 @@ struct VxHipContext {
     char last_variant[96] = "";  // a copy: the launchers' name buffers are per thread, not per context
     int cu_count = 0;
     uint32_t activation_layout = 0;  // VXHIP_ACTIVATIONS_*: what the prepare entry points write for rows <= 32
+    // grow-only device staging of the host-pointer entry points' activations and outputs
+    void* io_in = nullptr;
+    void* io_out = nullptr;
+    size_t io_in_bytes = 0, io_out_bytes = 0;
 };
 
 struct VxHipQLinear {
