@@ -794,6 +794,23 @@ def test_host_pointer_entry_points_keep_weights_resident(oracle):
     assert st == 0 and same_f32(z, zwant) and lib.vxhip_resident_weights_bytes() == grown
     lib.vxhip_resident_weights_clear()
     assert lib.vxhip_resident_weights_bytes() == 0
+    # a byte limit: the least recently used weight leaves, a weight above the limit is not kept at all
+    import os
+    os.environ["VXHIP_RESIDENT_WEIGHT_BYTES"] = str(held + held // 2)
+    try:
+        vx.qlinear_i8u8(*args())
+        other = np.ascontiguousarray(np.roll(w, 3, axis=1))
+        _, want3 = oracle.qlinear(c["x"], other, c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], I8, I8, I8)
+        ok, y = vx.qlinear_i8u8(c["x"], other, c["scales"], c["zps"], c["bias"], 9, 512, 160, c["s_in"], c["zp_in"], c["s_out"],
+                                c["zp_out"], I8, I8, I8)
+        assert ok == 1 and (y == want3).all() and lib.vxhip_resident_weights_bytes() == held
+        os.environ["VXHIP_RESIDENT_WEIGHT_BYTES"] = "1024"
+        lib.vxhip_resident_weights_clear()
+        ok, y = vx.qlinear_i8u8(*args())
+        assert ok == 1 and (y == want2).all() and lib.vxhip_resident_weights_bytes() == 0
+    finally:
+        del os.environ["VXHIP_RESIDENT_WEIGHT_BYTES"]
+        lib.vxhip_resident_weights_clear()
 
 
 def test_declines_leave_output_untouched():
