@@ -384,6 +384,37 @@ int vxhip_packed_linear_forward_f32(VxHipContext* context,
                                     const float* input_dev, float* output_dev,
                                     uint32_t rows);
 
+/* The fused single-row decode forms of the reference's device route
+ * (native/src/backends/cuda/kernels/cuda_forward_gemv_pair_kernels.inc:
+ * vx_cuda_rmsnorm_packed_linear_triple_decode_a8 :1136,
+ * vx_cuda_rmsnorm_packed_linear_pair_silu_mul_decode_a8 :1424,
+ * vx_cuda_packed_linear_pair_silu_mul_decode_a8 :408,
+ * vx_cuda_packed_linear_add_decode_a8 :672), as one entry: the row operation in
+ * front of the linear, the dynamic preparation, the linear and the residual add
+ * behind it in ONE launch, for one or two rows.
+ *   row_op VXHIP_ROW_OP_NONE:    input [rows, k]
+ *          VXHIP_ROW_OP_RMSNORM: input [rows, k], gain [k], eps; the input is
+ *                                f32(x * (1/sqrt(mean(x^2) + eps)) * gain), in double
+ *          VXHIP_ROW_OP_SWIGLU:  input [rows, 2k] = [gate | up]; the input is
+ *                                silu(gate) * up
+ *   add_to_dev [rows, n] or NULL: output = add_to + (linear + bias); it may be
+ *   output_dev itself (the residual stream updated in place).
+ * The bits are those of the separate launches (vxhip_rmsnorm_prepare_i8 /
+ * vxhip_swiglu_prepare_i8 / vxhip_packed_linear_forward_f32, then the add).
+ * Returns 1 handled; 0 declined, nothing launched (more than two rows, k above
+ * 4096 (8192 without RMSNorm), k below 1024 with RMSNorm, a panel count the
+ * eight-wave kernel does not take): the caller runs the separate launches;
+ * -1 on an invalid argument. */
+#define VXHIP_ROW_OP_NONE 0u
+#define VXHIP_ROW_OP_RMSNORM 1u
+#define VXHIP_ROW_OP_SWIGLU 2u
+int vxhip_packed_linear_forward_fused(VxHipContext* context,
+                                      const VxHipPackedLinear* linear,
+                                      const float* input_dev, uint32_t rows,
+                                      uint32_t row_op, const float* gain_dev,
+                                      double eps, const float* add_to_dev,
+                                      float* output_dev);
+
 /* vxhip_packed_linear_forward_f32 for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc): it has no counterpart in the reference.  Same arguments, same

@@ -195,6 +195,38 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows", [1, 2])
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_of_one_or_two_rows_takes_the_fused_linears(oracle, rows, use_graph):
+    """One or two rows decode through the fused single-row linears (five launches per layer): the logits are
+    bit for bit those of the nine-launch layer, the tokens those of the CPU restatement."""
+    import torch
+    from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights, rope_tables
+    cfg = DecoderConfig(layers=2, hidden=1024, q_heads=8, kv_heads=4, head_dim=64, inter=1536, vocab=2000, group=128,
+                        max_seq=32)
+    weights = init_weights(cfg, 5)
+    prompt_len, new = 4, 6
+    prompt = np.random.default_rng(8).integers(0, cfg.vocab, (rows, prompt_len))
+    want_tokens, _ = DecoderRef(cfg, weights, oracle, rope_tables).generate(prompt, new)
+    pd = torch.from_numpy(prompt).cuda()
+    results = []
+    for fuse in (True, False):
+        dec = W8A8Decoder(cfg, weights, rows, fuse_rows=fuse)
+        assert dec.rows_fused == fuse
+        torch.cuda.synchronize()
+        dec.prefill(pd)
+        if use_graph:
+            dec.capture()
+        got = dec.decode(new - 1).cpu().numpy()
+        results.append((got, dec.last_logits.cpu().numpy(), dec.ctx.last_variant))
+        dec.close()
+    (fused_tokens, fused_logits, fused_route), (plain_tokens, plain_logits, _) = results
+    assert (fused_tokens == want_tokens).all() and (plain_tokens == want_tokens).all()
+    assert (fused_logits.view(np.uint32) == plain_logits.view(np.uint32)).all()
+    assert "-rmsnorm" in fused_route or "a8-" in fused_route
+
+
+@pytest.mark.gpu
 def test_decoder_stages_at_benchmark_dimensions(oracle):
     """Two layers of the benchmark decoder at its own dimensions (hidden 1024, 16 query / 8 KV heads
     of 128, SwiGLU 3072, vocabulary 32000), 32 rows, 128-token prompts, every stage of the prompt
@@ -381,6 +413,104 @@ def test_fused_decode_attention_equals_the_two_kernels(ctx, rows, start, q_heads
     ctx.synchronize()
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
     assert torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [1, 2])
+@pytest.mark.parametrize("op,k,n,group,bits,add", [
+    ("rmsnorm", 1024, 4096, 128, 8, False),    # the decoder's q/k/v and gate/up shapes
+    ("rmsnorm", 1024, 6144, 128, 8, False),
+    ("rmsnorm", 4096, 1056, 64, 8, True),
+    ("rmsnorm", 2048, 512, 32, 4, False),
+    ("rmsnorm", 1100, 200, 256, 8, False),     # ragged k and n
+    ("swiglu", 3072, 1024, 128, 8, True),      # the decoder's down projection
+    ("swiglu", 1000, 300, 64, 4, True),
+    ("swiglu", 4096, 4096, 128, 8, False),
+    ("none", 2048, 1024, 128, 8, True),        # the decoder's output projection
+    ("none", 520, 96, 32, 8, True),
+])
+def test_fused_decode_linears_equal_the_separate_launches(ctx, oracle, rows, op, k, n, group, bits, add):
+    """[RMSNorm | SwiGLU] -> preparation -> PackedLinear [-> residual add] as one launch
+    (vxhip_packed_linear_forward_fused) gives the bits of the row kernel, the linear and the add run one
+    after the other."""
+    import torch
+    import volvoxai_amd as vxa
+    import volvoxai_amd.w8a8 as vx
+    rng = np.random.default_rng(k * 7 + n + rows)
+    w = rng.integers(-8, 8, (n, k)).astype(np.int8) if bits == 4 else rng.integers(-128, 128, (n, k)).astype(np.int8)
+    words = oracle.pack_w4_words(w) if bits == 4 else oracle.pack_w8_words(w)
+    groups = (k + group - 1) // group
+    scales = rng.uniform(0.002, 0.01, (n, groups)).astype(np.float32)
+    bias = rng.normal(0, 0.1, n).astype(np.float32)
+    pl = vxa.PackedLinear(words, scales, bias, k, n, group, weight_bits=bits)
+    try:
+        width = 2 * k if op == "swiglu" else k
+        x = _dev((rng.normal(0, 2, (rows, width)) * rng.uniform(0.1, 30, (rows, 1))).astype(np.float32))
+        gain = _dev(rng.uniform(0.5, 1.5, k).astype(np.float32))
+        resid = _dev(rng.normal(0, 1, (rows, n)).astype(np.float32))
+        if op == "rmsnorm":
+            a8, sc = vx.rmsnorm_prepare_i8(ctx, x.clone(), gain, 1e-6)
+        elif op == "swiglu":
+            a8, sc = vx.swiglu_prepare_i8(ctx, x)
+        else:
+            a8, sc = None, None
+        if a8 is None:
+            st, want = pl.forward_f32(ctx, x)
+        else:
+            st, want = pl.forward_a8(ctx, a8, sc)
+        assert st == 0
+        if add:
+            want = resid + want
+        code = {"none": vxa.ROW_OP_NONE, "rmsnorm": vxa.ROW_OP_RMSNORM, "swiglu": vxa.ROW_OP_SWIGLU}[op]
+        out = resid.clone() if add else None
+        handled, got = pl.forward_fused(ctx, x, code, gain=gain, eps=1e-6, add_to=out, out=out)   # in place when adding
+        ctx.synchronize()
+        assert handled == 1, vx.library().vxhip_last_error()
+        route = ctx.last_variant
+        assert "-prep" in route and (op == "none" or f"-{op}" in route) and route.endswith("-add") == add
+        assert (got.cpu().numpy().view(np.uint32) == want.cpu().numpy().view(np.uint32)).all(), route
+        # a row that is not finite: NaN outputs from both
+        x2 = x.clone()
+        x2[0, 5] = float("inf")
+        if op == "rmsnorm":
+            a8, sc = vx.rmsnorm_prepare_i8(ctx, x2.clone(), gain, 1e-6)
+            _, want2 = pl.forward_a8(ctx, a8, sc)
+        elif op == "swiglu":
+            a8, sc = vx.swiglu_prepare_i8(ctx, x2)
+            _, want2 = pl.forward_a8(ctx, a8, sc)
+        else:
+            _, want2 = pl.forward_f32(ctx, x2)
+        handled, got2 = pl.forward_fused(ctx, x2, code, gain=gain, eps=1e-6)
+        ctx.synchronize()
+        g2, w2 = got2.cpu().numpy(), want2.cpu().numpy()
+        assert handled == 1 and (np.isnan(g2) == np.isnan(w2)).all() and np.isnan(g2[0]).all()
+        assert (g2[~np.isnan(g2)].view(np.uint32) == w2[~np.isnan(w2)].view(np.uint32)).all()
+    finally:
+        pl.close()
+
+
+@pytest.mark.gpu
+def test_fused_decode_linear_declines_what_it_does_not_take(ctx, oracle):
+    import volvoxai_amd as vxa
+    rng = np.random.default_rng(1)
+    k, n = 512, 64
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    pl = vxa.PackedLinear(oracle.pack_w8_words(w), rng.uniform(0.002, 0.01, (n, k // 128)).astype(np.float32), None, k, n, 128)
+    try:
+        gain = _dev(np.ones(k, np.float32))
+        out = _dev(np.full((3, n), 7.0, np.float32))
+        handled, _ = pl.forward_fused(ctx, _dev(np.ones((3, k), np.float32)), vxa.ROW_OP_NONE, out=out)   # three rows
+        assert handled == 0
+        handled, _ = pl.forward_fused(ctx, _dev(np.ones((1, k), np.float32)), vxa.ROW_OP_RMSNORM, gain=gain, eps=1e-6,
+                                      out=out[:1])                                                       # k < 1024
+        ctx.synchronize()
+        assert handled == 0 and (out.cpu().numpy() == 7.0).all()
+        with pytest.raises(ValueError):
+            pl.forward_fused(ctx, _dev(np.ones((1, k), np.float32)), vxa.ROW_OP_SWIGLU)                  # needs [gate | up]
+        with pytest.raises(ValueError):
+            pl.forward_fused(ctx, _dev(np.ones((1, k), np.float32)), vxa.ROW_OP_RMSNORM)                 # no gain
+    finally:
+        pl.close()
 
 
 @pytest.mark.gpu

@@ -679,8 +679,8 @@ def test_few_f32_rows_are_prepared_inside_the_gemv(ctx, oracle, rows, k, n, grou
     pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=bits)
     st, y = pl.forward_f32(ctx, dev(x))
     ctx.synchronize()
-    # (more rows, or a K too short for eight wavefronts per workgroup, keep the two launches)
-    assert st == 0 and ctx.last_variant.endswith("-prep") == (k >= 1000 and rows <= 2) and "gemv-mfma" in ctx.last_variant, ctx.last_variant
+    # (more rows keep the two launches)
+    assert st == 0 and ctx.last_variant.endswith("-prep") == (rows <= 2) and "gemv-mfma" in ctx.last_variant, ctx.last_variant
     assert same_f32(y.cpu().numpy(), want)
     vx.force_variant("gemv.noprep")
     try:
@@ -716,7 +716,7 @@ def test_qlinear_on_f32_rows_equals_the_three_nodes(ctx, oracle, rows, k, n, idt
         lin = vx.QLinear(c["w"], c["scales"], c["zps"], c["bias"], I8)
         got = lin.forward_f32(ctx, dev(x), c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, want_bytes=True)
         assert got[0] == 1 and (got[2].cpu().numpy() == q).all() and same_f32(got[1].cpu().numpy(), want), ctx.last_variant
-        inside = rows <= 2 and k >= 1000 and zero_weight_zp
+        inside = rows <= 2 and zero_weight_zp
         assert ctx.last_variant.endswith("-prep") == inside, ctx.last_variant
         ok2, only_bytes = lin.forward_f32(ctx, dev(x), c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, want_f32=False,
                                           want_bytes=True)[::2]

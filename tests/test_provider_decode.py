@@ -207,19 +207,22 @@ def test_prefill_and_steps_through_the_decode_callbacks(libs, oracle, tmp_path, 
 
 
 @pytest.mark.gpu
-def test_decode_callbacks_at_benchmark_widths_match_the_python_wiring(libs, tmp_path):
+@pytest.mark.parametrize("slots", [32, 1, 2])
+def test_decode_callbacks_at_benchmark_widths_match_the_python_wiring(libs, tmp_path, slots):
     """Two layers at the benchmark decoder's widths (hidden 1024, 16 query / 8 KV heads of 128,
     SwiGLU 3072, vocabulary 32000), 32 slots, a 24-token prompt and 4 steps: the SPI route and
     volvoxai_amd.decoder.W8A8Decoder launch the same kernels in the same order, so their ids are
-    identical (the CPU restatement pins those kernels stage by stage in tests/test_decoder.py)."""
+    identical (the CPU restatement pins those kernels stage by stage in tests/test_decoder.py).
+    One and two slots: both take the fused single-row linears in their steps."""
     import torch
     from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
     mock, _ = libs
     cfg = DecoderConfig(layers=2, max_seq=64)
     weights = init_weights(cfg, 21)
-    slots, capacity, prompt_len, steps = 32, cfg.max_seq, 24, 4
+    capacity, prompt_len, steps = cfg.max_seq, 24, 4
     prompt = np.random.default_rng(4).integers(0, cfg.vocab, (slots, prompt_len))
     dec = W8A8Decoder(cfg, weights, slots)
+    assert dec.rows_fused == (slots <= 2)
     first = dec.prefill(torch.from_numpy(prompt).cuda()).cpu().numpy()
     want = dec.decode(steps).cpu().numpy()
     dec.close()

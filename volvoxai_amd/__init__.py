@@ -10,4 +10,5 @@ from .w8a8 import (  # noqa: F401
     DTYPE_I8, DTYPE_U8, Context, QLinear, PackedLinear, qlinear_i8u8,
     packed_linear_f32, quantize_typed_f32_i8u8, dequantize_typed_i8u8_f32,
     requantize_linear_i8u8, requantize_forward, kernel_variants, force_variant,
+    ROW_OP_NONE, ROW_OP_RMSNORM, ROW_OP_SWIGLU,
 )

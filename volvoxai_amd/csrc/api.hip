@@ -1056,13 +1056,24 @@ int vxhip_packed_linear_forward_a8(VxHipContext* ctx, const VxHipPackedLinear* p
 
 // Few f32 rows: one launch, the GEMV preparing the rows itself (gemv_stream.hip, PREP).  0: ran; -2: no
 // such kernel takes the call (shape, forced variant) and nothing was launched.
-static int packed_run_f32_rows(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* x, float* y, uint32_t rows) {
+struct RowOps {
+    const float* gain = nullptr;  // RMSNorm in front of the preparation
+    double eps = 0.0;
+    bool swiglu = false;          // the rows are [gate | up]
+    const float* add_to = nullptr;
+};
+static int packed_run_f32_rows(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* x, float* y, uint32_t rows,
+                               const RowOps& ops = RowOps{}) {
     const char* force = forced_variant();
     if (rows > kMaxPrepRows || (force && (!strstr(force, "gemv") || strstr(force, "noprep")))) return -2;
     LinearArgs a{};
     a.mode = Epilogue::DequantF32;
     a.x_f32 = x;
-    a.ldx = pl->w.k;
+    a.ldx = ops.swiglu ? 2u * pl->w.k : pl->w.k;
+    a.row_gain = ops.gain;
+    a.row_eps = ops.eps;
+    a.row_swiglu = ops.swiglu ? 1u : 0u;
+    a.add_to = ops.add_to;
     a.rows = rows;
     a.n = pl->w.n;
     a.k = pl->w.k;
@@ -1114,6 +1125,24 @@ int vxhip_packed_linear_forward_f32(VxHipContext* ctx, const VxHipPackedLinear* 
     if (launch_prepare_i8(ctx->stream, input_dev, rows, k, prepared, ActivationLayout{ld, 0u}, row_scales) != VXHIP_OK)
         return -1;
     return packed_run_a8(ctx, pl, prepared, ld, false, row_scales, output_dev, nullptr, nullptr, rows);
+}
+
+int vxhip_packed_linear_forward_fused(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,
+                                      uint32_t rows, uint32_t row_op, const float* gain_dev, double eps,
+                                      const float* add_to_dev, float* output_dev) {
+    if (!ctx || !pl || !input_dev || !output_dev || row_op > VXHIP_ROW_OP_SWIGLU ||
+        (row_op == VXHIP_ROW_OP_RMSNORM && (!gain_dev || !(eps >= 0.0)))) {
+        set_error("packed_linear_forward_fused: null handle or tensor, unknown row operation, or RMSNorm without gain");
+        return -1;
+    }
+    if (!rows) return 1;
+    if (!same_device(ctx, pl->device, "packed_linear_forward_fused") || !use_device(ctx->device)) return -1;
+    RowOps ops;
+    ops.gain = row_op == VXHIP_ROW_OP_RMSNORM ? gain_dev : nullptr;
+    ops.eps = eps;
+    ops.swiglu = row_op == VXHIP_ROW_OP_SWIGLU;
+    ops.add_to = add_to_dev;
+    return packed_run_f32_rows(ctx, pl, input_dev, output_dev, rows, ops) == 0 ? 1 : 0;
 }
 
 int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,

@@ -14,6 +14,7 @@
 // All are row-sized, latency-bound kernels; none of them is on the int8 roofline.
 #include "common.h"
 #include "device_math.h"
+#include "row_math.h"
 #include "wave_ops.h"
 
 #include <math.h>
@@ -92,11 +93,10 @@ __global__ __launch_bounds__(1024) void rmsnorm_prepare_kernel(float* __restrict
     __syncthreads();
     double total = 0.0;
     for (uint32_t w = 0; w < blockDim.x / 64u; w++) total += dslots[w];
-    const double var = total / (double)d;
-    const double inv_std = 1.0 / sqrt(var + eps);
+    const double inv_std = rms_inverse(total, d, eps);
     for (uint32_t j = threadIdx.x; j < d; j += blockDim.x) {
         const float gj = j == threadIdx.x ? gain_first : gain[j];
-        const float y = (float)((double)vals[j] * inv_std * (double)gj);
+        const float y = rms_scaled(vals[j], inv_std, gj);
         vals[j] = y;
         if (normalized) normalized[(size_t)row * d + j] = y;
     }
@@ -115,9 +115,7 @@ __global__ __launch_bounds__(1024) void swiglu_prepare_kernel(const float* __res
     const float* gate = gate_up + (size_t)row * 2u * inter;
     const float* up = gate + inter;
     for (uint32_t j = threadIdx.x; j < inter; j += blockDim.x) {
-        const float g = gate[j];
-        const float s = __fdiv_rn(g, __fadd_rn(1.0f, expf(-g)));
-        const float y = __fmul_rn(s, up[j]);
+        const float y = swiglu_value(gate[j], up[j]);
         vals[j] = y;
         if (activated) activated[(size_t)row * inter + j] = y;
     }

@@ -24,6 +24,7 @@
 #include "common.h"
 #include "device_math.h"
 #include "epilogue.h"
+#include "row_math.h"
 #include "wave_ops.h"
 
 #include <stdio.h>
@@ -66,9 +67,15 @@ __device__ __forceinline__ v4i load_stream(const int8_t* p) {
 // 16 KiB reads that hit L2, issued behind the first weight requests -- and the linear is one launch
 // instead of two: the single-row route of the reference (packed_linear_ops.inc:1471-1535) also
 // quantizes the row and multiplies in one call.
-template <int MODE, int GK, int WAVES, bool W4, int SPLIT, bool PREP>
-__global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs a) {
+constexpr int kRowsPrepared = 0, kRowsF32 = 1, kRowsNorm = 2, kRowsSwiglu = 3;
+
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT, int ROWOP>
+__global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) void gemv_panel_kernel(const LinearArgs a) {
     constexpr bool F = MODE == (int)Epilogue::DequantF32;
+    // ROWOP: kRowsPrepared (0) int8 rows; kRowsF32 f32 rows prepared here; kRowsNorm, kRowsSwiglu: with
+    // RMSNorm or SwiGLU in front of the preparation
+    constexpr bool PREP = ROWOP != kRowsPrepared, NORM = ROWOP == kRowsNorm, SWIGLU = ROWOP == kRowsSwiglu;
+    static_assert(F || !(NORM || SWIGLU), "row operations ride in front of the dynamic preparation only");
     static_assert(MODE != (int)Epilogue::RequantRow || !PREP, "f32 activations: PackedLinear, or QLinear behind a QuantizeLinear");
     constexpr int CH = 32 / SPLIT;     // channels of this workgroup
     constexpr int QUADS = 4 / SPLIT;   // accumulator quads (8 channels each) of this workgroup
@@ -130,7 +137,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     // they would arrive with it, in front of it they are L2 hits whose preparation then runs while the
     // first weight blocks are on their way) and stay in registers for the two passes.
     constexpr int PREP_ROWS = PREP ? (int)kMaxPrepRows : 1, PREP_KEPT = PREP ? kPrepPerThread : 1;
+    // A row operation of the decoder may ride in front of the preparation (F only): RMSNorm with
+    // a.row_gain, or SwiGLU over rows that hold [gate | up]; its other operands travel with the rows.
+    constexpr bool ROWOPS = PREP && F;
+    // pass i of row r holds elements (whole 16-byte chunks of codes are written, so up to the padded end)
+    const uint32_t prep_end = (a.k + 15u) / 16u * 16u;
+    auto live = [&](int r, int i) { return (uint32_t)r < rows && (uint32_t)(i * WAVES * 64) < prep_end; };
     float xrows[PREP_ROWS][PREP_KEPT];
+    float xup[SWIGLU ? PREP_ROWS : 1][SWIGLU ? PREP_KEPT : 1];
+    float xgain[NORM ? PREP_KEPT : 1];
     if constexpr (PREP) {
 #pragma unroll
         for (int r = 0; r < PREP_ROWS; r++) {
@@ -138,21 +153,39 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
 #pragma unroll
             for (int i = 0; i < PREP_KEPT; i++) {
                 const uint32_t j = threadIdx.x + i * WAVES * 64;
-                xrows[r][i] = ((uint32_t)r < rows && j < a.k) ? src[j] : 0.0f;
+                xrows[r][i] = 0.0f;
+                if constexpr (SWIGLU) xup[r][i] = 0.0f;
+                if (live(r, i)) {  // (scalar: whole passes past the row end, and rows not given, cost nothing)
+                    xrows[r][i] = j < a.k ? src[j] : 0.0f;
+                    if constexpr (SWIGLU) xup[r][i] = j < a.k ? src[a.k + j] : 0.0f;
+                }
+            }
+        }
+        if constexpr (NORM) {
+#pragma unroll
+            for (int i = 0; i < PREP_KEPT; i++) {
+                const uint32_t j = threadIdx.x + i * WAVES * 64;
+                xgain[i] = 0.0f;
+                if (live(0, i)) xgain[i] = j < a.k ? a.row_gain[j] : 0.0f;
             }
         }
     }
 
     // The tail's per-output operands (activation scale, bias) are requested now, so that their
     // latency hides behind the stream instead of following it.
-    constexpr int TAIL_ITERS = ((int)kMaxGemvRows * CH + WAVES * 64 - 1) / (WAVES * 64);
-    float tail_rs[F ? TAIL_ITERS : 1], tail_bias[F ? TAIL_ITERS : 1];
+    constexpr int TAIL_ITERS = ((int)(PREP ? kMaxPrepRows : kMaxGemvRows) * CH + WAVES * 64 - 1) / (WAVES * 64);
+    float tail_rs[F ? TAIL_ITERS : 1], tail_bias[F ? TAIL_ITERS : 1], tail_add[ROWOPS ? TAIL_ITERS : 1];
     if constexpr (F) {
 #pragma unroll
         for (int it = 0; it < TAIL_ITERS; it++) {
             const uint32_t o = threadIdx.x + it * WAVES * 64;
             tail_rs[it] = PREP ? 0.0f : a.row_scale[min(o / CH, rows - 1u)];
             tail_bias[it] = a.bias_f32[ch0 + o % CH];  // padded to whole panels
+            if constexpr (ROWOPS) {
+                // the residual the output is added to: this thread's element, read before anything writes it
+                const uint32_t om = o / CH, on = ch0 + o % CH;
+                tail_add[it] = (a.add_to && om < rows && on < a.n) ? a.add_to[(size_t)om * a.n + on] : 0.0f;
+            }
         }
     }
 
@@ -217,6 +250,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
                 if ((uint32_t)r >= rows) break;
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
+                    if (!live(r, i)) continue;
                     const uint32_t j = threadIdx.x + i * WAVES * 64;
                     const float v = xrows[r][i];
                     int32_t q = a.input_zp + shift;
@@ -229,13 +263,58 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
             }
             __syncthreads();  // every wave reads every row's codes
         }
+        if constexpr (SWIGLU) {
+#pragma unroll
+            for (int r = 0; r < PREP_ROWS; r++)
+#pragma unroll
+                for (int i = 0; i < PREP_KEPT; i++)
+                    if (live(r, i)) xrows[r][i] = swiglu_value(xrows[r][i], xup[r][i]);
+        }
+        if constexpr (NORM) {
+            {
+                // The row's sum of squares in the order of rmsnorm_prepare_kernel's 1024 threads: this
+                // thread stands for VT of them (elements 1024 apart belong to the same one).
+                constexpr int VT = (int)kNormThreads / (WAVES * 64);
+                static_assert(VT >= 1 && PREP_KEPT % VT == 0, "a thread holds whole virtual threads");
+                __shared__ double norm_slots[PREP_ROWS][kNormThreads / 64];
+#pragma unroll
+                for (int r = 0; r < PREP_ROWS; r++) {
+                    if ((uint32_t)r >= rows) break;
+                    double vs[VT];
+#pragma unroll
+                    for (int v = 0; v < VT; v++) vs[v] = 0.0;
+#pragma unroll
+                    for (int i = 0; i < PREP_KEPT; i++)
+                        if (live(r, i)) vs[i % VT] += (double)xrows[r][i] * (double)xrows[r][i];
+#pragma unroll
+                    for (int v = 0; v < VT; v++) {
+                        const double part = wave_sum_to_lane0(vs[v]);
+                        if (lane == 0) norm_slots[r][wave + v * WAVES] = part;
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < PREP_ROWS; r++) {
+                    if ((uint32_t)r >= rows) break;
+                    double total = 0.0;
+#pragma unroll
+                    for (uint32_t w = 0; w < kNormThreads / 64u; w++) total += norm_slots[r][w];
+                    const double inv_std = rms_inverse(total, a.k, a.row_eps);
+#pragma unroll
+                    for (int i = 0; i < PREP_KEPT; i++)
+                        if (live(r, i)) xrows[r][i] = rms_scaled(xrows[r][i], inv_std, xgain[i]);
+                }
+            }
+        }
         if constexpr (PREP && F) {
 #pragma unroll
             for (int r = 0; r < PREP_ROWS; r++) {
+                if ((uint32_t)r >= rows) break;
                 float maximum = 0.0f;
                 uint32_t bad = 0u;
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
+                    if (!live(r, i)) continue;
                     bad |= finite_f32(xrows[r][i]) ? 0u : 1u;
                     maximum = fmaxf(maximum, fabsf(xrows[r][i]));  // fmaxf ignores a NaN operand; `bad` records it
                 }
@@ -261,6 +340,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
                 if (scale < 0x1p-126f) scale = 0x1p-126f;
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
+                    if (!live(r, i)) continue;
                     const uint32_t j = threadIdx.x + i * WAVES * 64;
                     // (elements past k were loaded as zeros: the padding of the last 16-byte chunk)
                     if (j < ldk) prep_codes[(size_t)r * ldk + j] = (int8_t)(bad ? 0 : packed_round_i8(__fdiv_rn(xrows[r][i], scale)));
@@ -372,7 +452,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
             }
             for (; g < a.groups; g++)
                 sum = __fadd_rn(sum, __fmul_rn((float)dp[(size_t)g * slab], __fmul_rn(rs, sp[g * CH])));
-            if (on < a.n) ((float*)a.y)[(size_t)om * a.n + on] = __fadd_rn(sum, tail_bias[it]);
+            float out = __fadd_rn(sum, tail_bias[it]);
+            if constexpr (ROWOPS)
+                if (a.add_to) out = __fadd_rn(tail_add[it], out);
+            if (on < a.n) ((float*)a.y)[(size_t)om * a.n + on] = out;
         }
     } else {
         for (uint32_t o = threadIdx.x; o < rows * CH; o += WAVES * 64) {
@@ -387,9 +470,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_panel_kernel(const LinearArgs
     }
 }
 
-template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, bool PREP = false>
+template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, int ROWOP = kRowsPrepared>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
-    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT, PREP>;
+    auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT, ROWOP>;
     if (lds > 64u * 1024u) {
         static std::atomic<uint64_t> configured{0};
         if (!raise_lds_limit((const void*)kern, 160 * 1024, configured)) return false;
@@ -398,11 +481,11 @@ bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int MODE, int GK, int WAVES, bool W4, bool PREP = false>
+template <int MODE, int GK, int WAVES, bool W4, int ROWOP = kRowsPrepared>
 bool launch_split(hipStream_t s, const LinearArgs& a, size_t lds, int split) {
-    if (split == 4) return launch_panel<MODE, GK, WAVES, W4, 4, PREP>(s, a, lds);
-    if (split == 2) return launch_panel<MODE, GK, WAVES, W4, 2, PREP>(s, a, lds);
-    return launch_panel<MODE, GK, WAVES, W4, 1, PREP>(s, a, lds);
+    if (split == 4) return launch_panel<MODE, GK, WAVES, W4, 4, ROWOP>(s, a, lds);
+    if (split == 2) return launch_panel<MODE, GK, WAVES, W4, 2, ROWOP>(s, a, lds);
+    return launch_panel<MODE, GK, WAVES, W4, 1, ROWOP>(s, a, lds);
 }
 
 template <int MODE, int GK, bool W4 = false>
@@ -424,6 +507,8 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
     else if (force && strstr(force, "wv8")) waves = 8;
     else if (force && strstr(force, "wv4")) waves = 4;
     else if (force && strstr(force, "wv2")) waves = 2;
+    // f32 rows are prepared by workgroups of eight waves or more (waves past the end of a short row idle)
+    if (a.x_f32 && waves < 8) waves = 8;
     // Fewer panels than half the compute units: two or four workgroups share each panel's
     // channels (only the 8- and 16-wave kernels are built that way; such shapes have them
     // unless K is tiny).
@@ -445,14 +530,33 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
             a.k > (uint32_t)kPrepPerThread * (uint32_t)waves * 64u || (MODE != (int)Epilogue::DequantF32 && a.zw))
             return nullptr;
         lds += (size_t)a.rows * ((a.k + 15u) / 16u * 16u) + (size_t)a.rows * 4u + 16u;
+        // RMSNorm in front: the sum of squares follows the 1024-thread row kernel, which rows of 1024
+        // elements and more get
+        if (a.row_gain && a.k < kNormThreads) return nullptr;
+        // (that form is built for eight waves only: its double arithmetic does not fit the registers of sixteen)
+        if (a.row_gain) {
+            if (a.k > (uint32_t)kPrepPerThread * 8u * 64u) return nullptr;
+            waves = 8;
+        }
     }
     // the MFMA GEMM takes shapes whose group dots or scales do not fit
     if (lds > 156u * 1024u) return nullptr;
     bool ok = false;
     if constexpr (MODE != (int)Epilogue::RequantRow) {
         if (prep) {
-            ok = waves == 16 ? launch_split<MODE, GK, 16, W4, true>(s, a, lds, split)
-                             : launch_split<MODE, GK, 8, W4, true>(s, a, lds, split);
+            if constexpr (MODE == (int)Epilogue::DequantF32) {
+                if (a.row_gain)
+                    ok = launch_split<MODE, GK, 8, W4, kRowsNorm>(s, a, lds, split);
+                else if (a.row_swiglu)
+                    ok = waves == 16 ? launch_split<MODE, GK, 16, W4, kRowsSwiglu>(s, a, lds, split)
+                                     : launch_split<MODE, GK, 8, W4, kRowsSwiglu>(s, a, lds, split);
+                else
+                    ok = waves == 16 ? launch_split<MODE, GK, 16, W4, kRowsF32>(s, a, lds, split)
+                                     : launch_split<MODE, GK, 8, W4, kRowsF32>(s, a, lds, split);
+            } else {
+                ok = waves == 16 ? launch_split<MODE, GK, 16, W4, kRowsF32>(s, a, lds, split)
+                                 : launch_split<MODE, GK, 8, W4, kRowsF32>(s, a, lds, split);
+            }
             if (!ok) return nullptr;
             static const char* const prep_names[3][2] = {{"wv8-prep", "wv16-prep"},
                                                          {"wv8c16-prep", "wv16c16-prep"},
@@ -476,8 +580,11 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (cu_count <= 0) cu_count = 256;
     if (a.rows == 0u || a.rows > kMaxGemvRows) return nullptr;
+    const bool row_ops = a.row_gain || a.row_swiglu || a.add_to;
+    if (row_ops && (!a.x_f32 || a.mode != Epilogue::DequantF32 || (a.row_gain && a.row_swiglu))) return nullptr;
     if (a.x_f32) {
         if (a.ldx < a.k) return nullptr;  // f32 rows of ldx elements
+        if (a.row_swiglu && a.ldx < 2u * a.k) return nullptr;  // [gate | up]
     } else {
         if (((uintptr_t)a.x % 16u) != 0u) return nullptr;
         if (!a.x_operand_order && (a.ldx < 16u || (a.ldx % 16u) != 0u)) return nullptr;
@@ -519,7 +626,8 @@ const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count,
     }
     if (!kind) return nullptr;
     static thread_local char name[96];
-    snprintf(name, sizeof name, "%s.%s", family, kind);
+    snprintf(name, sizeof name, "%s.%s%s%s", family, kind, a.row_gain ? "-rmsnorm" : a.row_swiglu ? "-swiglu" : "",
+             a.add_to ? "-add" : "");
     return name;
 }
 

@@ -110,9 +110,13 @@ def rope_tables(cfg: DecoderConfig):
 
 
 class W8A8Decoder:
-    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None):
+    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None, fuse_rows=True):
         import torch
         self.torch, self.cfg, self.rows = torch, cfg, rows
+        # one or two rows: a decode step runs the fused single-row forms (five launches per layer instead of
+        # nine) where the library takes every linear of a layer that way
+        self.rows_fused = (fuse_rows and rows <= 2 and 1024 <= cfg.hidden <= 4096 and cfg.q_dim <= 8192
+                           and cfg.inter <= 8192)
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
         # prepared activations of up to 32 rows travel between the glue kernels and the GEMVs in
@@ -194,12 +198,40 @@ class W8A8Decoder:
         a8, sc = vx.swiglu_prepare_i8(self.ctx, gu)
         return self._linear_a8(L["down"], a8, sc)
 
+    def _fused(self, pl, x, row_op, gain=None, add_to=None):
+        handled, out = pl.forward_fused(self.ctx, x, row_op, gain=gain, eps=self.cfg.eps, add_to=add_to, out=add_to)
+        if not handled:
+            raise RuntimeError(f"the fused decode linear declined k={pl.k} n={pl.n} rows={x.shape[0]}: "
+                               + _library().vxhip_last_error().decode())
+        return out
+
+    def _layer_rows_fused(self, li, x2, positions, rows):
+        """One layer of a decode step of one or two rows in five launches, the fused forms of the reference's
+        device route (cuda_forward_gemv_pair_kernels.inc:1136,672,1424,408): RMSNorm rides in front of the
+        q/k/v and gate/up linears, SwiGLU in front of the down projection, and the two residual adds
+        behind the output and down projections, which update x2 in place.  Same bits as `_layer`."""
+        cfg, L = self.cfg, self.layers[li]
+        qkv = self._fused(L["qkv"], x2, vx.ROW_OP_RMSNORM, gain=L["gain1"])
+        attn = vx.rope_gqa_attention_decode(self.ctx, qkv, self.cos, self.sin, positions, cfg.q_heads, cfg.kv_heads,
+                                            cfg.head_dim, self.k_cache[li], self.v_cache[li])
+        self._fused(L["o"], attn, vx.ROW_OP_NONE, add_to=x2)
+        gu = self._fused(L["gate_up"], x2, vx.ROW_OP_RMSNORM, gain=L["gain2"])
+        self._fused(L["down"], gu, vx.ROW_OP_SWIGLU, add_to=x2)
+
     def _forward(self, tokens, positions, next_tokens=None, advance=None):
         """tokens int32 [rows, t] -> logits of the last position and their argmax (int32, written
         to `next_tokens` when given; `advance` counters are incremented by the same launch)."""
         cfg = self.cfg
         rows, t = tokens.shape
         x2 = vx.embedding_gather(self.ctx, tokens.reshape(-1), self.embedding)
+        if t == 1 and self.rows_fused:
+            for li in range(cfg.layers):
+                self._layer_rows_fused(li, x2, positions, rows)
+            handled, logits = self.lm_head.forward_fused(self.ctx, x2, vx.ROW_OP_RMSNORM, gain=self.gain_f, eps=cfg.eps)
+            if not handled:
+                a8, sc = vx.rmsnorm_prepare_i8(self.ctx, x2, self.gain_f, cfg.eps)
+                logits = self._linear_a8(self.lm_head, a8, sc)
+            return logits, vx.argmax_rows(self.ctx, logits, out=next_tokens, advance=advance)
         delta = None
         for li in range(cfg.layers):
             delta = self._layer(li, x2, delta, positions, rows, t)

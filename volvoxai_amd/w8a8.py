@@ -256,6 +256,9 @@ class QLinear:
         return (ok, out, accumulators) if want_accumulators else (ok, out)
 
 
+ROW_OP_NONE, ROW_OP_RMSNORM, ROW_OP_SWIGLU = 0, 1, 2
+
+
 class PackedLinear:
     """Compiled scope of one PackedLinear node (weight_bits=8, DYNAMIC_I8)."""
 
@@ -298,6 +301,30 @@ class PackedLinear:
         entry = library().vxhip_packed_linear_forward_f32_noalloc if no_alloc else library().vxhip_packed_linear_forward_f32
         st = entry(ctx._h, self._h, _dp(x, "x", torch.float32), _dp(out, "out", torch.float32, (rows, self.n)), rows)
         return st, out
+
+    def forward_fused(self, ctx: Context, x, row_op=ROW_OP_NONE, gain=None, eps=0.0, add_to=None, out=None):
+        """One or two f32 rows through [RMSNorm | SwiGLU] -> preparation -> linear [-> residual add] in one
+        launch.  x is [rows, k], or [rows, 2k] = [gate | up] for ROW_OP_SWIGLU; add_to [rows, n] may be
+        `out` itself.  Returns (handled, out): handled 0 means nothing ran and the caller takes the
+        separate launches."""
+        import torch
+        width = 2 * self.k if row_op == ROW_OP_SWIGLU else self.k
+        if row_op not in (ROW_OP_NONE, ROW_OP_RMSNORM, ROW_OP_SWIGLU):
+            raise ValueError(f"row_op: {row_op}")
+        if x.ndim != 2 or x.shape[1] != width:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {width}]")
+        rows = x.shape[0]
+        if row_op == ROW_OP_RMSNORM and gain is None:
+            raise ValueError("gain: RMSNorm needs its gain vector")
+        if out is None:
+            out = torch.empty((rows, self.n), dtype=torch.float32, device=x.device)
+        handled = library().vxhip_packed_linear_forward_fused(
+            ctx._h, self._h, _dp(x, "x", torch.float32), rows, row_op,
+            _dp(gain if row_op == ROW_OP_RMSNORM else None, "gain", torch.float32, numel=self.k), float(eps),
+            _dp(add_to, "add_to", torch.float32, (rows, self.n)), _dp(out, "out", torch.float32, (rows, self.n)))
+        if handled < 0:
+            raise RuntimeError(library().vxhip_last_error().decode())
+        return handled, out
 
     def forward_a8(self, ctx: Context, a8, row_scales, out=None, want_accumulators=False,
                    accumulators=None):
