@@ -177,17 +177,6 @@ struct LinearArgs {
     // of the QLinear (input_scale, input_zp; x_f32_unsigned: that node writes U8)
     const float* x_f32;
     uint32_t x_f32_unsigned;
-    // what the kernel does to the f32 rows before it prepares them (DequantF32 only), the fused decode
-    // forms of the reference's device route
-    // (native/src/backends/cuda/kernels/cuda_forward_gemv_pair_kernels.inc:1136,1424,408,672):
-    // row_gain: RMSNorm with this gain [k] and row_eps, as rmsnorm_prepare_kernel computes it;
-    // row_swiglu: the rows are [gate | up] of 2k elements and the input is silu(gate) * up, as
-    // swiglu_prepare_kernel computes it.  add_to [rows][n] (may be y itself): the output is
-    // add_to + (linear + bias), the residual add behind the linear.
-    const float* row_gain;
-    double row_eps;
-    uint32_t row_swiglu;
-    const float* add_to;
     uint32_t ldx;
     uint32_t x_operand_order;  // see ActivationLayout; rows <= 32
     uint32_t x_flip_mask;      // GEMV only: 0x80808080 when x holds unsigned bytes (the kernel flips their top bits), else 0
@@ -227,6 +216,18 @@ struct LinearArgs {
     float dq_scale;
     int32_t dq_zp;
     uint32_t* fault;
+    // (behind everything else: the kernels that do not use them find their arguments where they were)
+    // what the kernel does to the f32 rows before it prepares them (DequantF32 only), the fused decode
+    // forms of the reference's device route
+    // (native/src/backends/cuda/kernels/cuda_forward_gemv_pair_kernels.inc:1136,1424,408,672):
+    // row_gain: RMSNorm with this gain [k] and row_eps, as rmsnorm_prepare_kernel computes it;
+    // row_swiglu: the rows are [gate | up] of 2k elements and the input is silu(gate) * up, as
+    // swiglu_prepare_kernel computes it.  add_to [rows][n] (may be y itself): the output is
+    // add_to + (linear + bias), the residual add behind the linear.
+    const float* row_gain;
+    double row_eps;
+    uint32_t row_swiglu;
+    const float* add_to;
 };
 
 // gemm_mfma.hip / gemv_stream.hip: return the variant id that ran, or null if

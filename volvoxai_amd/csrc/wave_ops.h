@@ -58,13 +58,38 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
+// Lane i takes lane i + 32 (valid in lanes 0..31) or lane i + 16 (valid in lanes 0..15): the two
+// row-crossing steps of a shuffle-down tree as lane-permute swaps in the vector ALU.  A swap of a
+// register with a copy of itself leaves the upper half (the odd rows) of the copy in its lower half
+// (its even rows).
+__device__ __forceinline__ uint32_t lane_down32(uint32_t v) {
+    return __builtin_amdgcn_permlane32_swap(v, v, false, false)[1];
+}
+__device__ __forceinline__ uint32_t lane_down16(uint32_t v) {
+    return __builtin_amdgcn_permlane16_swap(v, v, false, false)[1];
+}
+__device__ __forceinline__ float lane_down32(float v) {
+    return __builtin_bit_cast(float, lane_down32(__builtin_bit_cast(uint32_t, v)));
+}
+__device__ __forceinline__ float lane_down16(float v) {
+    return __builtin_bit_cast(float, lane_down16(__builtin_bit_cast(uint32_t, v)));
+}
+__device__ __forceinline__ double lane_down32(double v) {
+    const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+    return __builtin_bit_cast(double, ((uint64_t)lane_down32((uint32_t)(bits >> 32)) << 32) | lane_down32((uint32_t)bits));
+}
+__device__ __forceinline__ double lane_down16(double v) {
+    const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+    return __builtin_bit_cast(double, ((uint64_t)lane_down16((uint32_t)(bits >> 32)) << 32) | lane_down16((uint32_t)bits));
+}
+
 // The sum over the 64 lanes in the order of a shuffle-down tree with offsets 32, 16, 8, 4, 2, 1
-// (bit for bit what that tree gives), valid in lane 0 only.  The two steps that cross rows are
-// shuffles; the four inside the row are DPP moves.
+// (bit for bit what that tree gives), valid in lane 0 only.  No step goes through LDS: the two
+// that cross rows are lane-permute swaps, the four inside the row DPP moves.
 template <typename T>
 __device__ __forceinline__ T wave_sum_to_lane0(T v) {
-    v += __shfl_down(v, 32, 64);
-    v += __shfl_down(v, 16, 64);
+    v += lane_down32(v);
+    v += lane_down16(v);
     v += lane_exchange<kDppRowShl + 8>(v);
     v += lane_exchange<kDppRowShl + 4>(v);
     v += lane_exchange<kDppRowShl + 2>(v);
