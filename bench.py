@@ -375,6 +375,23 @@ def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
     dec.graph = graph
     dec.close()
     total_s = prefill_s + decode_s
+    # one row (a single stream): a step through the fused single-row linears, five launches per layer,
+    # beside the nine-launch layer the 32 rows take
+    single = {}
+    weights = init_weights(cfg, 2024)
+    one = torch.from_numpy(np.random.default_rng(8).integers(0, cfg.vocab, (1, prompt_len))).cuda()
+    one_tokens = {}
+    for name, fuse in (("fused_linears", True), ("separate_launches", False)):
+        d1 = W8A8Decoder(cfg, weights, 1, fuse_rows=fuse)
+        d1.prefill(one)
+        d1.capture()
+        d1.stream.synchronize()
+        t0 = time.perf_counter()
+        one_tokens[name] = d1.decode(new_tokens - 1).cpu().numpy()
+        single[name] = {"ms_per_decode_step": (time.perf_counter() - t0) * 1e3 / (new_tokens - 1),
+                        "last_linear_variant": d1.ctx.last_variant}
+        d1.close()
+    single["tokens_equal"] = bool((one_tokens["fused_linears"] == one_tokens["separate_launches"]).all())
     return {"workload": "configs[3]: 28-layer W8A8 decoder (hidden 1024, 16q/8kv x128, SwiGLU 3072, vocab 32000), "
                         "32 rows, prompt 128, 128 new tokens, greedy",
             "value": rows * new_tokens / total_s, "unit": "tokens/s",
@@ -386,6 +403,7 @@ def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
             "decode_linear_variant": step_variant, "prefill_linear_variant": prefill_variant,
             "weight_bytes_read_per_step": weight_bytes,
             "decode_hbm_GBs": weight_bytes / (decode_s / (new_tokens - 1)) / 1e9,
+            "single_row": single,
             "glue": "HIP kernels of the same library (embedding gather, residual+RMSNorm+prepare, RoPE+KV append, "
                     "prompt and decode GQA attention, SwiGLU+prepare, argmax+advance); "
                     "one HIP graph per decode step"}

@@ -104,6 +104,18 @@ def test_packed_linear_wrappers_refuse_wrong_tensors():
         pl.forward_a8(ctx, fake(3 * 128 - 1, dtype=torch.int8), fake(3), out=fake(3, 40))  # flat and too short
     with pytest.raises(ValueError, match="row_scales"):
         pl.forward_a8(ctx, fake(3, 128, dtype=torch.int8), fake(3, 1))
+    # the fused single-row forms
+    from volvoxai_amd.w8a8 import ROW_OP_NONE, ROW_OP_RMSNORM, ROW_OP_SWIGLU
+    with pytest.raises(ValueError, match=r"expected \[rows, 256\]"):
+        pl.forward_fused(ctx, fake(1, 128), ROW_OP_SWIGLU)                       # [gate | up] is 2k wide
+    with pytest.raises(ValueError, match="gain"):
+        pl.forward_fused(ctx, fake(1, 128), ROW_OP_RMSNORM, out=fake(1, 40))     # RMSNorm without its gain
+    with pytest.raises(ValueError, match="gain"):
+        pl.forward_fused(ctx, fake(1, 128), ROW_OP_RMSNORM, gain=fake(127), out=fake(1, 40))
+    with pytest.raises(ValueError, match="add_to: shape"):
+        pl.forward_fused(ctx, fake(2, 128), ROW_OP_NONE, add_to=fake(1, 40), out=fake(2, 40))
+    with pytest.raises(ValueError, match="row_op"):
+        pl.forward_fused(ctx, fake(1, 128), 7, out=fake(1, 40))
 
 
 def test_attention_wrappers_refuse_wrong_shapes():
