@@ -198,7 +198,7 @@ def test_decoder_tokens_agree_with_cpu_restatement(oracle, use_graph, fused):
 @pytest.mark.parametrize("rows", [1, 2])
 @pytest.mark.parametrize("use_graph", [False, True])
 def test_decode_of_one_or_two_rows_takes_the_fused_linears(oracle, rows, use_graph):
-    """One or two rows decode through the fused single-row linears (five launches per layer): the logits are
+    """One row (two on request) decodes through the fused single-row linears (five launches per layer): the logits are
     bit for bit those of the nine-launch layer, the tokens those of the CPU restatement."""
     import torch
     from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights, rope_tables
@@ -210,6 +210,9 @@ def test_decode_of_one_or_two_rows_takes_the_fused_linears(oracle, rows, use_gra
     want_tokens, _ = DecoderRef(cfg, weights, oracle, rope_tables).generate(prompt, new)
     pd = torch.from_numpy(prompt).cuda()
     results = []
+    by_default = W8A8Decoder(cfg, weights, rows)
+    assert by_default.rows_fused == (rows == 1)   # two rows run the fused forms no faster: on request only
+    by_default.close()
     for fuse in (True, False):
         dec = W8A8Decoder(cfg, weights, rows, fuse_rows=fuse)
         assert dec.rows_fused == fuse
@@ -469,6 +472,10 @@ def test_fused_decode_linears_equal_the_separate_launches(ctx, oracle, rows, op,
         route = ctx.last_variant
         assert "-prep" in route and (op == "none" or f"-{op}" in route) and route.endswith("-add") == add
         assert (got.cpu().numpy().view(np.uint32) == want.cpu().numpy().view(np.uint32)).all(), route
+        if add:  # and into a buffer of its own
+            handled, apart = pl.forward_fused(ctx, x, code, gain=gain, eps=1e-6, add_to=resid)
+            ctx.synchronize()
+            assert handled == 1 and (apart.cpu().numpy().view(np.uint32) == want.cpu().numpy().view(np.uint32)).all()
         # a row that is not finite: NaN outputs from both
         x2 = x.clone()
         x2[0, 5] = float("inf")

@@ -237,7 +237,11 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
     int8_t* prep_codes = reinterpret_cast<int8_t*>(gemv_lds) +
                          (F ? (size_t)a.groups * (rows + 1u) * CH * 4u : (size_t)WAVES * rows * CH * 4u);
     float* prep_scale = reinterpret_cast<float*>(prep_codes + (size_t)rows * ldk);
-    auto prepare_rows = [&]() {
+    // (NR, the number of rows, is a template tag: without a branch between the rows their chains of
+    // reductions interleave)
+    auto prepare_rows_of = [&](auto rows_tag) __attribute__((always_inline)) {
+        constexpr int NR = decltype(rows_tag)::value;
+        auto pass = [&](int i) { return (uint32_t)(i * WAVES * 64) < prep_end; };
         if constexpr (PREP && !F) {
             // QuantizeLinear in front of a QLinear: q = saturate(ties-to-even(f32(x / s) + f32(zp))), NaN -> zp
             // (native/src/kernels/quantize_linear_ops.inc:156-169), stored as the signed byte the MFMA takes
@@ -246,11 +250,10 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
             const float zp_f = (float)(a.input_zp + shift), lo_f = (float)(a.x_f32_unsigned ? 0 : -128),
                         hi_f = (float)(a.x_f32_unsigned ? 255 : 127);
 #pragma unroll
-            for (int r = 0; r < PREP_ROWS; r++) {
-                if ((uint32_t)r >= rows) break;
+            for (int r = 0; r < NR; r++) {
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
-                    if (!live(r, i)) continue;
+                    if (!pass(i)) continue;
                     const uint32_t j = threadIdx.x + i * WAVES * 64;
                     const float v = xrows[r][i];
                     int32_t q = a.input_zp + shift;
@@ -265,10 +268,10 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
         }
         if constexpr (SWIGLU) {
 #pragma unroll
-            for (int r = 0; r < PREP_ROWS; r++)
+            for (int r = 0; r < NR; r++)
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++)
-                    if (live(r, i)) xrows[r][i] = swiglu_value(xrows[r][i], xup[r][i]);
+                    if (pass(i)) xrows[r][i] = swiglu_value(xrows[r][i], xup[r][i]);
         }
         if constexpr (NORM) {
             {
@@ -278,14 +281,13 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
                 static_assert(VT >= 1 && PREP_KEPT % VT == 0, "a thread holds whole virtual threads");
                 __shared__ double norm_slots[PREP_ROWS][kNormThreads / 64];
 #pragma unroll
-                for (int r = 0; r < PREP_ROWS; r++) {
-                    if ((uint32_t)r >= rows) break;
+                for (int r = 0; r < NR; r++) {
                     double vs[VT];
 #pragma unroll
                     for (int v = 0; v < VT; v++) vs[v] = 0.0;
 #pragma unroll
                     for (int i = 0; i < PREP_KEPT; i++)
-                        if (live(r, i)) vs[i % VT] += (double)xrows[r][i] * (double)xrows[r][i];
+                        if (pass(i)) vs[i % VT] += (double)xrows[r][i] * (double)xrows[r][i];
 #pragma unroll
                     for (int v = 0; v < VT; v++) {
                         const double part = wave_sum_to_lane0(vs[v]);
@@ -294,27 +296,25 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
                 }
                 __syncthreads();
 #pragma unroll
-                for (int r = 0; r < PREP_ROWS; r++) {
-                    if ((uint32_t)r >= rows) break;
+                for (int r = 0; r < NR; r++) {
                     double total = 0.0;
 #pragma unroll
                     for (uint32_t w = 0; w < kNormThreads / 64u; w++) total += norm_slots[r][w];
                     const double inv_std = rms_inverse(total, a.k, a.row_eps);
 #pragma unroll
                     for (int i = 0; i < PREP_KEPT; i++)
-                        if (live(r, i)) xrows[r][i] = rms_scaled(xrows[r][i], inv_std, xgain[i]);
+                        if (pass(i)) xrows[r][i] = rms_scaled(xrows[r][i], inv_std, xgain[i]);
                 }
             }
         }
         if constexpr (PREP && F) {
 #pragma unroll
-            for (int r = 0; r < PREP_ROWS; r++) {
-                if ((uint32_t)r >= rows) break;
+            for (int r = 0; r < NR; r++) {
                 float maximum = 0.0f;
                 uint32_t bad = 0u;
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
-                    if (!live(r, i)) continue;
+                    if (!pass(i)) continue;
                     bad |= finite_f32(xrows[r][i]) ? 0u : 1u;
                     maximum = fmaxf(maximum, fabsf(xrows[r][i]));  // fmaxf ignores a NaN operand; `bad` records it
                 }
@@ -327,8 +327,7 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
             }
             __syncthreads();
 #pragma unroll
-            for (int r = 0; r < PREP_ROWS; r++) {
-                if ((uint32_t)r >= rows) break;
+            for (int r = 0; r < NR; r++) {
                 float maximum = slot_max[r][0];
                 uint32_t bad = slot_bad[r][0];
 #pragma unroll
@@ -340,7 +339,7 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
                 if (scale < 0x1p-126f) scale = 0x1p-126f;
 #pragma unroll
                 for (int i = 0; i < PREP_KEPT; i++) {
-                    if (!live(r, i)) continue;
+                    if (!pass(i)) continue;
                     const uint32_t j = threadIdx.x + i * WAVES * 64;
                     // (elements past k were loaded as zeros: the padding of the last 16-byte chunk)
                     if (j < ldk) prep_codes[(size_t)r * ldk + j] = (int8_t)(bad ? 0 : packed_round_i8(__fdiv_rn(xrows[r][i], scale)));
@@ -348,6 +347,12 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
                 if (threadIdx.x == 0) prep_scale[r] = bad ? __builtin_nanf("") : scale;
             }
             __syncthreads();  // every wave reads every row's codes
+        }
+    };
+    auto prepare_rows = [&]() __attribute__((always_inline)) {
+        if constexpr (PREP) {
+            if (rows >= 2u) prepare_rows_of(std::integral_constant<int, PREP_ROWS>{});
+            else prepare_rows_of(std::integral_constant<int, 1>{});
         }
     };
 

@@ -110,12 +110,14 @@ def rope_tables(cfg: DecoderConfig):
 
 
 class W8A8Decoder:
-    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None, fuse_rows=True):
+    def __init__(self, cfg: DecoderConfig, weights: dict, rows: int, stream=None, fuse_rows=None):
         import torch
         self.torch, self.cfg, self.rows = torch, cfg, rows
-        # one or two rows: a decode step runs the fused single-row forms (five launches per layer instead of
-        # nine) where the library takes every linear of a layer that way
-        self.rows_fused = (fuse_rows and rows <= 2 and 1024 <= cfg.hidden <= 4096 and cfg.q_dim <= 8192
+        # One row: a decode step runs the fused single-row forms (five launches per layer instead of nine)
+        # where the library takes every linear of a layer that way.  They take two rows as well, at the
+        # speed of the separate launches (fuse_rows=True asks for them; None decides by the row count).
+        wanted = rows == 1 if fuse_rows is None else bool(fuse_rows)
+        self.rows_fused = (wanted and rows <= 2 and 1024 <= cfg.hidden <= 4096 and cfg.q_dim <= 8192
                            and cfg.inter <= 8192)
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
