@@ -44,8 +44,8 @@ PEAK_HBM_GBS = 8000.0     # HBM3E, MI355X
 # profiles/ (each counter scaled by what it reads for a 512 MiB copy kernel).  A counter run
 # cannot share a process with the timed run, so the measured values are carried here.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_4096x4096x4096": 101_190_827 + 16_860_089,
-    "gemv_1x4096x14336": 60_759_162 + 57_344,
+    "gemm_4096x4096x4096": 101_154_209 + 16_851_373,
+    "gemv_1x4096x14336": 60_764_410 + 57_344,
 }
 
 
@@ -342,7 +342,30 @@ def bench_other_configs(torch, vx, cases, ctx):
     return res
 
 
-def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
+def bench_single_row(torch, prompt_len=128, new_tokens=128):
+    """The decoder benchmark's model at one row (a single stream): a step through the fused single-row
+    linears, five launches per layer, beside the nine-launch layer the 32 rows take."""
+    from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
+    cfg = DecoderConfig()
+    single = {}
+    weights = init_weights(cfg, 2024)
+    one = torch.from_numpy(np.random.default_rng(8).integers(0, cfg.vocab, (1, prompt_len))).cuda()
+    one_tokens = {}
+    for name, fuse in (("fused_linears", True), ("separate_launches", False)):
+        d1 = W8A8Decoder(cfg, weights, 1, fuse_rows=fuse)
+        d1.prefill(one)
+        d1.capture()
+        d1.stream.synchronize()
+        t0 = time.perf_counter()
+        one_tokens[name] = d1.decode(new_tokens - 1).cpu().numpy()
+        single[name] = {"ms_per_decode_step": (time.perf_counter() - t0) * 1e3 / (new_tokens - 1),
+                        "last_linear_variant": d1.ctx.last_variant}
+        d1.close()
+    single["tokens_equal"] = bool((one_tokens["fused_linears"] == one_tokens["separate_launches"]).all())
+    return single
+
+
+def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128, single_row=True):
     """The decoder benchmark: random-init W8A8 decoder, every linear on the PackedLinear kernels,
     greedy decode of 32 concurrent rows, 128-token prompts, 128 new tokens each."""
     from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
@@ -375,23 +398,7 @@ def bench_decoder(torch, rows=32, prompt_len=128, new_tokens=128):
     dec.graph = graph
     dec.close()
     total_s = prefill_s + decode_s
-    # one row (a single stream): a step through the fused single-row linears, five launches per layer,
-    # beside the nine-launch layer the 32 rows take
-    single = {}
-    weights = init_weights(cfg, 2024)
-    one = torch.from_numpy(np.random.default_rng(8).integers(0, cfg.vocab, (1, prompt_len))).cuda()
-    one_tokens = {}
-    for name, fuse in (("fused_linears", True), ("separate_launches", False)):
-        d1 = W8A8Decoder(cfg, weights, 1, fuse_rows=fuse)
-        d1.prefill(one)
-        d1.capture()
-        d1.stream.synchronize()
-        t0 = time.perf_counter()
-        one_tokens[name] = d1.decode(new_tokens - 1).cpu().numpy()
-        single[name] = {"ms_per_decode_step": (time.perf_counter() - t0) * 1e3 / (new_tokens - 1),
-                        "last_linear_variant": d1.ctx.last_variant}
-        d1.close()
-    single["tokens_equal"] = bool((one_tokens["fused_linears"] == one_tokens["separate_launches"]).all())
+    single = bench_single_row(torch, prompt_len, new_tokens) if single_row else {}
     return {"workload": "configs[3]: 28-layer W8A8 decoder (hidden 1024, 16q/8kv x128, SwiGLU 3072, vocab 32000), "
                         "32 rows, prompt 128, 128 new tokens, greedy",
             "value": rows * new_tokens / total_s, "unit": "tokens/s",
@@ -415,7 +422,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "copy", "other"], default=None,
+    ap.add_argument("--no-single-row", action="store_true",
+                    help="decoder leg: the 32-row workload only (keeps a kernel profile of it unmixed)")
+    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "decoder_single_row", "copy", "other"], default=None,
                     help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
                          "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
@@ -581,8 +590,13 @@ def main():
             out["other_configs"] = bench_other_configs(torch, vx, cases, ctx)
 
     # ---- config 4: 28-layer decoder, 32 rows, greedy decode ------------------------
+    if args.only == "decoder_single_row":
+        out["decoder_single_row"] = bench_single_row(torch)
+        out.update(value=1e3 / out["decoder_single_row"]["fused_linears"]["ms_per_decode_step"], unit="tokens/s",
+                   ms_per_step=out["decoder_single_row"]["fused_linears"]["ms_per_decode_step"],
+                   config={"workload": "configs[3]'s model at one row, prompt 128, 128 new tokens, greedy"})
     if args.only in (None, "decoder"):
-        out["decoder"] = bench_decoder(torch)
+        out["decoder"] = bench_decoder(torch, single_row=not args.no_single_row)
         if args.only == "decoder":
             out.update(value=out["decoder"]["value"], unit="tokens/s", ms_per_step=out["decoder"]["ms_per_decode_step"],
                        config={"workload": out["decoder"]["workload"]})
