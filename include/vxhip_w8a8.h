@@ -72,6 +72,28 @@ VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags,
                                  VxHipContext** out_context);
 void vxhip_context_destroy(VxHipContext* context);
 VxHipStatus vxhip_context_synchronize(VxHipContext* context);
+
+/* Recording and replay.  Between begin and end the launches this context's entry
+ * points make are recorded instead of run; end hands back the recording,
+ * instantiated; vxhip_replay_launch runs it on the context's stream.  The
+ * reference's device route does the same with its forward pass
+ * (native/src/backends/cuda/host/cuda_graph_lifecycle_host.inc:184-188
+ * cuStreamBeginCapture, :236-262 instantiate and first launch, :285-290
+ * replay).  What may be recorded: the *_forward*, prepare, row, attention,
+ * gather and argmax entry points on device pointers, after the same calls have
+ * run once unrecorded (that run sizes the context's scratch; a recording that
+ * would have to grow it fails).  Not recordable: anything that copies to or from
+ * the host or synchronizes (memcpy, fault_flags, the host-pointer drop-ins).
+ * A replay reads and writes the device addresses of the recorded calls; values
+ * that change between replays (ids, positions) live in device memory.  end with
+ * out_replay NULL abandons the recording. */
+typedef struct VxHipReplay VxHipReplay;
+VxHipStatus vxhip_context_begin_recording(VxHipContext* context);
+VxHipStatus vxhip_context_end_recording(VxHipContext* context,
+                                        VxHipReplay** out_replay);
+VxHipStatus vxhip_replay_launch(VxHipContext* context,
+                                const VxHipReplay* replay);
+void vxhip_replay_destroy(VxHipReplay* replay);
 /* Kernel-variant id chosen by the last launch on this context, e.g.
  * "hip.qlinear.mfma-i8.t256x256" -- the string a provider reports as
  * route_evidence (runtime/public_api_model_lifecycle.inc:748-751). */

@@ -12,6 +12,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 static VxBackendProvider g_provider;
 static char g_name[VX_BACKEND_NAME_CAPACITY];
@@ -522,6 +523,8 @@ typedef struct MockDecode {
     char message[VX_REPORT_MESSAGE_CAPACITY];
     char compile_route[VX_REPORT_ROUTE_CAPACITY];
     char execute_route[VX_REPORT_ROUTE_CAPACITY];
+    int32_t replayed_steps; /* steps whose route evidence says they were a replay of the recorded step */
+    double step_seconds;    /* wall time of the steps after the second (those that can be replays), summed */
 } MockDecode;
 
 typedef struct DecodeSink {
@@ -593,7 +596,8 @@ int32_t mock_host_run_decode(MockDecode* run) {
     if (!g_registered) return run->status = VX_STATUS_NOT_FOUND;
     if (!g_provider.context_decode_prefill || !g_provider.context_decode_step || !g_provider.context_decode_reset)
         return run->status = VX_STATUS_BACKEND_UNSUPPORTED;
-    run->writes = run->sink_mismatch = run->wrong_step_refused = run->reset_repeats = run->attested = 0;
+    run->writes = run->sink_mismatch = run->wrong_step_refused = run->reset_repeats = run->attested = run->replayed_steps = 0;
+    run->step_seconds = 0.0;
     status = g_provider.runtime_create(g_provider.user_data, &runtime_options, &runtime, &report);
     run->failed_stage = VX_STAGE_RUNTIME_CREATE;
     if (status != VX_STATUS_OK) goto done;
@@ -682,9 +686,16 @@ int32_t mock_host_run_decode(MockDecode* run) {
         state.logits = NULL;
         state.ids_written = state.logits_written = 0;
         report = (VxReport)VX_REPORT_INIT;
-        status = g_provider.context_decode_step(context, position, &binding, 1, &sink, &report);
+        {
+            struct timespec t0, t1;
+            clock_gettime(CLOCK_MONOTONIC, &t0);
+            status = g_provider.context_decode_step(context, position, &binding, 1, &sink, &report);
+            clock_gettime(CLOCK_MONOTONIC, &t1);
+            if (i > 2) run->step_seconds += (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+        }
         if (status == VX_STATUS_OK && (run->writes != before + expected_writes || run->sink_mismatch))
             status = VX_STATUS_EXECUTION_FAILED;
+        if (status == VX_STATUS_OK && strstr(report.route_evidence, "+replay")) run->replayed_steps++;
     }
     if (status != VX_STATUS_OK) goto done;
     /* reset, then the same prefill again: the same first ids */

@@ -813,6 +813,65 @@ def test_host_pointer_entry_points_keep_weights_resident(oracle):
         lib.vxhip_resident_weights_clear()
 
 
+def test_recorded_launches_replay_on_new_values(oracle):
+    """A context records the launches of its entry points and replays them: a PackedLinear on two prepared rows and a
+    QLinear behind it, recorded once, replayed on three sets of activations written into the same device buffers;
+    every replay equals the oracle.  A recording that would have to grow the context's scratch is refused."""
+    import torch
+    import volvoxai_amd as vx
+    c = cases.decode_case(2, 512, 96, 128, 77)
+    words = oracle.pack_w8_words(c["w"])
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], 512, 96, 128)
+    q = cases.qlinear_random_case(5, 256, 64, 31, I8, I8, I8, False)
+    lin = vx.QLinear(q["w"], q["scales"], q["zps"], q["bias"], I8)
+    stream = torch.cuda.Stream()
+    ctx = vx.Context(0, stream)
+    try:
+        a8, rs = dev(c["a8"]), dev(c["row_scales"])
+        xq = dev(q["x"])
+        y = torch.empty((2, 96), dtype=torch.float32, device="cuda")
+        yq = torch.empty((5, 64), dtype=torch.int8, device="cuda")
+
+        def calls():
+            st, _ = pl.forward_a8(ctx, a8, rs, out=y)
+            ok = lin.forward(ctx, xq, q["s_in"], q["zp_in"], q["s_out"], q["zp_out"], I8, I8, out=yq)[0]
+            assert st == 0 and ok == 1
+
+        # unwarmed: the QLinear's first call needs scratch, which a recording may not allocate
+        fresh = vx.Context(0, stream)
+        fresh.begin_recording()
+        big = cases.qlinear_random_case(300, 256, 64, 32, I8, I8, I8, False)
+        refused = lin.forward(fresh, dev(big["x"]), big["s_in"], big["zp_in"], big["s_out"], big["zp_out"], I8, I8)[0]
+        abandoned = vx.library().vxhip_context_end_recording(fresh._h, None)
+        assert refused == 0 and abandoned == 0 and "recorded" in vx.library().vxhip_last_error().decode()
+        fresh.close()
+
+        calls()                      # the unrecorded run sizes the scratch
+        ctx.synchronize()
+        ctx.begin_recording()
+        calls()
+        replay = ctx.end_recording()
+        rng = np.random.default_rng(5)
+        for trial in range(3):
+            na8 = rng.integers(-127, 128, c["a8"].shape).astype(np.int8)
+            nrs = rng.uniform(0.01, 0.05, 2).astype(np.float32)
+            nx = rng.integers(-127, 128, q["x"].shape).astype(np.int8)
+            with torch.cuda.stream(stream):
+                a8.copy_(torch.from_numpy(na8)); rs.copy_(torch.from_numpy(nrs)); xq.copy_(torch.from_numpy(nx))
+                y.zero_(); yq.zero_()
+            replay.launch(ctx)
+            ctx.synchronize()
+            _, want, _ = oracle.packed_linear_a8(na8, nrs, words, c["scales"], c["bias"], 96, 128)
+            _, wantq = oracle.qlinear(nx, q["w"], q["bias"], q["scales"], q["zps"], q["s_in"], q["zp_in"], q["s_out"], q["zp_out"],
+                                      I8, I8, I8)
+            assert same_f32(y.cpu().numpy(), want) and (yq.cpu().numpy() == wantq).all(), trial
+        replay.close()
+    finally:
+        ctx.close()
+        pl.close()
+        lin.close()
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

@@ -23,7 +23,8 @@ class MockDecode(C.Structure):
                 ("generated", C.c_void_p), ("first_logits", C.c_void_p),
                 ("status", C.c_int32), ("failed_stage", C.c_int32), ("writes", C.c_int32), ("sink_mismatch", C.c_int32),
                 ("wrong_step_refused", C.c_int32), ("reset_repeats", C.c_int32), ("attested", C.c_int32),
-                ("message", C.c_char * 256), ("compile_route", C.c_char * 512), ("execute_route", C.c_char * 512)]
+                ("message", C.c_char * 256), ("compile_route", C.c_char * 512), ("execute_route", C.c_char * 512),
+                ("replayed_steps", C.c_int32), ("step_seconds", C.c_double)]
 
 
 def decoder_package(tmp, cfg, weights, slots, capacity, with_logits=True, mutate=None):
@@ -198,6 +199,7 @@ def test_prefill_and_steps_through_the_decode_callbacks(libs, oracle, tmp_path, 
     assert (generated == want_tokens).all(), (generated, want_tokens)
     assert run.wrong_step_refused == 1 and run.reset_repeats == 1 and run.attested == 1
     assert run.writes == (steps + 2) * (2 if with_logits else 1)
+    assert run.replayed_steps == steps - 1   # every step after the first runs from the recording of the second
     assert b"hip.decoder.w8a8-packed-linear.layers2" in run.compile_route and b"nodes=36" in run.execute_route
     # the generated ids were fed back into the id rows behind the prompt
     assert (ids[:, prompt_len:prompt_len + steps] == want_tokens[:steps].T).all()
@@ -237,3 +239,5 @@ def test_decode_callbacks_at_benchmark_widths_match_the_python_wiring(libs, tmp_
     assert st == 0 and run.failed_stage == 0, (st, run.failed_stage, run.message)
     assert (generated == want).all()
     assert run.wrong_step_refused == 1 and run.reset_repeats == 1 and run.attested == 1
+    # the first step is launched plainly, the second is recorded and run from the recording, like every later one
+    assert run.replayed_steps == steps - 1

@@ -105,6 +105,10 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_dequantize_typed_i8u8_f32": (C.c_int, [vp, u32, f32, i32, u32, vp]),
         "vxhip_quantize_forward": (C.c_int, [vp, vp, u32, vp, f32, i32, u32]),
         "vxhip_dequantize_forward": (C.c_int, [vp, vp, u32, f32, i32, u32, vp]),
+        "vxhip_context_begin_recording": (C.c_int, [vp]),
+        "vxhip_context_end_recording": (C.c_int, [vp, C.POINTER(vp)]),
+        "vxhip_replay_launch": (C.c_int, [vp, vp]),
+        "vxhip_replay_destroy": (None, [vp]),
         "vxhip_resident_weights_clear": (None, []),
         "vxhip_resident_weights_bytes": (C.c_uint64, []),
         "vxhip_requantize_linear_i8u8": (C.c_int, [vp, u32, vp, u32, f32, i32, f32, i32, u32, u32]),

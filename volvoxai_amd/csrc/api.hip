@@ -54,6 +54,11 @@ static bool multiplier_ok(float s_in, float s_w, float s_out) {
 
 VxHipStatus ensure_scratch(VxHipContext* ctx, size_t bytes) {
     if (bytes <= ctx->scratch_bytes) return VXHIP_OK;
+    if (ctx->recording) {
+        set_error("the context's scratch would have to grow while its launches are being recorded: run the same "
+                  "calls once before recording them");
+        return VXHIP_INVALID_ARGUMENT;
+    }
     // The outgrown block is retired, not freed: launches in flight may still read it, and a HIP
     // graph captured on this context keeps its address and may be replayed after this call.
     // Growing at least doubles the block, so the retired ones add up to less than the live one.
@@ -381,6 +386,76 @@ VxHipStatus vxhip_context_synchronize(VxHipContext* ctx) {
     return VXHIP_OK;
 }
 
+// Recording and replay of a context's launches: the reference's device route captures a forward pass
+// on its stream and replays the instantiated graph on later passes
+// (native/src/backends/cuda/host/cuda_graph_lifecycle_host.inc:184-188 cuStreamBeginCapture, :236-262
+// instantiate and first launch, :285-290 replay).
+VxHipStatus vxhip_context_begin_recording(VxHipContext* ctx) {
+    if (!ctx || ctx->recording) {
+        set_error("context_begin_recording: null context, or a recording is already open");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!use_device(ctx->device)) return VXHIP_BACKEND_UNAVAILABLE;
+    VXHIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->recording = true;
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_context_end_recording(VxHipContext* ctx, VxHipReplay** out) {
+    if (out) *out = nullptr;
+    if (!ctx || !ctx->recording) {
+        set_error("context_end_recording: null context, or no recording is open");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    ctx->recording = false;
+    hipGraph_t graph = nullptr;
+    const hipError_t ended = hipStreamEndCapture(ctx->stream, &graph);
+    if (ended != hipSuccess || !graph) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        set_error("context_end_recording: the stream did not yield a graph (%s)", hipGetErrorString(ended));
+        return VXHIP_EXECUTION_FAILED;
+    }
+    if (!out) {  // the caller abandons the recording
+        (void)hipGraphDestroy(graph);
+        return VXHIP_OK;
+    }
+    hipGraphExec_t executable = nullptr;
+    const hipError_t made = hipGraphInstantiate(&executable, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (made != hipSuccess || !executable) {
+        (void)hipGetLastError();
+        set_error("context_end_recording: the recorded launches could not be instantiated (%s)", hipGetErrorString(made));
+        return VXHIP_EXECUTION_FAILED;
+    }
+    VxHipReplay* replay = new (std::nothrow) VxHipReplay();
+    if (!replay) {
+        (void)hipGraphExecDestroy(executable);
+        return VXHIP_OUT_OF_MEMORY;
+    }
+    replay->device = ctx->device;
+    replay->executable = executable;
+    *out = replay;
+    return VXHIP_OK;
+}
+
+VxHipStatus vxhip_replay_launch(VxHipContext* ctx, const VxHipReplay* replay) {
+    if (!ctx || !replay || !replay->executable || ctx->recording) {
+        set_error("replay_launch: null handle, or the context is recording");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    if (!same_device(ctx, replay->device, "replay_launch") || !use_device(ctx->device)) return VXHIP_INVALID_ARGUMENT;
+    VXHIP_TRY(hipGraphLaunch(replay->executable, ctx->stream));
+    return VXHIP_OK;
+}
+
+void vxhip_replay_destroy(VxHipReplay* replay) {
+    if (!replay) return;
+    (void)hipSetDevice(replay->device);
+    if (replay->executable) (void)hipGraphExecDestroy(replay->executable);
+    delete replay;
+}
+
 const char* vxhip_context_last_variant(const VxHipContext* ctx) { return ctx ? ctx->last_variant : ""; }
 
 VxHipStatus vxhip_context_fault_flags(VxHipContext* ctx, uint32_t* flags) {
@@ -554,6 +629,9 @@ static const uint32_t* division_proof(VxHipContext* ctx, float divisor, float re
     memcpy(&bits, &divisor, sizeof bits);
     for (int i = 0; i < ctx->div_used; i++)
         if (ctx->div_bits[i] == bits) return ctx->div_proof_dev + 2 * i;
+    // (a proof recorded rather than run would not have happened for the calls that find its slot later:
+    // a divisor first seen while recording stays unproved, and its launches divide the long way)
+    if (ctx->recording) return nullptr;
     const int slot = ctx->div_next;
     uint32_t* counters = ctx->div_proof_dev + 2 * slot;
     ctx->div_bits[slot] = 0;  // +0.0 is never a divisor: the slot matches nothing until the launch succeeded

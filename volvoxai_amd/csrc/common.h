@@ -88,6 +88,13 @@ struct VxHipContext {
     void* io_in = nullptr;
     void* io_out = nullptr;
     size_t io_in_bytes = 0, io_out_bytes = 0;
+    bool recording = false;  // between vxhip_context_begin_recording and _end_recording: launches are recorded, not run
+};
+
+// The launches a context recorded, instantiated for replay.
+struct VxHipReplay {
+    int device = 0;
+    hipGraphExec_t executable = nullptr;
 };
 
 struct VxHipQLinear {

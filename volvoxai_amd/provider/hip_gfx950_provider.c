@@ -1384,7 +1384,11 @@ static VxStatus decoder_publish(HipContext* context, const VxBackendOutputSink* 
     }
     if (status != VX_STATUS_OK) return status;
     fill_report(report, context->compiled->runtime, VX_STATUS_OK, VX_STAGE_EXECUTE, VX_CODE_NONE, what);
-    attest(report, m->node_count, vxhip_context_last_variant(context->ctx));
+    {
+        char route[160];
+        snprintf(route, sizeof route, "%s%s", vxhip_context_last_variant(context->ctx), s->last_replayed ? "+replay" : "");
+        attest(report, m->node_count, route);
+    }
     return VX_STATUS_OK;
 }
 

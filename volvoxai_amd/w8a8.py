@@ -124,6 +124,15 @@ class Context:
     def clear_fault_flags(self):
         _check(library().vxhip_context_clear_fault_flags(self._h), "vxhip_context_clear_fault_flags")
 
+    def begin_recording(self):
+        """From here to end_recording() the launches of this context's entry points are recorded, not run."""
+        _check(library().vxhip_context_begin_recording(self._h), "context_begin_recording")
+
+    def end_recording(self) -> "Replay":
+        handle = C.c_void_p()
+        _check(library().vxhip_context_end_recording(self._h, C.byref(handle)), "context_end_recording")
+        return Replay(handle)
+
     def reserve_scratch(self, nbytes: int):
         _check(library().vxhip_context_reserve_scratch(self._h, int(nbytes)), "vxhip_context_reserve_scratch")
 
@@ -254,6 +263,27 @@ class QLinear:
             _dp(accumulators, "accumulators", torch.int32, (rows, self.d_out)), rows,
             float(np.float32(output_scale)), int(output_zero_point), output_dtype)
         return (ok, out, accumulators) if want_accumulators else (ok, out)
+
+
+class Replay:
+    """Launches recorded on a context (Context.begin_recording / end_recording), instantiated for replay."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    def launch(self, ctx: Context):
+        _check(library().vxhip_replay_launch(ctx._h, self._h), "replay_launch")
+
+    def close(self):
+        if self._h:
+            library().vxhip_replay_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 ROW_OP_NONE, ROW_OP_RMSNORM, ROW_OP_SWIGLU = 0, 1, 2
