@@ -123,35 +123,40 @@ __global__ __launch_bounds__(1024) void swiglu_prepare_kernel(const float* __res
     prepare_row(vals, inter, prepared, layout, row, row_scales + row, slots);
 }
 
-// grid (rows * t, q_heads + 2 * kv_heads), block head_dim.  Token (row, i) sits at cache slot
-// positions[i]; cos/sin are [max_seq][head_dim] tables indexed by that slot.
-__global__ void rope_append_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_table,
-                                   const float* __restrict__ sin_table, const int64_t* __restrict__ positions,
-                                   uint32_t t, uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
-                                   uint32_t max_seq, float* __restrict__ q_out, float* __restrict__ k_cache,
-                                   float* __restrict__ v_cache, uint32_t* __restrict__ fault) {
-    const uint32_t token = blockIdx.x, head = blockIdx.y, dd = threadIdx.x;
+// grid rows * t, one workgroup per token walking the elements of all its heads (a workgroup per head
+// is a launch of a hundred thousand workgroups that move 512 bytes each).  Token (row, i) sits at cache
+// slot positions[i]; cos/sin are [max_seq][head_dim] tables indexed by that slot.
+__global__ __launch_bounds__(256) void rope_append_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_table,
+                                                          const float* __restrict__ sin_table,
+                                                          const int64_t* __restrict__ positions, uint32_t t, uint32_t q_heads,
+                                                          uint32_t kv_heads, uint32_t head_dim, uint32_t max_seq,
+                                                          float* __restrict__ q_out, float* __restrict__ k_cache,
+                                                          float* __restrict__ v_cache, uint32_t* __restrict__ fault) {
+    const uint32_t token = blockIdx.x;
     const uint32_t row = token / t, i = token % t;
     const uint32_t width = (q_heads + 2u * kv_heads) * head_dim;
-    const float* src = qkv + (size_t)token * width + (size_t)head * head_dim;
     const uint64_t named = (uint64_t)positions[i];
     if (named >= max_seq) {  // outside the caches and the tables: touch nothing, say so
-        if (dd == 0) atomicOr(fault, (uint32_t)kFaultBadPosition);
+        if (threadIdx.x == 0) atomicOr(fault, (uint32_t)kFaultBadPosition);
         return;
     }
     const uint32_t slot = (uint32_t)named;
     const uint32_t half = head_dim / 2u;
-    const float v = src[dd];
-    if (head >= q_heads + kv_heads) {  // value head: plain append
-        const uint32_t h = head - q_heads - kv_heads;
-        v_cache[(((size_t)row * kv_heads + h) * max_seq + slot) * head_dim + dd] = v;
-        return;
+    for (uint32_t j = threadIdx.x; j < width; j += blockDim.x) {
+        const uint32_t head = j / head_dim, dd = j % head_dim;
+        const float* src = qkv + (size_t)token * width + (size_t)head * head_dim;
+        const float v = src[dd];
+        if (head >= q_heads + kv_heads) {  // value head: plain append
+            const uint32_t h = head - q_heads - kv_heads;
+            v_cache[(((size_t)row * kv_heads + h) * max_seq + slot) * head_dim + dd] = v;
+            continue;
+        }
+        const float partner = dd < half ? -src[dd + half] : src[dd - half];
+        const float c = cos_table[(size_t)slot * head_dim + dd], s = sin_table[(size_t)slot * head_dim + dd];
+        const float y = __fadd_rn(__fmul_rn(v, c), __fmul_rn(partner, s));
+        if (head < q_heads) q_out[((size_t)token * q_heads + head) * head_dim + dd] = y;
+        else k_cache[(((size_t)row * kv_heads + (head - q_heads)) * max_seq + slot) * head_dim + dd] = y;
     }
-    const float partner = dd < half ? -src[dd + half] : src[dd - half];
-    const float c = cos_table[(size_t)slot * head_dim + dd], s = sin_table[(size_t)slot * head_dim + dd];
-    const float y = __fadd_rn(__fmul_rn(v, c), __fmul_rn(partner, s));
-    if (head < q_heads) q_out[((size_t)token * q_heads + head) * head_dim + dd] = y;
-    else k_cache[(((size_t)row * kv_heads + (head - q_heads)) * max_seq + slot) * head_dim + dd] = y;
 }
 
 // grid (rows * t, q_heads / REP), block 256: a workgroup takes REP query heads that share one KV
@@ -1097,7 +1102,7 @@ VxHipStatus vxhip_rope_append_kv(VxHipContext* ctx, const float* qkv_dev, const 
     }
     if (!rows || !t) return VXHIP_OK;
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
-    hipLaunchKernelGGL(rope_append_kernel, dim3(rows * t, q_heads + 2u * kv_heads), dim3(head_dim), 0, ctx->stream,
+    hipLaunchKernelGGL(rope_append_kernel, dim3(rows * t), dim3(256), 0, ctx->stream,
                        qkv_dev, cos_dev, sin_dev, positions_dev, t, q_heads, kv_heads, head_dim, max_seq, q_out_dev,
                        k_cache_dev, v_cache_dev, ctx->fault_dev);
     VXHIP_TRY(hipGetLastError());
