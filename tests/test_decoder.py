@@ -497,6 +497,48 @@ def test_fused_decode_linears_equal_the_separate_launches(ctx, oracle, rows, op,
 
 
 @pytest.mark.gpu
+def test_fused_decode_linears_random_shapes(ctx, oracle):
+    """Sixty random shapes (ragged k and n, every group size, 8- and 4-bit weights, one and two rows, with and
+    without bias and residual) through the fused forms and through the separate launches: the same bits."""
+    import volvoxai_amd as vxa
+    import volvoxai_amd.w8a8 as vx
+    rng = np.random.default_rng(20240)
+    for case in range(60):
+        op = ("none", "rmsnorm", "swiglu")[case % 3]
+        rows, group, bits = int(rng.integers(1, 3)), int(rng.choice([32, 64, 128, 256])), int(rng.choice([8, 8, 4]))
+        k = int(rng.integers(1024, 4097)) if op == "rmsnorm" else int(rng.integers(16, 8193))
+        n, add = int(rng.integers(1, 2500)), bool(rng.integers(0, 2))
+        w = rng.integers(-8, 8, (n, k)).astype(np.int8) if bits == 4 else rng.integers(-128, 128, (n, k)).astype(np.int8)
+        words = oracle.pack_w4_words(w) if bits == 4 else oracle.pack_w8_words(w)
+        scales = rng.uniform(0.002, 0.01, (n, (k + group - 1) // group)).astype(np.float32)
+        bias = rng.normal(0, 0.1, n).astype(np.float32) if rng.integers(0, 2) else None
+        pl = vxa.PackedLinear(words, scales, bias, k, n, group, weight_bits=bits)
+        x = _dev((rng.normal(0, 2, (rows, 2 * k if op == "swiglu" else k)) * rng.uniform(0.01, 50, (rows, 1))).astype(np.float32))
+        gain = _dev(rng.uniform(0.5, 1.5, k).astype(np.float32))
+        resid = _dev(rng.normal(0, 1, (rows, n)).astype(np.float32))
+        if op == "rmsnorm":
+            a8, sc = vx.rmsnorm_prepare_i8(ctx, x.clone(), gain, 1e-5)
+            st, want = pl.forward_a8(ctx, a8, sc)
+        elif op == "swiglu":
+            a8, sc = vx.swiglu_prepare_i8(ctx, x)
+            st, want = pl.forward_a8(ctx, a8, sc)
+        else:
+            st, want = pl.forward_f32(ctx, x)
+        assert st == 0
+        if add:
+            want = resid + want
+        out = resid.clone() if add else None
+        handled, got = pl.forward_fused(ctx, x, {"none": vxa.ROW_OP_NONE, "rmsnorm": vxa.ROW_OP_RMSNORM, "swiglu": vxa.ROW_OP_SWIGLU}[op],
+                                        gain=gain, eps=1e-5, add_to=out, out=out)
+        ctx.synchronize()
+        assert handled == 1, (op, rows, k, n, group, bits)
+        assert (got.cpu().numpy().view(np.uint32) == want.cpu().numpy().view(np.uint32)).all(), (op, rows, k, n, group, bits, add,
+                                                                                                  ctx.last_variant)
+        pl.close()
+    assert ctx.fault_flags() == 0
+
+
+@pytest.mark.gpu
 def test_fused_decode_linear_declines_what_it_does_not_take(ctx, oracle):
     import volvoxai_amd as vxa
     rng = np.random.default_rng(1)
