@@ -923,7 +923,12 @@ uint32_t row_block(uint32_t rows, uint32_t d) {
 // ahead of their use the kernel is bound by those reads, and two heads per workgroup (half the
 // requests, half the workgroups) run a 32-row decode step of 16 heads 3 % faster than one; before
 // that rewrite the kernel was latency bound and one head per workgroup was the faster choice.
-uint32_t heads_per_workgroup(uint32_t rep) {
+// Few rows: while one head per workgroup still leaves no compute unit with two workgroups the launch
+// is latency bound again, and the heads are faster apart (28 layers of 16 query / 8 KV heads of 128,
+// per decode step: 1 row 1.13 -> 1.10 ms, 16 rows 1.385 -> 1.348; 32 rows 1.49 with two heads
+// together, 1.55 apart).
+uint32_t heads_per_workgroup(uint32_t rep, uint32_t query_heads_in_launch, int compute_units) {
+    if (query_heads_in_launch <= (uint32_t)(compute_units > 0 ? compute_units : 256)) return 1u;
     return rep >= 8u && rep % 4u == 0u ? 4u : rep % 2u == 0u ? 2u : 1u;
 }
 
@@ -1170,7 +1175,7 @@ VxHipStatus vxhip_gqa_attention(VxHipContext* ctx, const float* q_dev, const flo
             return VXHIP_OK;
         }
     }
-    const uint32_t together = heads_per_workgroup(rep);
+    const uint32_t together = heads_per_workgroup(rep, rows * t * q_heads, ctx->cu_count);
     const size_t lds = (size_t)together * (9u * head_dim + max_seq) * sizeof(float);
     if (lds > 60u * 1024u) {
         set_error("gqa_attention: head_dim/max_seq too large for the score buffer");
@@ -1198,7 +1203,7 @@ VxHipStatus vxhip_rope_gqa_attention_decode(VxHipContext* ctx, const float* qkv_
     if (!device_ready(ctx)) return VXHIP_BACKEND_UNAVAILABLE;
     const float scale = (float)(1.0 / sqrt((double)head_dim));
     const uint32_t rep = q_heads / kv_heads;
-    const uint32_t together = heads_per_workgroup(rep);
+    const uint32_t together = heads_per_workgroup(rep, rows * q_heads, ctx->cu_count);
     const size_t lds = ((size_t)together * (9u * head_dim + max_seq) + 2u * head_dim) * sizeof(float);
     if (lds > 60u * 1024u) {
         set_error("rope_gqa_attention_decode: head_dim/max_seq too large for the score buffer");
