@@ -3,6 +3,7 @@ with the committed outputs of the reference's C kernels.  Integer, byte and
 f32 results are all held bit-exact (the f32 epilogue reproduces the
 reference's operation order, so no tolerance is needed; the north-star
 tolerance of 1e-5 rel / 1e-6 abs is therefore met with margin zero)."""
+import ctypes as C
 import hashlib
 import json
 from pathlib import Path
@@ -850,6 +851,11 @@ def test_recorded_launches_replay_on_new_values(oracle):
         ctx.synchronize()
         ctx.begin_recording()
         calls()
+        # waits and host copies cannot be recorded: refused, the recording stays open
+        flags = C.c_uint32(0)
+        assert vx.library().vxhip_context_synchronize(ctx._h) != 0
+        assert vx.library().vxhip_context_fault_flags(ctx._h, C.byref(flags)) != 0
+        assert "recording" in vx.library().vxhip_last_error().decode()
         replay = ctx.end_recording()
         rng = np.random.default_rng(5)
         for trial in range(3):

@@ -262,6 +262,13 @@ static VxHipContext* default_context() {
     return ctx;
 }
 
+// Entry points that copy to or from the host or wait for the stream have no place in a recording.
+static bool not_recording(const VxHipContext* ctx, const char* who) {
+    if (!ctx->recording) return true;
+    set_error("%s: the context is recording its launches; host copies and waits cannot be recorded", who);
+    return false;
+}
+
 // A compiled weight is used on the device it was created on.
 static bool same_device(const VxHipContext* ctx, int handle_device, const char* who) {
     if (ctx->device == handle_device) return true;
@@ -369,6 +376,11 @@ VxHipStatus vxhip_context_create(int32_t device, void* stream, uint32_t flags, V
 void vxhip_context_destroy(VxHipContext* ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
+    if (ctx->recording) {  // an open recording is abandoned
+        hipGraph_t graph = nullptr;
+        if (hipStreamEndCapture(ctx->stream, &graph) == hipSuccess && graph) (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+    }
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
@@ -382,6 +394,7 @@ void vxhip_context_destroy(VxHipContext* ctx) {
 
 VxHipStatus vxhip_context_synchronize(VxHipContext* ctx) {
     if (!ctx) return VXHIP_INVALID_ARGUMENT;
+    if (!not_recording(ctx, "context_synchronize")) return VXHIP_INVALID_ARGUMENT;
     VXHIP_TRY(hipStreamSynchronize(ctx->stream));
     return VXHIP_OK;
 }
@@ -459,7 +472,7 @@ void vxhip_replay_destroy(VxHipReplay* replay) {
 const char* vxhip_context_last_variant(const VxHipContext* ctx) { return ctx ? ctx->last_variant : ""; }
 
 VxHipStatus vxhip_context_fault_flags(VxHipContext* ctx, uint32_t* flags) {
-    if (!ctx || !flags) return VXHIP_INVALID_ARGUMENT;
+    if (!ctx || !flags || !not_recording(ctx, "context_fault_flags")) return VXHIP_INVALID_ARGUMENT;
     VXHIP_TRY(hipMemcpyAsync(flags, ctx->fault_dev, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     VXHIP_TRY(hipStreamSynchronize(ctx->stream));
     return VXHIP_OK;
@@ -502,7 +515,7 @@ void vxhip_device_free(void* p) {
 }
 
 VxHipStatus vxhip_memcpy_to_device(VxHipContext* ctx, void* dst, const void* src, size_t bytes) {
-    if (!ctx || (bytes && (!dst || !src))) return VXHIP_INVALID_ARGUMENT;
+    if (!ctx || (bytes && (!dst || !src)) || !not_recording(ctx, "memcpy_to_device")) return VXHIP_INVALID_ARGUMENT;
     if (!bytes) return VXHIP_OK;
     VXHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
     VXHIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -510,7 +523,7 @@ VxHipStatus vxhip_memcpy_to_device(VxHipContext* ctx, void* dst, const void* src
 }
 
 VxHipStatus vxhip_memcpy_to_host(VxHipContext* ctx, void* dst, const void* src, size_t bytes) {
-    if (!ctx || (bytes && (!dst || !src))) return VXHIP_INVALID_ARGUMENT;
+    if (!ctx || (bytes && (!dst || !src)) || !not_recording(ctx, "memcpy_to_host")) return VXHIP_INVALID_ARGUMENT;
     if (!bytes) return VXHIP_OK;
     VXHIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
     VXHIP_TRY(hipStreamSynchronize(ctx->stream));
