@@ -1002,6 +1002,7 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restri
                                                            int32_t* __restrict__ out, int64_t* advance,
                                                            uint32_t advance_count) {
     const float* row = x + (size_t)blockIdx.x * n;
+    const float first = row[0];  // (requested with the row, not after the reduction)
     float bv = -INFINITY;
     uint32_t bi = 0xffffffffu;
     auto offer = [&](float v, uint32_t i) {
@@ -1011,12 +1012,27 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restri
         }
     };
     if ((n & 3u) == 0u && ((uintptr_t)row & 15u) == 0u) {
-        for (uint32_t j = threadIdx.x * 4u; j < n; j += blockDim.x * 4u) {
-            const float4 v = *reinterpret_cast<const float4*>(row + j);
-            offer(v.x, j);
-            offer(v.y, j + 1u);
-            offer(v.z, j + 2u);
-            offer(v.w, j + 3u);
+        // eight loads go out together: one round trip for 32 elements a thread instead of eight (the
+        // branches of `offer` keep the compiler from overlapping the loads of a plain loop)
+        constexpr uint32_t U = 8;
+        const uint32_t pitch = blockDim.x * 4u;
+        for (uint32_t j0 = threadIdx.x * 4u; j0 < n; j0 += pitch * U) {
+            float4 v[U];
+#pragma unroll
+            for (uint32_t u = 0; u < U; u++) {
+                const uint32_t j = j0 + u * pitch;
+                v[u] = j < n ? *reinterpret_cast<const float4*>(row + j) : float4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < U; u++) {
+                const uint32_t j = j0 + u * pitch;
+                if (j < n) {
+                    offer(v[u].x, j);
+                    offer(v[u].y, j + 1u);
+                    offer(v[u].z, j + 2u);
+                    offer(v[u].w, j + 3u);
+                }
+            }
         }
     } else {
         for (uint32_t j = threadIdx.x; j < n; j += blockDim.x) offer(row[j], j);
@@ -1036,7 +1052,6 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restri
     __syncthreads();
     if (threadIdx.x == 0) {
         for (uint32_t w = 1; w < waves; w++) offer(wave_v[w], wave_i[w]);
-        const float first = row[0];
         out[blockIdx.x] = (first != first || bi == 0xffffffffu) ? 0 : (int32_t)bi;
     }
     if (blockIdx.x == 0 && advance && threadIdx.x < advance_count) advance[threadIdx.x] += 1;
