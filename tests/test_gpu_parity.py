@@ -631,7 +631,7 @@ def test_quantize_dequantize_match_oracle(oracle):
 
 
 @pytest.mark.parametrize("rows,k,n", [(1, 96, 40), (17, 4096, 300), (32, 1024, 1024), (33, 200, 72), (200, 777, 130),
-                                      (600, 1024, 512)])
+                                      (600, 1024, 512), (2048, 192, 4096), (4000, 128, 4096)])  # the last two: the large tiles
 @pytest.mark.parametrize("idt,odt", [(I8, I8), (U8, U8), (I8, U8)])
 def test_qlinear_dequantized_equals_the_two_nodes(ctx, oracle, rows, k, n, idt, odt):
     """QLinear with the DequantizeLinear behind it folded into its epilogue
@@ -651,6 +651,8 @@ def test_qlinear_dequantized_equals_the_two_nodes(ctx, oracle, rows, k, n, idt, 
         got = lin.forward_dequantized(ctx, xd, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt, dequant_scale=dq_scale,
                                       dequant_zero_point=dq_zp, want_bytes=True)
         assert got[0] == 1 and same_f32(got[1].cpu().numpy(), want) and (got[2].cpu().numpy() == q).all(), ctx.last_variant
+        if rows >= 2048 and rows % 2 == 0:   # no weight zero points: the 16x16x64 tiles, dequantizing in their own epilogue
+            assert ctx.last_variant.endswith("k64-dq"), ctx.last_variant
         ok2, only = lin.forward_dequantized(ctx, xd, c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], idt, odt,
                                             dequant_scale=dq_scale, dequant_zero_point=dq_zp)
         assert ok2 == 1 and same_f32(only.cpu().numpy(), want)

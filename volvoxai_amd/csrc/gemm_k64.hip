@@ -33,7 +33,9 @@ extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
 // requantizing Epilogue.  Two LDS stages of 128 k-bytes, i.e. two 64-wide MFMA steps each.
 // FLIP: the activation bytes are unsigned; each activation fragment has its top bits flipped (one XOR per
 // dword) in front of the first MFMA row of the step that uses it, so that a U8 input needs no pass of its own.
-template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false>
+// DQ: the DequantizeLinear behind the QLinear rides in the epilogue -- each byte's value goes out as
+// f32((q - dq_zp) * dq_scale) (a.dq_out, 16 bytes a lane and tile), the bytes themselves only if a.y is set.
+template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false, bool DQ = false>
 __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams p) {
     static_assert(MODE != (int)Epilogue::DequantF32, "requantizing epilogues only");
     static_assert(TN % 4 == 0, "the epilogue transposes four channel tiles at a time");
@@ -215,6 +217,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
     // ---- epilogue: requantize, pack, transpose across the four lane groups, 16-byte stores ----
     const float zp_f = (float)a.out_zp, lo_f = (float)a.out_lo, hi_f = (float)a.out_hi;
     const float so = a.output_scale, sr = a.output_scale_recip;
+    [[maybe_unused]] const float dq_zp_f = (float)a.dq_zp;
     uint32_t mrow[TM];
     int32_t rsum[TM];
     uint32_t miss1 = 1, miss2 = 1;
@@ -266,6 +269,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
                     uint32_t u[4];
+                    v4f dq;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         uint32_t total = (uint32_t)acc[h * 4 + t][j][e];
@@ -283,7 +287,17 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
                         if (MODE == (int)Epilogue::RequantRow && (BARE || a.bias_row)) v = __fadd_rn(v, bo[t][e]);
                         // clamp, then ties-to-even by adding 1.5 * 2^23: the low mantissa bits are the integer
                         v = __builtin_amdgcn_fmed3f(v, lo_f, hi_f);
-                        u[e] = __float_as_uint(__fadd_rn(v, 12582912.0f));
+                        const float rounded = __fadd_rn(v, 12582912.0f);
+                        u[e] = __float_as_uint(rounded);
+                        if constexpr (DQ) {
+                            // the byte's value as a float (exact), then the DequantizeLinear's one rounding
+                            const float qf = __fsub_rn(rounded, 12582912.0f);
+                            dq[e] = __fmul_rn(__fsub_rn(qf, dq_zp_f), a.dq_scale);
+                        }
+                    }
+                    if constexpr (DQ) {
+                        const uint32_t nq = n0 + (wave_n * TN + h * 4 + t) * 16 + (lane >> 4) * 4;
+                        if (mrow[j] < a.rows && nq < a.n) *reinterpret_cast<v4f*>(a.dq_out + (size_t)mrow[j] * a.n + nq) = dq;
                     }
                     const uint32_t p01 = __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u);
                     const uint32_t p23 = __builtin_amdgcn_perm(u[3], u[2], 0x0c0c0400u);
@@ -296,7 +310,7 @@ __global__ __launch_bounds__(WN* WM * 64) void gemm_k64_kernel(const GemmParams 
                 const auto r01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
                 const auto r23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
                 const uint32_t n16 = n0 + (wave_n * TN + h * 4 + (lane >> 4)) * 16;
-                if (mrow[j] < a.rows && n16 < a.n) {
+                if ((!DQ || a.y) && mrow[j] < a.rows && n16 < a.n) {
                     const uint4 v = make_uint4(r01[0], r01[1], r23[0], r23[1]);
                     *reinterpret_cast<uint4*>((uint8_t*)a.y + (size_t)mrow[j] * a.n + n16) = v;
                 }
@@ -550,13 +564,13 @@ bool launch_f32_as(hipStream_t s, const LinearArgs& a) {
     return hipGetLastError() == hipSuccess;
 }
 
-template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false>
+template <int WN, int WM, int TN, int TM, int MODE, bool FLIP = false, bool DQ = false>
 bool launch_one(hipStream_t s, const LinearArgs& a) {
     constexpr int BN = WN * TN * 16, BM = WM * TM * 16;
     constexpr int LDS = 2 * ((BN / 32) * 4 + BM / 8) * 1024 + BN * 16;
     static_assert(LDS <= 160 * 1024, "stages do not fit the LDS");
     static std::atomic<uint64_t> configured{0};
-    auto kern = gemm_k64_kernel<WN, WM, TN, TM, MODE, FLIP>;
+    auto kern = gemm_k64_kernel<WN, WM, TN, TM, MODE, FLIP, DQ>;
     if (!raise_lds_limit((const void*)kern, LDS, configured)) return false;
     GemmParams p;
     p.a = a;
@@ -577,18 +591,22 @@ const char* launch_gemm_k64(hipStream_t s, const LinearArgs& a, int tile) {
     const bool row = a.mode == Epilogue::RequantRow;
     if (a.mode == Epilogue::DequantF32) return nullptr;
     constexpr int T = (int)Epilogue::RequantTensor, R = (int)Epilogue::RequantRow;
+    const bool dq = a.dq_out != nullptr;
+    bool ok = false;
     if (a.x_flip_mask) {
         // unsigned activation bytes, flipped in the kernel (the per-tensor form only: per-token scales come with I8 rows)
         if (row) return nullptr;
-        if (tile == 0) return launch_one<2, 4, 8, 4, T, true>(s, a) ? "t256x256k64" : nullptr;
-        return launch_one<2, 4, 8, 2, T, true>(s, a) ? "t256x128k64" : nullptr;
+        if (tile == 0) ok = dq ? launch_one<2, 4, 8, 4, T, true, true>(s, a) : launch_one<2, 4, 8, 4, T, true>(s, a);
+        else ok = dq ? launch_one<2, 4, 8, 2, T, true, true>(s, a) : launch_one<2, 4, 8, 2, T, true>(s, a);
+    } else if (tile == 0) {
+        ok = row ? (dq ? launch_one<2, 4, 8, 4, R, false, true>(s, a) : launch_one<2, 4, 8, 4, R>(s, a))
+                 : (dq ? launch_one<2, 4, 8, 4, T, false, true>(s, a) : launch_one<2, 4, 8, 4, T>(s, a));
+    } else {
+        ok = row ? (dq ? launch_one<2, 4, 8, 2, R, false, true>(s, a) : launch_one<2, 4, 8, 2, R>(s, a))
+                 : (dq ? launch_one<2, 4, 8, 2, T, false, true>(s, a) : launch_one<2, 4, 8, 2, T>(s, a));
     }
-    if (tile == 0) {
-        const bool ok = row ? launch_one<2, 4, 8, 4, R>(s, a) : launch_one<2, 4, 8, 4, T>(s, a);
-        return ok ? "t256x256k64" : nullptr;
-    }
-    const bool ok = row ? launch_one<2, 4, 8, 2, R>(s, a) : launch_one<2, 4, 8, 2, T>(s, a);
-    return ok ? "t256x128k64" : nullptr;
+    if (!ok) return nullptr;
+    return tile == 0 ? (dq ? "t256x256k64-dq" : "t256x256k64") : (dq ? "t256x128k64-dq" : "t256x128k64");
 }
 
 // The dequantizing GEMM on 16x16x64 MFMAs; group sizes 64, 128 and 256.  deep: one workgroup of

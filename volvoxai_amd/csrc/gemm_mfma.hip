@@ -649,7 +649,9 @@ const char* dispatch_tile(hipStream_t s, const LinearArgs& a, int cu_count, cons
         if (forced("t64x64")) pick = 4;
         // The two large tiles run on the 16x16x64 MFMA (gemm_k64.hip) when the straight-line epilogue
         // applies; a forced tile name without "k64" keeps the 32x32x32 kernel of this file.
-        const bool fast_ok = (a.n % 16u) == 0u && a.y && !a.acc_out && !a.dq_out && ((uintptr_t)a.y % 16u) == 0u;
+        // (with a.dq_out the dequantized values go out as well, or alone)
+        const bool fast_ok = (a.n % 16u) == 0u && (a.y || a.dq_out) && !a.acc_out && ((uintptr_t)a.y % 16u) == 0u &&
+                             ((uintptr_t)a.dq_out % 16u) == 0u;
         const bool named = forced("t256x") || forced("t128x") || forced("t64x");
         if (pick <= 1 && fast_ok && (forced("k64") || !named)) return launch_gemm_k64(s, a, pick);
         if (a.x_flip_mask) return nullptr;  // only those kernels flip unsigned bytes themselves: the caller stages them
