@@ -319,6 +319,15 @@ def bench_other_configs(torch, vx, cases, ctx):
     ms = region_ms(lambda i: lins[i % 24].forward_f32(ctx, xq, q["s_in"], q["zp_in"], q["s_out"], q["zp_out"]), 96, torch)
     res["qlinear_sandwich_f32_row_M1_K4096_N4096"] = {"ms": ms, "variant": ctx.last_variant,
                                                       "includes": "QuantizeLinear and DequantizeLinear, in the same launch"}
+    # QLinear with the DequantizeLinear behind it at the prompt shape: 4096 int8 rows in, f32 out, one launch
+    xb = torch.from_numpy(np.random.default_rng(10).integers(-127, 128, (4096, 4096)).astype(np.int8)).cuda()
+    yf = torch.empty((4096, 4096), dtype=torch.float32, device="cuda")
+    ms = region_ms(lambda i: lins[0].forward_dequantized(ctx, xb, q["s_in"], q["zp_in"], q["s_out"], q["zp_out"], out=yf), 40, torch)
+    ops = 2.0 * 4096 ** 3
+    res["qlinear_dequantized_M4096_K4096_N4096"] = {"ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12,
+                                                    "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                                                    "variant": ctx.last_variant,
+                                                    "includes": "DequantizeLinear, in the GEMM's epilogue (f32 output)"}
     for l in lins:
         l.close()
     # outlier-heavy large-K GEMM: f32 activations, dynamic per-token quantization, f32 out
