@@ -220,6 +220,8 @@ static std::shared_ptr<ResidentWeights> resident_find(const ResidentKey& key) {
 
 static void resident_insert(const ResidentKey& key, const std::shared_ptr<ResidentWeights>& weights, size_t bytes) {
     std::lock_guard<std::mutex> lock(g_resident_mutex);
+    for (const ResidentSlot& slot : g_resident)
+        if (slot.key == key) return;  // another thread packed the same weight meanwhile: this copy serves its call only
     const size_t limit = resident_limit_bytes();
     if (bytes > limit) return;  // used for this call only
     size_t held = bytes;
