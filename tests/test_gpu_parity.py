@@ -880,6 +880,37 @@ def test_recorded_launches_replay_on_new_values(oracle):
         lin.close()
 
 
+def test_host_pointer_entry_point_from_several_threads(oracle):
+    """Four threads call vxhip_qlinear_i8u8 at once, two weights among them: every thread has its own context and
+    stream, the resident set is shared, and every call returns the oracle's bytes."""
+    import threading
+    import volvoxai_amd as vx
+    lib = vx.library()
+    lib.vxhip_resident_weights_clear()
+    weights = [cases.qlinear_random_case(5, 384, 64, 700 + i, I8, I8, I8, False) for i in range(2)]
+    wants = [oracle.qlinear(c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"],
+                            I8, I8, I8)[1] for c in weights]
+    failures = []
+
+    def worker(index):
+        for call in range(12):
+            c, want = weights[(index + call) % 2], wants[(index + call) % 2]
+            ok, y = vx.qlinear_i8u8(c["x"], c["w"], c["scales"], c["zps"], c["bias"], 5, 384, 64, c["s_in"], c["zp_in"], c["s_out"],
+                                    c["zp_out"], I8, I8, I8)
+            if ok != 1 or not (y == want).all():
+                failures.append((index, call))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    assert not failures and not any(t.is_alive() for t in threads)
+    one = lib.vxhip_resident_weights_bytes()
+    assert one > 0
+    lib.vxhip_resident_weights_clear()
+
+
 def test_declines_leave_output_untouched():
     import volvoxai_amd as vx
     c = cases.qlinear_random_case(2, 16, 4, 3)

@@ -11,6 +11,8 @@
 #include <string.h>
 
 #include <memory>
+#include <sys/syscall.h>
+#include <unistd.h>
 #include <mutex>
 #include <vector>
 
@@ -257,8 +259,18 @@ static bool io_staging(VxHipContext* ctx, size_t in_bytes, size_t out_bytes) {
     return true;
 }
 
+// The context of the host-pointer entry points: one per calling thread, released when that thread ends.
+// (Not on the main thread, whose thread-local objects die at process exit, when nothing should be
+// asked of the runtime any more.)
+struct ThreadContext {
+    VxHipContext* ctx = nullptr;
+    ~ThreadContext() {
+        if (ctx && (pid_t)syscall(SYS_gettid) != getpid()) vxhip_context_destroy(ctx);
+    }
+};
 static VxHipContext* default_context() {
-    static thread_local VxHipContext* ctx = nullptr;
+    static thread_local ThreadContext holder;
+    VxHipContext*& ctx = holder.ctx;
     if (!ctx && vxhip_context_create(0, nullptr, VXHIP_CONTEXT_OWN_STREAM, &ctx) != VXHIP_OK) ctx = nullptr;
     if (ctx && !use_device(ctx->device)) return nullptr;
     return ctx;
