@@ -490,7 +490,10 @@ int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
  * few hundred samples), so a buffer that is refilled is packed again.  A caller
  * that rewrites individual weights in place clears the set.  Entries are dropped
  * least recently used first beyond 256 entries or VXHIP_RESIDENT_WEIGHT_BYTES
- * bytes (environment, default 4 GiB).  No counterpart in the reference's ABI. */
+ * bytes (environment, default 4 GiB).  The two entry points may be called from
+ * several threads at once: the resident set is shared, each calling thread
+ * has a context of its own (stream, staging buffers), released when the
+ * thread ends.  No counterpart in the reference's ABI. */
 void vxhip_resident_weights_clear(void);
 uint64_t vxhip_resident_weights_bytes(void);
 
