@@ -41,6 +41,7 @@ extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
 constexpr int kDepth = 4;  // 1 KiB blocks in flight per wave
 constexpr int kPrepPerThread = 8;  // f32 elements of a row that a thread of a preparing kernel holds
+constexpr uint32_t kFitLdsRows = 4;  // the exact-fit kernel keeps the activation rows in LDS up to this many rows
 
 __device__ __forceinline__ v4i load_stream(const int8_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
@@ -475,6 +476,214 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
     }
 }
 
+// The exact-fit form of the dequantizing kernel: a panel's blocks divide evenly into WAVES runs of BPW
+// blocks, each a whole number of scale groups, so the whole stream is straight-line code -- the same
+// split of K over the wavefronts, the same integer group dots, the same ascending f32 sum, with
+// everything that is not the stream moved out of its way:
+//   * the first weight blocks are requested before anything else is looked at;
+//   * XLDS (few rows): a wave copies its own slice of the activation rows (32 bytes per block and row)
+//     into LDS once and reads the MFMA's activation operand from there, so the weight blocks are the
+//     only vector loads of the loop;
+//   * the wave that closes a group turns its dots into the products f32(dot) * (s_a * s_w[n][g])
+//     itself, lane-parallel over its own groups (its scales were requested mid-stream and wait in
+//     registers or in the wave's own LDS corner), so that behind the one barrier a thread per output
+//     only adds GROUPS products in ascending order -- the sum the reference forms
+//     (packed_linear_ops.inc:1498-1504), bit for bit.
+// Measured at M=1, K=4096, N=14336 (sixteen waves of eight blocks): 10.3 us against 12.5 us for the
+// general kernel, with a plain read of the same bytes at 9.3-9.6 us.
+template <int GK, int WAVES, int BPW, bool XLDS>
+__global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArgs a) {
+    static_assert(BPW % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
+    constexpr int GPW = BPW / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t panel = blockIdx.x, rows = a.rows;
+    const uint32_t t0 = (uint32_t)wave * BPW, g0 = (uint32_t)wave * GPW;
+    const uint32_t half = lane >> 5;
+    const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
+    const uint32_t last_chunk = (a.k - 1u) / 16u;
+    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + t0) * 1024u + (uint32_t)lane * 16u;
+
+    // LDS: products [GROUPS][rows][32] (int32 dots first) | per wave: scales [GPW][32], row scales [32] |
+    // per wave (XLDS): activation slice [2 * BPW chunks][rows] of 16 bytes
+    int32_t* dots = reinterpret_cast<int32_t*>(gemv_lds);
+    float* wave_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)GROUPS * rows * 32u + (size_t)wave * (GPW * 32 + 32);
+    float* wave_rs = wave_scales + GPW * 32;
+    char* xslice = gemv_lds + ((size_t)GROUPS * rows * 32u + (size_t)WAVES * (GPW * 32 + 32)) * 4u +
+                   (size_t)wave * (2 * BPW) * rows * 16u;
+
+    // (XLDS) this wave's activation chunks are requested first: they are cache hits and return ahead
+    // of the weight stream
+    constexpr int XPL = XLDS ? (2 * BPW * (int)kFitLdsRows + 63) / 64 : 1;  // chunks per lane
+    v4i xstage[XPL];
+    if constexpr (XLDS) {
+#pragma unroll
+        for (int j = 0; j < XPL; j++) {
+            const uint32_t e = min((uint32_t)lane + 64u * j, 2u * BPW * rows - 1u);
+            const uint32_t c = min(t0 * 2u + e / rows, last_chunk), r = e % rows;
+            xstage[j] = *reinterpret_cast<const v4i*>(
+                a.x + (a.x_operand_order ? ((size_t)c * kOperandOrderRows + r) * 16u : (size_t)r * a.ldx + (size_t)c * 16u));
+        }
+    }
+    const int8_t* xp = a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
+    const uint32_t x_chunk_pitch = a.x_operand_order ? 16u * kOperandOrderRows : 16u;
+    v4i wbuf[kDepth], xbuf[XLDS ? 1 : kDepth];
+    auto issue = [&](int slot, uint32_t b) {
+        wbuf[slot] = load_stream(wp + (size_t)b * 1024u);
+        if constexpr (!XLDS) {
+            const uint32_t chunk = min((t0 + b) * 2u + half, last_chunk);
+            xbuf[slot] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) issue(i, i);
+
+    // what the tail needs, requested behind the first blocks: the wave's group scales, lane e <-> (group
+    // g0 + e / 32, channel e % 32); the row scales; the bias of this thread's outputs
+    constexpr int SPL = (GPW * 32 + 63) / 64;
+    float sreg[SPL];
+#pragma unroll
+    for (int u = 0; u < SPL; u++) {
+        const uint32_t e = min((uint32_t)lane + 64u * u, GPW * 32u - 1u);
+        sreg[u] = a.scales_t[(size_t)(g0 + e / 32u) * a.n_pad + panel * 32u + e % 32u];
+    }
+    const float rs_lane = a.row_scale[min((uint32_t)lane, rows - 1u)];
+    constexpr int OPT_ = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);  // outputs per thread
+    float bias_t[OPT_];
+#pragma unroll
+    for (int it = 0; it < OPT_; it++) bias_t[it] = a.bias_f32[panel * 32u + (threadIdx.x + it * WAVES * 64) % 32u];
+
+    if constexpr (XLDS) {
+#pragma unroll
+        for (int j = 0; j < XPL; j++) {
+            const uint32_t e = (uint32_t)lane + 64u * j;
+            if (e < 2u * BPW * rows) *reinterpret_cast<v4i*>(xslice + (size_t)e * 16u) = xstage[j];
+        }
+    }
+
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    const bool row_live = (uint32_t)(lane & 31) < rows;
+#pragma unroll
+    for (int b = 0; b < BPW; b++) {
+        const int slot = b % kDepth;
+        v4i xop;
+        if constexpr (XLDS) xop = *reinterpret_cast<const v4i*>(xslice + ((size_t)(2 * b + half) * rows + m) * 16u);
+        else xop = xbuf[slot];
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wbuf[slot], xop, acc, 0, 0, 0);
+        if (b + kDepth < BPW) issue(slot, b + kDepth);
+        if ((b + 1) % GK == 0) {
+            if (row_live) {
+                int32_t* dp = dots + ((size_t)(g0 + b / GK) * rows + (lane & 31)) * 32u + half * 4u;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    *reinterpret_cast<v4i*>(dp + q * 8) = v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = 0;
+        }
+    }
+
+    // products of this wave's groups, in place: element e of its region is (group g0 + e / (rows * 32),
+    // row (e / 32) % rows, channel e % 32)
+    float* prod = reinterpret_cast<float*>(dots) + (size_t)g0 * rows * 32u;
+    if (rows == 1u) {
+#pragma unroll
+        for (int u = 0; u < SPL; u++) {
+            const uint32_t e = (uint32_t)lane + 64u * u;
+            if (e < GPW * 32u)
+                prod[e] = __fmul_rn((float)reinterpret_cast<const int32_t*>(prod)[e], __fmul_rn(rs_lane, sreg[u]));
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < SPL; u++) {
+            const uint32_t e = (uint32_t)lane + 64u * u;
+            if (e < GPW * 32u) wave_scales[e] = sreg[u];
+        }
+        if ((uint32_t)lane < rows) wave_rs[lane] = rs_lane;
+        const uint32_t per_group = rows * 32u;
+        for (uint32_t e = lane; e < GPW * per_group; e += 64u) {
+            const float sw = wave_scales[(e / per_group) * 32u + e % 32u];
+            const float rs = wave_rs[(e / 32u) % rows];
+            prod[e] = __fmul_rn((float)reinterpret_cast<const int32_t*>(prod)[e], __fmul_rn(rs, sw));
+        }
+    }
+    __syncthreads();
+    const float* products = reinterpret_cast<const float*>(dots);
+#pragma unroll
+    for (int it = 0; it < OPT_; it++) {
+        const uint32_t o = threadIdx.x + it * WAVES * 64;
+        if (o >= rows * 32u) break;
+        // (sixteen products are requested before the first add needs one)
+        constexpr int BATCH = GROUPS % 16 == 0 ? 16 : 8;
+        static_assert(GROUPS % BATCH == 0, "the groups of a panel come in whole batches");
+        float sum = 0.0f;
+#pragma unroll
+        for (int gb = 0; gb < GROUPS; gb += BATCH) {
+            float p[BATCH];
+#pragma unroll
+            for (int g = 0; g < BATCH; g++) p[g] = products[(size_t)(gb + g) * rows * 32u + o];
+#pragma unroll
+            for (int g = 0; g < BATCH; g++) sum = __fadd_rn(sum, p[g]);
+        }
+        const uint32_t on = panel * 32u + o % 32u;
+        if (on < a.n) ((float*)a.y)[(size_t)(o / 32u) * a.n + on] = __fadd_rn(sum, bias_t[it]);
+    }
+}
+
+template <int GK, int WAVES, int BPW>
+bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds) {
+    auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true> : gemv_fit_kernel<GK, WAVES, BPW, false>;
+    if (lds > 64u * 1024u) {
+        static std::atomic<uint64_t> configured[2] = {{0}, {0}};
+        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[xlds ? 1 : 0])) return false;
+    }
+    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
+    return hipGetLastError() == hipSuccess;
+}
+
+// The exact-fit kernel takes: the dequantizing epilogue on prepared int8 rows, eight-bit weights, enough
+// panels to fill the device without sharing one, and a K whose blocks are WAVES x BPW of an instance with
+// whole groups in every run.  Returns the variant suffix, or null when the general kernel has to run.
+template <int GK>
+const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
+    if (force && strstr(force, "nofit")) return nullptr;
+    if (a.x_f32 || a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != 8u || a.x_flip_mask) return nullptr;
+    const uint32_t panels = (a.n + 31u) / 32u;
+    const bool forced = force && strstr(force, "fit");
+    // (more rows than the LDS copy takes: measured slower than the general kernel -- 16 rows 16.8 against
+    // 13.8 us at K=4096, N=14336 -- so they come here only when asked for by name)
+    if ((panels * 4u < (uint32_t)cu_count * 3u || a.rows > kFitLdsRows) && !forced) return nullptr;
+    if (a.groups * GK != a.ksteps) return nullptr;  // (no padding group: every group of the stream has its scales)
+    const bool xlds = a.rows <= kFitLdsRows;
+    auto lds_for = [&](uint32_t waves, uint32_t bpw) {
+        const size_t groups = (size_t)waves * bpw / GK;
+        return groups * a.rows * 128u + (size_t)waves * (bpw / GK * 32u + 32u) * 4u +
+               (xlds ? (size_t)waves * 2u * bpw * a.rows * 16u : 0u);
+    };
+    const char* name = nullptr;
+    bool ok = false;
+    auto run = [&](auto waves_tag, auto bpw_tag, const char* id) {
+        constexpr int W = decltype(waves_tag)::value, B = decltype(bpw_tag)::value;
+        if constexpr (B % GK == 0) {
+            if (name || a.ksteps != (uint32_t)(W * B)) return;
+            const size_t lds = lds_for(W, B);
+            if (lds > 156u * 1024u) return;
+            ok = launch_fit<GK, W, B>(s, a, lds, xlds);
+            name = id;
+        }
+    };
+    using std::integral_constant;
+    run(integral_constant<int, 16>{}, integral_constant<int, 4>{}, "fit16x4");
+    run(integral_constant<int, 16>{}, integral_constant<int, 8>{}, "fit16x8");
+    run(integral_constant<int, 16>{}, integral_constant<int, 16>{}, "fit16x16");
+    run(integral_constant<int, 16>{}, integral_constant<int, 28>{}, "fit16x28");
+    run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, "fit8x4");
+    run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, "fit8x12");
+    return ok ? name : nullptr;
+}
+
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, int ROWOP = kRowsPrepared>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT, ROWOP>;
@@ -495,6 +704,9 @@ bool launch_split(hipStream_t s, const LinearArgs& a, size_t lds, int split) {
 
 template <int MODE, int GK, bool W4 = false>
 const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
+    if constexpr (MODE == (int)Epilogue::DequantF32 && !W4) {
+        if (const char* fit = launch_fit_mode<GK>(s, a, cu_count, force)) return fit;
+    }
     // blocks of the stream per panel, and the units a wave's run is made of
     constexpr uint32_t SPB = W4 ? 2 : 1, UNIT = GK > SPB ? GK : SPB;
     const uint32_t steps = ((a.k + 31u) / 32u + SPB - 1u) / SPB;  // 1 KiB blocks per panel
