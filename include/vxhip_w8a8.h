@@ -406,6 +406,22 @@ int vxhip_packed_linear_forward_f32(VxHipContext* context,
                                     const float* input_dev, float* output_dev,
                                     uint32_t rows);
 
+/* The same with the reference's output window (src/kernels/llm_ops.h:48-52,
+ * src/kernels/packed_linear_ops.inc:1550-1553, 1593-1596) on resident tensors:
+ * input_dev [rows, k] and output_dev [rows, n] are the whole tensors, units
+ * [first_unit, first_unit + unit_count) of the row-major output are written
+ * (unit_count 0: all of it), every other element keeps its value.  Only the
+ * rows the window touches are computed; a window that begins or ends inside a
+ * row is computed into the context's staging buffer and its elements copied
+ * (one device-to-device copy on the context's stream).  Returns 0, or -1 for a
+ * window that does not fit or a rejected descriptor. */
+int vxhip_packed_linear_forward_f32_window(VxHipContext* context,
+                                           const VxHipPackedLinear* linear,
+                                           const float* input_dev,
+                                           float* output_dev, uint32_t rows,
+                                           uint64_t first_unit,
+                                           uint64_t unit_count);
+
 /* The fused single-row decode forms of the reference's device route
  * (native/src/backends/cuda/kernels/cuda_forward_gemv_pair_kernels.inc:
  * vx_cuda_rmsnorm_packed_linear_triple_decode_a8 :1136,
@@ -472,14 +488,21 @@ int vxhip_packed_linear_forward_a8(VxHipContext* context,
  * entry takes the same values as plain arguments: x=input f32 [rows,k],
  * packed_weight, scale, bias (optional), y=out [rows,n], key_dim=k,
  * value_dim=n, rate=group_size, groups=weight_bits (8, 4, 3 or 2; 0 means 4
- * as in the reference), normalize=8.  The packed weight stays resident
- * between calls (see vxhip_resident_weights_clear).
+ * as in the reference), normalize=8, and the output window first_unit /
+ * unit_count (src/kernels/llm_ops.h:48-52): units are elements of the row-major
+ * output, [first_unit, first_unit + unit_count) are written and every other
+ * element of `output` is left as it was; unit_count 0 stands for the whole
+ * output ("a zero unit_count preserves whole-graph dispatch"); a window that
+ * does not fit rows * n is refused (src/kernels/packed_linear_ops.inc:1550-1553).
+ * `input` and `output` are the whole tensors, as in the reference.  The packed
+ * weight stays resident between calls (see vxhip_resident_weights_clear).
  * Returns 0 / -1 like vx_llm_forward_f32 (src/kernels/llm_ops.inc:41-56). */
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight,
                             const float* scale, const float* bias,
                             float* output, uint64_t rows, int32_t key_dim,
                             int32_t value_dim, int32_t rate, int32_t groups,
-                            int32_t normalize);
+                            int32_t normalize, uint64_t first_unit,
+                            uint64_t unit_count);
 
 /* The host-pointer entry points (vxhip_qlinear_i8u8, vxhip_packed_linear_f32) keep
  * the weights they are given resident on the device -- prepacked, with scales,

@@ -111,6 +111,9 @@ class Oracle:
         L.vxo_packed_linear_forward_bits.restype = C.c_int
         L.vxo_packed_linear_forward_bits.argtypes = (
             list(L.vxo_packed_linear_forward.argtypes) + [C.c_uint32])
+        L.vxo_packed_linear_forward_window.restype = C.c_int
+        L.vxo_packed_linear_forward_window.argtypes = (
+            list(L.vxo_packed_linear_forward.argtypes) + [C.c_uint32, C.c_uint64, C.c_uint64])
         L.vxo_packed_linear_a8_bits.restype = C.c_int
         L.vxo_packed_linear_a8_bits.argtypes = (
             list(L.vxo_packed_linear_a8.argtypes) + [C.c_uint32])
@@ -179,6 +182,13 @@ class Oracle:
             _ptr(x, _f32p), _ptr(packed, _u32p), _ptr(scales, _f32p),
             _ptr(bias, _f32p), _ptr(y, _f32p), rows, k, n, group, bits)
         return st, y
+
+    def packed_linear_window(self, x, packed, scales, bias, out, group, first_unit, unit_count, bits=8):
+        """Writes the window's elements of `out` [rows, n] in place; returns the status."""
+        rows, k = x.shape
+        return self.lib.vxo_packed_linear_forward_window(
+            _ptr(x, _f32p), _ptr(packed, _u32p), _ptr(scales, _f32p), _ptr(bias, _f32p), _ptr(out, _f32p),
+            rows, k, out.shape[1], group, bits, int(first_unit), int(unit_count))
 
     def packed_linear_a8(self, a, row_scales, packed, scales, bias, n, group,
                          row_finite=None, bits=8):
@@ -430,10 +440,13 @@ class Reference:
             rows, k, n, w_dtype, int(zero_zp)))
 
     # PackedLinear -----------------------------------------------------------
-    def packed_linear(self, x, packed, scales, bias, n, group, bits=8):
+    def packed_linear(self, x, packed, scales, bias, n, group, bits=8, first_unit=0, unit_count=0, out=None):
+        """vx_llm_forward_f32 on a PackedLinear node; with `out` given it is written in place, so a
+        window (first_unit, unit_count) shows what the reference leaves untouched."""
         rows, k = x.shape
-        y = np.zeros((rows, n), dtype=np.float32)
+        y = np.zeros((rows, n), dtype=np.float32) if out is None else out
         a = _LLMOpArgs()
+        a.first_unit, a.unit_count = int(first_unit), int(unit_count)
         a.kind = OP_PACKED_LINEAR
         a.batch, a.sequence = 1, rows
         a.key_dim, a.value_dim = k, n

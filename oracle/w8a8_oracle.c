@@ -326,6 +326,47 @@ int vxo_packed_linear_forward_bits(const float* input, const uint32_t* packed,
     return status;
 }
 
+/* vx_packed_linear_forward with its output window (packed_linear_ops.inc:1550-1553:
+ * units are elements of the row-major output; unit_count 0 = rows * n; a window
+ * past the end is refused; :1555 the rows first / n .. ceil((first + units) / n);
+ * :1593-1596 per row the columns [begin, end) that lie inside the window).  Every
+ * element outside the window keeps its value. */
+int vxo_packed_linear_forward_window(const float* input, const uint32_t* packed,
+                                     const float* scales, const float* bias,
+                                     float* output, uint64_t rows, uint32_t k,
+                                     uint32_t n, uint32_t group_size,
+                                     uint32_t weight_bits, uint64_t first_unit,
+                                     uint64_t unit_count) {
+    if (!input || !k || !n || !group_size_ok(group_size)) return -1;
+    const uint64_t first = first_unit;
+    const uint64_t units = unit_count ? unit_count : rows * n;
+    if (first > rows * n || units > rows * n - first) return -1;
+    int8_t* prepared = (int8_t*)malloc(k);
+    float* whole = (float*)malloc((size_t)n * sizeof(float));
+    if (!prepared || !whole) {
+        free(prepared);
+        free(whole);
+        return -1;
+    }
+    int status = 0;
+    for (uint64_t row = first / n; row < (first + units + n - 1u) / n && status == 0; row++) {
+        float as;
+        const uint8_t finite =
+            (uint8_t)vxo_packed_prepare_i8(input + row * k, k, prepared, &as);
+        status = vxo_packed_linear_a8_bits(prepared, &as, &finite, packed, scales,
+                                           bias, whole, NULL, 1u, k, n,
+                                           group_size, weight_bits);
+        const uint32_t begin = first > row * n ? (uint32_t)(first - row * n) : 0u;
+        const uint32_t end = first + units < (row + 1u) * n
+                                 ? (uint32_t)(first + units - row * n) : n;
+        for (uint32_t c = begin; c < end && status == 0; c++)
+            output[row * n + c] = whole[c];
+    }
+    free(prepared);
+    free(whole);
+    return status;
+}
+
 int vxo_packed_linear_forward(const float* input, const uint32_t* packed,
                               const float* scales, const float* bias,
                               float* output, uint64_t rows, uint32_t k,

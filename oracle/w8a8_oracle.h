@@ -114,6 +114,19 @@ int vxo_packed_linear_forward_bits(const float* input, const uint32_t* packed,
                                    float* output, uint64_t rows, uint32_t k,
                                    uint32_t n, uint32_t group_size,
                                    uint32_t weight_bits);
+/* vx_packed_linear_forward restricted to its output window (VxLLMOpArgs
+ * first_unit / unit_count, src/kernels/llm_ops.h:48-52; the bounds check, the row
+ * range and the per-row column range of src/kernels/packed_linear_ops.inc:
+ * 1550-1553, 1555, 1593-1596): units are elements of the row-major output,
+ * unit_count 0 = all rows * n, elements outside the window are not written.
+ * Pinned by the reference's own window cases (native/tests/
+ * test_packed_linear_i8.c:186-188 and :263-278) against oracle/_ref. */
+int vxo_packed_linear_forward_window(const float* input, const uint32_t* packed,
+                                     const float* scales, const float* bias,
+                                     float* output, uint64_t rows, uint32_t k,
+                                     uint32_t n, uint32_t group_size,
+                                     uint32_t weight_bits, uint64_t first_unit,
+                                     uint64_t unit_count);
 int vxo_packed_linear_a8_bits(const int8_t* activation, const float* row_scales,
                               const uint8_t* row_finite, const uint32_t* packed,
                               const float* scales, const float* bias,

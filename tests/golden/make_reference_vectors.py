@@ -76,6 +76,20 @@ PACKED_CASES = [dict(rows=r, k=k, n=n, group=g, seed=s, with_bias=b, special_row
     (200, 768, 136, 256, 44, True, True)]]
 
 
+# Output windows (VxLLMOpArgs.first_unit / unit_count): the reference's own window list for 11 rows of n
+# (native/tests/test_packed_linear_i8.c:263-265) and its small case (:186-187), on seeded inputs; the whole
+# output array, pre-filled with the guard value 12345, is what gets digested.
+WINDOW_GUARD = 12345.0
+PACKED_WINDOW_CASES = [dict(rows=11, k=k, n=n, group=g, seed=s, bits=b) for (k, n, g, s, b) in [
+    (257, 19, 64, 61, 8), (1283, 5, 128, 62, 8), (320, 13, 32, 63, 4), (96, 1, 32, 64, 8)]]
+
+
+def window_list(rows, n):
+    firsts = [0, 1, n - 1, n + 2, n, 3]
+    counts = [0, rows * n - 2, 4 * n + 2, 3 * n - 2, 8 * n, 14]
+    return [(f, c) for f, c in zip(firsts, counts) if f <= rows * n and (c or rows * n) <= rows * n - f]
+
+
 REQUANTIZE_CASES = [dict(elements=e, seed=s, input_dtype=i, output_dtype=o) for (e, s, i, o) in [
     (4096, 51, I8, I8), (4096, 52, I8, U8), (4096, 53, U8, I8), (4096, 54, U8, U8), (100003, 55, I8, I8), (7, 56, U8, I8)]]
 
@@ -94,7 +108,7 @@ def main():
     out = {"_comment": "Outputs of the reference's C kernels on the seeded inputs of tests/_cases.py; "
                        "written by tests/golden/make_reference_vectors.py.",
            "qlinear": [], "rowscale": [], "packed": [], "packed_w4": [], "packed_w3": [], "packed_w2": [],
-           "requantize": []}
+           "requantize": [], "packed_window": []}
     for kind, params in QLINEAR_CASES:
         c = build_case(kind, params)
         args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
@@ -134,6 +148,21 @@ def main():
             st, y = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits)
             assert st == 0
             out[f"packed_w{bits}"].append({"params": params, "expected": digest(y)})
+    for params in PACKED_WINDOW_CASES:
+        bits = params["bits"]
+        c = cases.packed_case(**{k: v for k, v in params.items() if k != "bits"}, special_rows=True)
+        words = orc.pack_w8_words(c["w"]) if bits == 8 else orc.pack_w4_words(cases.four_bit(c["w"]))
+        for first, count in window_list(params["rows"], params["n"]):
+            y = np.full((params["rows"], params["n"]), WINDOW_GUARD, np.float32)
+            st, _ = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits,
+                                      first_unit=first, unit_count=count, out=y)
+            assert st == 0
+            out["packed_window"].append({"params": params, "first_unit": first, "unit_count": count, "expected": digest(y)})
+        # a window that does not fit is refused and nothing is written
+        y = np.full((params["rows"], params["n"]), WINDOW_GUARD, np.float32)
+        st, _ = ref.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=bits,
+                                  first_unit=2, unit_count=params["rows"] * params["n"] - 1, out=y)
+        assert st == -1 and (y == WINDOW_GUARD).all()
     for params in REQUANTIZE_CASES:
         c = cases.requantize_case(**params)
         ok, y = ref.requantize_linear(c["x"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"], c["out_dtype"])

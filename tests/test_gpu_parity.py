@@ -1129,3 +1129,84 @@ def test_operand_order_activations(oracle, rows, k, n, group):
         blocked.synchronize()
         assert st == 0 and same_f32(host(y), want_big)
     pl.close(), plain.close(), blocked.close()
+
+
+@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (2048, 32, "fit16x4"),
+                                              (3072, 128, "fit8x12"), (4096, 128, "fit16x8"), (4096, 256, "fit16x8"),
+                                              (4090, 64, "fit16x8"), (8192, 128, "fit16x16"), (14336, 128, "fit16x28")])
+def test_exact_fit_gemv(oracle, k, group, instance):
+    """The straight-line streaming kernel for a K whose blocks divide evenly over the waves: every
+    instance, rows on both sides of its LDS-copy limit (more rows only when named), both activation
+    layouts, a row whose scale is NaN, an n that ends inside a panel -- the oracle's bits each time;
+    and the general kernel still gives them when the exact-fit one is ruled out by name."""
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    n = 6150 if k <= 4096 else 70  # 193 panels: taken without being named; the long rows only by name
+    plain, blocked = vx.Context(0, None), vx.Context(0, None)
+    blocked.set_activation_layout(True)
+    c = cases.packed_case(32, k, n, group, 4000 + k + group, True, special_rows=True)
+    words = oracle.pack_w8_words(c["w"])
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+    waves, bpw = (int(v) for v in instance[3:].split("x"))
+    groups = (k + group - 1) // group
+    try:
+        for rows in (1, 2, 4, 5, 16, 32):
+            # (the products of every group, the waves' scales and, for few rows, their activation slices share LDS)
+            lds = groups * rows * 128 + waves * (groups // waves * 32 + 32) * 4 + (waves * 2 * bpw * rows * 16 if rows <= 4 else 0)
+            if lds > 156 * 1024:
+                continue
+            x = c["x"][:rows].copy()
+            if rows >= 2:
+                x[-1, 7 % k] = np.nan  # a row that is not finite: a NaN scale, a NaN output row
+            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
+            for ctx in (plain, blocked):
+                codes, scales = packed_prepare_i8(ctx, dev(x))
+                for force in (None, "gemv.fit", "gemv.nofit"):
+                    vx.force_variant(force)
+                    st, y = pl.forward_a8(ctx, codes, scales)
+                    ctx.synchronize()
+                    assert st == 0 and same_f32(host(y), want), (rows, force, ctx.last_variant)
+                    named = force == "gemv.fit" or (force is None and rows <= 4 and n >= 6144)
+                    assert ctx.last_variant.endswith(instance) == named, (rows, force, ctx.last_variant)
+    finally:
+        vx.force_variant(None)
+        pl.close(), plain.close(), blocked.close()
+
+
+def test_packed_output_window(ctx, oracle):
+    """first_unit / unit_count of the PackedLinear descriptor (llm_ops.h:48-52) on both entry points: the
+    reference's window list on 11 rows (test_packed_linear_i8.c:263-265), the whole output array --
+    guard values included -- against the oracle's; a window that does not fit is refused untouched."""
+    import torch
+    import volvoxai_amd as vx
+    for k, n, group, bits in [(257, 19, 64, 8), (1283, 5, 128, 8), (320, 13, 32, 4), (4096, 6150, 128, 8)]:
+        rows = 11 if n < 100 else 3
+        c = cases.packed_case(rows, k, n, group, 4100 + k, True, special_rows=rows >= 5)
+        words = oracle.pack_w8_words(c["w"]) if bits == 8 else oracle.pack_w4_words(cases.four_bit(c["w"]))
+        pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=bits)
+        xd = dev(c["x"])
+        windows = [(0, 0), (1, rows * n - 2), (n - 1, 4 * n + 2), (n + 2, 3 * n - 2), (n, 8 * n), (3, 14), (2 * n, n), (0, 1)]
+        for first, count in windows:
+            if first > rows * n or (count or rows * n) > rows * n - first:
+                continue
+            want = np.full((rows, n), 12345.0, np.float32)
+            assert oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], want, group, first, count, bits=bits) == 0
+            got = np.full((rows, n), 12345.0, np.float32)
+            st, _ = vx.packed_linear_f32(c["x"], words, c["scales"], c["bias"], k, n, group, groups=bits,
+                                         first_unit=first, unit_count=count, out=got)
+            assert st == 0 and (got.view(np.uint32) == want.view(np.uint32)).all(), (k, n, first, count)
+            yd = torch.full((rows, n), 12345.0, dtype=torch.float32, device="cuda")
+            st = pl.forward_f32_window(ctx, xd, yd, first, count)
+            ctx.synchronize()
+            assert st == 0 and (host(yd).view(np.uint32) == want.view(np.uint32)).all(), (k, n, first, count, ctx.last_variant)
+        for first, count in [(rows * n + 1, 0), (2, rows * n - 1), (rows * n, 0)]:
+            got = np.full((rows, n), 12345.0, np.float32)
+            st, _ = vx.packed_linear_f32(c["x"], words, c["scales"], c["bias"], k, n, group, groups=bits,
+                                         first_unit=first, unit_count=count, out=got)
+            assert st == -1 and (got == 12345.0).all()
+            yd = torch.full((rows, n), 12345.0, dtype=torch.float32, device="cuda")
+            assert pl.forward_f32_window(ctx, xd, yd, first, count) == -1
+            ctx.synchronize()
+            assert (host(yd) == 12345.0).all()
+        pl.close()
+    vx.library().vxhip_resident_weights_clear()

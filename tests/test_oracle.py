@@ -171,6 +171,66 @@ def test_packed_w4_matches_reference_vectors(oracle, entry):
     check_digest(y, entry["expected"])
 
 
+def window_case(entry, oracle):
+    params = entry["params"]
+    c = cases.packed_case(**{k: v for k, v in params.items() if k != "bits"}, special_rows=True)
+    words = oracle.pack_w8_words(c["w"]) if params["bits"] == 8 else oracle.pack_w4_words(cases.four_bit(c["w"]))
+    return c, words
+
+
+@pytest.mark.parametrize("entry", VECTORS["packed_window"],
+                         ids=lambda e: f"{'x'.join(str(v) for v in e['params'].values())}-{e['first_unit']}+{e['unit_count']}")
+def test_packed_output_window_matches_reference_vectors(oracle, entry):
+    """first_unit / unit_count: the window's elements are the full call's, everything else keeps the
+    guard value -- the whole array against what the reference's kernel left in it."""
+    c, words = window_case(entry, oracle)
+    y = np.full((entry["params"]["rows"], c["n"]), 12345.0, np.float32)
+    st = oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], y, c["group"], entry["first_unit"],
+                                     entry["unit_count"], bits=entry["params"]["bits"])
+    assert st == 0
+    check_digest(y, entry["expected"])
+    # and what the rule fixes without any reference: window = slice of the full output, rest = guard
+    _, full = oracle.packed_linear(c["x"], words, c["scales"], c["bias"], c["n"], c["group"], bits=entry["params"]["bits"])
+    first, count = entry["first_unit"], entry["unit_count"] or full.size
+    flat, want = y.reshape(-1), full.reshape(-1)
+    inside = np.zeros(full.size, bool)
+    inside[first:first + count] = True
+    assert (flat[~inside] == 12345.0).all()
+    nan = np.isnan(want)
+    assert (np.isnan(flat[inside]) == nan[inside]).all()
+    assert (flat.view(np.uint32)[inside & ~nan] == want.view(np.uint32)[inside & ~nan]).all()
+
+
+def test_packed_output_window_refusals(oracle):
+    c = cases.packed_case(4, 64, 6, 32, 5)
+    words = oracle.pack_w8_words(c["w"])
+    for first, count in [(25, 0), (0, 25), (2, 23), (24, 1)]:  # 24 units in all
+        y = np.full((4, 6), 12345.0, np.float32)
+        assert oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], y, 32, first, count) == -1
+        assert (y == 12345.0).all()
+    y = np.full((4, 6), 12345.0, np.float32)
+    assert oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], y, 32, 24, 0) == -1  # 0 units = all 24: past the end
+    assert oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], y, 32, 23, 1) == 0
+    assert (y.reshape(-1)[:23] == 12345.0).all() and y[3, 5] != 12345.0
+
+
+def test_live_reference_packed_output_window(oracle, reference):
+    rng = np.random.default_rng(77)
+    for trial in range(40):
+        rows, k, n = int(rng.integers(1, 9)), int(rng.choice([31, 64, 200])), int(rng.integers(1, 12))
+        group = int(rng.choice([32, 64, 128, 256]))
+        c = cases.packed_case(rows, k, n, group, 300 + trial, with_bias=bool(trial % 2), special_rows=True)
+        words = oracle.pack_w8_words(c["w"])
+        first = int(rng.integers(0, rows * n + 2))
+        count = int(rng.integers(0, rows * n + 2))
+        a = np.full((rows, n), 12345.0, np.float32)
+        b = a.copy()
+        sa = oracle.packed_linear_window(c["x"], words, c["scales"], c["bias"], a, group, first, count)
+        sb, _ = reference.packed_linear(c["x"], words, c["scales"], c["bias"], n, group, first_unit=first, unit_count=count, out=b)
+        assert sa == sb, (trial, first, count)
+        assert (a.view(np.uint32) == b.view(np.uint32)).all(), (trial, first, count)
+
+
 @pytest.mark.parametrize("bits", [3, 2])
 def test_packed_low_bit_matches_reference_vectors(oracle, bits):
     for entry in VECTORS[f"packed_w{bits}"]:

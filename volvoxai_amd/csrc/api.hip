@@ -1291,13 +1291,61 @@ int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* ctx, const VxHipPacked
     return packed_run_a8(ctx, pl, prepared, ld, false, row_scales, output_dev, nullptr, nullptr, rows);
 }
 
+// The output window of vx_packed_linear_forward (packed_linear_ops.inc:1550-1553): units are elements of
+// the row-major output, [first, first + count); a count of 0 stands for the whole output (and then only
+// first = 0 fits).  False for a window the reference refuses.
+static bool unit_window(uint64_t rows, uint32_t n, uint64_t first_unit, uint64_t unit_count, uint64_t* first,
+                        uint64_t* units) {
+    const uint64_t all = rows * n;
+    *first = first_unit;
+    *units = unit_count ? unit_count : all;
+    return first_unit <= all && *units <= all - first_unit;
+}
+
+int vxhip_packed_linear_forward_f32_window(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,
+                                           float* output_dev, uint32_t rows, uint64_t first_unit, uint64_t unit_count) {
+    if (!ctx || !pl || !input_dev || !output_dev) {
+        set_error("packed_linear_forward_f32_window: null handle or tensor");
+        return -1;
+    }
+    const uint32_t n = pl->w.n, k = pl->w.k;
+    uint64_t first = 0, units = 0;
+    if (!unit_window(rows, n, first_unit, unit_count, &first, &units)) {
+        set_error("packed_linear_forward_f32_window: units [%llu, +%llu) do not fit %u rows of %u", (unsigned long long)first_unit,
+                  (unsigned long long)unit_count, rows, n);
+        return -1;
+    }
+    if (!units) return 0;
+    // the rows the window touches; whole rows are computed, the window's elements are what gets written
+    const uint64_t r0 = first / n, r1 = (first + units + n - 1u) / n;
+    const float* x = input_dev + r0 * k;
+    if (first % n == 0u && (first + units) % n == 0u)
+        return vxhip_packed_linear_forward_f32(ctx, pl, x, output_dev + first, (uint32_t)(r1 - r0));
+    if (!use_device(ctx->device)) return -1;
+    if (ctx->recording && (size_t)(r1 - r0) * n * 4u > ctx->io_out_bytes) {
+        set_error("packed_linear_forward_f32_window: a recording cannot grow the staging buffer");
+        return -1;
+    }
+    if (!io_staging(ctx, 0, (size_t)(r1 - r0) * n * 4u)) return -1;
+    float* staged = (float*)ctx->io_out;
+    const int st = vxhip_packed_linear_forward_f32(ctx, pl, x, staged, (uint32_t)(r1 - r0));
+    if (st != 0) return st;
+    if (hipMemcpyAsync(output_dev + first, staged + (first - r0 * n), (size_t)units * 4u, hipMemcpyDeviceToDevice,
+                       ctx->stream) != hipSuccess)
+        return -1;
+    return 0;
+}
+
 int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, const float* scale,
                             const float* bias, float* output, uint64_t rows, int32_t key_dim,
-                            int32_t value_dim, int32_t rate, int32_t groups, int32_t normalize) {
+                            int32_t value_dim, int32_t rate, int32_t groups, int32_t normalize,
+                            uint64_t first_unit, uint64_t unit_count) {
     // descriptor checks of vx_packed_linear_forward (packed_linear_ops.inc:1545-1554)
     if (!input || !packed_weight || !scale || !output || key_dim <= 0 || value_dim <= 0 || !rows ||
         rows > 0x7fffffffull)
         return -1;
+    uint64_t first = 0, units = 0;
+    if (!unit_window(rows, (uint32_t)value_dim, first_unit, unit_count, &first, &units)) return -1;
     const uint32_t bits = groups ? (uint32_t)groups : 4u;
     if ((bits != 8u && bits != 4u && bits != 3u && bits != 2u) || normalize != 8) {
         set_error("packed_linear_f32: this backend runs weight_bits 2, 3, 4 and 8 under DYNAMIC_I8 only");
@@ -1327,11 +1375,19 @@ int vxhip_packed_linear_f32(const float* input, const uint32_t* packed_weight, c
             return -1;
         resident_insert(key, held, (size_t)vxhip_packed_linear_resident_bytes(held->packed));
     }
-    const size_t in_bytes = (size_t)rows * key_dim * 4u, out_bytes = (size_t)rows * value_dim * 4u;
+    if (!units) return 0;
+    // Only the rows the window touches travel; they are computed whole and the window's elements, which
+    // are one run of the row-major output, are what is copied back: everything else in `output` stays
+    // as it was (the reference writes columns [begin, end) of the first and last row, :1593-1596).
+    const uint64_t r0 = first / n, r1 = (first + units + n - 1u) / n;
+    const size_t in_bytes = (size_t)(r1 - r0) * k * 4u, out_bytes = (size_t)(r1 - r0) * n * 4u;
     int st = -1;
-    if (io_staging(ctx, in_bytes, out_bytes) && vxhip_memcpy_to_device(ctx, ctx->io_in, input, in_bytes) == VXHIP_OK) {
-        st = vxhip_packed_linear_forward_f32(ctx, held->packed, (const float*)ctx->io_in, (float*)ctx->io_out, (uint32_t)rows);
-        if (st == 0 && vxhip_memcpy_to_host(ctx, output, ctx->io_out, out_bytes) != VXHIP_OK) st = -1;
+    if (io_staging(ctx, in_bytes, out_bytes) && vxhip_memcpy_to_device(ctx, ctx->io_in, input + r0 * k, in_bytes) == VXHIP_OK) {
+        st = vxhip_packed_linear_forward_f32(ctx, held->packed, (const float*)ctx->io_in, (float*)ctx->io_out,
+                                             (uint32_t)(r1 - r0));
+        if (st == 0 && vxhip_memcpy_to_host(ctx, output + first, (const float*)ctx->io_out + (first - r0 * n),
+                                            (size_t)units * 4u) != VXHIP_OK)
+            st = -1;
     }
     (void)hipStreamSynchronize(ctx->stream);
     return st;

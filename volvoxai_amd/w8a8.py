@@ -332,6 +332,17 @@ class PackedLinear:
         st = entry(ctx._h, self._h, _dp(x, "x", torch.float32), _dp(out, "out", torch.float32, (rows, self.n)), rows)
         return st, out
 
+    def forward_f32_window(self, ctx: Context, x, out, first_unit, unit_count):
+        """Writes units [first_unit, first_unit + unit_count) of the row-major `out` [rows, n] (0 units:
+        all of it) and leaves the rest of it alone: the reference's first_unit / unit_count."""
+        import torch
+        if x.ndim != 2 or x.shape[1] != self.k:
+            raise ValueError(f"x: shape {tuple(x.shape)}, expected [rows, {self.k}]")
+        rows = x.shape[0]
+        return library().vxhip_packed_linear_forward_f32_window(
+            ctx._h, self._h, _dp(x, "x", torch.float32), _dp(out, "out", torch.float32, (rows, self.n)), rows,
+            int(first_unit), int(unit_count))
+
     def forward_fused(self, ctx: Context, x, row_op=ROW_OP_NONE, gain=None, eps=0.0, add_to=None, out=None):
         """One or two f32 rows through [RMSNorm | SwiGLU] -> preparation -> linear [-> residual add] in one
         launch.  x is [rows, k], or [rows, 2k] = [gate | up] for ROW_OP_SWIGLU; add_to [rows, n] may be
@@ -551,16 +562,22 @@ def qlinear_i8u8(input, weight, weight_scales, weight_zero_points, bias, rows, d
     return int(ok), out
 
 
-def packed_linear_f32(x, packed_weight, scale, bias, key_dim, value_dim, rate, groups=8, normalize=8):
-    """vx_llm_forward_f32 for a PackedLinear node: (status, out[rows, value_dim])."""
+def packed_linear_f32(x, packed_weight, scale, bias, key_dim, value_dim, rate, groups=8, normalize=8,
+                      first_unit=0, unit_count=0, out=None):
+    """vx_llm_forward_f32 for a PackedLinear node: (status, out[rows, value_dim]).  first_unit /
+    unit_count: the reference's output window in elements of the row-major output (0 units = all);
+    `out`, when given, is written in place and keeps every element outside the window."""
     xx = _np(x, np.float32)
     rows = xx.shape[0]
     pw = _np(packed_weight, np.uint32)
     sc = _np(scale, np.float32)
     b = None if bias is None else _np(bias, np.float32)
-    out = np.zeros((rows, value_dim), dtype=np.float32)
+    if out is None:
+        out = np.zeros((rows, value_dim), dtype=np.float32)
+    elif out.dtype != np.float32 or out.shape != (rows, value_dim) or not out.flags.c_contiguous:
+        raise ValueError("out: a C-contiguous float32 array [rows, value_dim]")
     st = library().vxhip_packed_linear_f32(_hp(xx), _hp(pw), _hp(sc), _hp(b), _hp(out), rows,
-                                           key_dim, value_dim, rate, groups, normalize)
+                                           key_dim, value_dim, rate, groups, normalize, int(first_unit), int(unit_count))
     return int(st), out
 
 
