@@ -442,7 +442,9 @@ int vxhip_packed_linear_forward_f32_window(VxHipContext* context,
  * Returns 1 handled; 0 declined, nothing launched (more than two rows, k above
  * 4096 (8192 without RMSNorm), k below 1024 with RMSNorm, a panel count the
  * eight-wave kernel does not take): the caller runs the separate launches;
- * -1 on an invalid argument. */
+ * -1 on an invalid argument, which includes input rows that overlap the output
+ * or the residual (every workgroup reads the whole rows while others already
+ * store; add_to_dev == output_dev is the one overlap that is safe). */
 #define VXHIP_ROW_OP_NONE 0u
 #define VXHIP_ROW_OP_RMSNORM 1u
 #define VXHIP_ROW_OP_SWIGLU 2u
@@ -452,6 +454,18 @@ int vxhip_packed_linear_forward_fused(VxHipContext* context,
                                       uint32_t row_op, const float* gain_dev,
                                       double eps, const float* add_to_dev,
                                       float* output_dev);
+
+/* 1 if vxhip_packed_linear_forward_fused would run a call of this description
+ * (rows, row operation, with or without a residual) on this context, 0 if it
+ * would decline; nothing is launched.  It is the launcher's own decision, made
+ * without launching, so the two cannot disagree.  A caller that updates its
+ * residual stream in place asks for every linear of a model once, up front: after
+ * the first fused launch of a layer has overwritten the stream there is no way
+ * back to the separate launches.  No counterpart in the reference. */
+int vxhip_packed_linear_fused_takes(VxHipContext* context,
+                                    const VxHipPackedLinear* linear,
+                                    uint32_t rows, uint32_t row_op,
+                                    int with_residual);
 
 /* vxhip_packed_linear_forward_f32 for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid

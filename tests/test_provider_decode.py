@@ -241,3 +241,36 @@ def test_decode_callbacks_at_benchmark_widths_match_the_python_wiring(libs, tmp_
     assert run.wrong_step_refused == 1 and run.reset_repeats == 1 and run.attested == 1
     # the first step is launched plainly, the second is recorded and run from the recording, like every later one
     assert run.replayed_steps == steps - 1
+
+
+@pytest.mark.gpu
+def test_one_slot_with_a_linear_the_fused_form_declines(libs, tmp_path, monkeypatch):
+    """One slot, hidden 1024 (which the fused single-row forms take) and a SwiGLU width above what they
+    take (the down projection would decline after the stream had been updated in place): the route is
+    decided over every linear up front, so the steps run the separate launches and succeed, with the
+    ids of the Python wiring -- also with the recording switched off."""
+    import torch
+    from volvoxai_amd.decoder import DecoderConfig, W8A8Decoder, init_weights
+    mock, _ = libs
+    cfg = DecoderConfig(layers=2, hidden=1024, q_heads=8, kv_heads=4, head_dim=128, inter=8448, vocab=640, max_seq=48)
+    weights = init_weights(cfg, 31)
+    slots, capacity, prompt_len, steps = 1, cfg.max_seq, 9, 5
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, (slots, prompt_len))
+    dec = W8A8Decoder(cfg, weights, slots)
+    assert not dec.rows_fused
+    first = dec.prefill(torch.from_numpy(prompt).cuda()).cpu().numpy()
+    want = dec.decode(steps).cpu().numpy()
+    dec.close()
+    g, w = decoder_package(tmp_path / "dec", cfg, weights, slots, capacity, with_logits=False)
+    for no_replay in (False, True):
+        if no_replay:
+            monkeypatch.setenv("VXHIP_PROVIDER_NO_REPLAY", "1")
+        ids = np.zeros((slots, capacity), np.int32)
+        ids[:, :prompt_len] = prompt
+        generated = np.full((steps + 1, slots), -1, np.int32)
+        run = MockDecode(str(g).encode(), str(w).encode(), b"token_ids", b"next_token_ids", None, slots, capacity, cfg.vocab,
+                         prompt_len, steps, ids.ctypes.data, generated.ctypes.data, None)
+        st = mock.mock_host_run_decode(C.byref(run))
+        assert st == 0 and run.failed_stage == 0, (st, run.failed_stage, run.message)
+        assert (generated[0] == first).all() and (generated == want).all()
+        assert run.replayed_steps == (0 if no_replay else steps - 1)

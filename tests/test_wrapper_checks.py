@@ -116,6 +116,13 @@ def test_packed_linear_wrappers_refuse_wrong_tensors():
         pl.forward_fused(ctx, fake(2, 128), ROW_OP_NONE, add_to=fake(1, 40), out=fake(2, 40))
     with pytest.raises(ValueError, match="row_op"):
         pl.forward_fused(ctx, fake(1, 128), 7, out=fake(1, 40))
+    # an input that shares memory with the output or the residual would be read half updated
+    shared = fake(1, 128)
+    with pytest.raises(ValueError, match="overlaps out"):
+        pl.forward_fused(ctx, shared, ROW_OP_NONE, out=shared[:, :40].contiguous().set_(shared.untyped_storage(), 0, (1, 40)))
+    with pytest.raises(ValueError, match="overlaps add_to"):
+        pl.forward_fused(ctx, shared, ROW_OP_NONE, add_to=torch.Tensor().set_(shared.untyped_storage(), 8, (1, 40)).as_subclass(FakeDevice),
+                         out=fake(1, 40))
 
 
 def test_attention_wrappers_refuse_wrong_shapes():

@@ -99,6 +99,7 @@ def _declare(L: C.CDLL) -> None:
         "vxhip_packed_linear_forward_f32": (C.c_int, [vp, vp, vp, vp, u32]),
         "vxhip_packed_linear_forward_f32_noalloc": (C.c_int, [vp, vp, vp, vp, u32]),
         "vxhip_packed_linear_forward_fused": (C.c_int, [vp, vp, vp, u32, u32, vp, C.c_double, vp, vp]),
+        "vxhip_packed_linear_fused_takes": (C.c_int, [vp, vp, u32, u32, C.c_int]),
         "vxhip_packed_linear_forward_a8": (C.c_int, [vp, vp, vp, vp, vp, vp, u32]),
         "vxhip_packed_linear_f32": (C.c_int, [vp, vp, vp, vp, vp, u64, i32, i32, i32, i32, i32, u64, u64]),
         "vxhip_packed_linear_forward_f32_window": (C.c_int, [vp, vp, vp, vp, u32, u64, u64]),

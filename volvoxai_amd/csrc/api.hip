@@ -1242,12 +1242,45 @@ int vxhip_packed_linear_forward_fused(VxHipContext* ctx, const VxHipPackedLinear
     }
     if (!rows) return 1;
     if (!same_device(ctx, pl->device, "packed_linear_forward_fused") || !use_device(ctx->device)) return -1;
+    // Every workgroup reads the whole input rows while others already store their channels: an input that
+    // overlaps the output (or the residual it is added to, which may itself be the output) would be read
+    // half updated.
+    {
+        const uintptr_t x0 = (uintptr_t)input_dev;
+        const uintptr_t x1 = x0 + (size_t)rows * (row_op == VXHIP_ROW_OP_SWIGLU ? 2u : 1u) * pl->w.k * 4u;
+        const size_t out_bytes = (size_t)rows * pl->w.n * 4u;
+        const uintptr_t y0 = (uintptr_t)output_dev, a0 = (uintptr_t)add_to_dev;
+        if ((x0 < y0 + out_bytes && y0 < x1) || (add_to_dev && x0 < a0 + out_bytes && a0 < x1)) {
+            set_error("packed_linear_forward_fused: the input rows overlap the output or the residual");
+            return -1;
+        }
+    }
     RowOps ops;
     ops.gain = row_op == VXHIP_ROW_OP_RMSNORM ? gain_dev : nullptr;
     ops.eps = eps;
     ops.swiglu = row_op == VXHIP_ROW_OP_SWIGLU;
     ops.add_to = add_to_dev;
     return packed_run_f32_rows(ctx, pl, input_dev, output_dev, rows, ops) == 0 ? 1 : 0;
+}
+
+int vxhip_packed_linear_fused_takes(VxHipContext* ctx, const VxHipPackedLinear* pl, uint32_t rows, uint32_t row_op,
+                                    int with_residual) {
+    if (!ctx || !pl || !rows || row_op > VXHIP_ROW_OP_SWIGLU) return 0;
+    // the launcher's own decision, with nothing launched: stand-in addresses that are never dereferenced
+    static const float stand_in[4] = {0.f, 0.f, 0.f, 0.f};
+    static float stand_out[4];
+    RowOps ops;
+    ops.gain = row_op == VXHIP_ROW_OP_RMSNORM ? stand_in : nullptr;
+    ops.eps = 1e-6;
+    ops.swiglu = row_op == VXHIP_ROW_OP_SWIGLU;
+    ops.add_to = with_residual ? stand_out : nullptr;
+    char kept[sizeof ctx->last_variant];
+    memcpy(kept, ctx->last_variant, sizeof kept);
+    set_gemv_dry_run(true);
+    const int st = packed_run_f32_rows(ctx, pl, stand_in, stand_out, rows, ops);
+    set_gemv_dry_run(false);
+    memcpy(ctx->last_variant, kept, sizeof kept);
+    return st == 0 ? 1 : 0;
 }
 
 int vxhip_packed_linear_forward_f32_noalloc(VxHipContext* ctx, const VxHipPackedLinear* pl, const float* input_dev,

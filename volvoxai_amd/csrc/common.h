@@ -253,6 +253,9 @@ inline bool raise_lds_limit(const void* kernel, int bytes, std::atomic<uint64_t>
 }
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force);
+// While on (per thread), launch_gemv_stream chooses as always and launches nothing: its result tells
+// whether a call of that description would be taken.
+void set_gemv_dry_run(bool on);
 
 const char* forced_variant();
 

@@ -37,6 +37,10 @@ namespace vxhip {
 
 namespace {
 
+// While set on the calling thread the launchers of this file decide as always but launch nothing: what
+// launch_gemv_stream then returns tells whether (and as which variant) a call would run.
+thread_local bool gemv_dry_run = false;
+
 extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
 constexpr int kDepth = 4;  // 1 KiB blocks in flight per wave
@@ -635,6 +639,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 template <int GK, int WAVES, int BPW>
 bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds) {
     auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true> : gemv_fit_kernel<GK, WAVES, BPW, false>;
+    if (gemv_dry_run) return true;
     if (lds > 64u * 1024u) {
         static std::atomic<uint64_t> configured[2] = {{0}, {0}};
         if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[xlds ? 1 : 0])) return false;
@@ -687,6 +692,7 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, int ROWOP = kRowsPrepared>
 bool launch_panel(hipStream_t s, const LinearArgs& a, size_t lds) {
     auto kern = gemv_panel_kernel<MODE, GK, WAVES, W4, SPLIT, ROWOP>;
+    if (gemv_dry_run) return true;
     if (lds > 64u * 1024u) {
         static std::atomic<uint64_t> configured{0};
         if (!raise_lds_limit((const void*)kern, 160 * 1024, configured)) return false;
@@ -793,6 +799,8 @@ const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const 
 }
 
 }  // namespace
+
+void set_gemv_dry_run(bool on) { gemv_dry_run = on; }
 
 const char* launch_gemv_stream(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (cu_count <= 0) cu_count = 256;

@@ -117,8 +117,7 @@ class W8A8Decoder:
         # where the library takes every linear of a layer that way.  They take two rows as well, at the
         # speed of the separate launches (fuse_rows=True asks for them; None decides by the row count).
         wanted = rows == 1 if fuse_rows is None else bool(fuse_rows)
-        self.rows_fused = (wanted and rows <= 2 and 1024 <= cfg.hidden <= 4096 and cfg.q_dim <= 8192
-                           and cfg.inter <= 8192)
+        self.rows_fused = False  # settled below, once the linears exist: the library is asked about each one
         self.stream = stream if stream is not None else torch.cuda.Stream()
         self.ctx = vx.Context(0, self.stream)
         # prepared activations of up to 32 rows travel between the glue kernels and the GEMVs in
@@ -139,6 +138,13 @@ class W8A8Decoder:
                                 "gate_up": make(lw["gate_up"]), "down": make(lw["down"])})
         self.gain_f = torch.from_numpy(weights["norm_f"]).to(dev)
         self.lm_head = make(weights["lm_head"])
+        if wanted and rows <= 2:
+            # the residual stream is updated in place by the first fused launch of a layer, so every
+            # linear of every layer has to be taken that way, or none is
+            self.rows_fused = all(
+                L["qkv"].fused_takes(self.ctx, rows, vx.ROW_OP_RMSNORM, False) and L["o"].fused_takes(self.ctx, rows, vx.ROW_OP_NONE, True)
+                and L["gate_up"].fused_takes(self.ctx, rows, vx.ROW_OP_RMSNORM, False)
+                and L["down"].fused_takes(self.ctx, rows, vx.ROW_OP_SWIGLU, True) for L in self.layers)
         cos, sin = rope_tables(cfg)
         self.cos, self.sin = torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev)
         shape = (cfg.layers, rows, cfg.kv_heads, cfg.max_seq, cfg.head_dim)

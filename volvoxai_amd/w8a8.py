@@ -343,6 +343,10 @@ class PackedLinear:
             ctx._h, self._h, _dp(x, "x", torch.float32), _dp(out, "out", torch.float32, (rows, self.n)), rows,
             int(first_unit), int(unit_count))
 
+    def fused_takes(self, ctx: Context, rows, row_op=ROW_OP_NONE, with_residual=False) -> bool:
+        """Whether forward_fused would run a call of this description on ctx (nothing is launched)."""
+        return bool(library().vxhip_packed_linear_fused_takes(ctx._h, self._h, int(rows), int(row_op), 1 if with_residual else 0))
+
     def forward_fused(self, ctx: Context, x, row_op=ROW_OP_NONE, gain=None, eps=0.0, add_to=None, out=None):
         """One or two f32 rows through [RMSNorm | SwiGLU] -> preparation -> linear [-> residual add] in one
         launch.  x is [rows, k], or [rows, 2k] = [gate | up] for ROW_OP_SWIGLU; add_to [rows, n] may be
@@ -359,6 +363,12 @@ class PackedLinear:
             raise ValueError("gain: RMSNorm needs its gain vector")
         if out is None:
             out = torch.empty((rows, self.n), dtype=torch.float32, device=x.device)
+        # every workgroup reads the whole input rows while others already store: the input may not share
+        # memory with the output or the residual (add_to may be `out` itself)
+        x0, x1 = x.data_ptr(), x.data_ptr() + x.numel() * 4
+        for name, other in (("out", out), ("add_to", add_to)):
+            if other is not None and x0 < other.data_ptr() + other.numel() * 4 and other.data_ptr() < x1:
+                raise ValueError(f"x: overlaps {name}")
         handled = library().vxhip_packed_linear_forward_fused(
             ctx._h, self._h, _dp(x, "x", torch.float32), rows, row_op,
             _dp(gain if row_op == ROW_OP_RMSNORM else None, "gain", torch.float32, numel=self.k), float(eps),
