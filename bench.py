@@ -42,7 +42,8 @@ PEAK_INT8_TOPS = 5000.0   # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0     # HBM3E, MI355X
 # HBM-side bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under
 # profiles/ (each counter scaled by what it reads for a 512 MiB copy kernel).  A counter run
-# cannot share a process with the timed run, so the measured values are carried here.
+# cannot share a process with the timed run, so `roofline.traffic` is NOT measured by this run: the
+# values are carried here from those profiles, and the JSON line says so (`traffic_source`).
 MEASURED_TRAFFIC_BYTES = {
     "gemm_4096x4096x4096": 101_154_209 + 16_851_373,
     "gemv_1x4096x14336": 60_764_410 + 57_344,
@@ -78,14 +79,14 @@ def timed_region(fn, steps, torch, stream):
         e1.record(stream)
         stream.synchronize()
         once = max(e0.elapsed_time(e1), 1e-3)
-        rounds = max(1, int(np.ceil(MIN_TIMED_MS / once)))
+        singly_rounds = max(1, int(np.ceil(MIN_TIMED_MS / once)))
         e0.record(stream)
-        for _ in range(rounds):
+        for _ in range(singly_rounds):
             for i in range(steps):
                 fn(i)
         e1.record(stream)
         stream.synchronize()
-        res["singly_ms"] = e0.elapsed_time(e1) / (rounds * steps)
+        res["singly_ms"] = e0.elapsed_time(e1) / (singly_rounds * steps)
     try:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
@@ -95,6 +96,13 @@ def timed_region(fn, steps, torch, stream):
         with torch.cuda.stream(stream):
             graph.replay()
             stream.synchronize()
+            # the replay count comes from a timed replay of the graph itself (a replayed step is shorter
+            # than a singly launched one), with a margin, so that MIN_TIMED_MS are really timed
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            rounds = max(1, int(np.ceil(1.05 * MIN_TIMED_MS / max(e0.elapsed_time(e1), 1e-3))))
             marks = [event() for _ in range(rounds + 1)]
             marks[0].record(stream)
             for r in range(rounds):
@@ -106,7 +114,8 @@ def timed_region(fn, steps, torch, stream):
                    graph_replays=rounds)
     except RuntimeError as e:  # capture refused: report the singly launched figure only
         print(f"bench.py: HIP graph capture failed ({e}); timing single launches", file=sys.stderr)
-    res["timed_ms_total"] = (res["graph_ms"] if res["graph_ms"] is not None else res["singly_ms"]) * rounds * steps
+    res["timed_ms_total"] = (res["graph_ms"] * res["graph_replays"] if res["graph_ms"] is not None
+                             else res["singly_ms"] * singly_rounds) * steps
     return res
 
 
@@ -139,6 +148,21 @@ def host_cpu():
     allowed = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     share = int(os.environ.get("OMP_NUM_THREADS", "0")) or allowed
     return model, allowed, max(1, min(allowed, share))
+
+
+def host_physical_cores():
+    """Physical cores of the host as /proc/cpuinfo lists them (distinct (physical id, core id) pairs);
+    None if it does not say.  The baseline runs on this job's share of them, not on all."""
+    try:
+        cores, phys = set(), None
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("physical id"):
+                phys = line.split(":", 1)[1].strip()
+            elif line.startswith("core id"):
+                cores.add((phys, line.split(":", 1)[1].strip()))
+        return len(cores) or None
+    except OSError:
+        return None
 
 
 def _time_calls(call, seconds):
@@ -193,7 +217,10 @@ def cpu_baseline_gemm(rows, k, n, seed):
         one = None
     assert ok == 1
     return {"value": ops / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": kind, "sample": sample,
-            "ms_per_call": dt * 1e3, "single_thread": one, "cpu_model": model, "logical_cpus_allowed": allowed}
+            "ms_per_call": dt * 1e3, "single_thread": one, "cpu_model": model, "logical_cpus_allowed": allowed,
+            "host_physical_cores": host_physical_cores(),
+            "cores_note": "cores = the threads the baseline ran on: this job's share of the host (its OMP_NUM_THREADS), "
+                          "not every physical core of the host"}
 
 
 def cpu_baseline_gemv(k, n, seed):
@@ -223,7 +250,8 @@ def cpu_baseline_gemv(k, n, seed):
         kind, route = "port", "vxo_packed_linear_forward"
     return {"value": gb / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": kind,
             "sample": f"{route}, M=1 K={k} N={n} full size, {dt * 1e3:.2f} ms per call on {threads} threads",
-            "ms_per_call": dt * 1e3, "single_thread": one, "cpu_model": model, "logical_cpus_allowed": allowed}
+            "ms_per_call": dt * 1e3, "single_thread": one, "cpu_model": model, "logical_cpus_allowed": allowed,
+            "host_physical_cores": host_physical_cores()}
 
 
 def region_ms(fn, steps, torch, warmup=5):
@@ -501,7 +529,7 @@ def main():
         out["roofline"] = {"bound": "mfma", "achieved": ops / (wall_ms * 1e-3) / 1e12, "peak": PEAK_INT8_TOPS,
                            "unit": "TOP/s", "frac": ops / (wall_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                            "traffic": MEASURED_TRAFFIC_BYTES["gemm_4096x4096x4096"],
-                           "traffic_source": "profiles/gemm_k64_rowscale_4096x4096x4096.md (FETCH_SIZE + WRITE_SIZE runs)",
+                           "traffic_source": "carried from profiles/gemm_k64_rowscale_4096x4096x4096.md (separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs), not measured in this run",
                            "kernel": ctx.last_variant, "ops_per_launch": ops,
                            "avg_kernel_ms": wall_ms, "fastest_replay_kernel_ms": reg["graph_min_ms"],
                            "event_pair_per_launch_ms": {"mean": ev_mean, "median": ev_med, "min": ev_min},
@@ -532,9 +560,10 @@ def main():
     # ---- decode GEMV: M=1, K=4096, N=14336 -------------------------------------
     if args.only in (None, "gemv"):
         Mg, Kg, Ng, G = 1, 4096, 14336, 128
+        from volvoxai_amd.decoder import pack_w8_words
         d = cases.decode_case(Mg, Kg, Ng, G, 14336)
-        orc = Oracle()
-        words = orc.pack_w8_words(d["w"])
+        orc = Oracle()  # (the checker of the spot parity below, never part of what is timed)
+        words = pack_w8_words(d["w"])
         copies = 6  # 6 x 56 MiB > 256 MB Infinity Cache
         pls = [vx.PackedLinear(words, d["scales"], d["bias"], Kg, Ng, G) for _ in range(copies)]
         a8 = torch.from_numpy(d["a8"]).cuda()
@@ -579,7 +608,7 @@ def main():
         out["roofline_gemv"] = {"bound": "hbm", "achieved": gb / (gwall_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
                                 "unit": "GB/s", "frac": gb / (gwall_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                 "traffic": MEASURED_TRAFFIC_BYTES["gemv_1x4096x14336"],
-                                "traffic_source": "profiles/gemv_panel_1x4096x14336.md (FETCH_SIZE + WRITE_SIZE runs)",
+                                "traffic_source": "carried from profiles/gemv_fit_1x4096x14336.md (separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs), not measured in this run",
                                 "kernel": ctx.last_variant, "bytes_per_launch": gb, "avg_kernel_ms": gwall_ms,
                                 "fastest_replay_kernel_ms": greg["graph_min_ms"],
                                 "event_pair_per_launch_ms": {"mean": gmean, "median": gmed, "min": gmin},

@@ -22,6 +22,7 @@ HERE = Path(__file__).resolve().parent
 DTYPE_U8 = 5
 DTYPE_I8 = 6
 OP_PACKED_LINEAR = 1036  # src/generated/operator_vocabulary.h:127
+OP_ROTARY_EMBEDDING = 1030  # src/generated/operator_vocabulary.h:121
 
 _f32p = C.POINTER(C.c_float)
 _i32p = C.POINTER(C.c_int32)
@@ -463,6 +464,54 @@ class Reference:
         a.y_elements[0] = y.size
         st = self.lib.vx_llm_forward_f32(C.byref(a))
         return int(st), y
+
+    # decoder glue ----------------------------------------------------------------
+    def rmsnorm(self, x, gain, eps):
+        """rmsnorm_f32 (src/kernels/softmax_rmsnorm.inc:3-17)."""
+        out = np.zeros_like(x)
+        self.lib.rmsnorm_f32.restype = None
+        self.lib.rmsnorm_f32.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_double]
+        self.lib.rmsnorm_f32(_ptr(x, _f32p), _ptr(gain, _f32p), _ptr(out, _f32p), x.shape[0], x.shape[1], float(eps))
+        return out
+
+    def silu_mul(self, gate, up):
+        """silu_f32 then mul_f32 (src/kernels/elementwise_f32.inc:153-165): the SiLU and Mul nodes of a SwiGLU."""
+        gate, up = np.ascontiguousarray(gate), np.ascontiguousarray(up)
+        act, out = np.zeros_like(gate), np.zeros_like(gate)
+        self.lib.silu_f32.restype = None
+        self.lib.silu_f32.argtypes = [_f32p, _f32p, C.c_int]
+        self.lib.silu_f32(_ptr(gate, _f32p), _ptr(act, _f32p), gate.size)
+        self.lib.mul_f32.restype = None
+        self.lib.mul_f32.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+        self.lib.mul_f32(_ptr(act, _f32p), _ptr(up, _f32p), _ptr(out, _f32p), gate.size)
+        return out
+
+    def rotary(self, x, cos, sin):
+        """The RotaryEmbedding operator of vx_llm_forward_f32 (src/kernels/llm_math.h:256-274), half-split
+        pairs over the whole head: x [tokens, heads, d], cos and sin [tokens, d]."""
+        tokens, heads, d = x.shape
+        y = np.zeros_like(x)
+        a = _LLMOpArgs()
+        a.kind = OP_ROTARY_EMBEDDING
+        a.batch, a.sequence, a.heads, a.key_dim = 1, tokens, heads, d
+        a.rotary_dim, a.rotary_offset, a.interleaved = d, 0, 0
+        a.x[0], a.x[1], a.x[2] = x.ctypes.data, cos.ctypes.data, sin.ctypes.data
+        a.y[0] = y.ctypes.data
+        a.x_elements[0], a.x_elements[1], a.x_elements[2] = x.size, cos.size, sin.size
+        a.y_elements[0] = y.size
+        st = self.lib.vx_llm_forward_f32(C.byref(a))
+        return int(st), y
+
+    def attention(self, q, k, v, q_heads, kv_heads, head_dim, causal):
+        """cross_sdpa_gqa_f32 (src/kernels/cross_sdpa.inc:53) with scale f32(1/sqrt(head_dim)), no mask."""
+        out = np.zeros((q.shape[0], q_heads * head_dim), dtype=np.float32)
+        self.lib.cross_sdpa_gqa_f32.restype = None
+        self.lib.cross_sdpa_gqa_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_int]
+        self.lib.cross_sdpa_gqa_f32(_ptr(q, _f32p), _ptr(k, _f32p), _ptr(v, _f32p), _ptr(out, _f32p), q.shape[0], k.shape[0],
+                                    q.shape[1], k.shape[1], q_heads, kv_heads, head_dim,
+                                    float(np.float32(1.0 / np.sqrt(head_dim))), None, 0, int(causal))
+        return out
 
     def embedding(self, tokens, table):
         """embedding_f32 (src/kernels/embedding.inc:5-16); pointers travel as integers."""

@@ -27,14 +27,16 @@ class DecoderRef:
         return y
 
     def rmsnorm(self, x, gain):
-        xd = x.astype(np.float64)
-        inv = 1.0 / np.sqrt((xd * xd).mean(-1, keepdims=True) + self.cfg.eps)
-        return (xd * inv * gain.astype(np.float64)).astype(np.float32)
+        # the reference's own order of operations, pinned to rmsnorm_f32 bit for bit (tests/_glue_defs.py)
+        from _glue_defs import rmsnorm
+        return rmsnorm(x.reshape(-1, x.shape[-1]), gain, self.cfg.eps).reshape(x.shape)
 
     def rope(self, x, cos, sin):
-        half = self.cfg.head_dim // 2
-        partner = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
-        return (x * cos[None, :, None, :] + partner * sin[None, :, None, :]).astype(np.float32)
+        # x [rows, t, heads, d], tables [t, d]: the RotaryEmbedding operator's arithmetic, pinned the same way
+        from _glue_defs import rotary
+        rows, t = x.shape[:2]
+        y = rotary(x.reshape(rows * t, x.shape[2], x.shape[3]), np.tile(cos, (rows, 1)), np.tile(sin, (rows, 1)))
+        return y.reshape(x.shape)
 
     def forward(self, tokens, start, k_cache, v_cache, trace=None):
         """tokens [rows, t] at positions start..start+t-1; caches [layers][rows, kvh, seq, d] lists

@@ -4,7 +4,8 @@ Run in a container that has the reference tree:  the kernels are compiled from
 their sources by `make -C oracle ref` into oracle/_ref/libvxref.so, and every
 expected value below is an output of those kernels (qlinear_i8u8,
 vx_qlinear_i8u8_native, vx_qlinear_i8u8_packed, vx_llm_forward_f32,
-volvoxai_ptq_pack_bias_i32, requantize_linear_i8u8) on the seeded inputs of tests/_cases.py.  Large
+volvoxai_ptq_pack_bias_i32, requantize_linear_i8u8; for the decoder glue rmsnorm_f32, silu_f32, mul_f32,
+cross_sdpa_gqa_f32 and the RotaryEmbedding operator) on the seeded inputs of tests/_cases.py and tests/_glue_defs.py.  Large
 outputs are stored as a SHA-256 plus a leading slice; small ones whole.
 
     python tests/golden/make_reference_vectors.py
@@ -23,6 +24,7 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
 import _cases as cases  # noqa: E402
+import _glue_defs as glue  # noqa: E402
 from oracle.pyoracle import Oracle, Reference  # noqa: E402
 
 I8, U8 = cases.DTYPE_I8, cases.DTYPE_U8
@@ -108,7 +110,7 @@ def main():
     out = {"_comment": "Outputs of the reference's C kernels on the seeded inputs of tests/_cases.py; "
                        "written by tests/golden/make_reference_vectors.py.",
            "qlinear": [], "rowscale": [], "packed": [], "packed_w4": [], "packed_w3": [], "packed_w2": [],
-           "requantize": [], "packed_window": []}
+           "requantize": [], "packed_window": [], "glue": {}}
     for kind, params in QLINEAR_CASES:
         c = build_case(kind, params)
         args = (c["x"], c["w"], c["bias"], c["scales"], c["zps"], c["s_in"], c["zp_in"], c["s_out"],
@@ -168,6 +170,29 @@ def main():
         ok, y = ref.requantize_linear(c["x"], c["s_in"], c["zp_in"], c["s_out"], c["zp_out"], c["in_dtype"], c["out_dtype"])
         assert ok == 1
         out["requantize"].append({"params": params, "expected": digest(y)})
+    # The decoder glue: rmsnorm_f32, silu_f32 + mul_f32, the RotaryEmbedding operator of vx_llm_forward_f32 and
+    # cross_sdpa_gqa_f32 on the seeded inputs of tests/_glue_defs.py.  Outputs that a kernel is held to bit for
+    # bit are digested; those compared under a tolerance are stored whole (as their f32 bit patterns).
+    def bits(a):
+        return [int(v) for v in np.ascontiguousarray(a).reshape(-1).view(np.uint32)]
+
+    g = out["glue"]
+    g["rmsnorm"] = []
+    for params in glue.RMSNORM_CASES:
+        x, gain = glue.rmsnorm_case(**params)
+        g["rmsnorm"].append({"params": params, "eps": glue.EPS, "expected": digest(ref.rmsnorm(x, gain, glue.EPS))})
+    gu = glue.silu_mul_case()
+    half = gu.shape[1] // 2
+    g["silu_mul"] = {"shape": [gu.shape[0], half], "expected_bits": bits(ref.silu_mul(gu[:, :half], gu[:, half:]))}
+    x, cos, sin = glue.rotary_case()
+    st, y = ref.rotary(x, cos, sin)
+    assert st == 0
+    g["rotary"] = {"expected": digest(y)}
+    g["attention"] = []
+    for params in glue.ATTENTION_CASES:
+        q, k, v = glue.attention_case(**params)
+        y = ref.attention(q, k, v, params["q_heads"], params["kv_heads"], params["head_dim"], params["causal"])
+        g["attention"].append({"params": params, "shape": list(y.shape), "expected_bits": bits(y)})
     path = Path(__file__).with_name("reference_vectors.json")
     path.write_text(json.dumps(out, indent=1) + "\n")
     print("wrote", path, path.stat().st_size, "bytes")

@@ -232,8 +232,10 @@ def test_decode_of_one_or_two_rows_takes_the_fused_linears(oracle, rows, use_gra
 @pytest.mark.gpu
 def test_decoder_stages_at_benchmark_dimensions(oracle):
     """Two layers of the benchmark decoder at its own dimensions (hidden 1024, 16 query / 8 KV heads
-    of 128, SwiGLU 3072, vocabulary 32000), 32 rows, 128-token prompts, every stage of the prompt
-    pass fed with the CPU restatement's own intermediate tensors.  With identical inputs the integer
+    of 128, SwiGLU 3072, vocabulary 32000), 32 rows, 128-token prompts: every stage of the prompt
+    pass, then of one decode step behind it (cache length 129, the fused decode attention, the
+    32-row streaming linears) through the final norm, the lm_head and the argmax, each fed with the
+    CPU restatement's own intermediate tensors.  With identical inputs the integer
     work is exact (codes, scales, linears: same bits) and the f32 glue is within rounding noise.
     The stages are chained through the restatement's tensors because the assembled pipeline is
     chaotic in the last bit: a 1e-6 difference after attention moves an activation across a
@@ -252,7 +254,8 @@ def test_decoder_stages_at_benchmark_dimensions(oracle):
     kc = [np.zeros((rows, cfg.kv_heads, 0, cfg.head_dim), np.float32) for _ in range(cfg.layers)]
     vc = [np.zeros((rows, cfg.kv_heads, 0, cfg.head_dim), np.float32) for _ in range(cfg.layers)]
     trace = []
-    ref.forward(prompt, 0, kc, vc, trace)
+    prompt_logits = ref.forward(prompt, 0, kc, vc, trace)
+    rep = cfg.q_heads // cfg.kv_heads
     ctx = vx.Context(0, torch.cuda.current_stream())
     cos, sin = (_dev(a) for a in rope_tables(cfg))
     positions = torch.arange(t, dtype=torch.int64, device="cuda")
@@ -291,7 +294,6 @@ def test_decoder_stages_at_benchmark_dimensions(oracle):
         # f32 attention is no closer to the float64 value than the kernel is)
         got = attn.cpu().numpy().reshape(rows, t, cfg.q_heads, cfg.head_dim)
         q64, k64, v64 = q.cpu().numpy().astype(np.float64), kc[li].astype(np.float64), vc[li].astype(np.float64)
-        rep = cfg.q_heads // cfg.kv_heads
         truth, score_max = np.zeros(got.shape), 0.0
         for h in range(cfg.q_heads):
             sc64 = np.einsum("btd,bsd->bts", q64[:, :, h], k64[:, h // rep]) * float(np.float32(1.0 / np.sqrt(cfg.head_dim)))
@@ -331,6 +333,73 @@ def test_decoder_stages_at_benchmark_dimensions(oracle):
         assert np.abs(off).max() <= 1 and (off != 0).mean() < 1e-3, li
         down = linear(L["down"], _dev(ref_a8), _dev(ref_s))
         assert (bits(down) == bits(tr["down"])).all(), li
+
+    # ---- one decode step behind the prompt (cache length 129), stage by stage, through the head -----
+    first = prompt_logits.argmax(-1)
+    step = []
+    step_logits = ref.forward(first[:, None], t, kc, vc, step)
+    position = torch.full((1,), t, dtype=torch.int64, device="cuda")
+    for li, (L, tr) in enumerate(zip(weights["layers"], step)):
+        x_in = tr["x_in"].reshape(rows, cfg.hidden)
+        a8, sc = w8a8.rmsnorm_prepare_i8(ctx, _dev(x_in), _dev(L["norm1"]), cfg.eps)
+        want_a8, want_s = codes_of(ref.rmsnorm(x_in, L["norm1"]))
+        assert (a8.cpu().numpy() == want_a8).all() and (bits(sc.cpu().numpy()) == bits(want_s)).all(), li
+        qkv = linear(L["qkv"], a8, sc)   # 32 rows: the streaming kernel
+        assert (bits(qkv) == bits(tr["qkv"].reshape(rows, -1))).all(), li
+        # rotary embedding, append at slot 128 and attention over 129 slots in the one decode launch
+        kd = torch.zeros((rows, cfg.kv_heads, cfg.max_seq, cfg.head_dim), dtype=torch.float32, device="cuda")
+        vd = torch.zeros_like(kd)
+        kd[:, :, :t] = _dev(kc[li][:, :, :t])
+        vd[:, :, :t] = _dev(vc[li][:, :, :t])
+        attn = w8a8.rope_gqa_attention_decode(ctx, _dev(tr["qkv"].reshape(rows, -1)), cos, sin, position, cfg.q_heads,
+                                              cfg.kv_heads, cfg.head_dim, kd, vd)
+        ctx.synchronize()
+        assert (bits(kd[:, :, :t + 1].cpu().numpy()) == bits(kc[li])).all() and (bits(vd[:, :, :t + 1].cpu().numpy()) == bits(vc[li])).all()
+        got = attn.cpu().numpy().reshape(rows, cfg.q_heads, cfg.head_dim)
+        qr = ref.rope(tr["qkv"].reshape(rows, 1, -1)[..., :cfg.q_dim].reshape(rows, 1, cfg.q_heads, cfg.head_dim),
+                      ref.cos[t:t + 1], ref.sin[t:t + 1])[:, 0].astype(np.float64)
+        k64, v64 = kc[li].astype(np.float64), vc[li].astype(np.float64)
+        truth, score_max = np.zeros(got.shape), 0.0
+        for h in range(cfg.q_heads):
+            sc64 = np.einsum("bd,bsd->bs", qr[:, h], k64[:, h // rep]) * float(np.float32(1.0 / np.sqrt(cfg.head_dim)))
+            score_max = max(score_max, float(np.abs(sc64).max()))
+            p64 = np.exp(sc64 - sc64.max(-1, keepdims=True))
+            p64 /= p64.sum(-1, keepdims=True)
+            truth[:, h] = np.einsum("bs,bsd->bd", p64, v64[:, h // rep])
+        bound = 4.0 * 2.0 ** -24 * max(score_max, 16.0) * np.abs(truth).max()
+        assert np.abs(got - truth).max() <= bound, (li, np.abs(got - truth).max(), bound)
+        plo = vx.PackedLinear(pack_w8_words(L["o"]["w"]), L["o"]["scales"], None, cfg.q_dim, cfg.hidden, cfg.group)
+        st, o = plo.forward_f32(ctx, _dev(tr["attn"]))
+        ctx.synchronize()
+        plo.close()
+        assert st == 0 and (bits(o.cpu().numpy()) == bits(tr["o"])).all(), li
+        resid = _dev(x_in)
+        a8, sc = w8a8.add_rmsnorm_prepare_i8(ctx, resid, _dev(tr["o"]), _dev(L["norm2"]), cfg.eps)
+        x_mid = tr["x_mid"].reshape(rows, cfg.hidden)
+        assert (bits(resid.cpu().numpy()) == bits(x_mid)).all(), li
+        want_a8, want_s = codes_of(ref.rmsnorm(x_mid, L["norm2"]))
+        assert (a8.cpu().numpy() == want_a8).all() and (bits(sc.cpu().numpy()) == bits(want_s)).all(), li
+        gu = linear(L["gate_up"], a8, sc)
+        assert (bits(gu) == bits(tr["gu"])).all(), li
+        a8, sc, act = w8a8.swiglu_prepare_i8(ctx, _dev(tr["gu"]), want_activated=True)
+        ctx.synchronize()
+        assert np.allclose(act.cpu().numpy(), tr["act"], rtol=1e-6, atol=1e-30), li
+        ref_a8, ref_s = codes_of(tr["act"])
+        down = linear(L["down"], _dev(ref_a8), _dev(ref_s))
+        assert (bits(down) == bits(tr["down"])).all(), li
+    # the head: last residual add + final RMSNorm + preparation, lm_head (32 rows x 32000 channels), argmax
+    last = step[-1]
+    resid = _dev(last["x_mid"].reshape(rows, cfg.hidden))
+    a8, sc = w8a8.add_rmsnorm_prepare_i8(ctx, resid, _dev(last["down"]), _dev(weights["norm_f"]), cfg.eps)
+    x_out = last["x_mid"].reshape(rows, cfg.hidden) + last["down"]
+    assert (bits(resid.cpu().numpy()) == bits(x_out)).all()
+    want_a8, want_s = codes_of(ref.rmsnorm(x_out, weights["norm_f"]))
+    assert (a8.cpu().numpy() == want_a8).all() and (bits(sc.cpu().numpy()) == bits(want_s)).all()
+    logits = linear(weights["lm_head"], a8, sc)
+    assert (bits(logits) == bits(step_logits)).all()
+    ids = w8a8.argmax_rows(ctx, _dev(step_logits))
+    ctx.synchronize()
+    assert (ids.cpu().numpy() == step_logits.argmax(-1)).all()
     ctx.close()
 
 
@@ -360,9 +429,20 @@ def test_decoder_at_benchmark_dimensions_end_to_end(oracle):
     dec.close()
     assert (eager == replayed).all() and "a8-" in variant
     scale = np.abs(want_logits[0]).max()
-    err = np.abs(first_logits - want_logits[0]).max(axis=1) / scale
+    row_err = np.abs(first_logits - want_logits[0]).max(axis=1)
+    err = row_err / scale
     assert err.max() < 0.1 and (err < 2e-4).mean() >= 0.5, np.sort(err)
-    assert (eager[0] == want_tokens[0]).mean() >= 0.75
+    # Row by row: the token is the restatement's, or the restatement's own logits put the chosen token
+    # within twice this row's measured logit error of its maximum -- a flip that the row's rounding
+    # noise explains.  Anything else is a real disagreement.
+    for r in range(rows):
+        if eager[0][r] != want_tokens[0][r]:
+            gap = want_logits[0][r].max() - want_logits[0][r][eager[0][r]]
+            assert gap <= 2.0 * row_err[r], (r, int(eager[0][r]), int(want_tokens[0][r]), float(gap), float(row_err[r]))
+    # rows whose logits agree to rounding noise must agree on the token unless the top two are that close
+    quiet = err < 2e-4
+    flips = quiet & (eager[0] != want_tokens[0])
+    assert flips.sum() <= 1, np.nonzero(flips)
 
 
 @pytest.mark.gpu

@@ -1485,17 +1485,15 @@ int vxhip_requantize_linear_i8u8(const void* input, uint32_t input_elements, voi
     if (a < b + output_elements && b < a + input_elements) return 0;
     VxHipContext* ctx = default_context();
     if (!ctx) return 0;
-    void *xd = nullptr, *yd = nullptr;
     int ok = 0;
-    if (hipMalloc(&xd, input_elements) == hipSuccess && hipMalloc(&yd, output_elements) == hipSuccess &&
-        vxhip_memcpy_to_device(ctx, xd, input, input_elements) == VXHIP_OK) {
-        ok = vxhip_requantize_forward(ctx, xd, input_elements, yd, input_scale, input_zp, output_scale, output_zp,
-                                      input_dtype, output_dtype);
-        if (ok && vxhip_memcpy_to_host(ctx, output, yd, output_elements) != VXHIP_OK) ok = 0;
+    // (the context's grow-only staging buffers, like the other host-pointer entry points)
+    if (io_staging(ctx, input_elements, output_elements) &&
+        vxhip_memcpy_to_device(ctx, ctx->io_in, input, input_elements) == VXHIP_OK) {
+        ok = vxhip_requantize_forward(ctx, ctx->io_in, input_elements, ctx->io_out, input_scale, input_zp, output_scale,
+                                      output_zp, input_dtype, output_dtype);
+        if (ok && vxhip_memcpy_to_host(ctx, output, ctx->io_out, output_elements) != VXHIP_OK) ok = 0;
     }
     (void)hipStreamSynchronize(ctx->stream);
-    if (xd) (void)hipFree(xd);
-    if (yd) (void)hipFree(yd);
     return ok;
 }
 
@@ -1505,16 +1503,13 @@ int vxhip_quantize_typed_f32_i8u8(const float* input, uint32_t elements, void* o
     if (!elements) return 1;
     VxHipContext* ctx = default_context();
     if (!ctx) return 0;
-    void *xd = nullptr, *yd = nullptr;
     int ok = 0;
-    if (hipMalloc(&xd, (size_t)elements * 4u) == hipSuccess && hipMalloc(&yd, elements) == hipSuccess &&
-        vxhip_memcpy_to_device(ctx, xd, input, (size_t)elements * 4u) == VXHIP_OK) {
-        ok = vxhip_quantize_forward(ctx, (const float*)xd, elements, yd, scale, zp, dtype);
-        if (ok && vxhip_memcpy_to_host(ctx, output, yd, elements) != VXHIP_OK) ok = 0;
+    if (io_staging(ctx, (size_t)elements * 4u, elements) &&
+        vxhip_memcpy_to_device(ctx, ctx->io_in, input, (size_t)elements * 4u) == VXHIP_OK) {
+        ok = vxhip_quantize_forward(ctx, (const float*)ctx->io_in, elements, ctx->io_out, scale, zp, dtype);
+        if (ok && vxhip_memcpy_to_host(ctx, output, ctx->io_out, elements) != VXHIP_OK) ok = 0;
     }
     (void)hipStreamSynchronize(ctx->stream);
-    if (xd) (void)hipFree(xd);
-    if (yd) (void)hipFree(yd);
     return ok;
 }
 
@@ -1524,16 +1519,13 @@ int vxhip_dequantize_typed_i8u8_f32(const void* input, uint32_t elements, float 
     if (!elements) return 1;
     VxHipContext* ctx = default_context();
     if (!ctx) return 0;
-    void *xd = nullptr, *yd = nullptr;
     int ok = 0;
-    if (hipMalloc(&xd, elements) == hipSuccess && hipMalloc(&yd, (size_t)elements * 4u) == hipSuccess &&
-        vxhip_memcpy_to_device(ctx, xd, input, elements) == VXHIP_OK) {
-        ok = vxhip_dequantize_forward(ctx, xd, elements, scale, zp, dtype, (float*)yd);
-        if (ok && vxhip_memcpy_to_host(ctx, output, yd, (size_t)elements * 4u) != VXHIP_OK) ok = 0;
+    if (io_staging(ctx, elements, (size_t)elements * 4u) &&
+        vxhip_memcpy_to_device(ctx, ctx->io_in, input, elements) == VXHIP_OK) {
+        ok = vxhip_dequantize_forward(ctx, ctx->io_in, elements, scale, zp, dtype, (float*)ctx->io_out);
+        if (ok && vxhip_memcpy_to_host(ctx, output, ctx->io_out, (size_t)elements * 4u) != VXHIP_OK) ok = 0;
     }
     (void)hipStreamSynchronize(ctx->stream);
-    if (xd) (void)hipFree(xd);
-    if (yd) (void)hipFree(yd);
     return ok;
 }
 
