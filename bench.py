@@ -379,6 +379,46 @@ def bench_other_configs(torch, vx, cases, ctx):
     return res
 
 
+def bench_gemm_budget(torch, vx, cases, ctx):
+    """Where the headline GEMM's time goes, from the product's own launches only (no instrumented
+    build): the M=N=4096 kernel at K = 1024 .. 8192 on random bytes gives a fixed part and a part per
+    k-byte (least squares over the four K); the same kernel on constant operands (all weights and
+    activations 1: the datapath does not toggle) against random ones separates what the data costs
+    from what the structure costs; the register-only MFMA loop of the same operation count is the
+    ceiling beside both."""
+    res = {"shape": "M=N=4096, per-token requantizing epilogue, f32 bias"}
+    rng = np.random.default_rng(4096)
+    M = N = 4096
+    scales = (rng.uniform(0.002, 0.01, N) / np.sqrt(4096) * 4).astype(np.float32)
+    row_scales = torch.from_numpy(rng.uniform(0.01, 0.05, M).astype(np.float32)).cuda()
+    bias = torch.from_numpy(rng.normal(0, 0.1, N).astype(np.float32)).cuda()
+    y = torch.empty((M, N), dtype=torch.int8, device="cuda")
+    times = {}
+    for label, constant in (("random", False), ("constant", True)):
+        for K in ((1024, 2048, 4096, 8192) if not constant else (4096,)):
+            w = np.ones((N, K), np.int8) if constant else rng.integers(-127, 128, (N, K)).astype(np.int8)
+            x = np.ones((M, K), np.int8) if constant else rng.integers(-127, 128, (M, K)).astype(np.int8)
+            lin = vx.QLinear(w, scales, np.zeros(N, np.int32), None, vx.DTYPE_I8)
+            xd = torch.from_numpy(x).cuda()
+            ms = region_ms(lambda i: lin.forward_rowscale(ctx, xd, row_scales, 0.05, 0, bias_f32=bias, out=y), 20, torch)
+            times[(label, K)] = ms * 1e3
+            res[f"{label}_operands_K{K}_us"] = ms * 1e3
+            res.setdefault("variants", {})[f"{label}_K{K}"] = ctx.last_variant
+            lin.close()
+            del xd
+    ks = np.array([1024, 2048, 4096, 8192], dtype=np.float64)
+    ts = np.array([times[("random", int(k))] for k in ks])
+    slope, fixed = np.polyfit(ks, ts, 1)
+    res["fit_random_operands"] = {"fixed_us": float(fixed), "us_per_k_block_of_128": float(slope * 128),
+                                  "loop_us_at_K4096": float(slope * 4096),
+                                  "loop_int8_TOPS_at_K4096": 2.0 * M * N * 4096 / (slope * 4096 * 1e-6) / 1e12,
+                                  "residuals_us": [float(v) for v in ts - (fixed + slope * ks)]}
+    res["register_only_mfma_same_operation_count"] = {
+        "random_operands": ctx.probe_mfma_rate(128, True, k64=True),
+        "constant_operands": ctx.probe_mfma_rate(128, False, k64=True)}
+    return res
+
+
 def bench_single_row(torch, prompt_len=128, new_tokens=128):
     """The decoder benchmark's model at one row (a single stream): a step through the fused single-row
     linears, five launches per layer, beside the nine-launch layer the 32 rows take."""
@@ -461,7 +501,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-single-row", action="store_true",
                     help="decoder leg: the 32-row workload only (keeps a kernel profile of it unmixed)")
-    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "decoder_single_row", "copy", "other"], default=None,
+    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "decoder_single_row", "copy", "other", "gemm_budget"], default=None,
                     help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
                          "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
@@ -626,6 +666,11 @@ def main():
                        config={"workload": out["gemv"]["workload"]}, roofline=out["roofline_gemv"])
         for p in pls:
             p.close()
+
+    if args.only == "gemm_budget":
+        with torch.cuda.stream(stream):
+            out["gemm_budget"] = bench_gemm_budget(torch, vx, cases, ctx)
+        out.update(value=None, config={"workload": "where the M=K=N=4096 GEMM's time goes (fixed part, loop, data)"})
 
     # ---- the other benchmark sizes, timed only (their parity is in tests/) -----
     if args.only in (None, "other"):

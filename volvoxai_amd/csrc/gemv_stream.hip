@@ -45,7 +45,7 @@ extern __shared__ __attribute__((aligned(16))) char gemv_lds[];
 
 constexpr int kDepth = 4;  // 1 KiB blocks in flight per wave
 constexpr int kPrepPerThread = 8;  // f32 elements of a row that a thread of a preparing kernel holds
-constexpr uint32_t kFitLdsRows = 4;  // the exact-fit kernel keeps the activation rows in LDS up to this many rows
+constexpr uint32_t kFitLdsRows = 8;  // the exact-fit kernel keeps the activation rows in LDS up to this many rows
 
 __device__ __forceinline__ v4i load_stream(const int8_t* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
@@ -657,12 +657,12 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
     if (a.x_f32 || a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != 8u || a.x_flip_mask) return nullptr;
     const uint32_t panels = (a.n + 31u) / 32u;
     const bool forced = force && strstr(force, "fit");
-    // (more rows than the LDS copy takes: measured slower than the general kernel -- 16 rows 16.8 against
-    // 13.8 us at K=4096, N=14336 -- so they come here only when asked for by name)
+    // (more rows than the LDS copy takes: measured slower than the general kernel -- 16 rows 15.4 against
+    // 13.5 us at K=4096, N=14336, where eight rows are 12.2 against 12.8 -- so they come here only when
+    // asked for by name)
     if ((panels * 4u < (uint32_t)cu_count * 3u || a.rows > kFitLdsRows) && !forced) return nullptr;
     if (a.groups * GK != a.ksteps) return nullptr;  // (no padding group: every group of the stream has its scales)
-    const bool xlds = a.rows <= kFitLdsRows;
-    auto lds_for = [&](uint32_t waves, uint32_t bpw) {
+    auto lds_for = [&](uint32_t waves, uint32_t bpw, bool xlds) {
         const size_t groups = (size_t)waves * bpw / GK;
         return groups * a.rows * 128u + (size_t)waves * (bpw / GK * 32u + 32u) * 4u +
                (xlds ? (size_t)waves * 2u * bpw * a.rows * 16u : 0u);
@@ -673,7 +673,13 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
         constexpr int W = decltype(waves_tag)::value, B = decltype(bpw_tag)::value;
         if constexpr (B % GK == 0) {
             if (name || a.ksteps != (uint32_t)(W * B)) return;
-            const size_t lds = lds_for(W, B);
+            // the activation rows go through LDS while two workgroups still fit a compute unit that way
+            bool xlds = a.rows <= kFitLdsRows;
+            size_t lds = lds_for(W, B, xlds);
+            if (xlds && lds > 80u * 1024u) {
+                xlds = false;
+                lds = lds_for(W, B, false);
+            }
             if (lds > 156u * 1024u) return;
             ok = launch_fit<GK, W, B>(s, a, lds, xlds);
             name = id;
