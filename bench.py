@@ -419,6 +419,38 @@ def bench_gemm_budget(torch, vx, cases, ctx):
     return res
 
 
+def bench_config5(torch, vx, ctx):
+    """configs[4] alone (M=2048, K=14336, N=4096, f32 rows in, f32 out): the call, its two launches
+    apart, and the probe that says what bounds the GEMM: matrix and vector instructions of a SIMD
+    take turns, so the MFMAs and the exact per-group fold add up."""
+    from volvoxai_amd.decoder import pack_w8_words
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    rows, k, n, G = 2048, 14336, 4096, 128
+    rng = np.random.default_rng(55)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[:, rng.choice(k, k // 100, replace=False)] *= 20.0
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    chan = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    pl = vx.PackedLinear(pack_w8_words(w), np.repeat(chan[:, None], k // G, axis=1).copy(),
+                         rng.normal(0, 0.1, n).astype(np.float32), k, n, G)
+    xd = torch.from_numpy(x).cuda()
+    y = torch.empty((rows, n), dtype=torch.float32, device="cuda")
+    ops = 2.0 * rows * k * n
+    ms = region_ms(lambda i: pl.forward_f32(ctx, xd, out=y), 20, torch)
+    a8, rs = packed_prepare_i8(ctx, xd)
+    ms_gemm = region_ms(lambda i: pl.forward_a8(ctx, a8, rs, out=y), 20, torch)
+    variant = ctx.last_variant
+    ms_prep = region_ms(lambda i: packed_prepare_i8(ctx, xd), 20, torch)
+    pl.close()
+    groups = k // G
+    return {"workload": "configs[4]: M=2048, K=14336, N=4096, dynamic per-token quantization, f32 dequant + bias",
+            "ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12, "frac_mfma": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+            "ms_gemm_alone": ms_gemm, "ms_preparation_alone": ms_prep, "variant": variant,
+            "per_simd": {"mfma_16x16x64": rows * n * k / (16 * 16 * 64) / 1024,
+                         "fold_vector_instructions": rows * n * groups * 3 / 64 / 1024},
+            "mfma_valu_overlap_probe": ctx.probe_mfma_valu_overlap(2000)}
+
+
 def bench_single_row(torch, prompt_len=128, new_tokens=128):
     """The decoder benchmark's model at one row (a single stream): a step through the fused single-row
     linears, five launches per layer, beside the nine-launch layer the 32 rows take."""
@@ -501,7 +533,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-single-row", action="store_true",
                     help="decoder leg: the 32-row workload only (keeps a kernel profile of it unmixed)")
-    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "decoder_single_row", "copy", "other", "gemm_budget"], default=None,
+    ap.add_argument("--only", choices=["gemm", "gemv", "decoder", "decoder_single_row", "copy", "other", "gemm_budget", "config5"], default=None,
                     help="run one leg only (for profiling a single kernel); 'copy' runs a plain "
                          "device copy of known size, the yardstick for the HBM traffic counters")
     args = ap.parse_args()
@@ -671,6 +703,11 @@ def main():
         with torch.cuda.stream(stream):
             out["gemm_budget"] = bench_gemm_budget(torch, vx, cases, ctx)
         out.update(value=None, config={"workload": "where the M=K=N=4096 GEMM's time goes (fixed part, loop, data)"})
+
+    if args.only == "config5":
+        with torch.cuda.stream(stream):
+            out["config5"] = bench_config5(torch, vx, ctx)
+        out.update(value=out["config5"]["TOPS"], ms_per_step=out["config5"]["ms"], config={"workload": out["config5"]["workload"]})
 
     # ---- the other benchmark sizes, timed only (their parity is in tests/) -----
     if args.only in (None, "other"):

@@ -246,6 +246,19 @@ VxHipStatus vxhip_probe_stream_read(VxHipContext* context, const void* const* bu
                                     uint32_t launches, double* gigabytes_per_second,
                                     double* microseconds);
 
+/* A third measurement aid without a counterpart in the reference: whether the
+ * matrix and the vector instructions of a SIMD run beside each other, which
+ * bounds the dequantizing GEMM (two MFMAs and twelve vector instructions per
+ * result tile and scale group of 128).  Four launches of `rounds` rounds, four
+ * waves per SIMD, random operand bytes: [0] the MFMAs of a 64 x 32 wave tile
+ * alone, [1] the folds of its accumulators alone, [2] both in every wave, [3]
+ * even waves the MFMAs and odd waves the folds (half the work of each kind).
+ * microseconds[4] and shader_mhz[4] (optional) receive time and clock of each.
+ * Synchronises the context's stream. */
+VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* context, uint32_t rounds,
+                                          double* microseconds,
+                                          double* shader_mhz);
+
 /* Device memory for hosts without HIP headers. */
 VxHipStatus vxhip_device_malloc(size_t bytes, void** out_device_pointer);
 void vxhip_device_free(void* device_pointer);

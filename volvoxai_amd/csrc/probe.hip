@@ -79,10 +79,129 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restric
     if (fold == 0x9e3779b9u) sink[0] = fold;  // keeps the loads alive; practically never true
 }
 
+// Do matrix and vector instructions of a SIMD run beside each other?  Four waves per SIMD, random 8-bit
+// operands.  A round of a wave is what a 64 x 32 wave tile of the dequantizing GEMM does per scale group of
+// 128: sixteen v_mfma_i32_16x16x64_i8 (two per result tile) and the fold of 32 accumulator registers,
+// sum += f32(dot) * c with each operation rounded on its own (three vector instructions per register; the
+// vector-only form needs a fourth, an integer add, to keep the conversion in the loop).
+// MODE 0: the MFMAs alone.  1: the folds alone.  2: both in every wave, the fold of a tile behind the MFMAs
+// of the next.  3: even waves run the MFMAs, odd waves the folds (half of each kind of work).
+template <int MODE>
+__global__ __launch_bounds__(1024) void mfma_valu_overlap_kernel(const v4i* __restrict__ operands, uint32_t rounds,
+                                                                uint64_t* __restrict__ clocks, float* sink) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    v4i a[2], b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        a[i] = operands[(threadIdx.x & 255u) + 256 * i];
+        b[i] = operands[(threadIdx.x & 255u) + 256 * (i + 2)];
+    }
+    v4i acc[8];
+    float sum[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = v4i{(int)threadIdx.x, i, 3, 4};
+#pragma unroll
+    for (int i = 0; i < 32; i++) sum[i] = 0.f;
+    const float c = __int_as_float(0x3a83126f + (int)(threadIdx.x & 7u));
+    auto mfmas = [&](int i) {
+        acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b[i & 1], acc[i], 0, 0, 0);
+        acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], b[(i + 1) & 1], acc[i], 0, 0, 0);
+    };
+    auto fold = [&](int j, bool alone) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            sum[j * 4 + e] = __fadd_rn(sum[j * 4 + e], __fmul_rn((float)acc[j][e], c));
+            if (alone) acc[j][e] += 0x01010101;
+        }
+    };
+    const uint64_t c0 = __builtin_readcyclecounter(), t0 = __builtin_amdgcn_s_memrealtime();
+    const bool folds_only = MODE == 1 || (MODE == 3 && (wave & 1));
+    if (folds_only) {
+        for (uint32_t r = 0; r < rounds; r++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) fold(i, true);
+    } else {
+        for (uint32_t r = 0; r < rounds; r++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                mfmas(i);
+                if constexpr (MODE == 2) fold((i + 7) & 7, false);
+            }
+    }
+    float f = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) f += sum[i];
+#pragma unroll
+    for (int i = 0; i < 8; i++) f += (float)(acc[i][0] ^ acc[i][1] ^ acc[i][2] ^ acc[i][3]);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        clocks[0] = __builtin_readcyclecounter() - c0;
+        clocks[1] = __builtin_amdgcn_s_memrealtime() - t0;
+    }
+    if (f == 1.2345f) sink[0] = f;
+}
+
 }  // namespace
 }  // namespace vxhip
 
 using namespace vxhip;
+
+extern "C" VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* ctx, uint32_t rounds, double* microseconds,
+                                                     double* shader_mhz) {
+    if (!ctx || !rounds || !microseconds) {
+        set_error("probe_mfma_valu_overlap: null context/result or zero rounds");
+        return VXHIP_INVALID_ARGUMENT;
+    }
+    VXHIP_TRY(hipSetDevice(ctx->device));
+    std::vector<uint32_t> host(4 * 256 * 4);
+    uint32_t lcg = 12345u;
+    for (auto& v : host) {
+        lcg = lcg * 1664525u + 1013904223u;
+        const uint32_t hi = lcg;
+        lcg = lcg * 1664525u + 1013904223u;
+        v = (hi & 0xffff0000u) | (lcg >> 16);
+    }
+    v4i* operands = nullptr;
+    uint64_t* clocks = nullptr;
+    float* sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    VxHipStatus st = VXHIP_OK;
+    auto check = [&](hipError_t e, const char* what) {
+        if (st == VXHIP_OK && e != hipSuccess) st = hip_status(e, what);
+    };
+    check(hipMalloc((void**)&operands, host.size() * 4), "hipMalloc");
+    check(hipMalloc((void**)&clocks, 16), "hipMalloc");
+    check(hipMalloc((void**)&sink, 64), "hipMalloc");
+    check(hipEventCreate(&e0), "hipEventCreate");
+    check(hipEventCreate(&e1), "hipEventCreate");
+    if (st == VXHIP_OK) {
+        check(hipMemcpyAsync(operands, host.data(), host.size() * 4, hipMemcpyHostToDevice, ctx->stream), "copy");
+        check(hipStreamSynchronize(ctx->stream), "sync");
+    }
+    const int groups = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    void (*const kernels[4])(const v4i*, uint32_t, uint64_t*, float*) = {
+        mfma_valu_overlap_kernel<0>, mfma_valu_overlap_kernel<1>, mfma_valu_overlap_kernel<2>, mfma_valu_overlap_kernel<3>};
+    for (int mode = 0; mode < 4 && st == VXHIP_OK; mode++) {
+        float ms = 0.0f;
+        // one launch to settle the clock, then the timed one
+        hipLaunchKernelGGL(kernels[mode], dim3(groups), dim3(1024), 0, ctx->stream, operands, rounds, clocks, sink);
+        check(hipEventRecord(e0, ctx->stream), "record");
+        hipLaunchKernelGGL(kernels[mode], dim3(groups), dim3(1024), 0, ctx->stream, operands, rounds, clocks, sink);
+        check(hipGetLastError(), "launch");
+        check(hipEventRecord(e1, ctx->stream), "record");
+        check(hipEventSynchronize(e1), "sync");
+        check(hipEventElapsedTime(&ms, e0, e1), "elapsed");
+        uint64_t c[2] = {0, 0};
+        check(hipMemcpy(c, clocks, sizeof c, hipMemcpyDeviceToHost), "read clocks");
+        microseconds[mode] = ms * 1e3;
+        if (shader_mhz) shader_mhz[mode] = c[1] ? (double)c[0] / ((double)c[1] / 100.0) : 0.0;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(operands);
+    (void)hipFree(clocks);
+    (void)hipFree(sink);
+    return st;
+}
 
 extern "C" VxHipStatus vxhip_probe_stream_read(VxHipContext* ctx, const void* const* buffers_dev,
                                                uint32_t buffer_count, size_t bytes_each, uint32_t launches,
