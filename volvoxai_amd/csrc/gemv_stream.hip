@@ -529,6 +529,10 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
                 a.x + (a.x_operand_order ? ((size_t)c * kOperandOrderRows + r) * 16u : (size_t)r * a.ldx + (size_t)c * 16u));
         }
     }
+    // (the order is kept by hand: loads come back in the order of their issue, and left to itself the
+    // scheduler puts the weight requests first, so that the wait for these few bytes becomes a wait for
+    // the first four blocks and the next four go out a memory round trip late)
+    __builtin_amdgcn_sched_barrier(0);
     const int8_t* xp = a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
     const uint32_t x_chunk_pitch = a.x_operand_order ? 16u * kOperandOrderRows : 16u;
     v4i wbuf[kDepth], xbuf[XLDS ? 1 : kDepth];
@@ -541,6 +545,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     };
 #pragma unroll
     for (int i = 0; i < kDepth; i++) issue(i, i);
+    __builtin_amdgcn_sched_barrier(0);
 
     // what the tail needs, requested behind the first blocks: the wave's group scales, lane e <-> (group
     // g0 + e / 32, channel e % 32); the row scales; the bias of this thread's outputs
