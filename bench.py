@@ -102,7 +102,7 @@ def timed_region(fn, steps, torch, stream):
             graph.replay()
             e1.record(stream)
             stream.synchronize()
-            rounds = max(1, int(np.ceil(1.05 * MIN_TIMED_MS / max(e0.elapsed_time(e1), 1e-3))))
+            rounds = max(1, int(np.ceil(1.2 * MIN_TIMED_MS / max(e0.elapsed_time(e1), 1e-3))))
             marks = [event() for _ in range(rounds + 1)]
             marks[0].record(stream)
             for r in range(rounds):
