@@ -1168,6 +1168,22 @@ def test_exact_fit_gemv(oracle, k, group, instance):
                     assert st == 0 and same_f32(host(y), want), (rows, force, ctx.last_variant)
                     named = force == "gemv.fit" or (force is None and rows <= 8 and n >= 6144)
                     assert ctx.last_variant.endswith(instance) == named, (rows, force, ctx.last_variant)
+        # one and two f32 rows: the kernel prepares them itself (the reference's single-row route in one launch);
+        # a zero row, a row with an infinity, a plain one
+        for rows, special in ((1, None), (1, "zero"), (2, "inf"), (2, None)):
+            x = c["x"][5:5 + rows].copy()
+            if special == "zero":
+                x[0] = 0.0
+            if special == "inf":
+                x[1, k // 3] = np.inf
+            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
+            for force in (None, "gemv.nofit"):
+                vx.force_variant(force)
+                st, y = pl.forward_f32(plain, dev(x))
+                plain.synchronize()
+                assert st == 0 and same_f32(host(y), want), (rows, special, force, plain.last_variant)
+                prepared_here = force is None and n >= 6144 and k % 32 == 0
+                assert plain.last_variant.endswith(instance + "-prep") == prepared_here, (rows, force, plain.last_variant)
     finally:
         vx.force_variant(None)
         pl.close(), plain.close(), blocked.close()

@@ -495,9 +495,15 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
 //     (packed_linear_ops.inc:1498-1504), bit for bit.
 // Measured at M=1, K=4096, N=14336 (sixteen waves of eight blocks): 10.3 us against 12.5 us for the
 // general kernel, with a plain read of the same bytes at 9.3-9.6 us.
-template <int GK, int WAVES, int BPW, bool XLDS>
+// PREP: one or two f32 rows (a.x_f32) which the workgroup prepares itself, by prepare_i8_kernel's rule to the
+// letter, as the reference's single-row route quantizes the row and multiplies in one call
+// (packed_linear_ops.inc:1471-1535).  A wave's 64 lanes hold exactly the elements of the wave's own K-slice
+// (BPW / 2 consecutive ones per lane), so only the row maximum crosses the waves; the codes go straight into
+// the wave's LDS slice, where the MFMA's activation operand is read from.
+template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false>
 __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArgs a) {
     static_assert(BPW % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
+    static_assert(!PREP || (XLDS && BPW % 4 == 0), "prepared rows live in the LDS slices; a lane loads pairs of elements");
     constexpr int GPW = BPW / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -518,9 +524,22 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 
     // (XLDS) this wave's activation chunks are requested first: they are cache hits and return ahead
     // of the weight stream
-    constexpr int XPL = XLDS ? (2 * BPW * (int)kFitLdsRows + 63) / 64 : 1;  // chunks per lane
+    constexpr int XPL = XLDS && !PREP ? (2 * BPW * (int)kFitLdsRows + 63) / 64 : 1;  // chunks per lane
     v4i xstage[XPL];
-    if constexpr (XLDS) {
+    constexpr int EPL = BPW / 2;  // PREP: f32 elements of a row per lane
+    float xf[PREP ? (int)kMaxPrepRows : 1][PREP ? EPL : 1];
+    if constexpr (PREP) {
+#pragma unroll
+        for (int r = 0; r < (int)kMaxPrepRows; r++) {
+            const float* src = a.x_f32 + (size_t)min((uint32_t)r, rows - 1u) * a.ldx + (size_t)t0 * 32u + (uint32_t)lane * EPL;
+#pragma unroll
+            for (int i = 0; i < EPL; i += 2) {
+                const float2 v = *reinterpret_cast<const float2*>(src + i);
+                xf[r][i] = v.x;
+                xf[r][i + 1] = v.y;
+            }
+        }
+    } else if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < XPL; j++) {
             const uint32_t e = min((uint32_t)lane + 64u * j, 2u * BPW * rows - 1u);
@@ -556,13 +575,61 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         const uint32_t e = min((uint32_t)lane + 64u * u, GPW * 32u - 1u);
         sreg[u] = a.scales_t[(size_t)(g0 + e / 32u) * a.n_pad + panel * 32u + e % 32u];
     }
-    const float rs_lane = a.row_scale[min((uint32_t)lane, rows - 1u)];
+    float rs_lane = 0.0f;
+    if constexpr (!PREP) rs_lane = a.row_scale[min((uint32_t)lane, rows - 1u)];
     constexpr int OPT_ = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);  // outputs per thread
     float bias_t[OPT_];
 #pragma unroll
     for (int it = 0; it < OPT_; it++) bias_t[it] = a.bias_f32[panel * 32u + (threadIdx.x + it * WAVES * 64) % 32u];
 
-    if constexpr (XLDS) {
+    if constexpr (PREP) {
+        // per row: scale = max|x| / 127 (true division; 1 for a zero row; floored at 2^-126), codes =
+        // ties-to-even(x / scale) clamped to +-127; a row that is not finite gets zero codes and a NaN scale
+        __shared__ float slot_max[kMaxPrepRows][WAVES];
+        __shared__ uint32_t slot_bad[kMaxPrepRows][WAVES];
+#pragma unroll
+        for (int r = 0; r < (int)kMaxPrepRows; r++) {
+            float maximum = 0.0f;
+            uint32_t bad = 0u;
+#pragma unroll
+            for (int i = 0; i < EPL; i++) {
+                bad |= finite_f32(xf[r][i]) ? 0u : 1u;
+                maximum = fmaxf(maximum, fabsf(xf[r][i]));
+            }
+            maximum = wave_max(maximum);
+            bad = __builtin_amdgcn_ballot_w64(bad != 0u) != 0ull ? 1u : 0u;
+            if (lane == 0) {
+                slot_max[r][wave] = maximum;
+                slot_bad[r][wave] = bad;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < (int)kMaxPrepRows; r++) {
+            float maximum = slot_max[r][0];
+            uint32_t bad = slot_bad[r][0];
+#pragma unroll
+            for (int w = 1; w < WAVES; w++) {
+                maximum = fmaxf(maximum, slot_max[r][w]);
+                bad |= slot_bad[r][w];
+            }
+            float scale = maximum == 0.0f ? 1.0f : __fdiv_rn(maximum, 127.0f);
+            if (scale < 0x1p-126f) scale = 0x1p-126f;
+            if ((uint32_t)r < rows) {
+                // element j = lane * EPL + i of the slice lives in chunk j / 16 at byte j % 16: [chunk][row] of 16 bytes
+#pragma unroll
+                for (int i = 0; i < EPL; i += 2) {
+                    const uint32_t j = (uint32_t)lane * EPL + i;
+                    const int32_t q0 = bad ? 0 : packed_round_i8(__fdiv_rn(xf[r][i], scale));
+                    const int32_t q1 = bad ? 0 : packed_round_i8(__fdiv_rn(xf[r][i + 1], scale));
+                    *reinterpret_cast<uint16_t*>(xslice + ((size_t)(j / 16u) * rows + r) * 16u + j % 16u) =
+                        (uint16_t)((uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8));
+                }
+            }
+            const float row_scale = bad ? __builtin_nanf("") : scale;
+            if (min((uint32_t)lane, rows - 1u) == (uint32_t)r) rs_lane = row_scale;  // (as the loaded scales: lane r carries row r's)
+        }
+    } else if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < XPL; j++) {
             const uint32_t e = (uint32_t)lane + 64u * j;
@@ -644,10 +711,13 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 template <int GK, int WAVES, int BPW>
 bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds) {
     auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true> : gemv_fit_kernel<GK, WAVES, BPW, false>;
+    if constexpr (BPW % 4 == 0) {
+        if (a.x_f32) kern = gemv_fit_kernel<GK, WAVES, BPW, true, true>;
+    }
     if (gemv_dry_run) return true;
     if (lds > 64u * 1024u) {
-        static std::atomic<uint64_t> configured[2] = {{0}, {0}};
-        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[xlds ? 1 : 0])) return false;
+        static std::atomic<uint64_t> configured[3] = {{0}, {0}, {0}};
+        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[a.x_f32 ? 2 : xlds ? 1 : 0])) return false;
     }
     hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError() == hipSuccess;
@@ -659,7 +729,11 @@ bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds) {
 template <int GK>
 const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     if (force && strstr(force, "nofit")) return nullptr;
-    if (a.x_f32 || a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != 8u || a.x_flip_mask) return nullptr;
+    if (a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != 8u || a.x_flip_mask) return nullptr;
+    // f32 rows (prepared in the kernel): one or two whole rows of exactly the stream's length, pairs of elements aligned
+    const bool prep = a.x_f32 != nullptr;
+    if (prep && (a.rows > kMaxPrepRows || a.k != a.ksteps * 32u || (a.ldx % 2u) != 0u || ((uintptr_t)a.x_f32 % 8u) != 0u))
+        return nullptr;
     const uint32_t panels = (a.n + 31u) / 32u;
     const bool forced = force && strstr(force, "fit");
     // (more rows than the LDS copy takes: measured slower than the general kernel -- 16 rows 15.4 against
@@ -681,11 +755,11 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
             // the activation rows go through LDS while two workgroups still fit a compute unit that way
             bool xlds = a.rows <= kFitLdsRows;
             size_t lds = lds_for(W, B, xlds);
-            if (xlds && lds > 80u * 1024u) {
+            if (xlds && lds > 80u * 1024u && !prep) {
                 xlds = false;
                 lds = lds_for(W, B, false);
             }
-            if (lds > 156u * 1024u) return;
+            if (lds > 156u * 1024u || (prep && B % 4 != 0)) return;
             ok = launch_fit<GK, W, B>(s, a, lds, xlds);
             name = id;
         }
@@ -697,7 +771,13 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
     run(integral_constant<int, 16>{}, integral_constant<int, 28>{}, "fit16x28");
     run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, "fit8x4");
     run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, "fit8x12");
-    return ok ? name : nullptr;
+    if (!ok) return nullptr;
+    if (!prep) return name;
+    static const char* const prep_names[6][2] = {{"fit16x4", "fit16x4-prep"}, {"fit16x8", "fit16x8-prep"}, {"fit16x16", "fit16x16-prep"},
+                                                 {"fit16x28", "fit16x28-prep"}, {"fit8x4", "fit8x4-prep"}, {"fit8x12", "fit8x12-prep"}};
+    for (const auto& pair : prep_names)
+        if (!strcmp(pair[0], name)) return pair[1];
+    return name;
 }
 
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, int ROWOP = kRowsPrepared>
