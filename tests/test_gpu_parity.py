@@ -1136,7 +1136,8 @@ def test_operand_order_activations(oracle, rows, k, n, group):
                                               (4090, 64, "fit16x8"), (8192, 128, "fit16x16"), (14336, 128, "fit16x28")])
 def test_exact_fit_gemv(oracle, k, group, instance):
     """The straight-line streaming kernel for a K whose blocks divide evenly over the waves: every
-    instance, rows on both sides of its LDS-copy limit (more rows only when named), both activation
+    instance, rows on both sides of its LDS-copy limit, both places where the products are formed
+    (lane-parallel over the parked dots, or by the parking wave in its accumulators), both activation
     layouts, a row whose scale is NaN, an n that ends inside a panel -- the oracle's bits each time;
     and the general kernel still gives them when the exact-fit one is ruled out by name."""
     import volvoxai_amd as vx
@@ -1161,12 +1162,12 @@ def test_exact_fit_gemv(oracle, k, group, instance):
             _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
             for ctx in (plain, blocked):
                 codes, scales = packed_prepare_i8(ctx, dev(x))
-                for force in (None, "gemv.fit", "gemv.nofit"):
+                for force in (None, "gemv.fit.lprod", "gemv.fit.rprod", "gemv.nofit"):
                     vx.force_variant(force)
                     st, y = pl.forward_a8(ctx, codes, scales)
                     ctx.synchronize()
                     assert st == 0 and same_f32(host(y), want), (rows, force, ctx.last_variant)
-                    named = force == "gemv.fit" or (force is None and rows <= 8 and n >= 6144)
+                    named = force in ("gemv.fit.lprod", "gemv.fit.rprod") or (force is None and n >= 6144)
                     assert ctx.last_variant.endswith(instance) == named, (rows, force, ctx.last_variant)
         # one and two f32 rows: the kernel prepares them itself (the reference's single-row route in one launch);
         # a zero row, a row with an infinity, a plain one

@@ -500,10 +500,11 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
 // (packed_linear_ops.inc:1471-1535).  A wave's 64 lanes hold exactly the elements of the wave's own K-slice
 // (BPW / 2 consecutive ones per lane), so only the row maximum crosses the waves; the codes go straight into
 // the wave's LDS slice, where the MFMA's activation operand is read from.
-template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false>
+template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false, bool RPROD = false>
 __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArgs a) {
     static_assert(BPW % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
     static_assert(!PREP || (XLDS && BPW % 4 == 0), "prepared rows live in the LDS slices; a lane loads pairs of elements");
+    static_assert(!(PREP && RPROD), "one or two rows form their products lane-parallel");
     constexpr int GPW = BPW / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -575,8 +576,9 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         const uint32_t e = min((uint32_t)lane + 64u * u, GPW * 32u - 1u);
         sreg[u] = a.scales_t[(size_t)(g0 + e / 32u) * a.n_pad + panel * 32u + e % 32u];
     }
+    // (RPROD: the scale of the row whose dots the lane holds in its accumulators; else lane r carries row r's)
     float rs_lane = 0.0f;
-    if constexpr (!PREP) rs_lane = a.row_scale[min((uint32_t)lane, rows - 1u)];
+    if constexpr (!PREP) rs_lane = a.row_scale[RPROD ? m : min((uint32_t)lane, rows - 1u)];
     constexpr int OPT_ = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);  // outputs per thread
     float bias_t[OPT_];
 #pragma unroll
@@ -649,12 +651,37 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         else xop = xbuf[slot];
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wbuf[slot], xop, acc, 0, 0, 0);
         if (b + kDepth < BPW) issue(slot, b + kDepth);
+        if constexpr (RPROD) {
+            // the wave's group scales go to its LDS strip once they are here (they were requested behind
+            // the first kDepth blocks), in time for the first group that closes
+            if (b == (GK > kDepth ? kDepth : GK) - 1) {
+#pragma unroll
+                for (int u = 0; u < SPL; u++) {
+                    const uint32_t e = (uint32_t)lane + 64u * u;
+                    if (e < GPW * 32u) wave_scales[e] = sreg[u];
+                }
+            }
+        }
         if ((b + 1) % GK == 0) {
             if (row_live) {
                 int32_t* dp = dots + ((size_t)(g0 + b / GK) * rows + (lane & 31)) * 32u + half * 4u;
+                if constexpr (RPROD) {
+                    // many rows: the products are formed here, in the accumulators' own layout (a lane holds
+                    // its row's dots of sixteen channels), and parked as floats
+                    const float* sw = wave_scales + (b / GK) * 32 + half * 4u;
 #pragma unroll
-                for (int q = 0; q < 4; q++)
-                    *reinterpret_cast<v4i*>(dp + q * 8) = v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+                    for (int q = 0; q < 4; q++) {
+                        const v4f s4 = *reinterpret_cast<const v4f*>(sw + q * 8);
+                        v4f p;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) p[i] = __fmul_rn((float)acc[q * 4 + i], __fmul_rn(rs_lane, s4[i]));
+                        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(dp) + q * 8) = p;
+                    }
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        *reinterpret_cast<v4i*>(dp + q * 8) = v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+                }
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = 0;
@@ -664,7 +691,9 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     // products of this wave's groups, in place: element e of its region is (group g0 + e / (rows * 32),
     // row (e / 32) % rows, channel e % 32)
     float* prod = reinterpret_cast<float*>(dots) + (size_t)g0 * rows * 32u;
-    if (rows == 1u) {
+    if constexpr (RPROD) {
+        (void)prod;
+    } else if (rows == 1u) {
 #pragma unroll
         for (int u = 0; u < SPL; u++) {
             const uint32_t e = (uint32_t)lane + 64u * u;
@@ -709,15 +738,16 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 }
 
 template <int GK, int WAVES, int BPW>
-bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds) {
+bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds, bool rprod) {
     auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true> : gemv_fit_kernel<GK, WAVES, BPW, false>;
+    if (rprod) kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, true> : gemv_fit_kernel<GK, WAVES, BPW, false, false, true>;
     if constexpr (BPW % 4 == 0) {
         if (a.x_f32) kern = gemv_fit_kernel<GK, WAVES, BPW, true, true>;
     }
     if (gemv_dry_run) return true;
     if (lds > 64u * 1024u) {
-        static std::atomic<uint64_t> configured[3] = {{0}, {0}, {0}};
-        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[a.x_f32 ? 2 : xlds ? 1 : 0])) return false;
+        static std::atomic<uint64_t> configured[5] = {{0}, {0}, {0}, {0}, {0}};
+        if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[a.x_f32 ? 4 : (rprod ? 2 : 0) + (xlds ? 1 : 0)])) return false;
     }
     hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError() == hipSuccess;
@@ -736,16 +766,18 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
         return nullptr;
     const uint32_t panels = (a.n + 31u) / 32u;
     const bool forced = force && strstr(force, "fit");
-    // (more rows than the LDS copy takes: measured slower than the general kernel -- 16 rows 15.4 against
-    // 13.5 us at K=4096, N=14336, where eight rows are 12.2 against 12.8 -- so they come here only when
-    // asked for by name)
-    if ((panels * 4u < (uint32_t)cu_count * 3u || a.rows > kFitLdsRows) && !forced) return nullptr;
+    if (panels * 4u < (uint32_t)cu_count * 3u && !forced) return nullptr;
     if (a.groups * GK != a.ksteps) return nullptr;  // (no padding group: every group of the stream has its scales)
     auto lds_for = [&](uint32_t waves, uint32_t bpw, bool xlds) {
         const size_t groups = (size_t)waves * bpw / GK;
         return groups * a.rows * 128u + (size_t)waves * (bpw / GK * 32u + 32u) * 4u +
                (xlds ? (size_t)waves * 2u * bpw * a.rows * 16u : 0u);
     };
+    // where the products are formed: lane-parallel over the parked dots (few rows), or by the parking wave
+    // in its accumulators' layout (many rows)
+    // (measured at K=4096, N=14336: one row 10.8 us either way, 2 / 4 / 8 / 16 / 32 rows 10.8 / 10.9 / 11.0 / 11.9 / 16.3 us
+    // against 11.1 / 11.3 / 12.9 / 15.9 / 27.9 lane-parallel and 12.5 / 12.6 / 12.8 / 13.5 / 18.4 in the general kernel)
+    const bool rprod = !prep && (force && strstr(force, "rprod") ? true : force && strstr(force, "lprod") ? false : a.rows > 1u);
     const char* name = nullptr;
     bool ok = false;
     auto run = [&](auto waves_tag, auto bpw_tag, const char* id) {
@@ -760,7 +792,7 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
                 lds = lds_for(W, B, false);
             }
             if (lds > 156u * 1024u || (prep && B % 4 != 0)) return;
-            ok = launch_fit<GK, W, B>(s, a, lds, xlds);
+            ok = launch_fit<GK, W, B>(s, a, lds, xlds, rprod);
             name = id;
         }
     };
