@@ -448,7 +448,8 @@ def bench_config5(torch, vx, ctx):
             "ms_gemm_alone": ms_gemm, "ms_preparation_alone": ms_prep, "variant": variant,
             "per_simd": {"mfma_16x16x64": rows * n * k / (16 * 16 * 64) / 1024,
                          "fold_vector_instructions": rows * n * groups * 3 / 64 / 1024},
-            "mfma_valu_overlap_probe": ctx.probe_mfma_valu_overlap(2000)}
+            "mfma_valu_overlap_probe": ctx.probe_mfma_valu_overlap(2000),
+            "mfma_valu_overlap_probe_constant_operands": ctx.probe_mfma_valu_overlap(2000, constant_operands=True)}
 
 
 def bench_single_row(torch, prompt_len=128, new_tokens=128):

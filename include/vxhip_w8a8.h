@@ -254,8 +254,11 @@ VxHipStatus vxhip_probe_stream_read(VxHipContext* context, const void* const* bu
  * alone, [1] the folds of its accumulators alone, [2] both in every wave, [3]
  * even waves the MFMAs and odd waves the folds (half the work of each kind).
  * microseconds[4] and shader_mhz[4] (optional) receive time and clock of each.
+ * constant_operands != 0: every operand byte is 1 instead of random (the matrix
+ * pipes then draw less power and the clock stays higher).
  * Synchronises the context's stream. */
 VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* context, uint32_t rounds,
+                                          uint32_t constant_operands,
                                           double* microseconds,
                                           double* shader_mhz);
 

@@ -76,7 +76,7 @@ def _declare(L: C.CDLL) -> None:
                                         C.POINTER(C.c_double)]),
         "vxhip_probe_stream_read": (i32, [vp, C.POINTER(C.c_void_p), u32, sz, u32, C.POINTER(C.c_double),
                                           C.POINTER(C.c_double)]),
-        "vxhip_probe_mfma_valu_overlap": (i32, [vp, u32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "vxhip_probe_mfma_valu_overlap": (i32, [vp, u32, u32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "vxhip_context_set_activation_layout": (i32, [vp, u32]),
         "vxhip_context_prepared_bytes": (sz, [vp, u32, u32]),
         "vxhip_device_malloc": (i32, [sz, pp]),

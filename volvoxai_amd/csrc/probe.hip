@@ -145,8 +145,8 @@ __global__ __launch_bounds__(1024) void mfma_valu_overlap_kernel(const v4i* __re
 
 using namespace vxhip;
 
-extern "C" VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* ctx, uint32_t rounds, double* microseconds,
-                                                     double* shader_mhz) {
+extern "C" VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* ctx, uint32_t rounds, uint32_t constant_operands,
+                                                     double* microseconds, double* shader_mhz) {
     if (!ctx || !rounds || !microseconds) {
         set_error("probe_mfma_valu_overlap: null context/result or zero rounds");
         return VXHIP_INVALID_ARGUMENT;
@@ -158,7 +158,7 @@ extern "C" VxHipStatus vxhip_probe_mfma_valu_overlap(VxHipContext* ctx, uint32_t
         lcg = lcg * 1664525u + 1013904223u;
         const uint32_t hi = lcg;
         lcg = lcg * 1664525u + 1013904223u;
-        v = (hi & 0xffff0000u) | (lcg >> 16);
+        v = constant_operands ? 0x01010101u : (hi & 0xffff0000u) | (lcg >> 16);
     }
     v4i* operands = nullptr;
     uint64_t* clocks = nullptr;

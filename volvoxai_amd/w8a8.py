@@ -144,11 +144,12 @@ class Context:
                                                C.byref(mhz), C.byref(us)), "vxhip_probe_mfma_rate")
         return {"tops": tops.value, "shader_mhz": mhz.value, "microseconds": us.value}
 
-    def probe_mfma_valu_overlap(self, rounds=2000) -> dict:
+    def probe_mfma_valu_overlap(self, rounds=2000, constant_operands=False) -> dict:
         """Time and clock of the MFMAs alone, the folds alone, both in every wave, and split over
-        alternate waves (vxhip_probe_mfma_valu_overlap)."""
+        alternate waves (vxhip_probe_mfma_valu_overlap), on random operand bytes or on ones."""
         us, mhz = (C.c_double * 4)(), (C.c_double * 4)()
-        _check(library().vxhip_probe_mfma_valu_overlap(self._h, rounds, us, mhz), "vxhip_probe_mfma_valu_overlap")
+        _check(library().vxhip_probe_mfma_valu_overlap(self._h, rounds, 1 if constant_operands else 0, us, mhz),
+               "vxhip_probe_mfma_valu_overlap")
         names = ("mfma_only", "folds_only", "both_in_every_wave", "mfma_waves_beside_fold_waves_half_the_work_each")
         return {n: {"microseconds": us[i], "shader_mhz": mhz[i]} for i, n in enumerate(names)}
 
