@@ -1131,12 +1131,15 @@ def test_operand_order_activations(oracle, rows, k, n, group):
     pl.close(), plain.close(), blocked.close()
 
 
-@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (2048, 32, "fit16x4"),
-                                              (3072, 128, "fit8x12"), (4096, 128, "fit16x8"), (4096, 256, "fit16x8"),
-                                              (4090, 64, "fit16x8"), (8192, 128, "fit16x16"), (14336, 128, "fit16x28")])
-def test_exact_fit_gemv(oracle, k, group, instance):
+@pytest.mark.parametrize("k,group,instance,bits",
+                         [(1024, 128, "fit8x4", 8), (2048, 64, "fit16x4", 8), (2048, 32, "fit16x4", 8), (3072, 128, "fit8x12", 8),
+                          (4096, 128, "fit16x8", 8), (4096, 256, "fit16x8", 8), (4090, 64, "fit16x8", 8), (8192, 128, "fit16x16", 8),
+                          (14336, 128, "fit16x28", 8),
+                          (1024, 128, "fit4x4", 4), (2048, 64, "fit8x4", 4), (3072, 128, "fit8x6", 4), (4096, 128, "fit16x4", 4),
+                          (4096, 32, "fit16x4", 4), (4070, 256, "fit16x4", 4), (8192, 128, "fit16x8", 4), (14336, 128, "fit16x14", 4)])
+def test_exact_fit_gemv(oracle, k, group, instance, bits):
     """The straight-line streaming kernel for a K whose blocks divide evenly over the waves: every
-    instance, rows on both sides of its LDS-copy limit, both places where the products are formed
+    instance for eight- and four-bit weights, rows on both sides of its LDS-copy limit, both places where the products are formed
     (lane-parallel over the parked dots, or by the parking wave in its accumulators), both activation
     layouts, a row whose scale is NaN, an n that ends inside a panel -- the oracle's bits each time;
     and the general kernel still gives them when the exact-fit one is ruled out by name."""
@@ -1146,8 +1149,8 @@ def test_exact_fit_gemv(oracle, k, group, instance):
     plain, blocked = vx.Context(0, None), vx.Context(0, None)
     blocked.set_activation_layout(True)
     c = cases.packed_case(32, k, n, group, 4000 + k + group, True, special_rows=True)
-    words = oracle.pack_w8_words(c["w"])
-    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+    words = oracle.pack_w8_words(c["w"]) if bits == 8 else oracle.pack_w4_words(cases.four_bit(c["w"]))
+    pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group, weight_bits=bits)
     waves, bpw = (int(v) for v in instance[3:].split("x"))
     groups = (k + group - 1) // group
     try:
@@ -1159,7 +1162,7 @@ def test_exact_fit_gemv(oracle, k, group, instance):
             x = c["x"][:rows].copy()
             if rows >= 2:
                 x[-1, 7 % k] = np.nan  # a row that is not finite: a NaN scale, a NaN output row
-            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
+            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group, bits=bits)
             for ctx in (plain, blocked):
                 codes, scales = packed_prepare_i8(ctx, dev(x))
                 for force in (None, "gemv.fit.lprod", "gemv.fit.rprod", "gemv.nofit"):
@@ -1167,7 +1170,8 @@ def test_exact_fit_gemv(oracle, k, group, instance):
                     st, y = pl.forward_a8(ctx, codes, scales)
                     ctx.synchronize()
                     assert st == 0 and same_f32(host(y), want), (rows, force, ctx.last_variant)
-                    named = force in ("gemv.fit.lprod", "gemv.fit.rprod") or (force is None and n >= 6144)
+                    # (unnamed it takes enough panels to fill the device, and four-bit weights only while the rows fit LDS)
+                    named = force in ("gemv.fit.lprod", "gemv.fit.rprod") or (force is None and n >= 6144 and (bits == 8 or rows <= 8))
                     assert ctx.last_variant.endswith(instance) == named, (rows, force, ctx.last_variant)
         # one and two f32 rows: the kernel prepares them itself (the reference's single-row route in one launch);
         # a zero row, a row with an infinity, a plain one
@@ -1177,13 +1181,13 @@ def test_exact_fit_gemv(oracle, k, group, instance):
                 x[0] = 0.0
             if special == "inf":
                 x[1, k // 3] = np.inf
-            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
+            _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group, bits=bits)
             for force in (None, "gemv.nofit"):
                 vx.force_variant(force)
                 st, y = pl.forward_f32(plain, dev(x))
                 plain.synchronize()
                 assert st == 0 and same_f32(host(y), want), (rows, special, force, plain.last_variant)
-                prepared_here = force is None and n >= 6144 and k % 32 == 0
+                prepared_here = force is None and n >= 6144 and k % (32 if bits == 8 else 64) == 0
                 assert plain.last_variant.endswith(instance + "-prep") == prepared_here, (rows, force, plain.last_variant)
     finally:
         vx.force_variant(None)

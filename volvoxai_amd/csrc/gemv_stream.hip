@@ -500,34 +500,37 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
 // (packed_linear_ops.inc:1471-1535).  A wave's 64 lanes hold exactly the elements of the wave's own K-slice
 // (BPW / 2 consecutive ones per lane), so only the row maximum crosses the waves; the codes go straight into
 // the wave's LDS slice, where the MFMA's activation operand is read from.
-template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false, bool RPROD = false>
+// W4: four-bit weights; a 1 KiB block then carries two k-steps (low nibbles, then high nibbles, each moved to
+// the top of its byte: operands with a factor 16, which the exact dot sheds with a shift when it is parked).
+template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false, bool RPROD = false, bool W4 = false>
 __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArgs a) {
-    static_assert(BPW % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
-    static_assert(!PREP || (XLDS && BPW % 4 == 0), "prepared rows live in the LDS slices; a lane loads pairs of elements");
+    constexpr int SPB = W4 ? 2 : 1, STEPS = BPW * SPB;  // k-steps per block, per wave
+    static_assert(STEPS % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
+    static_assert(!PREP || (XLDS && STEPS % 4 == 0), "prepared rows live in the LDS slices; a lane loads pairs of elements");
     static_assert(!(PREP && RPROD), "one or two rows form their products lane-parallel");
-    constexpr int GPW = BPW / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
+    constexpr int GPW = STEPS / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t panel = blockIdx.x, rows = a.rows;
-    const uint32_t t0 = (uint32_t)wave * BPW, g0 = (uint32_t)wave * GPW;
+    const uint32_t t0 = (uint32_t)wave * STEPS, g0 = (uint32_t)wave * GPW;  // first k-step, first group
     const uint32_t half = lane >> 5;
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
     const uint32_t last_chunk = (a.k - 1u) / 16u;
-    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + t0) * 1024u + (uint32_t)lane * 16u;
+    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + (uint32_t)wave * BPW) * 1024u + (uint32_t)lane * 16u;
 
     // LDS: products [GROUPS][rows][32] (int32 dots first) | per wave: scales [GPW][32], row scales [32] |
-    // per wave (XLDS): activation slice [2 * BPW chunks][rows] of 16 bytes
+    // per wave (XLDS): activation slice [2 * STEPS chunks][rows] of 16 bytes
     int32_t* dots = reinterpret_cast<int32_t*>(gemv_lds);
     float* wave_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)GROUPS * rows * 32u + (size_t)wave * (GPW * 32 + 32);
     float* wave_rs = wave_scales + GPW * 32;
     char* xslice = gemv_lds + ((size_t)GROUPS * rows * 32u + (size_t)WAVES * (GPW * 32 + 32)) * 4u +
-                   (size_t)wave * (2 * BPW) * rows * 16u;
+                   (size_t)wave * (2 * STEPS) * rows * 16u;
 
     // (XLDS) this wave's activation chunks are requested first: they are cache hits and return ahead
     // of the weight stream
-    constexpr int XPL = XLDS && !PREP ? (2 * BPW * (int)kFitLdsRows + 63) / 64 : 1;  // chunks per lane
+    constexpr int XPL = XLDS && !PREP ? (2 * STEPS * (int)kFitLdsRows + 63) / 64 : 1;  // chunks per lane
     v4i xstage[XPL];
-    constexpr int EPL = BPW / 2;  // PREP: f32 elements of a row per lane
+    constexpr int EPL = STEPS / 2;  // PREP: f32 elements of a row per lane
     float xf[PREP ? (int)kMaxPrepRows : 1][PREP ? EPL : 1];
     if constexpr (PREP) {
 #pragma unroll
@@ -543,7 +546,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     } else if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < XPL; j++) {
-            const uint32_t e = min((uint32_t)lane + 64u * j, 2u * BPW * rows - 1u);
+            const uint32_t e = min((uint32_t)lane + 64u * j, 2u * STEPS * rows - 1u);
             const uint32_t c = min(t0 * 2u + e / rows, last_chunk), r = e % rows;
             xstage[j] = *reinterpret_cast<const v4i*>(
                 a.x + (a.x_operand_order ? ((size_t)c * kOperandOrderRows + r) * 16u : (size_t)r * a.ldx + (size_t)c * 16u));
@@ -555,12 +558,15 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     __builtin_amdgcn_sched_barrier(0);
     const int8_t* xp = a.x + (size_t)m * (a.x_operand_order ? 16u : a.ldx);
     const uint32_t x_chunk_pitch = a.x_operand_order ? 16u * kOperandOrderRows : 16u;
-    v4i wbuf[kDepth], xbuf[XLDS ? 1 : kDepth];
+    v4i wbuf[kDepth], xbuf[XLDS ? 1 : kDepth][SPB];
     auto issue = [&](int slot, uint32_t b) {
         wbuf[slot] = load_stream(wp + (size_t)b * 1024u);
         if constexpr (!XLDS) {
-            const uint32_t chunk = min((t0 + b) * 2u + half, last_chunk);
-            xbuf[slot] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
+#pragma unroll
+            for (int h = 0; h < SPB; h++) {
+                const uint32_t chunk = min((t0 + b * SPB + h) * 2u + half, last_chunk);
+                xbuf[slot][h] = *reinterpret_cast<const v4i*>(xp + (size_t)chunk * x_chunk_pitch);
+            }
         }
     };
 #pragma unroll
@@ -635,7 +641,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 #pragma unroll
         for (int j = 0; j < XPL; j++) {
             const uint32_t e = (uint32_t)lane + 64u * j;
-            if (e < 2u * BPW * rows) *reinterpret_cast<v4i*>(xslice + (size_t)e * 16u) = xstage[j];
+            if (e < 2u * STEPS * rows) *reinterpret_cast<v4i*>(xslice + (size_t)e * 16u) = xstage[j];
         }
     }
 
@@ -646,45 +652,56 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 #pragma unroll
     for (int b = 0; b < BPW; b++) {
         const int slot = b % kDepth;
-        v4i xop;
-        if constexpr (XLDS) xop = *reinterpret_cast<const v4i*>(xslice + ((size_t)(2 * b + half) * rows + m) * 16u);
-        else xop = xbuf[slot];
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wbuf[slot], xop, acc, 0, 0, 0);
-        if (b + kDepth < BPW) issue(slot, b + kDepth);
-        if constexpr (RPROD) {
-            // the wave's group scales go to its LDS strip once they are here (they were requested behind
-            // the first kDepth blocks), in time for the first group that closes
-            if (b == (GK > kDepth ? kDepth : GK) - 1) {
 #pragma unroll
-                for (int u = 0; u < SPL; u++) {
-                    const uint32_t e = (uint32_t)lane + 64u * u;
-                    if (e < GPW * 32u) wave_scales[e] = sreg[u];
-                }
+        for (int h = 0; h < SPB; h++) {
+            const int t = b * SPB + h;  // the wave's k-step
+            v4i xop, wop = wbuf[slot];
+            if constexpr (XLDS) xop = *reinterpret_cast<const v4i*>(xslice + ((size_t)(2 * t + half) * rows + m) * 16u);
+            else xop = xbuf[slot][h];
+            if constexpr (W4) {
+#pragma unroll
+                for (int d = 0; d < 4; d++) wop[d] = (h == 0 ? wbuf[slot][d] << 4 : wbuf[slot][d]) & (int)0xf0f0f0f0u;
             }
-        }
-        if ((b + 1) % GK == 0) {
-            if (row_live) {
-                int32_t* dp = dots + ((size_t)(g0 + b / GK) * rows + (lane & 31)) * 32u + half * 4u;
-                if constexpr (RPROD) {
-                    // many rows: the products are formed here, in the accumulators' own layout (a lane holds
-                    // its row's dots of sixteen channels), and parked as floats
-                    const float* sw = wave_scales + (b / GK) * 32 + half * 4u;
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wop, xop, acc, 0, 0, 0);
+            if (h == SPB - 1 && b + kDepth < BPW) issue(slot, b + kDepth);
+            if constexpr (RPROD) {
+                // the wave's group scales go to its LDS strip once they are here (they were requested behind
+                // the first kDepth blocks), in time for the first group that closes
+                if (t == (GK > kDepth * SPB ? kDepth * SPB : GK) - 1) {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const v4f s4 = *reinterpret_cast<const v4f*>(sw + q * 8);
-                        v4f p;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) p[i] = __fmul_rn((float)acc[q * 4 + i], __fmul_rn(rs_lane, s4[i]));
-                        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(dp) + q * 8) = p;
+                    for (int u = 0; u < SPL; u++) {
+                        const uint32_t e = (uint32_t)lane + 64u * u;
+                        if (e < GPW * 32u) wave_scales[e] = sreg[u];
                     }
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; q++)
-                        *reinterpret_cast<v4i*>(dp + q * 8) = v4i{acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
                 }
             }
+            if ((t + 1) % GK == 0) {
+                if (row_live) {
+                    int32_t* dp = dots + ((size_t)(g0 + t / GK) * rows + (lane & 31)) * 32u + half * 4u;
+                    if constexpr (RPROD) {
+                        // many rows: the products are formed here, in the accumulators' own layout (a lane holds
+                        // its row's dots of sixteen channels), and parked as floats
+                        const float* sw = wave_scales + (t / GK) * 32 + half * 4u;
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[r] = 0;
+                        for (int q = 0; q < 4; q++) {
+                            const v4f s4 = *reinterpret_cast<const v4f*>(sw + q * 8);
+                            v4f p;
+#pragma unroll
+                            for (int i = 0; i < 4; i++)
+                                p[i] = __fmul_rn((float)(acc[q * 4 + i] >> (W4 ? 4 : 0)), __fmul_rn(rs_lane, s4[i]));
+                            *reinterpret_cast<v4f*>(reinterpret_cast<float*>(dp) + q * 8) = p;
+                        }
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            *reinterpret_cast<v4i*>(dp + q * 8) =
+                                v4i{acc[q * 4] >> (W4 ? 4 : 0), acc[q * 4 + 1] >> (W4 ? 4 : 0), acc[q * 4 + 2] >> (W4 ? 4 : 0),
+                                    acc[q * 4 + 3] >> (W4 ? 4 : 0)};
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r] = 0;
+            }
         }
     }
 
@@ -721,7 +738,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         const uint32_t o = threadIdx.x + it * WAVES * 64;
         if (o >= rows * 32u) break;
         // (sixteen products are requested before the first add needs one)
-        constexpr int BATCH = GROUPS % 16 == 0 ? 16 : 8;
+        constexpr int BATCH = GROUPS % 16 == 0 ? 16 : GROUPS % 8 == 0 ? 8 : GROUPS % 4 == 0 ? 4 : 1;
         static_assert(GROUPS % BATCH == 0, "the groups of a panel come in whole batches");
         float sum = 0.0f;
 #pragma unroll
@@ -737,12 +754,12 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     }
 }
 
-template <int GK, int WAVES, int BPW>
+template <int GK, int WAVES, int BPW, bool W4>
 bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds, bool rprod) {
-    auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true> : gemv_fit_kernel<GK, WAVES, BPW, false>;
-    if (rprod) kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, true> : gemv_fit_kernel<GK, WAVES, BPW, false, false, true>;
-    if constexpr (BPW % 4 == 0) {
-        if (a.x_f32) kern = gemv_fit_kernel<GK, WAVES, BPW, true, true>;
+    auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, false, W4> : gemv_fit_kernel<GK, WAVES, BPW, false, false, false, W4>;
+    if (rprod) kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, true, W4> : gemv_fit_kernel<GK, WAVES, BPW, false, false, true, W4>;
+    if constexpr ((BPW * (W4 ? 2 : 1)) % 4 == 0) {
+        if (a.x_f32) kern = gemv_fit_kernel<GK, WAVES, BPW, true, true, false, W4>;
     }
     if (gemv_dry_run) return true;
     if (lds > 64u * 1024u) {
@@ -753,63 +770,71 @@ bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds, bool 
     return hipGetLastError() == hipSuccess;
 }
 
-// The exact-fit kernel takes: the dequantizing epilogue on prepared int8 rows, eight-bit weights, enough
-// panels to fill the device without sharing one, and a K whose blocks are WAVES x BPW of an instance with
-// whole groups in every run.  Returns the variant suffix, or null when the general kernel has to run.
-template <int GK>
+// The exact-fit kernel takes: the dequantizing epilogue on prepared int8 rows (or one or two f32 rows), eight- or
+// four-bit weights, enough panels to fill the device without sharing one, and a K whose blocks are WAVES x BPW of
+// an instance with whole groups in every run.  Returns the variant suffix, or null when the general kernel has to run.
+template <int GK, bool W4>
 const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
+    constexpr uint32_t SPB = W4 ? 2u : 1u;
     if (force && strstr(force, "nofit")) return nullptr;
-    if (a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != 8u || a.x_flip_mask) return nullptr;
+    if (a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != (W4 ? 4u : 8u) || a.x_flip_mask) return nullptr;
     // f32 rows (prepared in the kernel): one or two whole rows of exactly the stream's length, pairs of elements aligned
     const bool prep = a.x_f32 != nullptr;
-    if (prep && (a.rows > kMaxPrepRows || a.k != a.ksteps * 32u || (a.ldx % 2u) != 0u || ((uintptr_t)a.x_f32 % 8u) != 0u))
+    if (prep && (a.rows > kMaxPrepRows || a.k != a.ksteps * 32u * SPB || (a.ldx % 2u) != 0u || ((uintptr_t)a.x_f32 % 8u) != 0u))
         return nullptr;
     const uint32_t panels = (a.n + 31u) / 32u;
     const bool forced = force && strstr(force, "fit");
     if (panels * 4u < (uint32_t)cu_count * 3u && !forced) return nullptr;
-    if (a.groups * GK != a.ksteps) return nullptr;  // (no padding group: every group of the stream has its scales)
-    auto lds_for = [&](uint32_t waves, uint32_t bpw, bool xlds) {
-        const size_t groups = (size_t)waves * bpw / GK;
-        return groups * a.rows * 128u + (size_t)waves * (bpw / GK * 32u + 32u) * 4u +
-               (xlds ? (size_t)waves * 2u * bpw * a.rows * 16u : 0u);
+    // (four-bit weights with more rows than the LDS copy takes: the stream is half as long and the activation loads
+    // per block weigh twice as much -- 16 rows 12.1 us here against 12.0 in the general kernel, 32 rows 17.5 against 17.7)
+    if (W4 && a.rows > kFitLdsRows && !forced) return nullptr;
+    if (a.groups * GK != a.ksteps * SPB) return nullptr;  // (no padding group: every group of the stream has its scales)
+    auto lds_for = [&](uint32_t waves, uint32_t steps, bool xlds) {
+        const size_t groups = (size_t)waves * steps / GK;
+        return groups * a.rows * 128u + (size_t)waves * (steps / GK * 32u + 32u) * 4u +
+               (xlds ? (size_t)waves * 2u * steps * a.rows * 16u : 0u);
     };
-    // where the products are formed: lane-parallel over the parked dots (few rows), or by the parking wave
-    // in its accumulators' layout (many rows)
+    // where the products are formed: lane-parallel over the parked dots (one row), or by the parking wave
+    // in its accumulators' layout (more rows)
     // (measured at K=4096, N=14336: one row 10.8 us either way, 2 / 4 / 8 / 16 / 32 rows 10.8 / 10.9 / 11.0 / 11.9 / 16.3 us
     // against 11.1 / 11.3 / 12.9 / 15.9 / 27.9 lane-parallel and 12.5 / 12.6 / 12.8 / 13.5 / 18.4 in the general kernel)
     const bool rprod = !prep && (force && strstr(force, "rprod") ? true : force && strstr(force, "lprod") ? false : a.rows > 1u);
-    const char* name = nullptr;
-    bool ok = false;
-    auto run = [&](auto waves_tag, auto bpw_tag, const char* id) {
-        constexpr int W = decltype(waves_tag)::value, B = decltype(bpw_tag)::value;
-        if constexpr (B % GK == 0) {
-            if (name || a.ksteps != (uint32_t)(W * B)) return;
+    static thread_local char name[24];
+    bool taken = false, ok = false;
+    auto run = [&](auto waves_tag, auto bpw_tag) {
+        constexpr int W = decltype(waves_tag)::value, B = decltype(bpw_tag)::value, STEPS = B * (int)SPB;
+        if constexpr (STEPS % GK == 0) {
+            if (taken || a.ksteps != (uint32_t)(W * B)) return;
             // the activation rows go through LDS while two workgroups still fit a compute unit that way
             bool xlds = a.rows <= kFitLdsRows;
-            size_t lds = lds_for(W, B, xlds);
+            size_t lds = lds_for(W, STEPS, xlds);
             if (xlds && lds > 80u * 1024u && !prep) {
                 xlds = false;
-                lds = lds_for(W, B, false);
+                lds = lds_for(W, STEPS, false);
             }
-            if (lds > 156u * 1024u || (prep && B % 4 != 0)) return;
-            ok = launch_fit<GK, W, B>(s, a, lds, xlds, rprod);
-            name = id;
+            if (lds > 156u * 1024u || (prep && STEPS % 4 != 0)) return;
+            ok = launch_fit<GK, W, B, W4>(s, a, lds, xlds, rprod);
+            taken = true;
+            snprintf(name, sizeof name, "fit%dx%d%s", W, B, prep ? "-prep" : "");
         }
     };
     using std::integral_constant;
-    run(integral_constant<int, 16>{}, integral_constant<int, 4>{}, "fit16x4");
-    run(integral_constant<int, 16>{}, integral_constant<int, 8>{}, "fit16x8");
-    run(integral_constant<int, 16>{}, integral_constant<int, 16>{}, "fit16x16");
-    run(integral_constant<int, 16>{}, integral_constant<int, 28>{}, "fit16x28");
-    run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, "fit8x4");
-    run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, "fit8x12");
-    if (!ok) return nullptr;
-    if (!prep) return name;
-    static const char* const prep_names[6][2] = {{"fit16x4", "fit16x4-prep"}, {"fit16x8", "fit16x8-prep"}, {"fit16x16", "fit16x16-prep"},
-                                                 {"fit16x28", "fit16x28-prep"}, {"fit8x4", "fit8x4-prep"}, {"fit8x12", "fit8x12-prep"}};
-    for (const auto& pair : prep_names)
-        if (!strcmp(pair[0], name)) return pair[1];
-    return name;
+    if constexpr (W4) {  // K = 1024, 2048, 3072, 4096, 8192, 14336
+        run(integral_constant<int, 4>{}, integral_constant<int, 4>{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 4>{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 6>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 4>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 8>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 14>{});
+    } else {  // K = 2048, 4096, 8192, 14336, 1024, 3072
+        run(integral_constant<int, 16>{}, integral_constant<int, 4>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 8>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 16>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 28>{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 4>{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 12>{});
+    }
+    return ok ? name : nullptr;
 }
 
 template <int MODE, int GK, int WAVES, bool W4, int SPLIT = 1, int ROWOP = kRowsPrepared>
@@ -833,8 +858,8 @@ bool launch_split(hipStream_t s, const LinearArgs& a, size_t lds, int split) {
 
 template <int MODE, int GK, bool W4 = false>
 const char* launch_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
-    if constexpr (MODE == (int)Epilogue::DequantF32 && !W4) {
-        if (const char* fit = launch_fit_mode<GK>(s, a, cu_count, force)) return fit;
+    if constexpr (MODE == (int)Epilogue::DequantF32) {
+        if (const char* fit = launch_fit_mode<GK, W4>(s, a, cu_count, force)) return fit;
     }
     // blocks of the stream per panel, and the units a wave's run is made of
     constexpr uint32_t SPB = W4 ? 2 : 1, UNIT = GK > SPB ? GK : SPB;
