@@ -235,6 +235,9 @@ struct LinearArgs {
     double row_eps;
     uint32_t row_swiglu;
     const float* add_to;
+    // set by the large-tile GEMM launchers for outputs of a size where it was measured to pay: the
+    // output leaves the L2 as it is stored (store_stream) instead of with the write-back at the end
+    uint32_t stream_out;
 };
 
 // gemm_mfma.hip / gemv_stream.hip: return the variant id that ran, or null if
