@@ -1194,6 +1194,44 @@ def test_exact_fit_gemv(oracle, k, group, instance, bits):
         pl.close(), plain.close(), blocked.close()
 
 
+@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (3072, 128, "fit8x12"),
+                                              (4096, 128, "fit16x8"), (4090, 32, "fit16x8")])
+def test_exact_fit_gemv_shared_panels(oracle, k, group, instance):
+    """Few panels: four (N = 1000) or two (N = 4090) workgroups of the straight-line kernel share a panel's
+    channels -- the decoder's projections at 32 rows.  Rows on both sides of the LDS-copy limit, both places
+    where the products are formed, both activation layouts, a NaN row: the oracle's bits each time."""
+    import volvoxai_amd as vx
+    from volvoxai_amd.w8a8 import packed_prepare_i8
+    plain, blocked = vx.Context(0, None), vx.Context(0, None)
+    blocked.set_activation_layout(True)
+    try:
+        for n, suffix in ((1000, "c8"), (4090, "c16")):
+            c = cases.packed_case(32, k, n, group, 4200 + k + n, True, special_rows=True)
+            words = oracle.pack_w8_words(c["w"])
+            pl = vx.PackedLinear(words, c["scales"], c["bias"], k, n, group)
+            waves = int(instance[3:].split("x")[0])
+            groups, ch = (k + group - 1) // group, 32 // (4 if suffix == "c8" else 2)
+            for rows in (1, 3, 8, 9, 32):
+                if groups * rows * ch * 4 + waves * (groups // waves * ch + 32) * 4 > 156 * 1024:
+                    continue  # (the products of every group do not fit the LDS: not a shape of the streaming kernels)
+                x = c["x"][:rows].copy()
+                if rows >= 2:
+                    x[-1, 11 % k] = np.nan
+                _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group)
+                for ctx in (plain, blocked):
+                    codes, scales = packed_prepare_i8(ctx, dev(x))
+                    for force in (None, "gemv.fit.lprod", "gemv.fit.rprod", "gemv.nofit"):
+                        vx.force_variant(force)
+                        st, y = pl.forward_a8(ctx, codes, scales)
+                        ctx.synchronize()
+                        assert st == 0 and same_f32(host(y), want), (n, rows, force, ctx.last_variant)
+                        assert ctx.last_variant.endswith(instance + suffix) == (force != "gemv.nofit"), (n, rows, force, ctx.last_variant)
+            pl.close()
+    finally:
+        vx.force_variant(None)
+        plain.close(), blocked.close()
+
+
 def test_packed_output_window(ctx, oracle):
     """first_unit / unit_count of the PackedLinear descriptor (llm_ops.h:48-52) on both entry points: the
     reference's window list on 11 rows (test_packed_linear_i8.c:263-265), the whole output array --

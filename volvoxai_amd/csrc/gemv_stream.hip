@@ -502,28 +502,35 @@ __global__ __launch_bounds__(WAVES * 64, (ROWOP == 2 && WAVES == 8) ? 4 : 1) voi
 // the wave's LDS slice, where the MFMA's activation operand is read from.
 // W4: four-bit weights; a 1 KiB block then carries two k-steps (low nibbles, then high nibbles, each moved to
 // the top of its byte: operands with a factor 16, which the exact dot sheds with a shift when it is parked).
-template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false, bool RPROD = false, bool W4 = false>
+template <int GK, int WAVES, int BPW, bool XLDS, bool PREP = false, bool RPROD = false, bool W4 = false, int SPLIT = 1>
 __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArgs a) {
     constexpr int SPB = W4 ? 2 : 1, STEPS = BPW * SPB;  // k-steps per block, per wave
     static_assert(STEPS % GK == 0 && BPW >= kDepth, "a wave's run is whole groups and at least one round");
     static_assert(!PREP || (XLDS && STEPS % 4 == 0), "prepared rows live in the LDS slices; a lane loads pairs of elements");
     static_assert(!(PREP && RPROD), "one or two rows form their products lane-parallel");
+    static_assert(SPLIT == 1 || SPLIT == 2 || SPLIT == 4, "workgroups per panel");
     constexpr int GPW = STEPS / GK, GROUPS = WAVES * GPW;  // groups per wave, per panel
+    // SPLIT workgroups share a panel, each taking CH of its channels, as in gemv_panel_kernel: a lane whose
+    // channel is another workgroup's loads the bytes of the lane that holds this workgroup's channel at the
+    // same offset, and only the accumulator quads of the workgroup's channels are parked
+    constexpr int CH = 32 / SPLIT, QUADS = 4 / SPLIT;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const uint32_t panel = blockIdx.x, rows = a.rows;
+    const uint32_t panel = blockIdx.x / SPLIT, sub = blockIdx.x % SPLIT, rows = a.rows;
+    const uint32_t ch0 = panel * 32u + sub * CH;
+    const uint32_t src_lane = SPLIT == 1 ? (uint32_t)lane : ((lane & 32) | (sub * CH + (lane & (CH - 1))));
     const uint32_t t0 = (uint32_t)wave * STEPS, g0 = (uint32_t)wave * GPW;  // first k-step, first group
     const uint32_t half = lane >> 5;
     const uint32_t m = min((uint32_t)(lane & 31), rows - 1u);
     const uint32_t last_chunk = (a.k - 1u) / 16u;
-    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + (uint32_t)wave * BPW) * 1024u + (uint32_t)lane * 16u;
+    const int8_t* wp = a.w + ((size_t)panel * a.ksteps + (uint32_t)wave * BPW) * 1024u + src_lane * 16u;
 
-    // LDS: products [GROUPS][rows][32] (int32 dots first) | per wave: scales [GPW][32], row scales [32] |
+    // LDS: products [GROUPS][rows][CH] (int32 dots first) | per wave: scales [GPW][CH], row scales [32] |
     // per wave (XLDS): activation slice [2 * STEPS chunks][rows] of 16 bytes
     int32_t* dots = reinterpret_cast<int32_t*>(gemv_lds);
-    float* wave_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)GROUPS * rows * 32u + (size_t)wave * (GPW * 32 + 32);
-    float* wave_rs = wave_scales + GPW * 32;
-    char* xslice = gemv_lds + ((size_t)GROUPS * rows * 32u + (size_t)WAVES * (GPW * 32 + 32)) * 4u +
+    float* wave_scales = reinterpret_cast<float*>(gemv_lds) + (size_t)GROUPS * rows * CH + (size_t)wave * (GPW * CH + 32);
+    float* wave_rs = wave_scales + GPW * CH;
+    char* xslice = gemv_lds + ((size_t)GROUPS * rows * CH + (size_t)WAVES * (GPW * CH + 32)) * 4u +
                    (size_t)wave * (2 * STEPS) * rows * 16u;
 
     // (XLDS) this wave's activation chunks are requested first: they are cache hits and return ahead
@@ -574,21 +581,21 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
     __builtin_amdgcn_sched_barrier(0);
 
     // what the tail needs, requested behind the first blocks: the wave's group scales, lane e <-> (group
-    // g0 + e / 32, channel e % 32); the row scales; the bias of this thread's outputs
-    constexpr int SPL = (GPW * 32 + 63) / 64;
+    // g0 + e / CH, channel e % CH); the row scales; the bias of this thread's outputs
+    constexpr int SPL = (GPW * CH + 63) / 64;
     float sreg[SPL];
 #pragma unroll
     for (int u = 0; u < SPL; u++) {
-        const uint32_t e = min((uint32_t)lane + 64u * u, GPW * 32u - 1u);
-        sreg[u] = a.scales_t[(size_t)(g0 + e / 32u) * a.n_pad + panel * 32u + e % 32u];
+        const uint32_t e = min((uint32_t)lane + 64u * u, (uint32_t)(GPW * CH) - 1u);
+        sreg[u] = a.scales_t[(size_t)(g0 + e / CH) * a.n_pad + ch0 + e % CH];
     }
     // (RPROD: the scale of the row whose dots the lane holds in its accumulators; else lane r carries row r's)
     float rs_lane = 0.0f;
     if constexpr (!PREP) rs_lane = a.row_scale[RPROD ? m : min((uint32_t)lane, rows - 1u)];
-    constexpr int OPT_ = ((int)kMaxGemvRows * 32 + WAVES * 64 - 1) / (WAVES * 64);  // outputs per thread
+    constexpr int OPT_ = ((int)kMaxGemvRows * CH + WAVES * 64 - 1) / (WAVES * 64);  // outputs per thread
     float bias_t[OPT_];
 #pragma unroll
-    for (int it = 0; it < OPT_; it++) bias_t[it] = a.bias_f32[panel * 32u + (threadIdx.x + it * WAVES * 64) % 32u];
+    for (int it = 0; it < OPT_; it++) bias_t[it] = a.bias_f32[ch0 + (threadIdx.x + it * WAVES * 64) % CH];
 
     if constexpr (PREP) {
         // per row: scale = max|x| / 127 (true division; 1 for a zero row; floored at 2^-126), codes =
@@ -671,32 +678,36 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 #pragma unroll
                     for (int u = 0; u < SPL; u++) {
                         const uint32_t e = (uint32_t)lane + 64u * u;
-                        if (e < GPW * 32u) wave_scales[e] = sreg[u];
+                        if (e < (uint32_t)(GPW * CH)) wave_scales[e] = sreg[u];
                     }
                 }
             }
             if ((t + 1) % GK == 0) {
                 if (row_live) {
-                    int32_t* dp = dots + ((size_t)(g0 + t / GK) * rows + (lane & 31)) * 32u + half * 4u;
+                    int32_t* dp = dots + ((size_t)(g0 + t / GK) * rows + (lane & 31)) * CH + half * 4u;
                     if constexpr (RPROD) {
                         // many rows: the products are formed here, in the accumulators' own layout (a lane holds
                         // its row's dots of sixteen channels), and parked as floats
-                        const float* sw = wave_scales + (t / GK) * 32 + half * 4u;
+                        const float* sw = wave_scales + (t / GK) * CH + half * 4u;
 #pragma unroll
                         for (int q = 0; q < 4; q++) {
-                            const v4f s4 = *reinterpret_cast<const v4f*>(sw + q * 8);
+                            // quad q holds channels 8q..8q+7 of the panel; the test is scalar
+                            if (SPLIT > 1 && (uint32_t)(q / QUADS) != sub) continue;
+                            const v4f s4 = *reinterpret_cast<const v4f*>(sw + (q % QUADS) * 8);
                             v4f p;
 #pragma unroll
                             for (int i = 0; i < 4; i++)
                                 p[i] = __fmul_rn((float)(acc[q * 4 + i] >> (W4 ? 4 : 0)), __fmul_rn(rs_lane, s4[i]));
-                            *reinterpret_cast<v4f*>(reinterpret_cast<float*>(dp) + q * 8) = p;
+                            *reinterpret_cast<v4f*>(reinterpret_cast<float*>(dp) + (q % QUADS) * 8) = p;
                         }
                     } else {
 #pragma unroll
-                        for (int q = 0; q < 4; q++)
-                            *reinterpret_cast<v4i*>(dp + q * 8) =
+                        for (int q = 0; q < 4; q++) {
+                            if (SPLIT > 1 && (uint32_t)(q / QUADS) != sub) continue;
+                            *reinterpret_cast<v4i*>(dp + (q % QUADS) * 8) =
                                 v4i{acc[q * 4] >> (W4 ? 4 : 0), acc[q * 4 + 1] >> (W4 ? 4 : 0), acc[q * 4 + 2] >> (W4 ? 4 : 0),
                                     acc[q * 4 + 3] >> (W4 ? 4 : 0)};
+                        }
                     }
                 }
 #pragma unroll
@@ -705,29 +716,29 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         }
     }
 
-    // products of this wave's groups, in place: element e of its region is (group g0 + e / (rows * 32),
-    // row (e / 32) % rows, channel e % 32)
-    float* prod = reinterpret_cast<float*>(dots) + (size_t)g0 * rows * 32u;
+    // products of this wave's groups, in place: element e of its region is (group g0 + e / (rows * CH),
+    // row (e / CH) % rows, channel e % CH)
+    float* prod = reinterpret_cast<float*>(dots) + (size_t)g0 * rows * CH;
     if constexpr (RPROD) {
         (void)prod;
     } else if (rows == 1u) {
 #pragma unroll
         for (int u = 0; u < SPL; u++) {
             const uint32_t e = (uint32_t)lane + 64u * u;
-            if (e < GPW * 32u)
+            if (e < (uint32_t)(GPW * CH))
                 prod[e] = __fmul_rn((float)reinterpret_cast<const int32_t*>(prod)[e], __fmul_rn(rs_lane, sreg[u]));
         }
     } else {
 #pragma unroll
         for (int u = 0; u < SPL; u++) {
             const uint32_t e = (uint32_t)lane + 64u * u;
-            if (e < GPW * 32u) wave_scales[e] = sreg[u];
+            if (e < (uint32_t)(GPW * CH)) wave_scales[e] = sreg[u];
         }
         if ((uint32_t)lane < rows) wave_rs[lane] = rs_lane;
-        const uint32_t per_group = rows * 32u;
+        const uint32_t per_group = rows * CH;
         for (uint32_t e = lane; e < GPW * per_group; e += 64u) {
-            const float sw = wave_scales[(e / per_group) * 32u + e % 32u];
-            const float rs = wave_rs[(e / 32u) % rows];
+            const float sw = wave_scales[(e / per_group) * CH + e % CH];
+            const float rs = wave_rs[(e / CH) % rows];
             prod[e] = __fmul_rn((float)reinterpret_cast<const int32_t*>(prod)[e], __fmul_rn(rs, sw));
         }
     }
@@ -736,7 +747,7 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
 #pragma unroll
     for (int it = 0; it < OPT_; it++) {
         const uint32_t o = threadIdx.x + it * WAVES * 64;
-        if (o >= rows * 32u) break;
+        if (o >= rows * CH) break;
         // (sixteen products are requested before the first add needs one)
         constexpr int BATCH = GROUPS % 16 == 0 ? 16 : GROUPS % 8 == 0 ? 8 : GROUPS % 4 == 0 ? 4 : 1;
         static_assert(GROUPS % BATCH == 0, "the groups of a panel come in whole batches");
@@ -745,20 +756,21 @@ __global__ __launch_bounds__(WAVES * 64, 8) void gemv_fit_kernel(const LinearArg
         for (int gb = 0; gb < GROUPS; gb += BATCH) {
             float p[BATCH];
 #pragma unroll
-            for (int g = 0; g < BATCH; g++) p[g] = products[(size_t)(gb + g) * rows * 32u + o];
+            for (int g = 0; g < BATCH; g++) p[g] = products[(size_t)(gb + g) * rows * CH + o];
 #pragma unroll
             for (int g = 0; g < BATCH; g++) sum = __fadd_rn(sum, p[g]);
         }
-        const uint32_t on = panel * 32u + o % 32u;
-        if (on < a.n) ((float*)a.y)[(size_t)(o / 32u) * a.n + on] = __fadd_rn(sum, bias_t[it]);
+        const uint32_t on = ch0 + o % CH;
+        if (on < a.n) ((float*)a.y)[(size_t)(o / CH) * a.n + on] = __fadd_rn(sum, bias_t[it]);
     }
 }
 
-template <int GK, int WAVES, int BPW, bool W4>
+template <int GK, int WAVES, int BPW, bool W4, int SPLIT = 1>
 bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds, bool rprod) {
-    auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, false, W4> : gemv_fit_kernel<GK, WAVES, BPW, false, false, false, W4>;
-    if (rprod) kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, true, W4> : gemv_fit_kernel<GK, WAVES, BPW, false, false, true, W4>;
-    if constexpr ((BPW * (W4 ? 2 : 1)) % 4 == 0) {
+    auto kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, false, W4, SPLIT> : gemv_fit_kernel<GK, WAVES, BPW, false, false, false, W4, SPLIT>;
+    if (rprod)
+        kern = xlds ? gemv_fit_kernel<GK, WAVES, BPW, true, false, true, W4, SPLIT> : gemv_fit_kernel<GK, WAVES, BPW, false, false, true, W4, SPLIT>;
+    if constexpr (SPLIT == 1 && (BPW * (W4 ? 2 : 1)) % 4 == 0) {
         if (a.x_f32) kern = gemv_fit_kernel<GK, WAVES, BPW, true, true, false, W4>;
     }
     if (gemv_dry_run) return true;
@@ -766,17 +778,18 @@ bool launch_fit(hipStream_t s, const LinearArgs& a, size_t lds, bool xlds, bool 
         static std::atomic<uint64_t> configured[5] = {{0}, {0}, {0}, {0}, {0}};
         if (!raise_lds_limit((const void*)kern, 160 * 1024, configured[a.x_f32 ? 4 : (rprod ? 2 : 0) + (xlds ? 1 : 0)])) return false;
     }
-    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL(kern, dim3((a.n + 31u) / 32u * SPLIT), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError() == hipSuccess;
 }
 
 // The exact-fit kernel takes: the dequantizing epilogue on prepared int8 rows (or one or two f32 rows), eight- or
-// four-bit weights, enough panels to fill the device without sharing one, and a K whose blocks are WAVES x BPW of
-// an instance with whole groups in every run.  Returns the variant suffix, or null when the general kernel has to run.
+// four-bit weights, and a K whose blocks are WAVES x BPW of an instance with whole groups in every run; with few
+// panels (eight-bit weights, prepared rows, K up to 4096) two or four workgroups share a panel's channels, as in
+// the general kernel.  Returns the variant suffix, or null when the general kernel has to run.
 template <int GK, bool W4>
 const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, const char* force) {
     constexpr uint32_t SPB = W4 ? 2u : 1u;
-    if (force && strstr(force, "nofit")) return nullptr;
+    if (force && (strstr(force, "nofit") || strstr(force, "wv"))) return nullptr;  // (wv..: a general-kernel name)
     if (a.row_gain || a.row_swiglu || a.add_to || a.weight_bits != (W4 ? 4u : 8u) || a.x_flip_mask) return nullptr;
     // f32 rows (prepared in the kernel): one or two whole rows of exactly the stream's length, pairs of elements aligned
     const bool prep = a.x_f32 != nullptr;
@@ -784,14 +797,24 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
         return nullptr;
     const uint32_t panels = (a.n + 31u) / 32u;
     const bool forced = force && strstr(force, "fit");
-    if (panels * 4u < (uint32_t)cu_count * 3u && !forced) return nullptr;
+    // workgroups per panel: the general kernel's rule (and its names: c8, c16 for the channels of a workgroup)
+    uint32_t split = 1;
+    if (!W4 && !prep && a.ksteps <= 128u) {
+        split = panels * 4u <= (uint32_t)cu_count ? 4u : panels * 2u <= (uint32_t)cu_count ? 2u : 1u;
+        if (force && strstr(force, "c8")) split = 4;
+        else if (force && strstr(force, "c16")) split = 2;
+        else if (force && strstr(force, "c32")) split = 1;
+    }
+    // (one workgroup per panel and panels for fewer than three quarters of the compute units: the general kernel)
+    if (split == 1u && panels * 4u < (uint32_t)cu_count * 3u && !forced) return nullptr;
     // (four-bit weights with more rows than the LDS copy takes: the stream is half as long and the activation loads
     // per block weigh twice as much -- 16 rows 12.1 us here against 12.0 in the general kernel, 32 rows 17.5 against 17.7)
     if (W4 && a.rows > kFitLdsRows && !forced) return nullptr;
     if (a.groups * GK != a.ksteps * SPB) return nullptr;  // (no padding group: every group of the stream has its scales)
+    const size_t ch = 32u / split;
     auto lds_for = [&](uint32_t waves, uint32_t steps, bool xlds) {
         const size_t groups = (size_t)waves * steps / GK;
-        return groups * a.rows * 128u + (size_t)waves * (steps / GK * 32u + 32u) * 4u +
+        return groups * a.rows * ch * 4u + (size_t)waves * (steps / GK * ch + 32u) * 4u +
                (xlds ? (size_t)waves * 2u * steps * a.rows * 16u : 0u);
     };
     // where the products are formed: lane-parallel over the parked dots (one row), or by the parking wave
@@ -801,8 +824,9 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
     const bool rprod = !prep && (force && strstr(force, "rprod") ? true : force && strstr(force, "lprod") ? false : a.rows > 1u);
     static thread_local char name[24];
     bool taken = false, ok = false;
-    auto run = [&](auto waves_tag, auto bpw_tag) {
+    auto run = [&](auto waves_tag, auto bpw_tag, auto splits_tag) {
         constexpr int W = decltype(waves_tag)::value, B = decltype(bpw_tag)::value, STEPS = B * (int)SPB;
+        constexpr bool SPLITS = decltype(splits_tag)::value;  // the instance is built for shared panels too
         if constexpr (STEPS % GK == 0) {
             if (taken || a.ksteps != (uint32_t)(W * B)) return;
             // the activation rows go through LDS while two workgroups still fit a compute unit that way
@@ -813,26 +837,35 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
                 lds = lds_for(W, STEPS, false);
             }
             if (lds > 156u * 1024u || (prep && STEPS % 4 != 0)) return;
-            ok = launch_fit<GK, W, B, W4>(s, a, lds, xlds, rprod);
+            if constexpr (SPLITS) {
+                if (split == 4u) ok = launch_fit<GK, W, B, W4, 4>(s, a, lds, xlds, rprod);
+                else if (split == 2u) ok = launch_fit<GK, W, B, W4, 2>(s, a, lds, xlds, rprod);
+                else ok = launch_fit<GK, W, B, W4>(s, a, lds, xlds, rprod);
+            } else {
+                if (split != 1u) return;
+                ok = launch_fit<GK, W, B, W4>(s, a, lds, xlds, rprod);
+            }
             taken = true;
-            snprintf(name, sizeof name, "fit%dx%d%s", W, B, prep ? "-prep" : "");
+            snprintf(name, sizeof name, "fit%dx%d%s%s", W, B, split == 4u ? "c8" : split == 2u ? "c16" : "", prep ? "-prep" : "");
         }
     };
     using std::integral_constant;
+    using std::true_type;
+    using std::false_type;
     if constexpr (W4) {  // K = 1024, 2048, 3072, 4096, 8192, 14336
-        run(integral_constant<int, 4>{}, integral_constant<int, 4>{});
-        run(integral_constant<int, 8>{}, integral_constant<int, 4>{});
-        run(integral_constant<int, 8>{}, integral_constant<int, 6>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 4>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 8>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 14>{});
+        run(integral_constant<int, 4>{}, integral_constant<int, 4>{}, false_type{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, false_type{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 6>{}, false_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 4>{}, false_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 8>{}, false_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 14>{}, false_type{});
     } else {  // K = 2048, 4096, 8192, 14336, 1024, 3072
-        run(integral_constant<int, 16>{}, integral_constant<int, 4>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 8>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 16>{});
-        run(integral_constant<int, 16>{}, integral_constant<int, 28>{});
-        run(integral_constant<int, 8>{}, integral_constant<int, 4>{});
-        run(integral_constant<int, 8>{}, integral_constant<int, 12>{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 4>{}, true_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 8>{}, true_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 16>{}, false_type{});
+        run(integral_constant<int, 16>{}, integral_constant<int, 28>{}, false_type{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, true_type{});
+        run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, true_type{});
     }
     return ok ? name : nullptr;
 }
