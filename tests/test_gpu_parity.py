@@ -1155,6 +1155,9 @@ def test_exact_fit_gemv(oracle, k, group, instance, bits):
     groups = (k + group - 1) // group
     try:
         for rows in (1, 2, 4, 5, 8, 9, 16, 32):
+            if k == 3072 and bits == 8:  # two instances: eight waves of twelve blocks up to eight rows, then twelve of eight
+                instance = "fit8x12" if rows <= 8 else "fit12x8"
+                waves = int(instance[3:].split("x")[0])
             # (the products of every group, the waves' scales and, for few rows, their activation slices share LDS)
             fixed = groups * rows * 128 + waves * (groups // waves * 32 + 32) * 4
             if fixed > 156 * 1024:  # (with the activation slices on top, while that stays within 80 KiB)
@@ -1165,6 +1168,12 @@ def test_exact_fit_gemv(oracle, k, group, instance, bits):
             _, want = oracle.packed_linear(x, words, c["scales"], c["bias"], n, group, bits=bits)
             for ctx in (plain, blocked):
                 codes, scales = packed_prepare_i8(ctx, dev(x))
+                if k == 3072 and bits == 8:  # either instance, named in full
+                    for named_instance in ("fit8x12", "fit12x8"):
+                        vx.force_variant("gemv." + named_instance)
+                        st, y = pl.forward_a8(ctx, codes, scales)
+                        ctx.synchronize()
+                        assert st == 0 and same_f32(host(y), want) and ctx.last_variant.endswith(named_instance), (rows, ctx.last_variant)
                 for force in (None, "gemv.fit.lprod", "gemv.fit.rprod", "gemv.nofit"):
                     vx.force_variant(force)
                     st, y = pl.forward_a8(ctx, codes, scales)
@@ -1188,13 +1197,15 @@ def test_exact_fit_gemv(oracle, k, group, instance, bits):
                 plain.synchronize()
                 assert st == 0 and same_f32(host(y), want), (rows, special, force, plain.last_variant)
                 prepared_here = force is None and n >= 6144 and k % (32 if bits == 8 else 64) == 0
+                if k == 3072 and bits == 8:
+                    instance = "fit8x12"
                 assert plain.last_variant.endswith(instance + "-prep") == prepared_here, (rows, force, plain.last_variant)
     finally:
         vx.force_variant(None)
         pl.close(), plain.close(), blocked.close()
 
 
-@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (3072, 128, "fit8x12"),
+@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (3072, 128, "fit12x8"),
                                               (4096, 128, "fit16x8"), (4090, 32, "fit16x8")])
 def test_exact_fit_gemv_shared_panels(oracle, k, group, instance):
     """Few panels: four (N = 1000) or two (N = 4090) workgroups of the straight-line kernel share a panel's

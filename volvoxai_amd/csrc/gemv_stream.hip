@@ -829,6 +829,11 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
         constexpr bool SPLITS = decltype(splits_tag)::value;  // the instance is built for shared panels too
         if constexpr (STEPS % GK == 0) {
             if (taken || a.ksteps != (uint32_t)(W * B)) return;
+            // (an instance named in full, "fit12x8", rules the others out)
+            char id[16];
+            snprintf(id, sizeof id, "fit%dx%d", W, B);
+            if (const char* named = force ? strstr(force, "fit") : nullptr)
+                if (named[3] >= '0' && named[3] <= '9' && strncmp(named, id, strlen(id)) != 0) return;
             // the activation rows go through LDS while two workgroups still fit a compute unit that way
             bool xlds = a.rows <= kFitLdsRows;
             size_t lds = lds_for(W, STEPS, xlds);
@@ -865,6 +870,11 @@ const char* launch_fit_mode(hipStream_t s, const LinearArgs& a, int cu_count, co
         run(integral_constant<int, 16>{}, integral_constant<int, 16>{}, false_type{});
         run(integral_constant<int, 16>{}, integral_constant<int, 28>{}, false_type{});
         run(integral_constant<int, 8>{}, integral_constant<int, 4>{}, true_type{});
+        // K = 3072, measured at N = 1024 (four workgroups a panel) and N = 6144: twelve waves of eight blocks are
+        // faster with shared panels (1 / 32 rows: 3.75 / 5.0 us against 4.1 / 5.9) and with many rows (32 rows at
+        // N = 6144: 7.2 against 10.2 us); eight waves of twelve by 0.1 us with up to eight rows on whole panels
+        if (split == 1u && a.rows <= kFitLdsRows) run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, true_type{});
+        run(integral_constant<int, 12>{}, integral_constant<int, 8>{}, true_type{});
         run(integral_constant<int, 8>{}, integral_constant<int, 12>{}, true_type{});
     }
     return ok ? name : nullptr;
