@@ -1205,8 +1205,9 @@ def test_exact_fit_gemv(oracle, k, group, instance, bits):
         pl.close(), plain.close(), blocked.close()
 
 
-@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (2048, 64, "fit16x4"), (3072, 128, "fit12x8"),
-                                              (4096, 128, "fit16x8"), (4090, 32, "fit16x8")])
+@pytest.mark.parametrize("k,group,instance", [(1024, 128, "fit8x4"), (1024, 32, "fit8x4"), (2048, 64, "fit16x4"), (2048, 32, "fit16x4"),
+                                              (3072, 128, "fit12x8"), (3072, 256, "fit12x8"), (4096, 128, "fit16x8"), (4096, 256, "fit16x8"),
+                                              (4090, 32, "fit16x8")])
 def test_exact_fit_gemv_shared_panels(oracle, k, group, instance):
     """Few panels: four (N = 1000) or two (N = 4090) workgroups of the straight-line kernel share a panel's
     channels -- the decoder's projections at 32 rows.  Rows on both sides of the LDS-copy limit, both places
