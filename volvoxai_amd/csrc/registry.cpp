@@ -30,13 +30,13 @@ const VxHipKernelVariant kVariants[] = {
     {"hip.packed-linear.a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32>|gemm_k64_f32_kernel",
      "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-gt32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300},
-    {"hip.packed-linear.a8-gemv-mfma", 0, kPackedLinear, "gemv_panel_kernel<DequantF32>",
+    {"hip.packed-linear.a8-gemv-mfma", 0, kPackedLinear, "gemv_fit_kernel|gemv_panel_kernel<DequantF32>",
      "hip.packed-linear.w8-dynamic-i8-g32-64-128-256-rows-le32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400},
     {"hip.packed-linear.w4a8-mfma", 0, kPackedLinear, "gemm_mfma_kernel<DequantF32, W4>|gemm_k64_f32_kernel<W4>",
      "hip.packed-linear.w4-dynamic-i8-g32-64-128-256-rows-gt32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.gfx950-mfma-i32-16x16x64-i8,hip.global-load-lds-b128", 300},
-    {"hip.packed-linear.w4a8-gemv-mfma", 0, kPackedLinear, "gemv_panel_kernel<DequantF32, W4>",
+    {"hip.packed-linear.w4a8-gemv-mfma", 0, kPackedLinear, "gemv_fit_kernel<W4>|gemv_panel_kernel<DequantF32, W4>",
      "hip.packed-linear.w4-dynamic-i8-g32-64-128-256-rows-le32",
      "hip.gfx950-mfma-i32-32x32x32-i8,hip.nontemporal-dwordx4", 400},
     {"hip.packed-linear.prepare-i8", 0, kPackedLinear, "prepare_i8_kernel|prepare_i8_rows_kernel",
