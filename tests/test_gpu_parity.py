@@ -471,6 +471,42 @@ def test_rowscale_epilogue_levels_and_divisors(ctx, oracle, s_out_bits, zp_out, 
     lin.close()
 
 
+@pytest.mark.parametrize("zp_out,int_bias", [(0, False), (3, True)])
+def test_streamed_output_stores(ctx, oracle, zp_out, int_bias):
+    """Byte outputs of 12 MiB and more leave the large 16x16x64 tiles through streamed stores, a copy of
+    the straight-line epilogue of its own (both of its levels here): 3072 rows x 4096 channels, exactly the
+    size at which they start, must equal the small tile's plainly stored output everywhere and the
+    oracle's bytes on random sub-blocks."""
+    import volvoxai_amd as vx
+    rows, k, n = 3072, 256, 4096
+    c = cases.rowscale_case(rows, k, n, 91)
+    bias_i32 = np.random.default_rng(6).integers(-3000, 3000, n).astype(np.int32) if int_bias else None
+    lin = vx.QLinear(c["w"], c["scales"], c["zps"], bias_i32, I8)
+    xd, sd, bd = dev(c["x"]), dev(c["row_scales"]), dev(c["bias_f32"])
+    got = {}
+    for force in ("mfma-i8-rowscale.t256x256k64", "mfma-i8-rowscale.t256x128k64", "mfma-i8-rowscale.t128x64"):
+        vx.force_variant(force)
+        try:
+            ok, y = lin.forward_rowscale(ctx, xd, sd, c["s_out"], zp_out, bias_f32=bd)
+            ctx.synchronize()
+        finally:
+            vx.force_variant(None)
+        assert ok == 1 and ("k64" in force) == ("k64" in ctx.last_variant), ctx.last_variant
+        got[force] = host(y)
+    plain = got["mfma-i8-rowscale.t128x64"]
+    assert (got["mfma-i8-rowscale.t256x256k64"] == plain).all() and (got["mfma-i8-rowscale.t256x128k64"] == plain).all()
+    rng = np.random.default_rng(12)
+    for _ in range(3):
+        rs = np.sort(rng.choice(rows, 24, replace=False))
+        cs = np.sort(rng.choice(n, 40, replace=False))
+        ok2, want, _ = oracle.qlinear_rowscale(c["x"][rs], c["w"][cs], c["scales"][cs], c["zps"][cs], c["row_scales"][rs],
+                                               c["s_out"], zp_out, bias_i32=None if bias_i32 is None else bias_i32[cs],
+                                               bias_f32=c["bias_f32"][cs])
+        assert ok2 == 1 and (plain[np.ix_(rs, cs)] == want).all()
+    assert ((plain == 127) | (plain == -128)).mean() < 0.5 and ctx.fault_flags() == 0
+    lin.close()
+
+
 def test_outlier_large_k_config5_reduced_rows(ctx, oracle):
     """K=14336, N=4096 with 1% outlier channels scaled x20 before the dynamic
     per-row quantization; 96 rows here (the oracle is scalar), full K and N."""
