@@ -264,7 +264,7 @@ def region_ms(fn, steps, torch, warmup=5):
 
 
 def bench_other_configs(torch, vx, cases, ctx):
-    """configs[1] at M=4,16, configs[2] at M=512,2048 and configs[4] (M=2048, K=14336, N=4096,
+    """configs[1] at M=4,8,16, configs[2] at M=512,2048 and configs[4] (M=2048, K=14336, N=4096,
     dynamic per-token scales, f32 dequant+bias): time per call with inputs resident."""
     from volvoxai_amd.decoder import pack_w8_words
     from volvoxai_amd.w8a8 import operand_order_codes
@@ -279,7 +279,7 @@ def bench_other_configs(torch, vx, cases, ctx):
     # order), which the GEMV loads as whole cache lines.  The row-major figure stays beside it.
     octx = vx.Context(0, torch.cuda.current_stream())
     octx.set_activation_layout(True)
-    for m in (4, 16):
+    for m in (4, 8, 16):
         a8 = torch.from_numpy(d["a8"][:m]).cuda()
         o8 = torch.from_numpy(operand_order_codes(d["a8"][:m])).cuda()
         ars = torch.from_numpy(d["row_scales"][:m]).cuda()
@@ -307,7 +307,7 @@ def bench_other_configs(torch, vx, cases, ctx):
     # (twelve copies: six of these 29 MB matrices would fit the 256 MB Infinity Cache)
     w4copies = 2 * copies
     pls = [vx.PackedLinear(w4words, d["scales"], d["bias"], Kg, Ng, G, weight_bits=4) for _ in range(w4copies)]
-    for m in (1, 16):
+    for m in (1, 4, 16):
         o8 = torch.from_numpy(operand_order_codes(d["a8"][:m])).cuda()
         ars = torch.from_numpy(d["row_scales"][:m]).cuda()
         y = torch.empty((m, Ng), dtype=torch.float32, device="cuda")
